@@ -1,0 +1,363 @@
+// Context, buffers, argument validation and the small elementwise operators
+// of the C ABI declared in include/leviathan_hip.h.
+#include "lev_common.hpp"
+
+#include <cmath>
+#include <new>
+
+// ---------------------------------------------------------------------------
+// errors
+// ---------------------------------------------------------------------------
+
+int lev_fail(lev_ctx *ctx, int status, const char *fmt, ...) {
+    if (ctx) {
+        char buf[512];
+        va_list ap;
+        va_start(ap, fmt);
+        vsnprintf(buf, sizeof(buf), fmt, ap);
+        va_end(ap);
+        ctx->last_error = buf;
+    }
+    return status;
+}
+
+int lev_hip_check(lev_ctx *ctx, hipError_t err, const char *what) {
+    if (err == hipSuccess) return LEV_OK;
+    return lev_fail(ctx, LEV_ERR_COMMAND_FAILED, "%s: %s", what, hipGetErrorString(err));
+}
+
+void *lev_scratch(lev_ctx *ctx, size_t bytes) {
+    if (bytes <= ctx->scratch_bytes) return ctx->scratch;
+    // Growing replaces the buffer; earlier kernels on the stream may still be
+    // using the old one, so drain the stream first.
+    if (ctx->scratch) {
+        if (hipStreamSynchronize(ctx->stream) != hipSuccess) return nullptr;
+        (void)hipFree(ctx->scratch);
+        ctx->scratch = nullptr;
+        ctx->scratch_bytes = 0;
+    }
+    size_t want = (bytes + 0xFFFFFu) & ~(size_t)0xFFFFFu;
+    void *p = nullptr;
+    if (hipMalloc(&p, want) != hipSuccess) return nullptr;
+    ctx->scratch = p;
+    ctx->scratch_bytes = want;
+    return p;
+}
+
+extern "C" int lev_hip_abi_version(void) { return 1; }
+
+extern "C" const char *lev_hip_status_name(int status) {
+    switch (status) {
+        case LEV_OK: return "ok";
+        case LEV_ERR_BAD_DIMENSIONS: return "badDimensions";
+        case LEV_ERR_WRONG_INPUT_COUNT: return "wrongInputCount";
+        case LEV_ERR_NON_FINITE_INPUT: return "nonFiniteInput";
+        case LEV_ERR_NON_FINITE_SCALE: return "nonFiniteScale";
+        case LEV_ERR_NON_FINITE_OUTPUT: return "nonFiniteOutput";
+        case LEV_ERR_EXCEEDS_MODEL_WORKLOAD: return "exceedsModelWorkload";
+        case LEV_ERR_INTEGER_OVERFLOW: return "integerOverflow";
+        case LEV_ERR_DEVICE_UNAVAILABLE: return "deviceUnavailable";
+        case LEV_ERR_KERNEL_LOAD_FAILED: return "kernelLoadFailed";
+        case LEV_ERR_FUNCTION_MISSING: return "functionMissing";
+        case LEV_ERR_COMMAND_FAILED: return "commandFailed";
+        case LEV_ERR_EXCEEDS_MAX_BUFFER_LENGTH: return "exceedsMaxBufferLength";
+        case LEV_ERR_EXCEEDS_WORKING_SET: return "exceedsWorkingSet";
+        case LEV_ERR_INVALID_ARGUMENT: return "invalidArgument";
+        default: return "unknown";
+    }
+}
+
+// ---------------------------------------------------------------------------
+// context + buffers
+// ---------------------------------------------------------------------------
+
+extern "C" int lev_hip_ctx_create(int device, void *stream, lev_ctx **out) {
+    if (!out) return LEV_ERR_INVALID_ARGUMENT;
+    *out = nullptr;
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess || count <= 0 || device < 0 || device >= count)
+        return LEV_ERR_DEVICE_UNAVAILABLE;
+    if (hipSetDevice(device) != hipSuccess) return LEV_ERR_DEVICE_UNAVAILABLE;
+    lev_ctx *ctx = new (std::nothrow) lev_ctx();
+    if (!ctx) return LEV_ERR_DEVICE_UNAVAILABLE;
+    ctx->device = device;
+    if (hipGetDeviceProperties(&ctx->props, device) != hipSuccess) {
+        delete ctx;
+        return LEV_ERR_DEVICE_UNAVAILABLE;
+    }
+    // This library carries gfx950 code objects only.
+    if (std::strncmp(ctx->props.gcnArchName, "gfx950", 6) != 0) {
+        delete ctx;
+        return LEV_ERR_KERNEL_LOAD_FAILED;
+    }
+    ctx->num_cus = ctx->props.multiProcessorCount;
+    if (stream != LEV_HIP_OWN_STREAM) {
+        ctx->stream = static_cast<hipStream_t>(stream);
+    } else {
+        if (hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking) != hipSuccess) {
+            delete ctx;
+            return LEV_ERR_DEVICE_UNAVAILABLE;
+        }
+        ctx->owns_stream = true;
+    }
+    if (hipMalloc(reinterpret_cast<void **>(&ctx->d_flag), sizeof(int)) != hipSuccess ||
+        hipHostMalloc(reinterpret_cast<void **>(&ctx->h_flag), sizeof(int), hipHostMallocDefault) !=
+            hipSuccess ||
+        hipMemset(ctx->d_flag, 0, sizeof(int)) != hipSuccess) {
+        lev_hip_ctx_destroy(ctx);
+        return LEV_ERR_DEVICE_UNAVAILABLE;
+    }
+    *ctx->h_flag = 0;
+    *out = ctx;
+    return LEV_OK;
+}
+
+extern "C" int lev_hip_ctx_destroy(lev_ctx *ctx) {
+    if (!ctx) return LEV_OK;
+    (void)hipSetDevice(ctx->device);
+    if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
+    if (ctx->scratch) (void)hipFree(ctx->scratch);
+    if (ctx->d_flag) (void)hipFree(ctx->d_flag);
+    if (ctx->h_flag) (void)hipHostFree(ctx->h_flag);
+    if (ctx->owns_stream && ctx->stream) (void)hipStreamDestroy(ctx->stream);
+    delete ctx;
+    return LEV_OK;
+}
+
+extern "C" int lev_hip_sync(lev_ctx *ctx) {
+    LEV_REQUIRE_CTX(ctx);
+    LEV_HIP(ctx, hipMemcpyAsync(ctx->h_flag, ctx->d_flag, sizeof(int), hipMemcpyDeviceToHost,
+                                ctx->stream));
+    LEV_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    if (*ctx->h_flag != 0) {
+        int flag = *ctx->h_flag;
+        *ctx->h_flag = 0;
+        LEV_HIP(ctx, hipMemsetAsync(ctx->d_flag, 0, sizeof(int), ctx->stream));
+        LEV_HIP(ctx, hipStreamSynchronize(ctx->stream));
+        return lev_fail(ctx, LEV_ERR_BAD_DIMENSIONS,
+                        "a kernel rejected device-resident arguments (code %d: expert ids must be "
+                        "distinct and below the expert count)",
+                        flag);
+    }
+    return LEV_OK;
+}
+
+extern "C" const char *lev_hip_last_error(lev_ctx *ctx) {
+    return ctx ? ctx->last_error.c_str() : "null context";
+}
+
+extern "C" int lev_hip_device_name(lev_ctx *ctx, char *out, size_t cap) {
+    LEV_REQUIRE_CTX(ctx);
+    if (!out || cap == 0) return LEV_ERR_INVALID_ARGUMENT;
+    std::snprintf(out, cap, "%s (%s)", ctx->props.name, ctx->props.gcnArchName);
+    return LEV_OK;
+}
+
+extern "C" int lev_hip_buf_alloc(lev_ctx *ctx, size_t bytes, void **d_out) {
+    LEV_REQUIRE_CTX(ctx);
+    if (!d_out) return LEV_ERR_INVALID_ARGUMENT;
+    *d_out = nullptr;
+    if (bytes == 0) return lev_fail(ctx, LEV_ERR_BAD_DIMENSIONS, "buf_alloc of 0 bytes");
+    if (bytes > ctx->props.totalGlobalMem)
+        return lev_fail(ctx, LEV_ERR_EXCEEDS_MAX_BUFFER_LENGTH, "buf_alloc %zu bytes > device %zu",
+                        bytes, (size_t)ctx->props.totalGlobalMem);
+    hipError_t e = hipMalloc(d_out, bytes);
+    if (e == hipErrorOutOfMemory)
+        return lev_fail(ctx, LEV_ERR_EXCEEDS_WORKING_SET, "buf_alloc %zu bytes: out of memory", bytes);
+    return lev_hip_check(ctx, e, "hipMalloc");
+}
+
+extern "C" int lev_hip_buf_free(lev_ctx *ctx, void *d_ptr) {
+    LEV_REQUIRE_CTX(ctx);
+    if (!d_ptr) return LEV_OK;
+    LEV_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    return lev_hip_check(ctx, hipFree(d_ptr), "hipFree");
+}
+
+extern "C" int lev_hip_buf_upload(lev_ctx *ctx, void *d_dst, const void *host_src, size_t bytes) {
+    LEV_REQUIRE_CTX(ctx);
+    if (!d_dst || !host_src) return LEV_ERR_INVALID_ARGUMENT;
+    LEV_HIP(ctx, hipMemcpyAsync(d_dst, host_src, bytes, hipMemcpyHostToDevice, ctx->stream));
+    return lev_hip_check(ctx, hipStreamSynchronize(ctx->stream), "upload");
+}
+
+extern "C" int lev_hip_buf_download(lev_ctx *ctx, void *host_dst, const void *d_src, size_t bytes) {
+    LEV_REQUIRE_CTX(ctx);
+    if (!host_dst || !d_src) return LEV_ERR_INVALID_ARGUMENT;
+    LEV_HIP(ctx, hipMemcpyAsync(host_dst, d_src, bytes, hipMemcpyDeviceToHost, ctx->stream));
+    return lev_hip_check(ctx, hipStreamSynchronize(ctx->stream), "download");
+}
+
+// ---------------------------------------------------------------------------
+// shared geometry validation
+// ---------------------------------------------------------------------------
+
+int lev_check_matvec(lev_ctx *ctx, const char *op, uint32_t block_values, uint32_t block_bytes,
+                     const void *d_w, size_t w_bytes, uint64_t w_off, const void *d_x,
+                     size_t x_count, uint64_t x_needed, const void *d_y, size_t y_capacity,
+                     uint64_t y_needed, uint64_t in_dim, uint64_t out_rows, lev_geom *g) {
+    if (!d_w || !d_x || !d_y) return lev_fail(ctx, LEV_ERR_INVALID_ARGUMENT, "%s: null pointer", op);
+    if (in_dim == 0 || out_rows == 0 || in_dim % block_values != 0 ||
+        in_dim > LEV_MAX_Q4_INPUT_DIM || out_rows > LEV_MAX_Q4_OUTPUT_DIM)
+        return lev_fail(ctx, LEV_ERR_BAD_DIMENSIONS, "%s: inDim %llu, outDim %llu", op,
+                        (unsigned long long)in_dim, (unsigned long long)out_rows);
+    g->blocks_per_row = in_dim / block_values;
+    uint64_t row_bytes, weight_bytes, w_end;
+    if (__builtin_mul_overflow(g->blocks_per_row, (uint64_t)block_bytes, &row_bytes) ||
+        __builtin_mul_overflow(out_rows, row_bytes, &weight_bytes) ||
+        __builtin_add_overflow(w_off, weight_bytes, &w_end))
+        return lev_fail(ctx, LEV_ERR_INTEGER_OVERFLOW, "%s: weight extent overflows", op);
+    if (weight_bytes > LEV_MAX_Q4_WEIGHT_BYTES)
+        return lev_fail(ctx, LEV_ERR_EXCEEDS_MODEL_WORKLOAD, "%s: %llu weight bytes", op,
+                        (unsigned long long)weight_bytes);
+    if (w_end > w_bytes)
+        return lev_fail(ctx, LEV_ERR_BAD_DIMENSIONS,
+                        "%s: weight bytes [%llu, %llu) beyond buffer extent %zu", op,
+                        (unsigned long long)w_off, (unsigned long long)w_end, w_bytes);
+    if (x_count != x_needed)
+        return lev_fail(ctx, LEV_ERR_WRONG_INPUT_COUNT, "%s: input %zu, expected %llu", op, x_count,
+                        (unsigned long long)x_needed);
+    if (y_capacity < y_needed)
+        return lev_fail(ctx, LEV_ERR_BAD_DIMENSIONS, "%s: y holds %zu floats, needs %llu", op,
+                        y_capacity, (unsigned long long)y_needed);
+    g->row_bytes = row_bytes;
+    g->weight_bytes = weight_bytes;
+    return LEV_OK;
+}
+
+// ---------------------------------------------------------------------------
+// elementwise operators
+// ---------------------------------------------------------------------------
+
+namespace {
+
+// One workgroup per vector.  Sum of squares in f32 per lane (strided), wave
+// DPP sums, f64 across waves; y = x * inv * w.
+__global__ void __launch_bounds__(256)
+rmsnorm_kernel(const float *__restrict__ x, float *__restrict__ y, const float *__restrict__ w,
+               uint32_t n, float eps) {
+    __shared__ float part[4];
+    const float *xv = x + (uint64_t)blockIdx.x * n;
+    float *yv = y + (uint64_t)blockIdx.x * n;
+    float ss = 0.f;
+    for (uint32_t i = threadIdx.x; i < n; i += 256) {
+        float v = xv[i];
+        ss = fmaf(v, v, ss);
+    }
+    ss = lev_wave_sum_broadcast(ss);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    double tot = ((double)part[0] + (double)part[1]) + ((double)part[2] + (double)part[3]);
+    float inv = (float)(1.0 / sqrt(tot / (double)n + (double)eps));
+    for (uint32_t i = threadIdx.x; i < n; i += 256) {
+        float v = xv[i] * inv;
+        yv[i] = w ? v * w[i] : v;
+    }
+}
+
+__global__ void __launch_bounds__(256)
+gelu_up_kernel(const float *__restrict__ gu, float *__restrict__ y, uint32_t n) {
+    uint32_t i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n) y[i] = lev_gelu_up_value(gu[i], gu[n + i]);
+}
+
+__global__ void __launch_bounds__(256)
+axpy_kernel(const float *__restrict__ x, float *__restrict__ y, float c, uint32_t n) {
+    uint32_t i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n) y[i] = fmaf(c, x[i], y[i]);
+}
+
+__global__ void __launch_bounds__(256)
+f32_to_f16_kernel(const float *__restrict__ x, uint16_t *__restrict__ out, size_t n) {
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) out[i] = __builtin_bit_cast(uint16_t, (_Float16)x[i]);
+}
+
+}  // namespace
+
+extern "C" int lev_hip_rmsnorm(lev_ctx *ctx, const float *d_x, float *d_y, uint32_t n,
+                               uint32_t vectors, const float *d_weight, float eps) {
+    LEV_REQUIRE_CTX(ctx);
+    if (!d_x || !d_y) return lev_fail(ctx, LEV_ERR_INVALID_ARGUMENT, "rmsnorm: null pointer");
+    if (n == 0 || vectors == 0 || !(eps >= 0.f))
+        return lev_fail(ctx, LEV_ERR_BAD_DIMENSIONS, "rmsnorm: n %u, vectors %u, eps %g", n, vectors,
+                        (double)eps);
+    hipLaunchKernelGGL(rmsnorm_kernel, dim3(vectors), dim3(256), 0, ctx->stream, d_x, d_y, d_weight,
+                       n, eps);
+    return lev_hip_check(ctx, hipGetLastError(), "rmsnorm launch");
+}
+
+extern "C" int lev_hip_gelu_up(lev_ctx *ctx, const float *d_gu, float *d_y, uint32_t n) {
+    LEV_REQUIRE_CTX(ctx);
+    if (!d_gu || !d_y) return lev_fail(ctx, LEV_ERR_INVALID_ARGUMENT, "gelu_up: null pointer");
+    if (n == 0) return lev_fail(ctx, LEV_ERR_BAD_DIMENSIONS, "gelu_up: n 0");
+    hipLaunchKernelGGL(gelu_up_kernel, dim3((n + 255) / 256), dim3(256), 0, ctx->stream, d_gu, d_y, n);
+    return lev_hip_check(ctx, hipGetLastError(), "gelu_up launch");
+}
+
+extern "C" int lev_hip_axpy(lev_ctx *ctx, const float *d_x, float *d_y, float c, uint32_t n) {
+    LEV_REQUIRE_CTX(ctx);
+    if (!d_x || !d_y) return lev_fail(ctx, LEV_ERR_INVALID_ARGUMENT, "axpy: null pointer");
+    if (n == 0) return lev_fail(ctx, LEV_ERR_BAD_DIMENSIONS, "axpy: n 0");
+    if (!std::isfinite(c)) return lev_fail(ctx, LEV_ERR_NON_FINITE_INPUT, "axpy: coefficient");
+    hipLaunchKernelGGL(axpy_kernel, dim3((n + 255) / 256), dim3(256), 0, ctx->stream, d_x, d_y, c, n);
+    return lev_hip_check(ctx, hipGetLastError(), "axpy launch");
+}
+
+extern "C" int lev_hip_f32_to_f16(lev_ctx *ctx, const float *d_x, uint16_t *d_out, size_t n) {
+    LEV_REQUIRE_CTX(ctx);
+    if (!d_x || !d_out) return lev_fail(ctx, LEV_ERR_INVALID_ARGUMENT, "f32_to_f16: null pointer");
+    if (n == 0 || n > ((size_t)1 << 40)) return lev_fail(ctx, LEV_ERR_BAD_DIMENSIONS, "f32_to_f16: n");
+    hipLaunchKernelGGL(f32_to_f16_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
+                       ctx->stream, d_x, d_out, n);
+    return lev_hip_check(ctx, hipGetLastError(), "f32_to_f16 launch");
+}
+
+// ---------------------------------------------------------------------------
+// streaming-read probe: what a plain 128-bit read loop achieves on this
+// device, stated next to the nominal HBM peak (the reference's `vk-bw`
+// command, rust/crates/lev-cli/src/main.rs:1876-1935).
+// ---------------------------------------------------------------------------
+
+namespace {
+
+__global__ void __launch_bounds__(256)
+stream_read_kernel(const lev_u32x4 *__restrict__ src, uint64_t n16, uint32_t *__restrict__ sink) {
+    uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    const uint64_t stride = (uint64_t)gridDim.x * 256;
+    lev_u32x4 a = {0, 0, 0, 0}, b = {0, 0, 0, 0}, c = {0, 0, 0, 0}, d = {0, 0, 0, 0};
+    for (; i + 3 * stride < n16; i += 4 * stride) {
+        lev_u32x4 v0 = src[i], v1 = src[i + stride], v2 = src[i + 2 * stride],
+                  v3 = src[i + 3 * stride];
+        a ^= v0;
+        b ^= v1;
+        c ^= v2;
+        d ^= v3;
+    }
+    for (; i < n16; i += stride) a ^= src[i];
+    a ^= b ^ c ^ d;
+    uint32_t r = a.x ^ a.y ^ a.z ^ a.w;
+    if (r == 0x9E3779B9u) sink[0] = r;   // practically never: keeps the loads alive
+}
+
+__global__ void empty_kernel() {}
+
+}  // namespace
+
+extern "C" int lev_hip_stream_read_probe(lev_ctx *ctx, const void *d_src, size_t bytes,
+                                         uint32_t *d_sink, uint32_t workgroups) {
+    LEV_REQUIRE_CTX(ctx);
+    if (!d_src || !d_sink) return lev_fail(ctx, LEV_ERR_INVALID_ARGUMENT, "probe: null pointer");
+    if (bytes < 16 || (reinterpret_cast<uintptr_t>(d_src) & 15u))
+        return lev_fail(ctx, LEV_ERR_BAD_DIMENSIONS, "probe: needs >= 16 bytes, 16-byte aligned");
+    if (workgroups == 0) workgroups = (uint32_t)ctx->num_cus * 8u;
+    hipLaunchKernelGGL(stream_read_kernel, dim3(workgroups), dim3(256), 0, ctx->stream,
+                       static_cast<const lev_u32x4 *>(d_src), (uint64_t)(bytes / 16), d_sink);
+    return lev_hip_check(ctx, hipGetLastError(), "probe launch");
+}
+
+extern "C" int lev_hip_empty_launch(lev_ctx *ctx) {
+    LEV_REQUIRE_CTX(ctx);
+    hipLaunchKernelGGL(empty_kernel, dim3(1), dim3(64), 0, ctx->stream);
+    return lev_hip_check(ctx, hipGetLastError(), "empty launch");
+}

@@ -1,0 +1,126 @@
+// Shared host + device helpers of the gfx950 quantized-matmul library.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <string>
+
+#include "../../include/leviathan_hip.h"
+
+// ---------------------------------------------------------------------------
+// context
+// ---------------------------------------------------------------------------
+
+struct lev_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    bool owns_stream = false;
+    hipDeviceProp_t props{};
+    int num_cus = 0;
+    std::string last_error;
+    // Engine-owned scratch (the reference sizes its MoE scratch once and keeps
+    // it, Gemma4.swift:2025-2059).  Grown on demand, never shrunk.
+    void *scratch = nullptr;
+    size_t scratch_bytes = 0;
+    // Device-side error flag written by kernels that validate device-resident
+    // arguments (expert ids); read back by lev_hip_sync.
+    int *d_flag = nullptr;
+    int *h_flag = nullptr;   // pinned
+};
+
+int lev_fail(lev_ctx *ctx, int status, const char *fmt, ...);
+int lev_hip_check(lev_ctx *ctx, hipError_t err, const char *what);
+// Returns device scratch of at least `bytes` (256-byte aligned) or nullptr.
+void *lev_scratch(lev_ctx *ctx, size_t bytes);
+
+#define LEV_REQUIRE_CTX(ctx)                         \
+    do {                                             \
+        if (!(ctx)) return LEV_ERR_INVALID_ARGUMENT; \
+    } while (0)
+
+#define LEV_HIP(ctx, expr)                                      \
+    do {                                                        \
+        int _st = lev_hip_check((ctx), (expr), #expr);          \
+        if (_st != LEV_OK) return _st;                          \
+    } while (0)
+
+// Geometry shared by every quantized matvec: dims, block multiple, workload
+// caps, weight extent inside [w_off, w_bytes), x count, y capacity.
+// Order of checks follows Q4.swift:168-193 and Gemma4.swift:2599-2627.
+struct lev_geom {
+    uint64_t blocks_per_row;
+    uint64_t row_bytes;
+    uint64_t weight_bytes;
+};
+int lev_check_matvec(lev_ctx *ctx, const char *op, uint32_t block_values, uint32_t block_bytes,
+                     const void *d_w, size_t w_bytes, uint64_t w_off, const void *d_x,
+                     size_t x_count, uint64_t x_needed, const void *d_y, size_t y_capacity,
+                     uint64_t y_needed, uint64_t in_dim, uint64_t out_rows, lev_geom *g);
+
+// ---------------------------------------------------------------------------
+// device helpers
+// ---------------------------------------------------------------------------
+
+#define LEV_WAVE 64
+
+typedef uint32_t lev_u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t lev_u32x2 __attribute__((ext_vector_type(2)));
+typedef float lev_f32x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 lev_f16x2 __attribute__((ext_vector_type(2)));
+
+// Loads that only promise the alignment the GGUF block layouts give
+// (Q4_0 and Q6_K blocks are 2-byte aligned; pairs of Q4_0 blocks 4-byte).
+struct __attribute__((packed, aligned(4))) lev_u32x4_a4 { uint32_t v[4]; };
+struct __attribute__((packed, aligned(4))) lev_u32_a4 { uint32_t v; };
+struct __attribute__((packed, aligned(2))) lev_u32_a2 { uint32_t v; };
+struct __attribute__((packed, aligned(2))) lev_u16_a2 { uint16_t v; };
+
+__device__ __forceinline__ float lev_f16_bits_to_f32(uint32_t bits16) {
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)bits16);
+}
+
+// Sum over the 64 lanes of a wave with DPP (no LDS traffic); every lane of
+// the last row-of-16 ends with partial results, lane 63 with the total.
+template <int CTRL, int ROW_MASK = 0xF, bool BOUND = true>
+__device__ __forceinline__ float lev_dpp_add(float v) {
+    int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xF, BOUND);
+    return v + __builtin_bit_cast(float, moved);
+}
+
+// Sum across groups of L consecutive lanes (L a power of two <= 64).  On
+// return lane (group_base + L - 1)... holds no special role: every lane of
+// the group holds the group's sum for L <= 16; for L = 32 / 64 use the value
+// from lane L-1 of the group (highest lane).
+template <int L>
+__device__ __forceinline__ float lev_group_sum(float v) {
+    if (L >= 2) v = lev_dpp_add<0xB1>(v);    // quad_perm [1,0,3,2]
+    if (L >= 4) v = lev_dpp_add<0x4E>(v);    // quad_perm [2,3,0,1]
+    if (L >= 8) v = lev_dpp_add<0x141>(v);   // row_half_mirror
+    if (L >= 16) v = lev_dpp_add<0x140>(v);  // row_mirror
+    if (L >= 32) v = lev_dpp_add<0x142, 0xA, false>(v);  // row_bcast:15 -> rows 1,3
+    if (L >= 64) v = lev_dpp_add<0x143, 0xC, false>(v);  // row_bcast:31 -> rows 2,3
+    return v;
+}
+
+__device__ __forceinline__ float lev_wave_sum_broadcast(float v) {
+    v = lev_group_sum<64>(v);
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+
+// Overflow-safe tanh and gelu_tanh(g)*u exactly as the reference kernels
+// spell them (g4_tanh / g4_gelu_up_value, Gemma4.swift:4364-4377).
+__device__ __forceinline__ float lev_stable_tanh(float x) {
+    float e = __expf(-2.0f * fabsf(x));
+    return copysignf((1.0f - e) / (1.0f + e), x);
+}
+
+__device__ __forceinline__ float lev_gelu_up_value(float g, float u) {
+    float inner = 0.7978845608028654f * (g + 0.044715f * g * g * g);
+    float gelu = 0.5f * g * (1.0f + lev_stable_tanh(inner));
+    return gelu * u;
+}

@@ -1,0 +1,238 @@
+// Q4_0 decode GEMV  y = W x  for gfx950.
+//
+// Stands in for g4_q4_matvec and its tiled / generated variants
+// (Sources/LeviathanCore/Gemma4.swift:3931, 4031; Q4Lowering.swift:541-664).
+//
+// HBM-bound: W is streamed exactly once (18 bytes per 32 weights), x is staged
+// once per workgroup into LDS and then lives in registers.  Mapping:
+//   - a lane owns one PAIR of adjacent blocks (36 B, two dwordx4 + one dword
+//     load), i.e. 64 consecutive activations, for R rows at a time;
+//   - L lanes cover one row (L = next power of two >= pairs per row, <= 64),
+//     so a wave's load instruction reads 64/L consecutive rows = contiguous
+//     bytes;
+//   - all R x 9 dword loads of a wave are issued before the first use, so a
+//     wave keeps R*2304 bytes in flight;
+//   - the L partial sums of a row are combined with DPP adds.
+#include "q4_0_device.hpp"
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWaves = kThreads / LEV_WAVE;
+
+// Resident workgroups per CU the persistent grid is sized for (tunable for
+// experiments through LEV_Q4_WG_PER_CU).
+uint32_t lev_q4_gemv_wg_per_cu() {
+    static uint32_t v = [] {
+        const char *e = getenv("LEV_Q4_WG_PER_CU");
+        int n = e ? atoi(e) : 0;
+        return (uint32_t)(n > 0 && n <= 16 ? n : 4);
+    }();
+    return v;
+}
+
+// Loads the R pairs a lane owns in the tile whose first row is `row0`.
+template <int L, int R>
+__device__ __forceinline__ void load_tile(const uint8_t *__restrict__ w, uint64_t row_bytes,
+                                          uint32_t row0, uint32_t rows, uint32_t p, bool p_ok,
+                                          uint32_t D[R][9]) {
+    constexpr int G = LEV_WAVE / L;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        uint32_t row = row0 + r * G;
+        if (p_ok && row < rows)
+            lev_q4_load_pair(w + row * row_bytes + (uint64_t)p * 36u, D[r]);
+        else
+            lev_q4_zero_pair(D[r]);
+    }
+}
+
+template <int L, int R, bool MULTI>
+__device__ __forceinline__ void finish_tile(const uint8_t *__restrict__ w, uint64_t row_bytes,
+                                            const lev_f32x4 *xs, float *__restrict__ y,
+                                            uint32_t row0, uint32_t rows, uint32_t pairs,
+                                            uint32_t lp, const lev_q4_pair_x &px0,
+                                            const uint32_t D[R][9]) {
+    constexpr int G = LEV_WAVE / L;
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r] = lev_q4_pair_dot(D[r], px0);
+
+    if (MULTI) {
+        // Rows longer than 64 pairs: further column chunks of the same rows.
+        for (uint32_t c = LEV_WAVE; c < pairs; c += LEV_WAVE) {
+            const uint32_t p = c + lp;
+            if (p < pairs) {
+                uint32_t E[R][9];
+                load_tile<L, R>(w, row_bytes, row0, rows, p, true, E);
+                lev_q4_pair_x px;
+                lev_q4_fetch_x(xs, pairs, p, px);
+#pragma unroll
+                for (int r = 0; r < R; ++r) acc[r] += lev_q4_pair_dot(E[r], px);
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        float s = lev_group_sum<L>(acc[r]);
+        uint32_t row = row0 + r * G;
+        if (lp == L - 1 && row < rows) y[row] = s;
+    }
+}
+
+// Persistent workgroups: each walks tiles of kWaves*G*R rows with a stride of
+// gridDim.x tiles, double-buffering the weight registers so that the loads
+// of tile t+1 are in flight while tile t is being multiplied.
+template <int L, int R, bool MULTI>
+__global__ void __launch_bounds__(kThreads)
+q4_0_gemv_pairs(const uint8_t *__restrict__ w, const float *__restrict__ x, float *__restrict__ y,
+                uint32_t pairs, uint32_t rows) {
+    extern __shared__ lev_f32x4 xs[];
+    constexpr int G = LEV_WAVE / L;                 // rows per wave-wide load
+    constexpr uint32_t kRowsPerTile = kWaves * G * R;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & (LEV_WAVE - 1);
+    const uint32_t wave = tid / LEV_WAVE;
+    const uint32_t grp = lane / L;
+    const uint32_t lp = lane % L;
+    const bool p_ok = lp < pairs;
+    const uint64_t row_bytes = (uint64_t)pairs * 36u;
+    const uint32_t in_tile = wave * (G * R) + grp;
+    const uint32_t step = gridDim.x * kRowsPerTile;
+
+    uint32_t base = blockIdx.x * kRowsPerTile;
+    if (base >= rows) return;
+
+    // Activations first (16 KB, L2 hits after the first workgroup), then the
+    // first tile's weights: the activations are staged and fetched while the
+    // weights are still in flight.
+    lev_f32x4 xv[kLevStageSlots];
+    lev_q4_stage_x_load(x, pairs, tid, kThreads, xv);
+    uint32_t Da[R][9], Db[R][9];
+    load_tile<L, R>(w, row_bytes, base + in_tile, rows, lp, p_ok, Da);
+    lev_q4_stage_x_store(x, xs, pairs, tid, kThreads, xv);
+    __syncthreads();
+
+    // Activations of the lane's first pair stay in registers for every tile.
+    lev_q4_pair_x px0;
+    if (p_ok) {
+        lev_q4_fetch_x(xs, pairs, lp, px0);
+    } else {
+#pragma unroll
+        for (int q = 0; q < 16; ++q) px0.xr[q] = lev_f32x4{0.f, 0.f, 0.f, 0.f};
+        px0.sum_a = px0.sum_b = 0.f;
+    }
+
+    while (true) {
+        uint32_t next = base + step;
+        if (next < rows) load_tile<L, R>(w, row_bytes, next + in_tile, rows, lp, p_ok, Db);
+        finish_tile<L, R, MULTI>(w, row_bytes, xs, y, base + in_tile, rows, pairs, lp, px0, Da);
+        if (next >= rows) break;
+        base = next;
+        next = base + step;
+        if (next < rows) load_tile<L, R>(w, row_bytes, next + in_tile, rows, lp, p_ok, Da);
+        finish_tile<L, R, MULTI>(w, row_bytes, xs, y, base + in_tile, rows, pairs, lp, px0, Db);
+        if (next >= rows) break;
+        base = next;
+    }
+}
+
+// Any geometry (odd block counts, rows that are only 2-byte aligned, rows too
+// long for LDS): one wave per row, 16-bit loads, activations from global
+// memory.  Correct everywhere, fast nowhere; the pair kernel covers every
+// shape the models on this path use.
+__global__ void __launch_bounds__(kThreads)
+q4_0_gemv_generic(const uint8_t *__restrict__ w, const float *__restrict__ x,
+                  float *__restrict__ y, uint32_t blocks_per_row, uint32_t rows) {
+    const uint32_t lane = threadIdx.x & (LEV_WAVE - 1);
+    const uint32_t row = blockIdx.x * kWaves + threadIdx.x / LEV_WAVE;
+    if (row >= rows) return;
+    const uint8_t *rp = w + (uint64_t)row * blocks_per_row * 18u;
+    float acc = 0.f;
+    for (uint32_t b = lane; b < blocks_per_row; b += LEV_WAVE) {
+        const uint16_t *h = reinterpret_cast<const uint16_t *>(rp + (uint64_t)b * 18u);
+        float d = lev_f16_bits_to_f32(h[0]);
+        const float *xb = x + (uint64_t)b * 32u;
+        float s = 0.f, xsum = 0.f;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            uint32_t two = h[1 + k];
+            float x0 = xb[2 * k], x1 = xb[2 * k + 1], x2 = xb[16 + 2 * k], x3 = xb[17 + 2 * k];
+            s = fmaf((float)(two & 0xF), x0, s);
+            s = fmaf((float)((two >> 8) & 0xF), x1, s);
+            s = fmaf((float)((two >> 4) & 0xF), x2, s);
+            s = fmaf((float)(two >> 12), x3, s);
+            xsum += (x0 + x1) + (x2 + x3);
+        }
+        acc = fmaf(d, fmaf(-8.0f, xsum, s), acc);
+    }
+    acc = lev_group_sum<64>(acc);
+    if (lane == LEV_WAVE - 1) y[row] = acc;
+}
+
+template <int L, int R, bool MULTI = false>
+hipError_t launch_pairs(lev_ctx *ctx, const uint8_t *w, const float *x, float *y, uint32_t pairs,
+                        uint32_t rows) {
+    constexpr uint32_t rows_per_tile = kWaves * (LEV_WAVE / L) * R;
+    uint32_t blocks = (rows + rows_per_tile - 1) / rows_per_tile;
+    // Persistent grid: as many workgroups as stay resident at once.
+    uint32_t cap = (uint32_t)ctx->num_cus * lev_q4_gemv_wg_per_cu();
+    if (blocks > cap) blocks = cap;
+    size_t lds = (size_t)16 * (pairs + 1) * sizeof(lev_f32x4);
+    if (lds > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&q4_0_gemv_pairs<L, R, MULTI>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+    }
+    hipLaunchKernelGGL((q4_0_gemv_pairs<L, R, MULTI>), dim3(blocks), dim3(kThreads), lds, ctx->stream, w, x,
+                       y, pairs, rows);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+// Enqueue without argument checks (callers validated the geometry).
+hipError_t lev_q4_0_gemv_launch(lev_ctx *ctx, const uint8_t *w, const float *x, float *y,
+                                uint32_t in_dim, uint32_t rows) {
+    const uint32_t nb = in_dim / 32u;
+    const bool pairable = (nb % 2u == 0u) && ((reinterpret_cast<uintptr_t>(w) & 3u) == 0u) &&
+                          (in_dim <= 32768u) && ((reinterpret_cast<uintptr_t>(x) & 15u) == 0u);
+    if (!pairable) {
+        uint32_t blocks = (rows + kWaves - 1) / kWaves;
+        hipLaunchKernelGGL(q4_0_gemv_generic, dim3(blocks), dim3(kThreads), 0, ctx->stream, w, x, y,
+                           nb, rows);
+        return hipGetLastError();
+    }
+    const uint32_t pairs = nb / 2u;
+    if (pairs > 32) {
+        static const int forced = [] {
+            const char *e = getenv("LEV_Q4_R");
+            return e ? atoi(e) : 0;
+        }();
+        if (pairs > 64) return launch_pairs<64, 2, true>(ctx, w, x, y, pairs, rows);
+        int r = forced;
+        // One row per wave and pass measured fastest at 4096 and 32768 rows:
+        // 100 VGPRs leave five waves per SIMD to hide the HBM latency.
+        if (r == 0) r = 1;
+        if (r == 1) return launch_pairs<64, 1>(ctx, w, x, y, pairs, rows);
+        if (r == 2) return launch_pairs<64, 2>(ctx, w, x, y, pairs, rows);
+        return launch_pairs<64, 4>(ctx, w, x, y, pairs, rows);
+    }
+    if (pairs > 16) return launch_pairs<32, 4>(ctx, w, x, y, pairs, rows);
+    if (pairs > 8) return launch_pairs<16, 4>(ctx, w, x, y, pairs, rows);
+    if (pairs > 4) return launch_pairs<8, 4>(ctx, w, x, y, pairs, rows);
+    return launch_pairs<4, 4>(ctx, w, x, y, pairs, rows);
+}
+
+extern "C" int lev_hip_q4_0_gemv(lev_ctx *ctx, const void *d_w, size_t w_bytes, uint64_t w_off,
+                                 const float *d_x, size_t x_count, float *d_y, size_t y_capacity,
+                                 uint32_t in_dim, uint32_t out_rows) {
+    LEV_REQUIRE_CTX(ctx);
+    lev_geom g;
+    int st = lev_check_matvec(ctx, "q4_0_gemv", 32, 18, d_w, w_bytes, w_off, d_x, x_count, in_dim,
+                              d_y, y_capacity, out_rows, in_dim, out_rows, &g);
+    if (st != LEV_OK) return st;
+    const uint8_t *w = static_cast<const uint8_t *>(d_w) + w_off;
+    return lev_hip_check(ctx, lev_q4_0_gemv_launch(ctx, w, d_x, d_y, in_dim, out_rows),
+                         "q4_0_gemv launch");
+}
