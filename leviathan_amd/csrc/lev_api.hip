@@ -44,6 +44,24 @@ void *lev_scratch(lev_ctx *ctx, size_t bytes) {
     return p;
 }
 
+namespace {
+__global__ void __launch_bounds__(256) zero_kernel(uint32_t *p, size_t n) {
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * 256;
+    for (; i < n; i += stride) p[i] = 0u;
+}
+}  // namespace
+
+hipError_t lev_zero_async(lev_ctx *ctx, void *d_ptr, size_t bytes) {
+    size_t n = bytes / 4;
+    if (n == 0) return hipSuccess;
+    unsigned blocks = (unsigned)((n + 255) / 256);
+    if (blocks > 4096u) blocks = 4096u;
+    hipLaunchKernelGGL(zero_kernel, dim3(blocks), dim3(256), 0, ctx->stream,
+                       static_cast<uint32_t *>(d_ptr), n);
+    return hipGetLastError();
+}
+
 extern "C" int lev_hip_abi_version(void) { return 1; }
 
 extern "C" const char *lev_hip_status_name(int status) {
@@ -132,7 +150,7 @@ extern "C" int lev_hip_sync(lev_ctx *ctx) {
     if (*ctx->h_flag != 0) {
         int flag = *ctx->h_flag;
         *ctx->h_flag = 0;
-        LEV_HIP(ctx, hipMemsetAsync(ctx->d_flag, 0, sizeof(int), ctx->stream));
+        LEV_HIP(ctx, lev_zero_async(ctx, ctx->d_flag, sizeof(int)));
         LEV_HIP(ctx, hipStreamSynchronize(ctx->stream));
         return lev_fail(ctx, LEV_ERR_BAD_DIMENSIONS,
                         "a kernel rejected device-resident arguments (code %d: expert ids must be "

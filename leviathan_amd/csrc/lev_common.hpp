@@ -37,6 +37,9 @@ int lev_fail(lev_ctx *ctx, int status, const char *fmt, ...);
 int lev_hip_check(lev_ctx *ctx, hipError_t err, const char *what);
 // Returns device scratch of at least `bytes` (256-byte aligned) or nullptr.
 void *lev_scratch(lev_ctx *ctx, size_t bytes);
+// Zero-fills `bytes` (a multiple of 4) with a small kernel on the context's
+// stream (safe to record into a HIP graph, unlike a memset node).
+hipError_t lev_zero_async(lev_ctx *ctx, void *d_ptr, size_t bytes);
 
 #define LEV_REQUIRE_CTX(ctx)                         \
     do {                                             \

@@ -1,0 +1,422 @@
+"""GPU parity: Q4_0 / Q6_K / Q4_K GEMV kernels against the CPU oracle.
+
+Every call goes through the C ABI (``libleviathan_hip.so`` via ctypes).
+Bars: dequantised weights and argmax bit-exact; outputs within the
+reference's normalised tolerance max|got-ref|/max(1,|ref|) < 1e-4 against the
+FP64 oracle (rust/crates/lev-cli/src/main.rs:12; 1e-5 for the tiled-Q4 shapes of
+Sources/leviathan-tests/main.swift:2503).
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-4
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    from leviathan_amd import ops
+    c = ops.Context(0)
+    yield c
+    c.close()
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def bits(a):
+    return np.ascontiguousarray(a, dtype=np.float32).view(np.uint32)
+
+
+def q4_gemv(ctx, w, x, rows, cols):
+    y = torch.full((rows,), float("nan"), device="cuda")      # NaN-filled output, must be overwritten
+    ctx.q4_0_gemv(dev(w), dev(x), cols, rows, y=y)
+    ctx.sync()
+    return y.cpu().numpy()
+
+
+# ---------------------------------------------------------------- Q4_0 ----
+
+def test_q4_0_dequant_bit_exact(ctx):
+    from leviathan_amd import capi
+    w = O.synth_q4_0(1, 4096 * 8)
+    got = ctx.dequant(capi.TYPE_Q4_0, dev(w), 4096 * 8)
+    ctx.sync()
+    assert np.array_equal(bits(got.cpu().numpy()), bits(O.q4_0_dequant(w)))
+    # the reference's known block (main.swift:706-721)
+    block = np.array([0x00, 0x3C] + list(range(16)), dtype=np.uint8)
+    got = ctx.dequant(capi.TYPE_Q4_0, dev(block), 1).cpu().numpy()
+    assert got.tolist() == [float(l) - 8 for l in range(16)] + [-8.0] * 16
+
+
+def test_q4_0_one_hot_gemv_reproduces_dequantised_weights_bit_exact(ctx):
+    rows, cols = 96, 4096
+    w = O.synth_q4_0(3, rows * cols // 32)
+    dq = O.q4_0_dequant(w).reshape(rows, cols)
+    for j in [0, 1, 15, 16, 31, 32, 63, 64, 100, 2048 + 17, 4095]:
+        x = np.zeros(cols, np.float32)
+        x[j] = 1.0
+        assert np.array_equal(bits(q4_gemv(ctx, w, x, rows, cols)), bits(dq[:, j].copy())), j
+
+
+def test_q4_0_reference_kats(ctx):
+    # 2 x 32 (main.swift:727-737): row 0 = -8*sum(x), row 1 = +8*sum(x)
+    w = np.array([0x00, 0x3C] + [0] * 16 + [0x00, 0xBC] + [0] * 16, dtype=np.uint8)
+    x = O.seeded_input(32, 1, 7)
+    y = q4_gemv(ctx, w, x, 2, 32)
+    sx = float(x.astype(np.float64).sum())
+    assert abs(y[0] + 8 * sx) < 1e-3 and abs(y[1] - 8 * sx) < 1e-3
+    # hand-computed -16 (main.swift:5106-5117)
+    block = np.array([0x00, 0x3C] + [(l | ((16 + l) << 4)) & 0xFF for l in range(16)], dtype=np.uint8)
+    assert q4_gemv(ctx, block, np.ones(32, np.float32), 1, 32)[0] == -16.0
+
+
+def test_q4_0_matches_scalar_oracle_128x256(ctx):
+    """main.swift:748-771: seeds 99 / 101, rel tol 1e-4 against the scalar oracle."""
+    w = H.swift_q4_0_blocks(99, 128 * 8)
+    x = O.seeded_input(256, 1, 101)
+    got = q4_gemv(ctx, w, x, 128, 256)
+    ref = O.q4_0_matvec_ref(w, 128, 256, x)
+    assert np.max(np.abs(got - ref) / np.maximum(1, np.abs(ref))) < TOL
+    assert O.max_rel_err(got, O.q4_0_matvec_f64(w, 128, 256, x)) < TOL
+
+
+@pytest.mark.parametrize("rows,cols", [(35, 128), (1, 32), (7, 64), (9, 96), (16, 704), (33, 2048),
+                                       (64, 2112), (40, 2816), (100, 768), (5, 8192), (3, 12288),
+                                       (1000, 4096), (2, 36864)])
+def test_q4_0_gemv_shapes_vs_fp64(ctx, rows, cols):
+    """Ragged rows, odd block counts (generic path), rows longer than one pass
+    (main.swift:964-985 ragged 35x128; :2381-2530 inDim 32/704/2112/2816)."""
+    rng = O.SplitMix64(0x5A4C4F57 + rows)
+    w = H.swift_synthetic_blocks(rng, rows * cols // 32) if rows * cols <= 1 << 16 \
+        else O.synth_q4_0(rows + cols, rows * cols // 32)
+    x = O.seeded_input(cols, 1, 70004)
+    got = q4_gemv(ctx, w, x, rows, cols)
+    assert O.max_rel_err(got, O.q4_0_matvec_f64(w, rows, cols, x)) < TOL
+
+
+def test_q4_0_mixed_sign_scales_alternating_input(ctx):
+    """main.swift:2381-2530: mixed-sign scales, alternating-sign x, tol 1e-5."""
+    rows, cols = 24, 2816
+    w = O.synth_q4_0(17, rows * cols // 32).reshape(-1, 18).copy()
+    w[1::2, 1] |= 0x80                                           # negate every other block scale
+    x = np.where(np.arange(cols) % 2 == 0, 1.0, -1.0).astype(np.float32) * O.seeded_input(cols, 1, 3)
+    got = q4_gemv(ctx, w.ravel(), x, rows, cols)
+    assert O.max_rel_err(got, O.q4_0_matvec_f64(w.ravel(), rows, cols, x)) < 1e-5
+
+
+def test_q4_0_config1_full_size(ctx):
+    w, x = H.config1()
+    got = q4_gemv(ctx, w, x, 4096, 4096)
+    ref = O.q4_0_matvec_f64(w, 4096, 4096, x)
+    assert O.max_rel_err(got, ref) < TOL
+    # the f32 CPU reference path sits inside the same contract
+    assert O.max_rel_err(O.q4_0_matvec_ref(w, 4096, 4096, x, threads=8), ref) < TOL
+    # linearity at full size: W(2x) == 2 W(x) exactly (power-of-two scaling)
+    assert np.array_equal(bits(q4_gemv(ctx, w, x * 2, 4096, 4096)), bits(got * 2))
+
+
+def test_q4_0_weight_offset_and_repeat_bit_identity(ctx):
+    """extraOffset selects an expert slice (Gemma4.swift:2583-2590); repeated
+    runs are bit-identical (main.swift:9053-9056)."""
+    rows, cols = 64, 2048
+    slices = [O.synth_q4_0(40 + e, rows * cols // 32) for e in range(3)]
+    pool = dev(np.concatenate(slices))
+    x = O.seeded_input(cols, 1, 5)
+    xd = dev(x)
+    for e in range(3):
+        y1 = ctx.q4_0_gemv(pool, xd, cols, rows, w_off=e * slices[0].size)
+        y2 = ctx.q4_0_gemv(pool, xd, cols, rows, w_off=e * slices[0].size)
+        ctx.sync()
+        assert torch.equal(y1, y2)
+        assert O.max_rel_err(y1.cpu().numpy(), O.q4_0_matvec_f64(slices[e], rows, cols, x)) < TOL
+
+
+def test_q4_0_guards_launch_nothing(ctx):
+    """Q4.swift:168-193 / Gemma4.swift:2599-2627: every bad geometry is rejected on the host."""
+    from leviathan_amd import capi
+    from leviathan_amd.ops import LevError
+    w = dev(np.zeros(8 * 18, np.uint8))
+    x = dev(np.zeros(32, np.float32))
+    y = torch.full((8,), 7.0, device="cuda")
+    cases = [
+        (dict(in_dim=33, out_rows=8), capi.BAD_DIMENSIONS),
+        (dict(in_dim=0, out_rows=8), capi.BAD_DIMENSIONS),
+        (dict(in_dim=32, out_rows=0), capi.BAD_DIMENSIONS),
+        (dict(in_dim=32, out_rows=9), capi.BAD_DIMENSIONS),          # weights too short
+        (dict(in_dim=32, out_rows=8, w_off=18), capi.BAD_DIMENSIONS),  # slice past the extent
+        (dict(in_dim=32, out_rows=8, x_count=3), capi.WRONG_INPUT_COUNT),
+    ]
+    for kw, status in cases:
+        with pytest.raises(LevError) as e:
+            ctx.q4_0_gemv(w, x, y=y, **kw)
+        assert e.value.status == status, kw
+    with pytest.raises(LevError) as e:                              # y too small
+        ctx.q4_0_gemv(w, x, 32, 8, y=torch.empty(4, device="cuda"))
+    assert e.value.status == capi.BAD_DIMENSIONS
+    ctx.sync()
+    assert torch.all(y == 7.0)                                      # nothing ran
+
+
+def test_q4_0_matvec_reporting_twin(ctx):
+    """Q4MetalBackend.matvecReporting twin: results, evidence, typed failures
+    (main.swift:762-796)."""
+    from leviathan_amd import capi, ops
+    w = H.swift_q4_0_blocks(99, 128 * 8)
+    x = O.seeded_input(256, 1, 101)
+    y, ev = ops.q4_0_matvec_reporting(w, 128, 256, x)
+    assert y.shape == (128,)
+    assert O.max_rel_err(y, O.q4_0_matvec_f64(w, 128, 256, x)) < TOL
+    assert ev.command_status == b"completed" and ev.device_name and ev.recommended_max_working_set_size > 0
+    assert ev.out_dim == 128 and ev.in_dim == 256
+    nanx = np.zeros(32, np.float32)
+    nanx[1] = np.inf
+    for args, status in [
+        (([], 8, 33, []), capi.BAD_DIMENSIONS),
+        (([], 8, 32, []), capi.BAD_DIMENSIONS),
+        ((np.zeros(8 * 18, np.uint8), 8, 32, [0, 0, 0]), capi.WRONG_INPUT_COUNT),
+        ((np.zeros(8 * 18, np.uint8), 8, 32, nanx), capi.NON_FINITE_INPUT),
+    ]:
+        with pytest.raises(ops.LevError) as e:
+            ops.q4_0_matvec_reporting(*args)
+        assert e.value.status == status
+    # a non-finite fp16 scale surfaces as a non-finite output (Q4.swift:260-268)
+    bad = np.zeros(18, np.uint8)
+    bad[1] = 0x7C
+    with pytest.raises(ops.LevError) as e:
+        ops.q4_0_matvec_reporting(bad, 1, 32, np.ones(32, np.float32))
+    assert e.value.status == capi.NON_FINITE_OUTPUT
+
+
+# ---------------------------------------------------------------- Q6_K ----
+
+def q6_gemv(ctx, w, x, rows, cols, argmax=False):
+    y = torch.full((rows,), float("nan"), device="cuda")
+    out = ctx.q6_k_gemv(dev(w), dev(x), cols, rows, y=y, argmax=argmax)
+    ctx.sync()
+    if argmax:
+        return y.cpu().numpy(), int(out[1].item()), float(out[2].item())
+    return y.cpu().numpy()
+
+
+def test_q6_k_dequant_bit_exact_and_known_levels(ctx):
+    from leviathan_amd import capi
+    w = O.synth_q6_k(2, 2048)
+    got = ctx.dequant(capi.TYPE_Q6_K, dev(w), 2048).cpu().numpy()
+    assert np.array_equal(bits(got), bits(O.q6_k_dequant(w)))
+    block = np.zeros(210, np.uint8)                      # main.swift:998-1018
+    block[208], block[209] = 0x00, 0x3C
+    block[192:208] = 1
+    block[0], block[128] = 0x21, 0x03
+    dq = ctx.dequant(capi.TYPE_Q6_K, dev(block), 1).cpu().numpy()
+    assert (dq[0], dq[32], dq[64], dq[96], dq[1]) == (17, -32, -30, -32, -32)
+    block[193] = 2
+    assert ctx.dequant(capi.TYPE_Q6_K, dev(block), 1).cpu().numpy()[20] == -64
+
+
+def test_q6_k_hand_computed_minus_315(ctx):
+    block, x = H.minus_315_block()
+    assert q6_gemv(ctx, block, x, 1, 256)[0] == -315.0
+    from leviathan_amd import ops
+    y, _ = ops.q6_k_matvec_reporting(block, 1, 256, x)
+    assert y[0] == -315.0
+
+
+def test_q6_k_one_hot_bit_exact(ctx):
+    rows, cols = 40, 4096
+    w = O.synth_q6_k(9, rows * cols // 256)
+    dq = O.q6_k_dequant(w).reshape(rows, cols)
+    for j in [0, 15, 16, 31, 32, 64, 96, 127, 128, 255, 256, 1000, 4095]:
+        x = np.zeros(cols, np.float32)
+        x[j] = 1.0
+        assert np.array_equal(bits(q6_gemv(ctx, w, x, rows, cols)), bits(dq[:, j].copy())), j
+
+
+def test_q6_k_random_64x512_vs_fp64(ctx):
+    """main.swift:1028-1085: seeds 555 / 202."""
+    w = H.swift_q6_k_blocks(555, 64 * 2)
+    x = O.seeded_input(512, 1, 202)
+    got = q6_gemv(ctx, w, x, 64, 512)
+    ref = O.q6_k_matvec_f64(w, 64, 512, x)
+    assert O.max_rel_err(got, ref) < TOL
+    assert O.max_rel_err(O.q6_k_matvec_ref(w, 64, 512, x), ref) < TOL
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 256), (5, 768), (33, 2048), (17, 2816), (21, 4096),
+                                       (6, 5120), (4, 8192), (3, 16384)])
+def test_q6_k_shapes_vs_fp64(ctx, rows, cols):
+    w = O.synth_q6_k(rows * 3 + cols, rows * cols // 256)
+    x = O.seeded_input(cols, 1, 11)
+    assert O.max_rel_err(q6_gemv(ctx, w, x, rows, cols), O.q6_k_matvec_f64(w, rows, cols, x)) < TOL
+
+
+def test_q6_k_saturated_bytes_every_fourth_block(ctx):
+    """main.swift:3865-4040: saturated code bytes in every 4th block."""
+    rows, cols = 12, 2816
+    w = O.synth_q6_k(5, rows * cols // 256).reshape(-1, 210).copy()
+    w[::4, :192] = 0xFF
+    x = O.seeded_input(cols, 1, 13)
+    got = q6_gemv(ctx, w.ravel(), x, rows, cols)
+    assert O.max_rel_err(got, O.q6_k_matvec_f64(w.ravel(), rows, cols, x)) < TOL
+
+
+def test_q6_k_config2_full_size_with_argmax(ctx):
+    w, x = H.config2()
+    got, idx, margin = q6_gemv(ctx, w, x, 32000, 4096, argmax=True)
+    ref64 = O.q6_k_matvec_f64(w, 32000, 4096, x)
+    assert O.max_rel_err(got, ref64) < TOL
+    ref32 = O.q6_k_matvec_ref(w, 32000, 4096, x, threads=8)      # reference CPU path
+    # the comparison is only meaningful if the CPU reference's own top-2 gap
+    # is far above the summation-order noise; assert it, then demand equality
+    cpu_margin = O.top_margin(ref32)
+    assert cpu_margin > 100 * float(np.max(np.abs(got - ref32)))
+    assert idx == O.argmax(ref32)
+    assert idx == O.argmax(got) and margin == O.top_margin(got)   # epilogue is exact on its input
+
+
+def test_argmax_ties_lowest_index_and_columns(ctx):
+    """rust/crates/lev-forge/src/ops.rs:508: lowest index on ties; margin = best - second."""
+    v = np.full((3, 5000), -1.0, np.float32)
+    v[0, [4000, 77, 3000]] = 2.5
+    v[1, 4999] = 9.0
+    v[1, 0] = 8.5
+    v[2] = O.normal(5000, 1)
+    idx, mg = ctx.argmax(dev(v), 5000, 3)
+    ctx.sync()
+    assert idx.cpu().tolist() == [77, 4999, O.argmax(v[2])]
+    assert mg.cpu().tolist() == [0.0, 0.5, O.top_margin(v[2])]
+
+
+# ---------------------------------------------------------------- Q4_K ----
+
+def q4k_gemv(ctx, w, x, rows, cols, ncol, gain=None, eps=1e-6):
+    y = torch.full((ncol, rows), float("nan"), device="cuda")
+    ctx.q4_k_gemv_ncol(dev(w), dev(x), cols, rows, ncol, gain=None if gain is None else dev(gain),
+                       eps=eps, y=y)
+    ctx.sync()
+    return y.cpu().numpy()
+
+
+def test_q4_k_dequant_bit_exact_and_hand_block(ctx):
+    from leviathan_amd import capi
+    w = O.synth_q4_k(3, 2048)
+    got = ctx.dequant(capi.TYPE_Q4_K, dev(w), 2048).cpu().numpy()
+    assert np.array_equal(bits(got), bits(O.q4_k_dequant(w)))
+    block = np.zeros(144, np.uint8)                      # lev-cpu/src/lib.rs:438-464
+    block[0:4] = [0x00, 0x3C, 0x00, 0x38]
+    block[4:16] = O.q4_k_pack_scale_min([1] * 8, [2] * 8)
+    block[16:] = 0x21
+    dq = ctx.dequant(capi.TYPE_Q4_K, dev(block), 1).cpu().numpy().reshape(4, 2, 32)
+    assert np.all(dq[:, 0] == 0.0) and np.all(dq[:, 1] == 1.0)
+
+
+def test_q4_k_one_hot_bit_exact(ctx):
+    rows, cols = 48, 4096
+    w = O.synth_q4_k(21, rows * cols // 256)
+    dq = O.q4_k_dequant(w).reshape(rows, cols)
+    for j in [0, 31, 32, 63, 64, 255, 256, 1234, 4095]:
+        x = np.zeros((1, cols), np.float32)
+        x[0, j] = 1.0
+        assert np.array_equal(bits(q4k_gemv(ctx, w, x, rows, cols, 1)[0]), bits(dq[:, j].copy())), j
+
+
+def test_q4_k_rust_fixture_16x1024(ctx):
+    """lev-cpu/src/lib.rs:466-476: SplitMix64(42), 16 x 1024."""
+    rng = O.SplitMix64(42)
+    w = H.rust_q4_k_blocks(rng, 16 * 4)
+    x = np.array([rng.next_signed_unit() for _ in range(1024)], np.float32)
+    got = q4k_gemv(ctx, w, x[None], 16, 1024, 1)[0]
+    assert O.max_rel_err(got, O.q4_k_matvec_f64(w, 16, 1024, x)) < TOL
+
+
+@pytest.mark.parametrize("ncol", [1, 2, 3, 4, 5, 8, 16])
+@pytest.mark.parametrize("rows,cols", [(37, 1024), (64, 4096), (20, 12288), (9, 256)])
+def test_q4_k_ncol_shapes_with_rmsnorm(ctx, rows, cols, ncol):
+    w, x, gain = H.config3(rows, cols, ncol, seed=rows + ncol)
+    got = q4k_gemv(ctx, w, x, rows, cols, ncol, gain)
+    xn = H.rmsnorm_rows(x, gain)
+    for c in range(ncol):
+        assert O.max_rel_err(got[c], O.q4_k_matvec_f64(w, rows, cols, xn[c])) < TOL, c
+    plain = q4k_gemv(ctx, w, x, rows, cols, ncol)                # no norm
+    for c in range(ncol):
+        assert O.max_rel_err(plain[c], O.q4_k_matvec_f64(w, rows, cols, x[c])) < TOL, c
+
+
+@pytest.mark.parametrize("ncol", [1, 2, 3, 4, 8])
+def test_q4_k_config3_full_size(ctx, ncol):
+    w, x, gain = H.config3(ncol=ncol)
+    got = q4k_gemv(ctx, w, x, 12288, 4096, ncol, gain)
+    xn = H.rmsnorm_rows(x, gain)
+    for c in range(ncol):
+        assert O.max_rel_err(got[c], O.q4_k_matvec_f64(w, 12288, 4096, xn[c])) < TOL, c
+    # columns are independent: column 0 alone gives the same bits
+    alone = q4k_gemv(ctx, w, x[:1], 12288, 4096, 1, gain)
+    if ncol <= 2:
+        assert np.array_equal(bits(alone[0]), bits(got[0]))
+    else:
+        assert O.max_rel_err(alone[0], got[0].astype(np.float64)) < 1e-5
+
+
+def test_q4_k_guards(ctx):
+    from leviathan_amd import capi
+    from leviathan_amd.ops import LevError
+    w = dev(np.zeros(144 * 4, np.uint8))
+    x = dev(np.zeros(2 * 256, np.float32))
+    for kw, status in [
+        (dict(in_dim=100, rows=4, ncol=1), capi.BAD_DIMENSIONS),
+        (dict(in_dim=256, rows=5, ncol=1), capi.BAD_DIMENSIONS),
+        (dict(in_dim=256, rows=4, ncol=3), capi.WRONG_INPUT_COUNT),
+        (dict(in_dim=256, rows=4, ncol=0), capi.BAD_DIMENSIONS),
+        (dict(in_dim=256, rows=4, ncol=17), capi.BAD_DIMENSIONS),
+    ]:
+        with pytest.raises(LevError) as e:
+            ctx.q4_k_gemv_ncol(w, x, **kw)
+        assert e.value.status == status, kw
+
+
+# ---------------------------------------------------------- elementwise ----
+
+def test_rmsnorm_operator(ctx):
+    x = O.normal(3 * 4096, 31).reshape(3, 4096)
+    g = O.normal(4096, 32, 1.0, 0.1)
+    y = ctx.rmsnorm(dev(x), 4096, 3, weight=dev(g)).cpu().numpy()
+    for r in range(3):
+        assert O.max_rel_err(y[r], O.rmsnorm_f64(x[r], g, 1e-6)) < 1e-5
+    y = ctx.rmsnorm(dev(x), 4096, 3).cpu().numpy()              # scale-free (router input)
+    assert O.max_rel_err(y[1], O.rmsnorm_f64(x[1], None, 1e-6)) < 1e-5
+    const = ctx.rmsnorm(dev(np.full(8, 2.0, np.float32)), 8, 1, weight=dev(np.full(8, 0.5, np.float32)))
+    assert np.all(np.abs(const.cpu().numpy() - 0.5) < 1e-5)     # lev-model/src/lib.rs:431-435
+
+
+def test_gelu_up_operator(ctx):
+    """main.swift:6630-6691: bounded, extreme and tail inputs stay finite;
+    main.swift:8947-8950 known values."""
+    n = 4096
+    g = np.array([(i % 97) / 13 - 3 for i in range(n)], np.float32)
+    u = O.seeded_input(n, 1, 9)
+    y = ctx.gelu_up(dev(np.concatenate([g, u])), n).cpu().numpy()
+    ref = np.array([O.gelu_up_f64(float(a), float(b)) for a, b in zip(g, u)])
+    assert O.max_rel_err(y, ref) < 2e-6
+    ext_g = np.array([1e30, -1e30, 1e-30, 0.5, -0.25, 8, -9.5, 1e20, 0, 1, -20], np.float32)
+    ext_u = np.array([1, 1, 2, -0.25, 8, -9.5, 1e20, 0, 0.5, 1, 3], np.float32)
+    y = ctx.gelu_up(dev(np.concatenate([ext_g, ext_u])), ext_g.size).cpu().numpy()
+    assert np.all(np.isfinite(y))
+    assert abs(y[9] - 0.841192) < 1e-6 and y[10] == 0
+
+
+def test_axpy_and_f16_operators(ctx):
+    x = O.seeded_input(1000, 1, 1)
+    y0 = O.seeded_input(1000, 1, 2)
+    y = ctx.axpy(dev(x), dev(y0), 0.37, 1000).cpu().numpy()
+    want = np.float32(0.37) * x.astype(np.float64) + y0
+    assert np.max(np.abs(y - want)) < 1e-6
+    v = np.concatenate([O.normal(5000, 3) * s for s in (1e-7, 1e-3, 1.0, 300.0, 1e5)]).astype(np.float32)
+    h = ctx.f32_to_f16(dev(v)).cpu().numpy()
+    with np.errstate(over="ignore"):
+        assert np.array_equal(h.view(np.uint16), v.astype(np.float16).view(np.uint16))
