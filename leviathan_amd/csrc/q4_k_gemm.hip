@@ -56,21 +56,33 @@ __device__ __forceinline__ void q4k_all_factors(const lev_u32x4 hdr, float d1[8]
     }
 }
 
+// One weight exactly as the reference rounds it: f32(d1*q - mm) first, THEN
+// round-to-nearest-even to fp16 (dequant_block_f32 followed by f32_to_f16_bits,
+// lev-cli/src/main.rs:1201-1217).  The empty asm pins the f32 value in a
+// register so that the compiler cannot merge the multiply-add with the
+// conversion into a single-rounding mixed-precision FMA, which differs from
+// the two-step rounding in about one weight in ten thousand.
+__device__ __forceinline__ _Float16 q4k_weight_f16(float d1, float code, float mm) {
+    float w32 = fmaf(d1, code, -mm);   // d1*code is exact (17 + 4 bits): one rounding, as in the reference
+    asm volatile("" : "+v"(w32));
+    return (_Float16)w32;
+}
+
 // 8 weights (one per code byte of the two dwords, nibble selected by `hi`)
-// -> fp16 B fragment, bit-exact with fp16(f32(d1*q) - mm).
+// -> fp16 B fragment, bit-exact with fp16(f32(d1*q - mm)).
 __device__ __forceinline__ f16x8 q4k_frag(uint32_t q0, uint32_t q1, bool hi, float d1, float mm) {
     uint32_t a = hi ? (q0 >> 4) : q0, b = hi ? (q1 >> 4) : q1;
     a &= 0x0F0F0F0Fu;
     b &= 0x0F0F0F0Fu;
     f16x8 f;
-    f[0] = (_Float16)fmaf(d1, (float)(a & 0xFFu), -mm);
-    f[1] = (_Float16)fmaf(d1, (float)((a >> 8) & 0xFFu), -mm);
-    f[2] = (_Float16)fmaf(d1, (float)((a >> 16) & 0xFFu), -mm);
-    f[3] = (_Float16)fmaf(d1, (float)(a >> 24), -mm);
-    f[4] = (_Float16)fmaf(d1, (float)(b & 0xFFu), -mm);
-    f[5] = (_Float16)fmaf(d1, (float)((b >> 8) & 0xFFu), -mm);
-    f[6] = (_Float16)fmaf(d1, (float)((b >> 16) & 0xFFu), -mm);
-    f[7] = (_Float16)fmaf(d1, (float)(b >> 24), -mm);
+    f[0] = q4k_weight_f16(d1, (float)(a & 0xFFu), mm);
+    f[1] = q4k_weight_f16(d1, (float)((a >> 8) & 0xFFu), mm);
+    f[2] = q4k_weight_f16(d1, (float)((a >> 16) & 0xFFu), mm);
+    f[3] = q4k_weight_f16(d1, (float)(a >> 24), mm);
+    f[4] = q4k_weight_f16(d1, (float)(b & 0xFFu), mm);
+    f[5] = q4k_weight_f16(d1, (float)((b >> 8) & 0xFFu), mm);
+    f[6] = q4k_weight_f16(d1, (float)((b >> 16) & 0xFFu), mm);
+    f[7] = q4k_weight_f16(d1, (float)(b >> 24), mm);
     return f;
 }
 

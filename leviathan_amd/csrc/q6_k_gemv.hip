@@ -58,13 +58,6 @@ __device__ __forceinline__ void q6_load_unit(const uint8_t *row, uint32_t g, q6_
     u.sc[1] = c.v[1];
 }
 
-__device__ __forceinline__ void q6_zero_unit(q6_unit_w &u) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) u.ql[i] = u.qh[i] = 0u;
-    u.sc[0] = u.sc[1] = 0u;
-    u.d = 0u;
-}
-
 // sum_i code_i * x_i over four code bytes packed in `c`, scaled by 2^-24.
 __device__ __forceinline__ float q6_dot4(uint32_t c, lev_f32x4 x, float acc) {
     lev_f16x2 e02 = __builtin_bit_cast(lev_f16x2, c & 0x00FF00FFu);
@@ -92,8 +85,8 @@ __device__ __forceinline__ float q6_unit_dot(const q6_unit_w &u, const q6_unit_x
     }
     // sub-scales: byte (v&1) + 2*pair for the low set, +4 for the high set
     const uint32_t bi = (v & 1u) + 2u * pair;
-    float s_lo = (float)__builtin_amdgcn_sbfe((int)u.sc[0], 8u * bi, 8u);
-    float s_hi = (float)__builtin_amdgcn_sbfe((int)u.sc[1], 8u * bi, 8u);
+    float s_lo = (float)(int)__builtin_amdgcn_sbfe((int)u.sc[0], 8u * bi, 8u);
+    float s_hi = (float)(int)__builtin_amdgcn_sbfe((int)u.sc[1], 8u * bi, 8u);
     float d = lev_f16_bits_to_f32(u.d);
     float t = fmaf(s_lo, fmaf(lo, 16777216.0f, -32.0f * x.sum_lo),
                    s_hi * fmaf(hi, 16777216.0f, -32.0f * x.sum_hi));
