@@ -1,0 +1,329 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X quantized-matmul hot path (one GPU).
+
+``python bench.py [--gpus 1] [--steps K] [--warmup W]`` prints ONE JSON line.
+
+Headline (``metric`` / ``value``): the Q4_0 4096x4096 decode GEMV of
+BASELINE.json, as achieved HBM GB/s = algorithmic bytes of one GEMV
+(weights + x + y = 9,469,952 B) / time of one step.  A step is one GEMV
+launch through the C ABI; successive steps use successive distinct copies of
+the weights out of a 604 MB ring, so every step streams its weights from HBM
+rather than from the 256 MB memory-side cache.  All inputs are resident in HBM
+before the timed region; timing is HIP events on the stream the kernels run on.
+
+The same line carries ``roofline`` (dominant kernel against the 8 TB/s HBM
+peak), ``cpu_baseline`` (the CPU restatement of the reference's path, timed on
+this host's cores on a bounded sample) and ``others`` (the remaining BASELINE
+configurations: Q6_K GEMV + argmax, RMSNorm + Q4_K N-column GEMV, Q4_K prefill
+GEMM on MFMA, MoE layer at T=1 and T=64, plus a plain streaming-read probe).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0                # MI355X published HBM3E peak
+MFMA_F16_PEAK_TFLOPS = 2500.0        # MI355X published dense fp16 / bf16 peak
+
+# HBM bytes per launch of the dominant kernel (q4_0_gemv_pairs<64,1,false>,
+# 4096x4096) from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by the
+# same counter on a plain copy kernel of known size; None until measured.
+MEASURED_TRAFFIC_BYTES = None
+
+
+def parse_args():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=2000)
+    p.add_argument("--warmup", type=int, default=200)
+    p.add_argument("--skip-others", action="store_true", help="headline only")
+    p.add_argument("--skip-cpu", action="store_true", help="no cpu_baseline leg")
+    p.add_argument("--only", default="", help="run one kernel family only (for profiling): "
+                   "q4_0 | q6_k | q4_k | gemm | moe1 | moe64 | copy")
+    return p.parse_args()
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this build runs on ONE GPU (got --gpus {args.gpus}); "
+              "multi-GPU sharding is described in DESIGN.md and not built.", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    from leviathan_amd import capi, ops          # raises if the HIP library is missing
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; there is no CPU path to measure.", file=sys.stderr)
+        sys.exit(2)
+    torch.cuda.set_device(0)
+    ctx = ops.Context(0)
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(1)
+
+    def timed(fn, steps, warmup):
+        """ms per call: `warmup` untimed calls, then exactly `steps` calls between
+        two HIP events on the launch stream, synchronised on both sides."""
+        for i in range(warmup):
+            fn(i)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(steps):
+            fn(warmup + i)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / steps
+
+    def rand_bytes(n):
+        return torch.randint(0, 256, (n,), dtype=torch.uint8, device=dev, generator=gen)
+
+    def half_scales(n, sigma):
+        s = (torch.randn(n, device=dev, generator=gen) * sigma).abs().to(torch.float16)
+        return s.view(torch.uint8).reshape(n, 2)
+
+    # ---- synthetic weights with the BASELINE distributions, built on the GPU ----
+    def make_q4_0(nblocks, sigma=0.02):
+        w = rand_bytes(nblocks * 18).reshape(nblocks, 18)
+        w[:, 0:2] = half_scales(nblocks, sigma)
+        return w.reshape(-1)
+
+    def make_q6_k(nblocks, sigma=0.01):
+        w = rand_bytes(nblocks * 210).reshape(nblocks, 210)
+        sc = torch.randint(-32, 32, (nblocks, 16), dtype=torch.int8, device=dev, generator=gen)
+        w[:, 192:208] = sc.view(torch.uint8)
+        w[:, 208:210] = half_scales(nblocks, sigma)
+        return w.reshape(-1)
+
+    def make_q4_k(nblocks, sigma=0.01):
+        w = rand_bytes(nblocks * 144).reshape(nblocks, 144)
+        w[:, 0:2] = half_scales(nblocks, sigma)
+        w[:, 2:4] = half_scales(nblocks, sigma)
+        return w.reshape(-1)
+
+    result = {}
+    others = {}
+    only = args.only
+
+    # ------------------------------------------------------------------ Q4_0
+    rows = cols = 4096
+    q4_bytes_w = rows * cols // 32 * 18
+    q4_alg_bytes = q4_bytes_w + cols * 4 + rows * 4            # 9,469,952
+    if only in ("", "q4_0"):
+        ncopy = 64                                             # 604 MB ring > 256 MB cache
+        ring = make_q4_0(ncopy * rows * cols // 32)
+        x = torch.randn(cols, device=dev, generator=gen)
+        y = torch.empty(rows, device=dev)
+        lib, c = ctx.lib, ctx.ctx
+        wp, wn, xp, yp = ring.data_ptr(), ring.numel(), x.data_ptr(), y.data_ptr()
+
+        def q4_step(i):
+            st = lib.lev_hip_q4_0_gemv(c, wp, wn, (i % ncopy) * q4_bytes_w, xp, cols, yp, rows, cols, rows)
+            if st:
+                raise RuntimeError(lib.lev_hip_last_error(c).decode())
+
+        ms = timed(q4_step, args.steps, args.warmup)
+        gbs = q4_alg_bytes / (ms * 1e-3) / 1e9
+        result.update(ms_per_step=ms, value=gbs)
+        # correctness of what was just timed, against the CPU restatement
+        check = {}
+        if not args.skip_cpu:
+            import oracle as O                                  # cpu_baseline leg only
+            q4_step(0)
+            torch.cuda.synchronize()
+            w0 = ring[:q4_bytes_w].cpu().numpy()
+            xh = x.cpu().numpy()
+            ref64 = O.q4_0_matvec_f64(w0, rows, cols, xh)
+            check["max_rel_err_vs_fp64"] = O.max_rel_err(y.cpu().numpy(), ref64)
+            ncores = os.cpu_count() or 1
+            threads = min(ncores, 64)
+
+            def cpu_rate(nthreads, budget_s):
+                n, t0 = 0, time.perf_counter()
+                while True:
+                    O.q4_0_matvec_ref(w0, rows, cols, xh, threads=nthreads)
+                    n += 1
+                    dt = time.perf_counter() - t0
+                    if dt >= budget_s:
+                        return n, q4_alg_bytes * n / dt / 1e9
+            n1, gbs1 = cpu_rate(0, 6.0)
+            nmt, gbsmt = cpu_rate(threads, 8.0)
+            result["cpu_baseline"] = {
+                "value": gbsmt, "unit": "GB/s", "cores": threads, "kind": "port",
+                "sample": f"{nmt} Q4_0 4096x4096 GEMVs, rows split over {threads} threads "
+                          f"(C restatement of Q4_0.matvecReference, gcc -O2, no FMA contraction)",
+                "single_thread": {"value": gbs1, "unit": "GB/s", "cores": 1, "sample": f"{n1} GEMVs"},
+            }
+        result["check"] = check
+        del ring
+
+    def run_other(name, fn, alg_bytes, steps, warmup, extra=None):
+        ms = timed(fn, steps, warmup)
+        entry = {"us_per_launch": ms * 1e3, "algorithmic_bytes": alg_bytes,
+                 "achieved_GBps": alg_bytes / (ms * 1e-3) / 1e9,
+                 "frac_of_hbm_peak": alg_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+        if extra:
+            entry.update(extra(ms))
+        others[name] = entry
+
+    lib, c = ctx.lib, ctx.ctx
+
+    def must(st):
+        if st:
+            raise RuntimeError(lib.lev_hip_last_error(c).decode())
+
+    if not args.skip_others or only:
+        # ---------------------------------------------------- streaming probe
+        if only in ("", "copy"):
+            buf = rand_bytes(1 << 30)
+            sink = torch.zeros(4, dtype=torch.int32, device=dev)
+            for nbytes, label in ((q4_bytes_w, "stream_read_9MiB_same_buffer"), (1 << 30, "stream_read_1GiB")):
+                run_other(label, lambda i: must(lib.lev_hip_stream_read_probe(
+                    c, buf.data_ptr(), nbytes, sink.data_ptr(), 512)), nbytes, 50, 10)
+            run_other("empty_kernel_launch", lambda i: must(lib.lev_hip_empty_launch(c)), 0, 1000, 100)
+            del buf
+
+        # ---------------------------------------------- Q4_0 large streaming
+        if only in ("", "q4_0"):
+            rows2 = 32768
+            nb2 = rows2 * cols // 32
+            ring2 = make_q4_0(8 * nb2)
+            x = torch.randn(cols, device=dev, generator=gen)
+            y2 = torch.empty(rows2, device=dev)
+            run_other("q4_0_gemv_32768x4096", lambda i: must(lib.lev_hip_q4_0_gemv(
+                c, ring2.data_ptr(), ring2.numel(), (i % 8) * nb2 * 18, x.data_ptr(), cols,
+                y2.data_ptr(), rows2, cols, rows2)), nb2 * 18 + cols * 4 + rows2 * 4, 100, 20)
+            del ring2
+
+        # ------------------------------------------------------ Q6_K + argmax
+        if only in ("", "q6_k"):
+            r6, nb6 = 32000, 32000 * 4096 // 256
+            ring6 = make_q6_k(6 * nb6)
+            x = torch.randn(cols, device=dev, generator=gen)
+            y6 = torch.empty(r6, device=dev)
+            idx = torch.empty(1, dtype=torch.int32, device=dev)
+            mg = torch.empty(1, device=dev)
+            run_other("q6_k_gemv_32000x4096_argmax", lambda i: must(lib.lev_hip_q6_k_gemv(
+                c, ring6.data_ptr(), ring6.numel(), (i % 6) * nb6 * 210, x.data_ptr(), cols,
+                y6.data_ptr(), r6, cols, r6, idx.data_ptr(), mg.data_ptr())),
+                nb6 * 210 + cols * 4 + r6 * 4 + 8, 100, 20)
+            run_other("q6_k_gemv_32000x4096_no_argmax", lambda i: must(lib.lev_hip_q6_k_gemv(
+                c, ring6.data_ptr(), ring6.numel(), (i % 6) * nb6 * 210, x.data_ptr(), cols,
+                y6.data_ptr(), r6, cols, r6, None, None)), nb6 * 210 + cols * 4 + r6 * 4, 100, 20)
+            del ring6
+
+        # ------------------------------------------- RMSNorm + Q4_K N columns
+        if only in ("", "q4_k", "gemm"):
+            r4, nb4 = 12288, 12288 * 4096 // 256
+            ncopy4 = 20
+            ring4 = make_q4_k(ncopy4 * nb4)
+        if only in ("", "q4_k"):
+            gain = 1.0 + 0.1 * torch.randn(cols, device=dev, generator=gen)
+            for n in (1, 2, 3, 4, 8):
+                xn = torch.randn(n, cols, device=dev, generator=gen)
+                yn = torch.empty(n, r4, device=dev)
+                run_other(f"rmsnorm_q4_k_gemv_12288x4096_N{n}", lambda i: must(lib.lev_hip_q4_k_gemv_ncol(
+                    c, ring4.data_ptr(), ring4.numel(), (i % ncopy4) * nb4 * 144, xn.data_ptr(),
+                    xn.numel(), gain.data_ptr(), 1e-6, yn.data_ptr(), yn.numel(), cols, r4, n)),
+                    nb4 * 144 + cols * 4 + n * (cols * 4 + r4 * 4), 200, 20)
+
+        # --------------------------------------------------- Q4_K prefill GEMM
+        if only in ("", "gemm"):
+            tokens = 512
+            xh = torch.randn(tokens, cols, device=dev, generator=gen).to(torch.float16)
+            yg = torch.empty(tokens, r4, device=dev)
+            flop = 2.0 * tokens * r4 * cols
+
+            def gemm_extra(ms):
+                tf = flop / (ms * 1e-3) / 1e12
+                return {"TFLOPs": tf, "mfma_frac_of_fp16_peak": tf / MFMA_F16_PEAK_TFLOPS,
+                        "bound": "mfma"}
+            run_other("q4_k_prefill_gemm_512x12288x4096", lambda i: must(lib.lev_hip_q4_k_gemm_prefill(
+                c, ring4.data_ptr(), ring4.numel(), (i % ncopy4) * nb4 * 144, xh.data_ptr(), xh.numel(),
+                yg.data_ptr(), yg.numel(), cols, r4, tokens)),
+                nb4 * 144 + tokens * cols * 2 + tokens * r4 * 4, 30, 5, gemm_extra)
+        if only in ("", "q4_k", "gemm"):
+            del ring4
+
+        # ------------------------------------------------------------- MoE
+        if only in ("", "moe1", "moe64"):
+            hidden, inter, experts, top_k = 2048, 768, 128, 8
+            gu = inter * (hidden // 32) * 18
+            dn = hidden * (inter // 32) * 18
+            npool = 2                                           # two distinct 340 MB pools
+            pools_t = [make_q4_0(experts * (2 * gu + dn) // 18) for _ in range(npool)]
+            wr = 0.02 * torch.randn(experts, hidden, device=dev, generator=gen)
+            pools = [ops.Context.moe_pools(p, hidden, inter, experts, 0, experts * gu, 2 * experts * gu)
+                     for p in pools_t]
+            import ctypes as C
+            for T in (1, 64):
+                if only and only != f"moe{T}":
+                    continue
+                xt = torch.randn(T, hidden, device=dev, generator=gen)
+                yt = torch.empty(T, hidden, device=dev)
+                ids = torch.empty(T, top_k, dtype=torch.int32, device=dev)
+                wts = torch.empty(T, top_k, device=dev)
+
+                def moe_step(i):
+                    must(lib.lev_hip_moe_layer_q4_0(c, C.byref(pools[i % npool]), wr.data_ptr(), None,
+                                                    xt.data_ptr(), yt.data_ptr(), ids.data_ptr(),
+                                                    wts.data_ptr(), top_k, T))
+                moe_step(0)
+                ctx.sync()
+                distinct = int(torch.unique(ids).numel())
+                alg = experts * hidden * 4 + distinct * (2 * gu + dn) + 2 * T * hidden * 4
+
+                def moe_extra(ms, T=T, distinct=distinct):
+                    return {"us_per_token": ms * 1e3 / T, "tokens": T, "distinct_experts": distinct,
+                            "ideal_us_at_hbm_peak": alg / HBM_PEAK_GBS / 1e3}
+                run_other(f"moe_layer_q4_0_T{T}", moe_step, alg, 200 if T == 1 else 50, 20, moe_extra)
+
+    if "value" not in result:                                  # --only run of another family
+        print(json.dumps({"only": only, "others": others}))
+        return
+
+    achieved = result["value"]
+    moe1 = others.get("moe_layer_q4_0_T1", {})
+    line = {
+        "metric": "Q4 GEMV achieved HBM GB/s (% of 8 TB/s); MoE layer us/token at T=1",
+        "value": achieved,
+        "unit": "GB/s",
+        "pct_of_hbm_peak": 100.0 * achieved / HBM_PEAK_GBS,
+        "moe_us_per_token_T1": moe1.get("us_per_token"),
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": result["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "Q4_0 decode GEMV y=W.x, W 4096x4096 GGUF Q4_0, x f32[4096], "
+                               "one launch per step, 64 distinct weight copies in rotation (604 MB)",
+                   "in_dim": cols, "out_rows": rows, "algorithmic_bytes_per_step": q4_alg_bytes},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES,
+                     "kernel": "q4_0_gemv_pairs<64,1,false>",
+                     "note": "achieved = 9,469,952 B / mean launch-to-launch time of the timed "
+                             "region (HIP events on the launch stream)"},
+        "cpu_baseline": result.get("cpu_baseline"),
+        "check": result.get("check"),
+        "device": ctx.device_name(),
+        "others": others,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
