@@ -98,6 +98,21 @@ int lev_hip_sync(lev_ctx *ctx);
 const char *lev_hip_last_error(lev_ctx *ctx);
 int lev_hip_device_name(lev_ctx *ctx, char *out, size_t cap);
 
+/* ---- recorded programs: record once, replay (Program / Step,
+ * rust/crates/lev-vulkan/src/engine.rs:94-141; deferred segments,
+ * Gemma4.swift:2313-2376) ----
+ * Between begin and end every operator call on the context is recorded
+ * instead of executed; run() replays the whole sequence with one submission.
+ * The context must own its stream or sit on a non-default stream.  Scratch
+ * is never grown while recording: run each MoE shape once before recording
+ * it.  Pointers and sizes are frozen into the program. */
+typedef struct lev_program lev_program;
+int lev_hip_program_begin(lev_ctx *ctx);
+int lev_hip_program_end(lev_ctx *ctx, lev_program **out);
+int lev_hip_program_run(lev_ctx *ctx, lev_program *program);
+int lev_hip_program_destroy(lev_ctx *ctx, lev_program *program);
+int lev_hip_program_node_count(lev_program *program, size_t *out);
+
 /* ---- buffers (device.makeBuffer, Q4.swift:223-231; Buf, engine.rs:10-40) ---- */
 int lev_hip_buf_alloc(lev_ctx *ctx, size_t bytes, void **d_out);
 int lev_hip_buf_free(lev_ctx *ctx, void *d_ptr);

@@ -60,6 +60,11 @@ SIGNATURES = {
     "lev_hip_sync": (_int, [_vp]),
     "lev_hip_last_error": (C.c_char_p, [_vp]),
     "lev_hip_device_name": (_int, [_vp, C.c_char_p, _sz]),
+    "lev_hip_program_begin": (_int, [_vp]),
+    "lev_hip_program_end": (_int, [_vp, C.POINTER(_vp)]),
+    "lev_hip_program_run": (_int, [_vp, _vp]),
+    "lev_hip_program_destroy": (_int, [_vp, _vp]),
+    "lev_hip_program_node_count": (_int, [_vp, C.POINTER(_sz)]),
     "lev_hip_buf_alloc": (_int, [_vp, _sz, C.POINTER(_vp)]),
     "lev_hip_buf_free": (_int, [_vp, _vp]),
     "lev_hip_buf_upload": (_int, [_vp, _vp, _vp, _sz]),

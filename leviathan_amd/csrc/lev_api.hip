@@ -28,6 +28,7 @@ int lev_hip_check(lev_ctx *ctx, hipError_t err, const char *what) {
 
 void *lev_scratch(lev_ctx *ctx, size_t bytes) {
     if (bytes <= ctx->scratch_bytes) return ctx->scratch;
+    if (ctx->recording) return nullptr;   // no allocation while a program is being recorded
     // Growing replaces the buffer; earlier kernels on the stream may still be
     // using the old one, so drain the stream first.
     if (ctx->scratch) {
@@ -144,6 +145,7 @@ extern "C" int lev_hip_ctx_destroy(lev_ctx *ctx) {
 
 extern "C" int lev_hip_sync(lev_ctx *ctx) {
     LEV_REQUIRE_CTX(ctx);
+    if (ctx->recording) return lev_fail(ctx, LEV_ERR_INVALID_ARGUMENT, "sync while recording a program");
     LEV_HIP(ctx, hipMemcpyAsync(ctx->h_flag, ctx->d_flag, sizeof(int), hipMemcpyDeviceToHost,
                                 ctx->stream));
     LEV_HIP(ctx, hipStreamSynchronize(ctx->stream));
@@ -378,4 +380,77 @@ extern "C" int lev_hip_empty_launch(lev_ctx *ctx) {
     LEV_REQUIRE_CTX(ctx);
     hipLaunchKernelGGL(empty_kernel, dim3(1), dim3(64), 0, ctx->stream);
     return lev_hip_check(ctx, hipGetLastError(), "empty launch");
+}
+
+// ---------------------------------------------------------------------------
+// recorded programs: record once, replay (Program / Step of
+// rust/crates/lev-vulkan/src/engine.rs:94-141; the deferred segment of
+// Gemma4.swift:2313-2376).  A program is a HIP graph captured from the
+// context's stream.
+// ---------------------------------------------------------------------------
+
+struct lev_program {
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    size_t nodes = 0;
+};
+
+extern "C" int lev_hip_program_begin(lev_ctx *ctx) {
+    LEV_REQUIRE_CTX(ctx);
+    if (ctx->stream == nullptr)
+        return lev_fail(ctx, LEV_ERR_INVALID_ARGUMENT,
+                        "program_begin: the default (null) stream cannot be captured; create the "
+                        "context on a stream of its own");
+    if (ctx->recording) return lev_fail(ctx, LEV_ERR_INVALID_ARGUMENT, "program_begin: already recording");
+    LEV_HIP(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
+    ctx->recording = true;
+    return LEV_OK;
+}
+
+extern "C" int lev_hip_program_end(lev_ctx *ctx, lev_program **out) {
+    LEV_REQUIRE_CTX(ctx);
+    if (!out) return LEV_ERR_INVALID_ARGUMENT;
+    *out = nullptr;
+    if (!ctx->recording) return lev_fail(ctx, LEV_ERR_INVALID_ARGUMENT, "program_end: not recording");
+    ctx->recording = false;
+    hipGraph_t graph = nullptr;
+    LEV_HIP(ctx, hipStreamEndCapture(ctx->stream, &graph));
+    lev_program *p = new (std::nothrow) lev_program();
+    if (!p) {
+        (void)hipGraphDestroy(graph);
+        return lev_fail(ctx, LEV_ERR_DEVICE_UNAVAILABLE, "program_end: out of host memory");
+    }
+    p->graph = graph;
+    (void)hipGraphGetNodes(graph, nullptr, &p->nodes);
+    hipError_t e = hipGraphInstantiate(&p->exec, graph, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+        (void)hipGraphDestroy(graph);
+        delete p;
+        return lev_hip_check(ctx, e, "hipGraphInstantiate");
+    }
+    *out = p;
+    return LEV_OK;
+}
+
+extern "C" int lev_hip_program_run(lev_ctx *ctx, lev_program *program) {
+    LEV_REQUIRE_CTX(ctx);
+    if (!program || !program->exec) return lev_fail(ctx, LEV_ERR_INVALID_ARGUMENT, "program_run: null program");
+    if (ctx->recording) return lev_fail(ctx, LEV_ERR_INVALID_ARGUMENT, "program_run: still recording");
+    return lev_hip_check(ctx, hipGraphLaunch(program->exec, ctx->stream), "hipGraphLaunch");
+}
+
+extern "C" int lev_hip_program_destroy(lev_ctx *ctx, lev_program *program) {
+    LEV_REQUIRE_CTX(ctx);
+    if (!program) return LEV_OK;
+    LEV_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    if (program->exec) (void)hipGraphExecDestroy(program->exec);
+    if (program->graph) (void)hipGraphDestroy(program->graph);
+    delete program;
+    return LEV_OK;
+}
+
+extern "C" int lev_hip_program_node_count(lev_program *program, size_t *out) {
+    if (!program || !out) return LEV_ERR_INVALID_ARGUMENT;
+    *out = program->nodes;
+    return LEV_OK;
 }

@@ -31,6 +31,9 @@ struct lev_ctx {
     // arguments (expert ids); read back by lev_hip_sync.
     int *d_flag = nullptr;
     int *h_flag = nullptr;   // pinned
+    // True between lev_hip_program_begin and lev_hip_program_end: the stream
+    // is being captured, so nothing may allocate or synchronise.
+    bool recording = false;
 };
 
 int lev_fail(lev_ctx *ctx, int status, const char *fmt, ...);

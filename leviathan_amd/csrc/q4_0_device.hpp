@@ -140,41 +140,104 @@ __device__ __forceinline__ void lev_q4_zero_pair(uint32_t D[9]) {
 // and the store: the loads are issued first (they are short and usually hit
 // L2), the caller's weight loads follow, and the wait for the activations
 // does not have to wait for the weights (VMEM returns in issue order).
-constexpr int kLevStageSlots = 4;   // float4 per thread covered in registers
+constexpr int kLevStageSlots = 4;   // default number of float4 per thread covered in registers
 
+// FULL: the caller guarantees pairs*16 == NS*nthreads (every slot in range,
+// nothing beyond), which removes every bounds test from the staging code.
+template <int NS = kLevStageSlots, bool FULL = false>
 __device__ __forceinline__ void lev_q4_stage_x_load(const float *__restrict__ x, uint32_t pairs,
                                                     uint32_t tid, uint32_t nthreads,
-                                                    lev_f32x4 v[kLevStageSlots]) {
+                                                    lev_f32x4 v[NS]) {
     const lev_f32x4 *x4 = reinterpret_cast<const lev_f32x4 *>(x);
     const uint32_t n4 = pairs * 16u;
+    if (FULL) {
 #pragma unroll
-    for (int k = 0; k < kLevStageSlots; ++k) {
+        for (int k = 0; k < NS; ++k) v[k] = x4[tid + k * nthreads];
+        return;
+    }
+    // Unconditional loads from clamped indices: a branch around a load makes
+    // the compiler wait for every outstanding load at the join, which would
+    // serialise these four.
+#pragma unroll
+    for (int k = 0; k < NS; ++k) {
         uint32_t i = tid + k * nthreads;
-        if (i < n4) v[k] = x4[i];
+        v[k] = x4[i < n4 ? i : n4 - 1u];
     }
 }
 
+template <int NS = kLevStageSlots>
 __device__ __forceinline__ void lev_q4_stage_x_store(const float *__restrict__ x, lev_f32x4 *xs,
                                                      uint32_t pairs, uint32_t tid,
                                                      uint32_t nthreads,
-                                                     const lev_f32x4 v[kLevStageSlots]) {
+                                                     const lev_f32x4 v[NS]) {
     const lev_f32x4 *x4 = reinterpret_cast<const lev_f32x4 *>(x);
     const uint32_t n4 = pairs * 16u;
 #pragma unroll
-    for (int k = 0; k < kLevStageSlots; ++k) {
+    for (int k = 0; k < NS; ++k) {
         uint32_t i = tid + k * nthreads;
         if (i < n4) xs[(i & 15u) * (pairs + 1u) + (i >> 4)] = v[k];
     }
-    // vectors longer than kLevStageSlots*nthreads float4 (rare): the rest
-    for (uint32_t i = tid + kLevStageSlots * nthreads; i < n4; i += nthreads)
+    // vectors longer than NS*nthreads float4 (rare): the rest
+    for (uint32_t i = tid + NS * nthreads; i < n4; i += nthreads)
         xs[(i & 15u) * (pairs + 1u) + (i >> 4)] = x4[i];
 }
 
 __device__ __forceinline__ void lev_q4_stage_x(const float *__restrict__ x, lev_f32x4 *xs,
                                                uint32_t pairs, uint32_t tid, uint32_t nthreads) {
     lev_f32x4 v[kLevStageSlots];
-    lev_q4_stage_x_load(x, pairs, tid, nthreads, v);
-    lev_q4_stage_x_store(x, xs, pairs, tid, nthreads, v);
+    lev_q4_stage_x_load<kLevStageSlots>(x, pairs, tid, nthreads, v);
+    lev_q4_stage_x_store<kLevStageSlots>(x, xs, pairs, tid, nthreads, v);
+}
+
+// As lev_q4_stage_x_store, and also writes the sum of every block of 32
+// activations to bsum[block] (a block is 8 consecutive float4, i.e. 8
+// consecutive threads of one pass, so the sum is three DPP steps).  nthreads
+// must be a multiple of 8.  bsum needs 2*pairs floats.
+template <int NS = kLevStageSlots, bool FULL = false>
+__device__ __forceinline__ void lev_q4_stage_x_store_sums(const float *__restrict__ x,
+                                                          lev_f32x4 *xs, float *bsum,
+                                                          uint32_t pairs, uint32_t tid,
+                                                          uint32_t nthreads,
+                                                          const lev_f32x4 v[NS]) {
+    const lev_f32x4 *x4 = reinterpret_cast<const lev_f32x4 *>(x);
+    const uint32_t n4 = pairs * 16u;
+    if (FULL) {
+#pragma unroll
+        for (int k = 0; k < NS; ++k) {
+            const uint32_t i = tid + k * nthreads;
+            float s4 = (v[k].x + v[k].y) + (v[k].z + v[k].w);
+            s4 = lev_group_sum<8>(s4);
+            xs[(i & 15u) * (pairs + 1u) + (i >> 4)] = v[k];
+            if ((i & 7u) == 7u) bsum[i >> 3] = s4;
+        }
+        return;
+    }
+    auto put = [&](uint32_t i, lev_f32x4 val) {
+        float s4 = (val.x + val.y) + (val.z + val.w);
+        s4 = lev_group_sum<8>(s4);
+        if (i < n4) {
+            xs[(i & 15u) * (pairs + 1u) + (i >> 4)] = val;
+            if ((i & 7u) == 7u) bsum[i >> 3] = s4;
+        }
+    };
+#pragma unroll
+    for (int k = 0; k < NS; ++k) put(tid + k * nthreads, v[k]);
+    const uint32_t covered = NS * nthreads;
+    if (n4 > covered) {   // longer vectors: whole extra passes, every thread takes part in the DPP sums
+        for (uint32_t base = covered; base < n4; base += nthreads) {
+            uint32_t i = base + tid;
+            put(i, x4[i < n4 ? i : n4 - 1u]);
+        }
+    }
+}
+
+// Fetches the activations of pair p with the block sums read from bsum.
+__device__ __forceinline__ void lev_q4_fetch_x_sums(const lev_f32x4 *xs, const float *bsum,
+                                                    uint32_t pairs, uint32_t p, lev_q4_pair_x &px) {
+#pragma unroll
+    for (int q = 0; q < 16; ++q) px.xr[q] = xs[q * (pairs + 1u) + p];
+    px.sum_a = bsum[2u * p];
+    px.sum_b = bsum[2u * p + 1u];
 }
 
 __device__ __forceinline__ void lev_q4_fetch_x(const lev_f32x4 *xs, uint32_t pairs, uint32_t p,

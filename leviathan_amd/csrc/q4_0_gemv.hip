@@ -17,7 +17,7 @@
 
 namespace {
 
-constexpr int kThreads = 256;
+constexpr int kThreads = 512;
 constexpr int kWaves = kThreads / LEV_WAVE;
 
 // Resident workgroups per CU the persistent grid is sized for (tunable for
@@ -26,34 +26,39 @@ uint32_t lev_q4_gemv_wg_per_cu() {
     static uint32_t v = [] {
         const char *e = getenv("LEV_Q4_WG_PER_CU");
         int n = e ? atoi(e) : 0;
-        return (uint32_t)(n > 0 && n <= 16 ? n : 4);
+        return (uint32_t)(n > 0 && n <= 16 ? n : 2);
     }();
     return v;
 }
 
 // Loads the R pairs a lane owns in the tile whose first row is `row0`.
+// Branch-free: lanes past the end of the row or of the matrix read a valid
+// pair from a clamped address; they multiply it by zero activations or
+// never store the result.
 template <int L, int R>
 __device__ __forceinline__ void load_tile(const uint8_t *__restrict__ w, uint64_t row_bytes,
-                                          uint32_t row0, uint32_t rows, uint32_t p, bool p_ok,
+                                          uint32_t row0, uint32_t rows, uint32_t pairs, uint32_t p,
                                           uint32_t D[R][9]) {
     constexpr int G = LEV_WAVE / L;
+    const uint32_t pc = p < pairs ? p : pairs - 1u;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         uint32_t row = row0 + r * G;
-        if (p_ok && row < rows)
-            lev_q4_load_pair(w + row * row_bytes + (uint64_t)p * 36u, D[r]);
-        else
-            lev_q4_zero_pair(D[r]);
+        lev_q4_load_pair(w + (row < rows ? row : rows - 1u) * row_bytes + (uint64_t)pc * 36u, D[r]);
     }
 }
 
+// Multiplies a tile and leaves the finished dot products of the workgroup's
+// kWaves*G*R rows in ysh; the first threads then store them contiguously.
 template <int L, int R, bool MULTI>
 __device__ __forceinline__ void finish_tile(const uint8_t *__restrict__ w, uint64_t row_bytes,
-                                            const lev_f32x4 *xs, float *__restrict__ y,
-                                            uint32_t row0, uint32_t rows, uint32_t pairs,
+                                            const lev_f32x4 *xs, const float *bsum, float *ysh,
+                                            float *__restrict__ y, uint32_t tile_base,
+                                            uint32_t in_tile, uint32_t rows, uint32_t pairs,
                                             uint32_t lp, const lev_q4_pair_x &px0,
                                             const uint32_t D[R][9]) {
     constexpr int G = LEV_WAVE / L;
+    constexpr uint32_t kRowsPerTile = kWaves * G * R;
     float acc[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) acc[r] = lev_q4_pair_dot(D[r], px0);
@@ -62,34 +67,86 @@ __device__ __forceinline__ void finish_tile(const uint8_t *__restrict__ w, uint6
         // Rows longer than 64 pairs: further column chunks of the same rows.
         for (uint32_t c = LEV_WAVE; c < pairs; c += LEV_WAVE) {
             const uint32_t p = c + lp;
-            if (p < pairs) {
-                uint32_t E[R][9];
-                load_tile<L, R>(w, row_bytes, row0, rows, p, true, E);
-                lev_q4_pair_x px;
-                lev_q4_fetch_x(xs, pairs, p, px);
+            uint32_t E[R][9];
+            load_tile<L, R>(w, row_bytes, tile_base + in_tile, rows, pairs, p, E);
+            lev_q4_pair_x px;
+            lev_q4_fetch_x_sums(xs, bsum, pairs, p < pairs ? p : pairs - 1u, px);
+            const float keep = p < pairs ? 1.0f : 0.0f;   // partial last chunk
 #pragma unroll
-                for (int r = 0; r < R; ++r) acc[r] += lev_q4_pair_dot(E[r], px);
-            }
+            for (int r = 0; r < R; ++r) acc[r] = fmaf(keep, lev_q4_pair_dot(E[r], px), acc[r]);
         }
     }
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         float s = lev_group_sum<L>(acc[r]);
-        uint32_t row = row0 + r * G;
-        if (lp == L - 1 && row < rows) y[row] = s;
+        if (lp == L - 1) ysh[in_tile + r * G] = s;
     }
+    __syncthreads();
+    if (threadIdx.x < kRowsPerTile && tile_base + threadIdx.x < rows)
+        y[tile_base + threadIdx.x] = ysh[threadIdx.x];
+    __syncthreads();   // ysh is reused by the next tile
 }
 
-// Persistent workgroups: each walks tiles of kWaves*G*R rows with a stride of
+// One tile per workgroup, straight-line code: used whenever the whole matrix
+// fits in one resident wave of workgroups (every decode-sized matrix).  EXACT
+// means pairs == L and pairs*16 == NS*kThreads: no padding lanes, no bounds
+// tests, so the compiler can wait for each weight load separately and start
+// multiplying as soon as the first one lands.
+template <int L, int R, int NS, bool EXACT>
+__global__ void __launch_bounds__(kThreads)
+q4_0_gemv_tile(const uint8_t *__restrict__ w, const float *__restrict__ x, float *__restrict__ y,
+               uint32_t pairs, uint32_t rows) {
+    extern __shared__ lev_f32x4 xs[];
+    constexpr int G = LEV_WAVE / L;
+    constexpr uint32_t kRowsPerTile = kWaves * G * R;
+    __shared__ float ysh[kRowsPerTile];
+    float *bsum = reinterpret_cast<float *>(xs + 16u * (pairs + 1u));
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & (LEV_WAVE - 1);
+    const uint32_t wave = tid / LEV_WAVE;
+    const uint32_t grp = lane / L;
+    const uint32_t lp = lane % L;
+    const uint64_t row_bytes = (uint64_t)pairs * 36u;
+    const uint32_t in_tile = wave * (G * R) + grp;
+    const uint32_t base = blockIdx.x * kRowsPerTile;
+
+    lev_f32x4 xv[NS];
+    lev_q4_stage_x_load<NS, EXACT>(x, pairs, tid, kThreads, xv);
+    uint32_t D[R][9];
+    load_tile<L, R>(w, row_bytes, base + in_tile, rows, pairs, lp, D);
+    lev_q4_stage_x_store_sums<NS, EXACT>(x, xs, bsum, pairs, tid, kThreads, xv);
+    __syncthreads();
+
+    lev_q4_pair_x px;
+    const bool p_ok = EXACT || lp < pairs;
+    lev_q4_fetch_x_sums(xs, bsum, pairs, p_ok ? lp : pairs - 1u, px);
+    if (!EXACT) {
+#pragma unroll
+        for (int q = 0; q < 16; ++q) px.xr[q] = p_ok ? px.xr[q] : lev_f32x4{0.f, 0.f, 0.f, 0.f};
+        px.sum_a = p_ok ? px.sum_a : 0.f;
+        px.sum_b = p_ok ? px.sum_b : 0.f;
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        float s = lev_group_sum<L>(lev_q4_pair_dot(D[r], px));
+        if (lp == L - 1) ysh[in_tile + r * G] = s;
+    }
+    __syncthreads();
+    if (tid < kRowsPerTile && base + tid < rows) y[base + tid] = ysh[tid];
+}
+
+// Workgroups of 8 waves walk tiles of kWaves*G*R rows with a stride of
 // gridDim.x tiles, double-buffering the weight registers so that the loads
 // of tile t+1 are in flight while tile t is being multiplied.
-template <int L, int R, bool MULTI>
+template <int L, int R, bool MULTI, int NS>
 __global__ void __launch_bounds__(kThreads)
 q4_0_gemv_pairs(const uint8_t *__restrict__ w, const float *__restrict__ x, float *__restrict__ y,
                 uint32_t pairs, uint32_t rows) {
     extern __shared__ lev_f32x4 xs[];
     constexpr int G = LEV_WAVE / L;                 // rows per wave-wide load
     constexpr uint32_t kRowsPerTile = kWaves * G * R;
+    __shared__ float ysh[kRowsPerTile];
+    float *bsum = reinterpret_cast<float *>(xs + 16u * (pairs + 1u));
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & (LEV_WAVE - 1);
     const uint32_t wave = tid / LEV_WAVE;
@@ -97,7 +154,7 @@ q4_0_gemv_pairs(const uint8_t *__restrict__ w, const float *__restrict__ x, floa
     const uint32_t lp = lane % L;
     const bool p_ok = lp < pairs;
     const uint64_t row_bytes = (uint64_t)pairs * 36u;
-    const uint32_t in_tile = wave * (G * R) + grp;
+    const uint32_t in_tile = wave * (G * R) + grp;   // rows of one wave are wave*(G*R) + r*G + grp
     const uint32_t step = gridDim.x * kRowsPerTile;
 
     uint32_t base = blockIdx.x * kRowsPerTile;
@@ -106,32 +163,38 @@ q4_0_gemv_pairs(const uint8_t *__restrict__ w, const float *__restrict__ x, floa
     // Activations first (16 KB, L2 hits after the first workgroup), then the
     // first tile's weights: the activations are staged and fetched while the
     // weights are still in flight.
-    lev_f32x4 xv[kLevStageSlots];
-    lev_q4_stage_x_load(x, pairs, tid, kThreads, xv);
+    lev_f32x4 xv[NS];
+    lev_q4_stage_x_load<NS>(x, pairs, tid, kThreads, xv);
     uint32_t Da[R][9], Db[R][9];
-    load_tile<L, R>(w, row_bytes, base + in_tile, rows, lp, p_ok, Da);
-    lev_q4_stage_x_store(x, xs, pairs, tid, kThreads, xv);
+    load_tile<L, R>(w, row_bytes, base + in_tile, rows, pairs, lp, Da);
+    lev_q4_stage_x_store_sums<NS>(x, xs, bsum, pairs, tid, kThreads, xv);
     __syncthreads();
 
-    // Activations of the lane's first pair stay in registers for every tile.
+    // Activations of the lane's first pair stay in registers for every tile;
+    // lanes past the end of the row hold zeros.
     lev_q4_pair_x px0;
-    if (p_ok) {
-        lev_q4_fetch_x(xs, pairs, lp, px0);
-    } else {
+    lev_q4_fetch_x_sums(xs, bsum, pairs, p_ok ? lp : pairs - 1u, px0);
 #pragma unroll
-        for (int q = 0; q < 16; ++q) px0.xr[q] = lev_f32x4{0.f, 0.f, 0.f, 0.f};
-        px0.sum_a = px0.sum_b = 0.f;
-    }
+    for (int q = 0; q < 16; ++q) px0.xr[q] = p_ok ? px0.xr[q] : lev_f32x4{0.f, 0.f, 0.f, 0.f};
+    px0.sum_a = p_ok ? px0.sum_a : 0.f;
+    px0.sum_b = p_ok ? px0.sum_b : 0.f;
 
+    if (step >= rows) {   // the grid covers every tile once: nothing to prefetch
+        finish_tile<L, R, MULTI>(w, row_bytes, xs, bsum, ysh, y, base, in_tile, rows, pairs, lp, px0, Da);
+        return;
+    }
+    // The prefetch is unconditional (past the last tile it re-reads the last
+    // row, which is harmless): a branch around it would make the compiler
+    // wait for the prefetched data before the current tile is multiplied.
     while (true) {
         uint32_t next = base + step;
-        if (next < rows) load_tile<L, R>(w, row_bytes, next + in_tile, rows, lp, p_ok, Db);
-        finish_tile<L, R, MULTI>(w, row_bytes, xs, y, base + in_tile, rows, pairs, lp, px0, Da);
+        load_tile<L, R>(w, row_bytes, next + in_tile, rows, pairs, lp, Db);
+        finish_tile<L, R, MULTI>(w, row_bytes, xs, bsum, ysh, y, base, in_tile, rows, pairs, lp, px0, Da);
         if (next >= rows) break;
         base = next;
         next = base + step;
-        if (next < rows) load_tile<L, R>(w, row_bytes, next + in_tile, rows, lp, p_ok, Da);
-        finish_tile<L, R, MULTI>(w, row_bytes, xs, y, base + in_tile, rows, pairs, lp, px0, Db);
+        load_tile<L, R>(w, row_bytes, next + in_tile, rows, pairs, lp, Da);
+        finish_tile<L, R, MULTI>(w, row_bytes, xs, bsum, ysh, y, base, in_tile, rows, pairs, lp, px0, Db);
         if (next >= rows) break;
         base = next;
     }
@@ -141,11 +204,11 @@ q4_0_gemv_pairs(const uint8_t *__restrict__ w, const float *__restrict__ x, floa
 // long for LDS): one wave per row, 16-bit loads, activations from global
 // memory.  Correct everywhere, fast nowhere; the pair kernel covers every
 // shape the models on this path use.
-__global__ void __launch_bounds__(kThreads)
+__global__ void __launch_bounds__(256)
 q4_0_gemv_generic(const uint8_t *__restrict__ w, const float *__restrict__ x,
                   float *__restrict__ y, uint32_t blocks_per_row, uint32_t rows) {
     const uint32_t lane = threadIdx.x & (LEV_WAVE - 1);
-    const uint32_t row = blockIdx.x * kWaves + threadIdx.x / LEV_WAVE;
+    const uint32_t row = blockIdx.x * 4u + threadIdx.x / LEV_WAVE;
     if (row >= rows) return;
     const uint8_t *rp = w + (uint64_t)row * blocks_per_row * 18u;
     float acc = 0.f;
@@ -170,21 +233,34 @@ q4_0_gemv_generic(const uint8_t *__restrict__ w, const float *__restrict__ x,
     if (lane == LEV_WAVE - 1) y[row] = acc;
 }
 
-template <int L, int R, bool MULTI = false>
+// NS = float4 of the activation vector each thread stages from registers.
+template <int L, int R, bool MULTI = false, int NS = 1>
 hipError_t launch_pairs(lev_ctx *ctx, const uint8_t *w, const float *x, float *y, uint32_t pairs,
                         uint32_t rows) {
     constexpr uint32_t rows_per_tile = kWaves * (LEV_WAVE / L) * R;
     uint32_t blocks = (rows + rows_per_tile - 1) / rows_per_tile;
+    if (!MULTI && blocks <= (uint32_t)ctx->num_cus * 4u) {
+        // every tile is resident at once: one straight-line tile per workgroup
+        size_t lds1 = (size_t)16 * (pairs + 1) * sizeof(lev_f32x4) + (size_t)2 * pairs * sizeof(float);
+        const bool exact = pairs == (uint32_t)L && pairs * 16u == (uint32_t)NS * kThreads;
+        if (exact)
+            hipLaunchKernelGGL((q4_0_gemv_tile<L, R, NS, true>), dim3(blocks), dim3(kThreads), lds1,
+                               ctx->stream, w, x, y, pairs, rows);
+        else
+            hipLaunchKernelGGL((q4_0_gemv_tile<L, R, NS, false>), dim3(blocks), dim3(kThreads), lds1,
+                               ctx->stream, w, x, y, pairs, rows);
+        return hipGetLastError();
+    }
     // Persistent grid: as many workgroups as stay resident at once.
     uint32_t cap = (uint32_t)ctx->num_cus * lev_q4_gemv_wg_per_cu();
     if (blocks > cap) blocks = cap;
-    size_t lds = (size_t)16 * (pairs + 1) * sizeof(lev_f32x4);
+    size_t lds = (size_t)16 * (pairs + 1) * sizeof(lev_f32x4) + (size_t)2 * pairs * sizeof(float);
     if (lds > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&q4_0_gemv_pairs<L, R, MULTI>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&q4_0_gemv_pairs<L, R, MULTI, NS>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
     }
-    hipLaunchKernelGGL((q4_0_gemv_pairs<L, R, MULTI>), dim3(blocks), dim3(kThreads), lds, ctx->stream, w, x,
+    hipLaunchKernelGGL((q4_0_gemv_pairs<L, R, MULTI, NS>), dim3(blocks), dim3(kThreads), lds, ctx->stream, w, x,
                        y, pairs, rows);
     return hipGetLastError();
 }
@@ -198,8 +274,8 @@ hipError_t lev_q4_0_gemv_launch(lev_ctx *ctx, const uint8_t *w, const float *x, 
     const bool pairable = (nb % 2u == 0u) && ((reinterpret_cast<uintptr_t>(w) & 3u) == 0u) &&
                           (in_dim <= 32768u) && ((reinterpret_cast<uintptr_t>(x) & 15u) == 0u);
     if (!pairable) {
-        uint32_t blocks = (rows + kWaves - 1) / kWaves;
-        hipLaunchKernelGGL(q4_0_gemv_generic, dim3(blocks), dim3(kThreads), 0, ctx->stream, w, x, y,
+        uint32_t blocks = (rows + 3u) / 4u;
+        hipLaunchKernelGGL(q4_0_gemv_generic, dim3(blocks), dim3(256), 0, ctx->stream, w, x, y,
                            nb, rows);
         return hipGetLastError();
     }
@@ -209,14 +285,14 @@ hipError_t lev_q4_0_gemv_launch(lev_ctx *ctx, const uint8_t *w, const float *x, 
             const char *e = getenv("LEV_Q4_R");
             return e ? atoi(e) : 0;
         }();
-        if (pairs > 64) return launch_pairs<64, 2, true>(ctx, w, x, y, pairs, rows);
+        if (pairs > 64) return launch_pairs<64, 2, true, 4>(ctx, w, x, y, pairs, rows);
         int r = forced;
         // One row per wave and pass measured fastest at 4096 and 32768 rows:
         // 100 VGPRs leave five waves per SIMD to hide the HBM latency.
         if (r == 0) r = 1;
-        if (r == 1) return launch_pairs<64, 1>(ctx, w, x, y, pairs, rows);
-        if (r == 2) return launch_pairs<64, 2>(ctx, w, x, y, pairs, rows);
-        return launch_pairs<64, 4>(ctx, w, x, y, pairs, rows);
+        if (r == 1) return launch_pairs<64, 1, false, 2>(ctx, w, x, y, pairs, rows);
+        if (r == 2) return launch_pairs<64, 2, false, 2>(ctx, w, x, y, pairs, rows);
+        return launch_pairs<64, 4, false, 2>(ctx, w, x, y, pairs, rows);
     }
     if (pairs > 16) return launch_pairs<32, 4>(ctx, w, x, y, pairs, rows);
     if (pairs > 8) return launch_pairs<16, 4>(ctx, w, x, y, pairs, rows);

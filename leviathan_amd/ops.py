@@ -81,6 +81,15 @@ class Context:
         self._check(self.lib.lev_hip_device_name(self.ctx, buf, 256))
         return buf.value.decode()
 
+    # -- recorded programs -------------------------------------------------
+    def program_begin(self):
+        self._check(self.lib.lev_hip_program_begin(self.ctx))
+
+    def program_end(self) -> "Program":
+        handle = C.c_void_p()
+        self._check(self.lib.lev_hip_program_end(self.ctx, C.byref(handle)))
+        return Program(self, handle)
+
     # -- dequantise -------------------------------------------------------
     def dequant(self, qtype: int, w: torch.Tensor, nblocks: int, w_off: int = 0) -> torch.Tensor:
         _dev(w, torch.uint8, "w")
@@ -222,6 +231,26 @@ class Context:
                                                     _ptr(expert_scale), _ptr(x), _ptr(y), _ptr(ids),
                                                     _ptr(weights), top_k, tokens))
         return y, ids, weights
+
+
+class Program:
+    """A recorded sequence of operator calls (``lev_program``), replayed with ``run()``."""
+
+    def __init__(self, ctx: Context, handle):
+        self.ctx, self.handle = ctx, handle
+
+    def run(self):
+        self.ctx._check(self.ctx.lib.lev_hip_program_run(self.ctx.ctx, self.handle))
+
+    def node_count(self) -> int:
+        n = C.c_size_t()
+        self.ctx._check(self.ctx.lib.lev_hip_program_node_count(self.handle, C.byref(n)))
+        return n.value
+
+    def destroy(self):
+        if self.handle:
+            self.ctx._check(self.ctx.lib.lev_hip_program_destroy(self.ctx.ctx, self.handle))
+            self.handle = None
 
 
 # -- host-array twins of the standalone backends --------------------------
