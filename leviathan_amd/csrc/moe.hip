@@ -8,9 +8,9 @@
 //   and the ordered g4_axpy merges (:2171-2175, :4459).
 //
 // Three launches per call, all HBM-bound:
-//   1. router: one wave per (token, expert) row, f64 accumulation; the last
-//      wave to finish a token runs softmax (f64), top-k (ties -> lower index)
-//      and renormalisation for that token.
+//   1. router: a workgroup per expert row, its waves take tokens in turn, f64
+//      accumulation; the wave that completes a token's last score runs softmax
+//      (f64), top-k (ties -> lower index) and renormalisation for that token.
 //   2. gate/up: a wave streams gate row i with lanes 0..31 and up row i with
 //      lanes 32..63 (a row of 2048 values is 32 block pairs), reduces both and
 //      writes act = gelu_tanh(g)*u.  x is staged once per workgroup.
@@ -28,115 +28,271 @@ constexpr int kFlagNonFiniteScore = 2;
 // router
 // ---------------------------------------------------------------------------
 
-__device__ __forceinline__ double wave_sum_f64(double v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
-    return v;
+// DPP lane exchange of a 64-bit value; lanes the control word does not write
+// keep their own value.
+template <int CTRL, int ROW_MASK = 0xF>
+__device__ __forceinline__ double dpp_move_f64(double v) {
+    int lo = __double2loint(v), hi = __double2hiint(v);
+    lo = __builtin_amdgcn_update_dpp(lo, lo, CTRL, ROW_MASK, 0xF, false);
+    hi = __builtin_amdgcn_update_dpp(hi, hi, CTRL, ROW_MASK, 0xF, false);
+    return __hiloint2double(hi, lo);
 }
 
-// grid (experts, tokens), 64 threads.  counters[tokens] must be zero on entry
-// and are zero again on exit (atomicInc wraps at experts-1).
-__global__ void __launch_bounds__(64)
-moe_router_kernel(const float *__restrict__ wr, const float *__restrict__ x,
-                  const float *__restrict__ expert_scale, float *__restrict__ scores,
-                  int32_t *__restrict__ ids, float *__restrict__ weights,
-                  uint32_t *__restrict__ counters, int *__restrict__ flag, uint32_t hidden,
-                  uint32_t experts, uint32_t top_k) {
-    const uint32_t e = blockIdx.x, t = blockIdx.y, lane = threadIdx.x;
-    const float *row = wr + (uint64_t)e * hidden;
-    const float *xv = x + (uint64_t)t * hidden;
-    double acc = 0.0;
-    if ((hidden & 3u) == 0u) {
-        const lev_f32x4 *r4 = reinterpret_cast<const lev_f32x4 *>(row);
-        const lev_f32x4 *x4 = reinterpret_cast<const lev_f32x4 *>(xv);
-        double a0 = 0.0, a1 = 0.0;
-        for (uint32_t i = lane; i < hidden / 4u; i += 64u) {
-            lev_f32x4 a = r4[i], b = x4[i];
-            a0 = fma((double)a.x, (double)b.x, a0);
-            a1 = fma((double)a.y, (double)b.y, a1);
-            a0 = fma((double)a.z, (double)b.z, a0);
-            a1 = fma((double)a.w, (double)b.w, a1);
-        }
-        acc = a0 + a1;
-    } else {
-        for (uint32_t i = lane; i < hidden; i += 64u) acc = fma((double)row[i], (double)xv[i], acc);
-    }
-    acc = wave_sum_f64(acc);
-    float *srow = scores + (uint64_t)t * experts;
-    uint32_t done = 0;
-    if (lane == 0) {
-        __hip_atomic_store(&srow[e], (float)acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __threadfence();
-        done = atomicInc(&counters[t], experts - 1u);
-    }
-    done = __shfl(done, 0);
-    if (done != experts - 1u) return;
-    __threadfence();
+__device__ __forceinline__ double lane63_f64(double v) {
+    int lo = __builtin_amdgcn_readlane(__double2loint(v), 63);
+    int hi = __builtin_amdgcn_readlane(__double2hiint(v), 63);
+    return __hiloint2double(hi, lo);
+}
 
-    // ---- last wave of this token: softmax + top-k (Gemma4.swift:3798-3810) ----
-    extern __shared__ double s_p[];                 // experts doubles
+// Sum / maximum over the 64 lanes, returned in every lane (wave-uniform).
+__device__ __forceinline__ double wave_sum_f64(double v) {
+    v += dpp_move_f64<0xB1>(v);
+    v += dpp_move_f64<0x4E>(v);
+    v += dpp_move_f64<0x141>(v);
+    v += dpp_move_f64<0x140>(v);
+    {   // row_bcast steps: lanes outside the mask must add nothing
+        int lo = __builtin_amdgcn_update_dpp(0, __double2loint(v), 0x142, 0xA, 0xF, false);
+        int hi = __builtin_amdgcn_update_dpp(0, __double2hiint(v), 0x142, 0xA, 0xF, false);
+        v += __hiloint2double(hi, lo);
+        lo = __builtin_amdgcn_update_dpp(0, __double2loint(v), 0x143, 0xC, 0xF, false);
+        hi = __builtin_amdgcn_update_dpp(0, __double2hiint(v), 0x143, 0xC, 0xF, false);
+        v += __hiloint2double(hi, lo);
+    }
+    return lane63_f64(v);
+}
+
+__device__ __forceinline__ float wave_max_f32(float v) {
+#define LEV_MAXSTEP(CTRL, MASK)                                                                   \
+    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(                           \
+                     __builtin_bit_cast(int, v), __builtin_bit_cast(int, v), CTRL, MASK, 0xF, false)))
+    LEV_MAXSTEP(0xB1, 0xF);
+    LEV_MAXSTEP(0x4E, 0xF);
+    LEV_MAXSTEP(0x141, 0xF);
+    LEV_MAXSTEP(0x140, 0xF);
+    LEV_MAXSTEP(0x142, 0xA);
+    LEV_MAXSTEP(0x143, 0xC);
+#undef LEV_MAXSTEP
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+
+// Orders one wave's LDS writes before its later LDS reads (the hardware runs
+// a wave's LDS accesses in order; this only restrains the compiler).
+__device__ __forceinline__ void wave_lds_fence() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// LDS the selection needs: a table of probabilities (experts rounded up to a
+// multiple of 64), as many rank counters, then 64 selected probabilities and ids.
+__host__ __device__ constexpr size_t router_lds_bytes(uint32_t experts) {
+    return (size_t)((experts + 63u) & ~63u) * 12u + 64u * 8u + 64u * 4u;
+}
+
+struct router_sel {
+    const double *sel_p;     // LDS: probabilities of the selected experts, selection order
+    const uint32_t *sel_id;  // LDS: their indices
+    bool ok;                 // false: a score was not finite, nothing selected
+};
+
+// softmax (f64) + top-k (ties -> lower index) for one token
+// (Gemma4.swift:3798-3810), run by a whole workgroup (every thread calls it;
+// blockDim a multiple of 64 and of the padded expert count when that is below
+// blockDim).  srow: the token's `experts` scores, written by an earlier kernel.
+//
+// Repeated extraction of the maximum with ties to the lower index is the same
+// as ordering by the strict total order "p larger, or p equal and index
+// lower"; an element's rank under that order is the number of elements that
+// come before it.  The workgroup counts ranks in parallel: the threads split
+// into blockDim/padded parts, each part compares every element against its
+// share of the table.
+//
+// J: each lane of a wave keeps experts j*64+lane, j < J, in registers, and
+// every wave computes the whole softmax for itself (same values, same order,
+// same result), so the only exchanges are the table, the ranks and the winners.
+template <int J>
+__device__ router_sel router_select_block(const float *__restrict__ srow, void *lds,
+                                          uint32_t experts, uint32_t top_k) {
+    constexpr uint32_t padded = 64u * J;
+    double *p_lds = static_cast<double *>(lds);
+    double *sel_p = p_lds + padded;
+    uint32_t *rank = reinterpret_cast<uint32_t *>(sel_p + 64);
+    uint32_t *sel_id = rank + padded;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    router_sel out{sel_p, sel_id, true};
+
+    float sc[J];
     float mx = -INFINITY;
     bool finite = true;
-    for (uint32_t i = lane; i < experts; i += 64u) {
-        float s = __hip_atomic_load(&srow[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        finite = finite && isfinite(s);
-        mx = fmaxf(mx, s);
-        s_p[i] = (double)s;
-    }
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
-    if (__any(!finite)) {
-        if (lane == 0) atomicOr(flag, kFlagNonFiniteScore);
-        for (uint32_t k = lane; k < top_k; k += 64u) {
-            ids[(uint64_t)t * top_k + k] = (int32_t)k;
-            weights[(uint64_t)t * top_k + k] = 0.f;
+    for (int j = 0; j < J; ++j) {
+        const uint32_t i = lane + 64u * j;
+        const bool valid = i < experts;
+        sc[j] = srow[valid ? i : experts - 1u];
+        finite = finite && isfinite(sc[j]);
+        mx = fmaxf(mx, sc[j]);
+    }
+    mx = wave_max_f32(mx);
+    if (__any(!finite)) {   // uniform over the workgroup
+        out.ok = false;
+        return out;
+    }
+    double p[J], sum = 0.0;
+#pragma unroll
+    for (int j = 0; j < J; ++j) {
+        const bool valid = lane + 64u * j < experts;
+        p[j] = valid ? exp((double)(sc[j] - mx)) : 0.0;   // subtraction in f32, exp in f64
+        sum += p[j];
+    }
+    sum = wave_sum_f64(sum);
+    if (wave == 0) {
+#pragma unroll
+        for (int j = 0; j < J; ++j) {
+            // padding entries hold 0 at indices above every real one: they rank last
+            p_lds[lane + 64u * j] = lane + 64u * j < experts ? p[j] / sum : 0.0;
+            rank[lane + 64u * j] = 0u;
+        }
+    }
+    __syncthreads();
+    auto count_before = [&](uint32_t i, uint32_t j0, uint32_t j1) {
+        const double pi = p_lds[i];
+        uint32_t before = 0;
+#pragma unroll 8
+        for (uint32_t j = j0; j < j1; ++j) {
+            const double pj = p_lds[j];   // same address across the wave: a broadcast read
+            before += (pj > pi || (pj == pi && j < i)) ? 1u : 0u;
+        }
+        return before;
+    };
+    if (blockDim.x > padded) {
+        const uint32_t parts = blockDim.x / padded, share = padded / parts;
+        const uint32_t i = tid % padded, part = tid / padded;
+        atomicAdd(&rank[i], count_before(i, part * share, (part + 1u) * share));
+    } else {
+        for (uint32_t i = tid; i < padded; i += blockDim.x) rank[i] = count_before(i, 0u, padded);
+    }
+    __syncthreads();
+    for (uint32_t i = tid; i < experts; i += blockDim.x) {
+        const uint32_t r = rank[i];
+        if (r < top_k) {
+            sel_id[r] = i;
+            sel_p[r] = p_lds[i];
+        }
+    }
+    __syncthreads();
+    return out;
+}
+
+// Renormalised weight of selection slot k (Gemma4.swift:3808-3810): the sum
+// runs over the slots in order, in f64.
+__device__ __forceinline__ float router_weight(const router_sel &r, const float *expert_scale,
+                                               uint32_t top_k, uint32_t k) {
+    double prob_sum = 0.0;
+    for (uint32_t m = 0; m < top_k; ++m) prob_sum += r.sel_p[m];
+    float wgt = (float)(r.sel_p[k] / prob_sum);
+    if (expert_scale) wgt *= expert_scale[r.sel_id[k]];
+    return wgt;
+}
+
+// Router scores, f64 accumulation rounded to f32 once.  Workgroup (e, g) owns
+// router row e.
+//   split = 1 (up to four tokens, gridDim.y = 1): the waves share the row, a
+//     part of the columns each, for every token, and meet in LDS.
+//   split = 0: wave w of group g scores the four tokens 4*(4g+w).. against the
+//     row, which it reads once for the four.
+constexpr uint32_t kScoreTokensPerWave = 4;
+
+__global__ void __launch_bounds__(256)
+moe_scores_kernel(const float *__restrict__ wr, const float *__restrict__ x,
+                  float *__restrict__ scores, uint32_t hidden, uint32_t experts, uint32_t tokens,
+                  int split) {
+    __shared__ double partial[4][4];
+    const uint32_t e = blockIdx.x, lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t waves = blockDim.x >> 6;
+    const float *row = wr + (uint64_t)e * hidden;
+    const bool vec = (hidden & 3u) == 0u &&
+                     ((reinterpret_cast<uintptr_t>(wr) | reinterpret_cast<uintptr_t>(x)) & 15u) == 0u;
+    if (split) {
+        for (uint32_t t = 0; t < tokens; ++t) {
+            const float *xv = x + (uint64_t)t * hidden;
+            double acc;
+            if (vec) {
+                const lev_f32x4 *r4 = reinterpret_cast<const lev_f32x4 *>(row);
+                const lev_f32x4 *x4 = reinterpret_cast<const lev_f32x4 *>(xv);
+                double a0 = 0.0, a1 = 0.0;
+                for (uint32_t i = threadIdx.x; i < hidden / 4u; i += blockDim.x) {
+                    lev_f32x4 a = r4[i], b = x4[i];
+                    a0 = fma((double)a.x, (double)b.x, a0);
+                    a1 = fma((double)a.y, (double)b.y, a1);
+                    a0 = fma((double)a.z, (double)b.z, a0);
+                    a1 = fma((double)a.w, (double)b.w, a1);
+                }
+                acc = a0 + a1;
+            } else {
+                acc = 0.0;
+                for (uint32_t i = threadIdx.x; i < hidden; i += blockDim.x)
+                    acc = fma((double)row[i], (double)xv[i], acc);
+            }
+            acc = wave_sum_f64(acc);
+            if (lane == 0) partial[t][wave] = acc;
+        }
+        __syncthreads();
+        if (threadIdx.x < tokens) {
+            double acc = partial[threadIdx.x][0];
+            for (uint32_t w = 1; w < waves; ++w) acc += partial[threadIdx.x][w];
+            scores[(uint64_t)threadIdx.x * experts + e] = (float)acc;
         }
         return;
     }
-    double sum = 0.0;
-    for (uint32_t i = lane; i < experts; i += 64u) {
-        double p = exp((double)((float)s_p[i] - mx));   // subtraction in f32, exp in f64
-        s_p[i] = p;
-        sum += p;
-    }
-    sum = wave_sum_f64(sum);
-    for (uint32_t i = lane; i < experts; i += 64u) s_p[i] = s_p[i] / sum;
-    __builtin_amdgcn_s_barrier();   // single wave: orders the LDS writes above
-    double prob_sum = 0.0;
-    double my_p = 0.0;              // lane k keeps the probability of slot k (top_k <= 64)
-    uint32_t my_id = 0;
-    for (uint32_t k = 0; k < top_k; ++k) {
-        double best = -1.0;
-        uint32_t bi = 0xFFFFFFFFu;
-        for (uint32_t i = lane; i < experts; i += 64u) {
-            double p = s_p[i];
-            if (p > best) {       // ascending i within a lane: ties keep the lower index
-                best = p;
-                bi = i;
-            }
-        }
+    constexpr uint32_t K = kScoreTokensPerWave;
+    const uint32_t t0 = (blockIdx.y * waves + wave) * K;
+    if (t0 >= tokens) return;
+    const float *xv[K];
 #pragma unroll
-        for (int off = 32; off > 0; off >>= 1) {
-            double ob = __shfl_xor(best, off);
-            uint32_t oi = __shfl_xor(bi, off);
-            if (ob > best || (ob == best && oi < bi)) {
-                best = ob;
-                bi = oi;
+    for (uint32_t k = 0; k < K; ++k)   // tokens past the end repeat the last one and are not stored
+        xv[k] = x + (uint64_t)(t0 + k < tokens ? t0 + k : tokens - 1u) * hidden;
+    double acc[K] = {};
+    if (vec) {
+        const lev_f32x4 *r4 = reinterpret_cast<const lev_f32x4 *>(row);
+#pragma unroll 2
+        for (uint32_t i = lane; i < hidden / 4u; i += 64u) {
+            const lev_f32x4 a = r4[i];
+#pragma unroll
+            for (uint32_t k = 0; k < K; ++k) {
+                const lev_f32x4 b = reinterpret_cast<const lev_f32x4 *>(xv[k])[i];
+                double lo = fma((double)a.x, (double)b.x, (double)a.y * (double)b.y);
+                double hi = fma((double)a.z, (double)b.z, (double)a.w * (double)b.w);
+                acc[k] += lo + hi;
             }
         }
-        prob_sum += best;          // slot order, as topIdx.reduce does
-        if (lane == k) {
-            my_p = best;
-            my_id = bi;
+    } else {
+        for (uint32_t i = lane; i < hidden; i += 64u) {
+            const float a = row[i];
+#pragma unroll
+            for (uint32_t k = 0; k < K; ++k) acc[k] = fma((double)a, (double)xv[k][i], acc[k]);
         }
-        if (lane == (bi & 63u)) s_p[bi] = -2.0;   // taken
-        __builtin_amdgcn_s_barrier();
     }
-    if (lane < top_k) {
-        float wgt = (float)(my_p / prob_sum);
-        if (expert_scale) wgt *= expert_scale[my_id];
-        ids[(uint64_t)t * top_k + lane] = (int32_t)my_id;
-        weights[(uint64_t)t * top_k + lane] = wgt;
+#pragma unroll
+    for (uint32_t k = 0; k < K; ++k) {
+        const double total = wave_sum_f64(acc[k]);
+        if (lane == 0 && t0 + k < tokens) scores[(uint64_t)(t0 + k) * experts + e] = (float)total;
+    }
+}
+
+// grid (tokens), 256 threads: selection for one token, written to global memory.
+template <int J>
+__global__ void __launch_bounds__(256)
+moe_topk_kernel(const float *__restrict__ scores, const float *__restrict__ expert_scale,
+                int32_t *__restrict__ ids, float *__restrict__ weights, int *__restrict__ flag,
+                uint32_t experts, uint32_t top_k) {
+    extern __shared__ double s_router[];
+    const uint32_t t = blockIdx.x;
+    const router_sel r = router_select_block<J>(scores + (uint64_t)t * experts, s_router, experts, top_k);
+    if (!r.ok && threadIdx.x == 0) atomicOr(flag, kFlagNonFiniteScore);
+    if (threadIdx.x < top_k) {
+        ids[(uint64_t)t * top_k + threadIdx.x] = r.ok ? (int32_t)r.sel_id[threadIdx.x] : (int32_t)threadIdx.x;
+        weights[(uint64_t)t * top_k + threadIdx.x] =
+            r.ok ? router_weight(r, expert_scale, top_k, threadIdx.x) : 0.f;
     }
 }
 
@@ -164,82 +320,135 @@ struct moe_args {
     uint32_t hidden, inter, experts, top_k;
 };
 
-constexpr int kGuThreads = 256;
+constexpr int kGuThreads = 512;
 constexpr int kGuWaves = kGuThreads / LEV_WAVE;
 
-// grid (chunks_per_slot, top_k, tokens).  P = passes of 32 pairs per row.
-template <int P>
+// Loads rows i0 + r (r < R) of the lane's half (gate or up): P pairs each.
+// Branch-free: rows and pairs past the end are clamped to valid ones.
+template <int P, int R>
+__device__ __forceinline__ void gu_load_rows(const uint8_t *__restrict__ wbase, uint64_t row_bytes,
+                                             uint32_t i0, uint32_t inter, uint32_t pairs, uint32_t lp,
+                                             uint32_t D[P][R][9]) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const uint32_t i = i0 + r;
+        const uint8_t *rp = wbase + (uint64_t)(i < inter ? i : inter - 1u) * row_bytes;
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+            const uint32_t pr = lp + 32u * p;
+            lev_q4_load_pair(rp + (uint64_t)(pr < pairs ? pr : pairs - 1u) * 36u, D[p][r]);
+        }
+    }
+}
+
+template <int P, int R>
+__device__ __forceinline__ void gu_finish_rows(const uint32_t D[P][R][9], const lev_q4_pair_x X[P],
+                                               float *__restrict__ arow, uint32_t i0, uint32_t i_end,
+                                               uint32_t lane) {
+    float mine = 0.f;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        float acc = 0.f;
+#pragma unroll
+        for (int p = 0; p < P; ++p) acc += lev_q4_pair_dot(D[p][r], X[p]);
+        acc = lev_group_sum<32>(acc);
+        float g = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, acc), 31));
+        float u = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, acc), 63));
+        float v = lev_gelu_up_value(g, u);
+        mine = lane == (uint32_t)r ? v : mine;
+    }
+    if (lane < (uint32_t)R && i0 + lane < i_end) arow[i0 + lane] = mine;   // R consecutive floats
+}
+
+// grid (chunks_per_slot, top_k, tokens), 8 waves.  Lanes 0..31 of a wave walk
+// gate row i and lanes 32..63 up row i; a wave has R such rows in flight and a
+// lane covers P pairs of each (rows of up to 64*32*P values).
+// ROUTE > 0 (the selection's register count, experts <= 64*ROUTE): the expert
+// ids come from this token's router scores, selected here by
+// the workgroup itself (every workgroup of a token repeats the selection, which
+// costs less than a kernel boundary); the first workgroup of a token publishes
+// ids and weights.  Otherwise the ids are read from `ids`.
+template <int P, int R, int NS, int ROUTE>
 __global__ void __launch_bounds__(kGuThreads)
-moe_gate_up_kernel(moe_args a, const float *__restrict__ x, const int32_t *__restrict__ ids,
-                   float *__restrict__ act, int *__restrict__ flag, uint32_t rows_per_block) {
+moe_gate_up_kernel(moe_args a, const float *__restrict__ x, const int32_t *ids,
+                   const float *__restrict__ scores, const float *__restrict__ expert_scale,
+                   int32_t *ids_out, float *weights_out, float *__restrict__ act,
+                   int *__restrict__ flag, uint32_t rows_per_block) {
     extern __shared__ lev_f32x4 xs[];
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t slot = blockIdx.y, t = blockIdx.z;
     const uint32_t pairs = a.hidden / 64u;
     const uint32_t half = lane >> 5, lp = lane & 31u;
-    const int32_t *tids = ids + (uint64_t)t * a.top_k;
-    if (!expert_ids_ok(tids, a.top_k, slot, a.experts)) {
-        if (tid == 0) atomicOr(flag, kFlagBadExpertId);
-        return;
+    float *bsum = reinterpret_cast<float *>(xs + 16u * (pairs + 1u));
+    const float *xt = x + (uint64_t)t * a.hidden;
+
+    lev_f32x4 xv[NS];
+    lev_q4_stage_x_load<NS>(xt, pairs, tid, kGuThreads, xv);
+
+    uint32_t e;
+    if constexpr (ROUTE > 0) {
+        void *rl = reinterpret_cast<void *>(bsum + 2u * pairs);
+        rl = reinterpret_cast<void *>((reinterpret_cast<uintptr_t>(rl) + 7u) & ~(uintptr_t)7u);
+        const router_sel r = router_select_block<ROUTE>(scores + (uint64_t)t * a.experts, rl,
+                                                        a.experts, a.top_k);
+        e = r.ok ? r.sel_id[slot] : slot;
+        if (blockIdx.x == 0 && slot == 0) {   // first workgroup of the token publishes the selection
+            if (!r.ok && tid == 0) atomicOr(flag, kFlagNonFiniteScore);
+            if (tid < a.top_k) {
+                ids_out[(uint64_t)t * a.top_k + tid] = r.ok ? (int32_t)r.sel_id[tid] : (int32_t)tid;
+                weights_out[(uint64_t)t * a.top_k + tid] =
+                    r.ok ? router_weight(r, expert_scale, a.top_k, tid) : 0.f;
+            }
+        }
+    } else {
+        const int32_t *tids = ids + (uint64_t)t * a.top_k;
+        if (!expert_ids_ok(tids, a.top_k, slot, a.experts)) {
+            if (tid == 0) atomicOr(flag, kFlagBadExpertId);
+            return;
+        }
+        e = (uint32_t)tids[slot];
     }
-    const uint32_t e = (uint32_t)tids[slot];
     const uint64_t row_bytes = (uint64_t)pairs * 36u;
-    // lanes 0..31 walk the gate row, lanes 32..63 the up row of the same index
     const uint8_t *wbase = a.base + (half ? a.up_off + e * a.up_stride : a.gate_off + e * a.gate_stride);
     const uint32_t i_begin = blockIdx.x * rows_per_block;
     const uint32_t i_end = min(i_begin + rows_per_block, a.inter);
+    constexpr uint32_t kStep = kGuWaves * R;
 
-    lev_f32x4 xv[kLevStageSlots];
-    const float *xt = x + (uint64_t)t * a.hidden;
-    lev_q4_stage_x_load(xt, pairs, tid, kGuThreads, xv);
-
-    uint32_t Da[P][9], Db[P][9];
-    auto load_row = [&](uint32_t i, uint32_t (&D)[P][9]) {
-        const uint8_t *rp = wbase + (uint64_t)(i < i_end ? i : i_end - 1u) * row_bytes;
-#pragma unroll
-        for (int p = 0; p < P; ++p) {
-            uint32_t pr = lp + 32u * p;
-            lev_q4_load_pair(rp + (uint64_t)(pr < pairs ? pr : pairs - 1u) * 36u, D[p]);
-        }
-    };
-    uint32_t i = i_begin + wave;
-    load_row(i, Da);
-    lev_q4_stage_x_store(xt, xs, pairs, tid, kGuThreads, xv);
+    uint32_t Da[P][R][9], Db[P][R][9];
+    uint32_t i0 = i_begin + wave * R;
+    gu_load_rows<P, R>(wbase, row_bytes, i0, a.inter, pairs, lp, Da);
+    lev_q4_stage_x_store_sums<NS>(xt, xs, bsum, pairs, tid, kGuThreads, xv);
     __syncthreads();
-    if (i >= i_end) return;
 
     lev_q4_pair_x X[P];
 #pragma unroll
     for (int p = 0; p < P; ++p) {
-        uint32_t pr = lp + 32u * p;
-        lev_q4_fetch_x(xs, pairs, pr < pairs ? pr : pairs - 1u, X[p]);
-        if (pr >= pairs) {   // padding lanes contribute nothing
+        const uint32_t pr = lp + 32u * p;
+        const bool p_ok = pr < pairs;
+        lev_q4_fetch_x_sums(xs, bsum, pairs, p_ok ? pr : pairs - 1u, X[p]);
 #pragma unroll
-            for (int q = 0; q < 16; ++q) X[p].xr[q] = lev_f32x4{0.f, 0.f, 0.f, 0.f};
-            X[p].sum_a = X[p].sum_b = 0.f;
-        }
+        for (int q = 0; q < 16; ++q) X[p].xr[q] = p_ok ? X[p].xr[q] : lev_f32x4{0.f, 0.f, 0.f, 0.f};
+        X[p].sum_a = p_ok ? X[p].sum_a : 0.f;   // padding lanes contribute nothing
+        X[p].sum_b = p_ok ? X[p].sum_b : 0.f;
     }
     float *arow = act + ((uint64_t)t * a.top_k + slot) * a.inter;
-    auto finish_row = [&](uint32_t i, const uint32_t (&D)[P][9]) {
-        float acc = 0.f;
-#pragma unroll
-        for (int p = 0; p < P; ++p) acc += lev_q4_pair_dot(D[p], X[p]);
-        acc = lev_group_sum<32>(acc);
-        float g = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, acc), 31));
-        float u = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, acc), 63));
-        if (lane == 0) arow[i] = lev_gelu_up_value(g, u);
-    };
+    if (rows_per_block <= kStep) {   // one step per wave: nothing to prefetch
+        gu_finish_rows<P, R>(Da, X, arow, i0, i_end, lane);
+        return;
+    }
+    // unconditional prefetch (clamped past the end): a branch around the loads
+    // would make the compiler wait for them before the current rows are used
     while (true) {
-        uint32_t next = i + kGuWaves;
-        if (next < i_end) load_row(next, Db);
-        finish_row(i, Da);
+        uint32_t next = i0 + kStep;
+        gu_load_rows<P, R>(wbase, row_bytes, next, a.inter, pairs, lp, Db);
+        gu_finish_rows<P, R>(Da, X, arow, i0, i_end, lane);
         if (next >= i_end) break;
-        i = next;
-        next = i + kGuWaves;
-        if (next < i_end) load_row(next, Da);
-        finish_row(i, Db);
+        i0 = next;
+        next = i0 + kStep;
+        gu_load_rows<P, R>(wbase, row_bytes, next, a.inter, pairs, lp, Da);
+        gu_finish_rows<P, R>(Db, X, arow, i0, i_end, lane);
         if (next >= i_end) break;
-        i = next;
+        i0 = next;
     }
 }
 
@@ -410,21 +619,46 @@ moe_down_generic(moe_args a, const float *__restrict__ act, const int32_t *__res
     if (lane == 0) y[(uint64_t)t * a.hidden + row] = accum;
 }
 
-template <int P>
-hipError_t launch_gate_up(lev_ctx *ctx, const moe_args &a, const float *x, const int32_t *ids,
+constexpr uint32_t kRouteInKernelMax = 256;   // experts the gate/up kernel selects by itself
+
+// Where the expert ids of the gate/up kernel come from.
+struct gu_route {
+    const int32_t *ids;          // given ids, or NULL: select from scores
+    const float *scores, *expert_scale;
+    int32_t *ids_out;
+    float *weights_out;
+};
+
+template <int P, int R, int NS>
+hipError_t launch_gate_up(lev_ctx *ctx, const moe_args &a, const float *x, const gu_route &rt,
                           float *act, uint32_t tokens) {
-    // rows per workgroup: enough workgroups to cover every CU a few times at
-    // one token, more rows per workgroup (less re-staging of x) at many.
+    // rows per workgroup: about two workgroups per CU at one token, more rows
+    // per workgroup (less re-staging of x) at many
+    constexpr uint32_t step = kGuWaves * R;
     uint64_t slots = (uint64_t)a.top_k * tokens;
-    uint32_t want_blocks_per_slot = (uint32_t)(((uint64_t)ctx->num_cus * 4u + slots - 1) / slots);
+    uint32_t want_blocks_per_slot = (uint32_t)(((uint64_t)ctx->num_cus * 2u + slots - 1) / slots);
     if (want_blocks_per_slot < 1) want_blocks_per_slot = 1;
     uint32_t rows_per_block = (a.inter + want_blocks_per_slot - 1) / want_blocks_per_slot;
-    if (rows_per_block < (uint32_t)kGuWaves * 2u) rows_per_block = kGuWaves * 2u;
-    rows_per_block = (rows_per_block + kGuWaves - 1) / kGuWaves * kGuWaves;
+    rows_per_block = (rows_per_block + step - 1) / step * step;
     uint32_t chunks = (a.inter + rows_per_block - 1) / rows_per_block;
-    size_t lds = (size_t)16 * (a.hidden / 64u + 1u) * sizeof(lev_f32x4);
-    hipLaunchKernelGGL((moe_gate_up_kernel<P>), dim3(chunks, a.top_k, tokens), dim3(kGuThreads), lds,
-                       ctx->stream, a, x, ids, act, ctx->d_flag, rows_per_block);
+    const uint32_t pairs = a.hidden / 64u;
+    size_t lds = (size_t)16 * (pairs + 1u) * sizeof(lev_f32x4) + (size_t)2 * pairs * sizeof(float);
+    dim3 grid(chunks, a.top_k, tokens);
+    if (rt.ids) {
+        hipLaunchKernelGGL((moe_gate_up_kernel<P, R, NS, 0>), grid, dim3(kGuThreads), lds, ctx->stream,
+                           a, x, rt.ids, nullptr, nullptr, nullptr, nullptr, act, ctx->d_flag,
+                           rows_per_block);
+    } else {
+        lds += 8 + router_lds_bytes(a.experts);
+        if (a.experts <= 128u)
+            hipLaunchKernelGGL((moe_gate_up_kernel<P, R, NS, 2>), grid, dim3(kGuThreads), lds, ctx->stream,
+                               a, x, nullptr, rt.scores, rt.expert_scale, rt.ids_out, rt.weights_out,
+                               act, ctx->d_flag, rows_per_block);
+        else   // callers keep experts <= kRouteInKernelMax
+            hipLaunchKernelGGL((moe_gate_up_kernel<P, R, NS, 4>), grid, dim3(kGuThreads), lds, ctx->stream,
+                               a, x, nullptr, rt.scores, rt.expert_scale, rt.ids_out, rt.weights_out,
+                               act, ctx->d_flag, rows_per_block);
+    }
     return hipGetLastError();
 }
 
@@ -493,18 +727,21 @@ int check_pools(lev_ctx *ctx, const lev_moe_experts *p, uint32_t top_k, uint32_t
     return LEV_OK;
 }
 
-bool pools_fast(const moe_args &a, const float *x) {
+bool experts_fast(const moe_args &a, const float *x) {
     auto al4 = [&](uint64_t v) { return ((reinterpret_cast<uintptr_t>(a.base) + v) & 3u) == 0; };
-    return a.hidden % 64u == 0 && a.inter % 64u == 0 && a.hidden <= 8192u && a.inter <= 4096u &&
+    return a.hidden % 64u == 0 && a.inter % 64u == 0 && a.hidden <= 4096u && a.inter <= 4096u &&
            al4(a.gate_off) && al4(a.up_off) && al4(a.down_off) && a.gate_stride % 4u == 0 &&
            a.up_stride % 4u == 0 && a.down_stride % 4u == 0 &&
            (reinterpret_cast<uintptr_t>(x) & 15u) == 0;
 }
 
-hipError_t run_experts(lev_ctx *ctx, const moe_args &a, const float *x, const int32_t *ids,
-                       const float *weights, float *y, float *act, uint32_t tokens) {
+// rt.ids == NULL (selection inside the gate/up kernel) is only valid on the
+// fast path: callers test experts_fast() first.
+hipError_t run_experts(lev_ctx *ctx, const moe_args &a, const float *x, const gu_route &rt,
+                       const int32_t *ids, const float *weights, float *y, float *act,
+                       uint32_t tokens, bool fast) {
     hipError_t e;
-    if (!pools_fast(a, x) || (reinterpret_cast<uintptr_t>(act) & 15u)) {
+    if (!fast) {
         hipLaunchKernelGGL(moe_gate_up_generic, dim3((a.inter + 3) / 4, a.top_k, tokens), dim3(256), 0,
                            ctx->stream, a, x, ids, act, ctx->d_flag);
         if ((e = hipGetLastError()) != hipSuccess) return e;
@@ -512,11 +749,8 @@ hipError_t run_experts(lev_ctx *ctx, const moe_args &a, const float *x, const in
                            ctx->stream, a, act, ids, weights, y, ctx->d_flag);
         return hipGetLastError();
     }
-    const uint32_t gp = a.hidden / 64u;
-    if (gp <= 32) e = launch_gate_up<1>(ctx, a, x, ids, act, tokens);
-    else if (gp <= 64) e = launch_gate_up<2>(ctx, a, x, ids, act, tokens);
-    else if (gp <= 96) e = launch_gate_up<3>(ctx, a, x, ids, act, tokens);
-    else e = launch_gate_up<4>(ctx, a, x, ids, act, tokens);
+    if (a.hidden <= 2048u) e = launch_gate_up<1, 3, 1>(ctx, a, x, rt, act, tokens);
+    else e = launch_gate_up<2, 1, 2>(ctx, a, x, rt, act, tokens);
     if (e != hipSuccess) return e;
     const uint32_t dp = a.inter / 64u;
     if (dp > 32) return launch_down<64>(ctx, a, act, ids, weights, y, tokens);
@@ -526,42 +760,49 @@ hipError_t run_experts(lev_ctx *ctx, const moe_args &a, const float *x, const in
     return launch_down<4>(ctx, a, act, ids, weights, y, tokens);
 }
 
-// scratch layout: [counters u32[tokens] | scores f32[tokens*experts] | act f32[tokens*top_k*inter]]
+// scratch layout: [scores f32[tokens*experts] | act f32[tokens*top_k*inter]]
 struct moe_scratch {
-    uint32_t *counters;
     float *scores;
     float *act;
 };
 
 int get_scratch(lev_ctx *ctx, uint32_t tokens, uint32_t experts, uint32_t top_k, uint32_t inter,
                 moe_scratch *s) {
-    // the counter region has a fixed size so that it never overlaps what an
-    // earlier call with other dimensions used for scores or activations
-    (void)tokens;
-    size_t c_bytes = (size_t)65536 * 4;
     size_t s_bytes = ((size_t)tokens * experts * 4 + 255) & ~(size_t)255;
     size_t a_bytes = (size_t)tokens * top_k * inter * 4;
-    size_t before = ctx->scratch_bytes;
-    char *p = static_cast<char *>(lev_scratch(ctx, c_bytes + s_bytes + a_bytes));
+    char *p = static_cast<char *>(lev_scratch(ctx, s_bytes + a_bytes));
     if (!p) return lev_fail(ctx, LEV_ERR_EXCEEDS_WORKING_SET, "moe: scratch allocation failed");
-    if (ctx->scratch_bytes != before) {
-        // fresh buffer: the router's counters must start at zero (they return
-        // to zero by themselves after every launch)
-        hipError_t e = lev_zero_async(ctx, p, c_bytes);
-        if (e != hipSuccess) return lev_hip_check(ctx, e, "moe scratch clear");
-    }
-    s->counters = reinterpret_cast<uint32_t *>(p);
-    s->scores = reinterpret_cast<float *>(p + c_bytes);
-    s->act = reinterpret_cast<float *>(p + c_bytes + s_bytes);
+    s->scores = reinterpret_cast<float *>(p);
+    s->act = reinterpret_cast<float *>(p + s_bytes);
     return LEV_OK;
 }
 
-hipError_t run_router(lev_ctx *ctx, const float *wr, const float *x, const float *scale,
-                      float *scores, int32_t *ids, float *weights, uint32_t *counters,
-                      uint32_t hidden, uint32_t experts, uint32_t top_k, uint32_t tokens) {
-    hipLaunchKernelGGL(moe_router_kernel, dim3(experts, tokens), dim3(64), experts * sizeof(double),
-                       ctx->stream, wr, x, scale, scores, ids, weights, counters, ctx->d_flag, hidden,
-                       experts, top_k);
+hipError_t run_scores(lev_ctx *ctx, const float *wr, const float *x, float *scores, uint32_t hidden,
+                      uint32_t experts, uint32_t tokens) {
+    const int split = tokens <= 4u;
+    const uint32_t per_group = 4u * kScoreTokensPerWave;
+    const uint32_t groups = split ? 1u : (tokens + per_group - 1u) / per_group;
+    hipLaunchKernelGGL(moe_scores_kernel, dim3(experts, groups), dim3(256), 0, ctx->stream, wr, x,
+                       scores, hidden, experts, tokens, split);
+    return hipGetLastError();
+}
+
+hipError_t run_topk(lev_ctx *ctx, const float *scores, const float *scale, int32_t *ids,
+                    float *weights, uint32_t experts, uint32_t top_k, uint32_t tokens) {
+    const size_t lds = router_lds_bytes(experts);
+#define LEV_TOPK(J)                                                                               \
+    hipLaunchKernelGGL((moe_topk_kernel<J>), dim3(tokens), dim3(256), lds, ctx->stream, scores,   \
+                       scale, ids, weights, ctx->d_flag, experts, top_k)
+    if (experts <= 128u) LEV_TOPK(2);
+    else if (experts <= 256u) LEV_TOPK(4);
+    else if (experts <= 1024u) LEV_TOPK(16);
+    else {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&moe_topk_kernel<64>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        LEV_TOPK(64);
+    }
+#undef LEV_TOPK
     return hipGetLastError();
 }
 
@@ -579,15 +820,19 @@ extern "C" int lev_hip_moe_route_topk(lev_ctx *ctx, const float *d_router_w, con
         return lev_fail(ctx, LEV_ERR_BAD_DIMENSIONS,
                         "moe_route_topk: hidden %u, experts %u, topK %u, tokens %u", hidden, experts,
                         top_k, tokens);
-    moe_scratch s;
-    int st = get_scratch(ctx, tokens, experts, top_k, 0, &s);
+    float *scores = d_scores;
+    if (!scores) {
+        moe_scratch s;
+        int st = get_scratch(ctx, tokens, experts, top_k, 0, &s);
+        if (st != LEV_OK) return st;
+        scores = s.scores;
+    }
+    int st = lev_hip_check(ctx, run_scores(ctx, d_router_w, d_x, scores, hidden, experts, tokens),
+                           "moe router scores launch");
     if (st != LEV_OK) return st;
-    // With caller-provided scores the counters still live in the scratch.
-    float *scores = d_scores ? d_scores : s.scores;
     return lev_hip_check(ctx,
-                         run_router(ctx, d_router_w, d_x, d_expert_scale, scores, d_ids, d_weights,
-                                    s.counters, hidden, experts, top_k, tokens),
-                         "moe router launch");
+                         run_topk(ctx, scores, d_expert_scale, d_ids, d_weights, experts, top_k, tokens),
+                         "moe router top-k launch");
 }
 
 extern "C" int lev_hip_moe_experts_q4_0(lev_ctx *ctx, const lev_moe_experts *pools, const float *d_x,
@@ -606,7 +851,9 @@ extern "C" int lev_hip_moe_experts_q4_0(lev_ctx *ctx, const lev_moe_experts *poo
         if (st != LEV_OK) return st;
         act = s.act;
     }
-    return lev_hip_check(ctx, run_experts(ctx, a, d_x, d_ids, d_weights, d_y, act, tokens),
+    const bool fast = experts_fast(a, d_x) && (reinterpret_cast<uintptr_t>(act) & 15u) == 0u;
+    gu_route rt{d_ids, nullptr, nullptr, nullptr, nullptr};
+    return lev_hip_check(ctx, run_experts(ctx, a, d_x, rt, d_ids, d_weights, d_y, act, tokens, fast),
                          "moe experts launch");
 }
 
@@ -624,11 +871,21 @@ extern "C" int lev_hip_moe_layer_q4_0(lev_ctx *ctx, const lev_moe_experts *pools
     moe_scratch s;
     st = get_scratch(ctx, tokens, a.experts, top_k, a.inter, &s);
     if (st != LEV_OK) return st;
-    st = lev_hip_check(ctx,
-                       run_router(ctx, d_router_w, d_x, d_expert_scale, s.scores, d_ids, d_weights,
-                                  s.counters, a.hidden, a.experts, top_k, tokens),
-                       "moe router launch");
+    st = lev_hip_check(ctx, run_scores(ctx, d_router_w, d_x, s.scores, a.hidden, a.experts, tokens),
+                       "moe router scores launch");
     if (st != LEV_OK) return st;
-    return lev_hip_check(ctx, run_experts(ctx, a, d_x, d_ids, d_weights, d_y, s.act, tokens),
+    const bool fast = experts_fast(a, d_x);
+    gu_route rt{d_ids, nullptr, nullptr, nullptr, nullptr};
+    if (fast && tokens <= 4u && a.experts <= kRouteInKernelMax) {
+        // few tokens: the gate/up workgroups select the experts themselves
+        rt = gu_route{nullptr, s.scores, d_expert_scale, d_ids, d_weights};
+    } else {
+        st = lev_hip_check(ctx,
+                           run_topk(ctx, s.scores, d_expert_scale, d_ids, d_weights, a.experts, top_k,
+                                    tokens),
+                           "moe router top-k launch");
+        if (st != LEV_OK) return st;
+    }
+    return lev_hip_check(ctx, run_experts(ctx, a, d_x, rt, d_ids, d_weights, d_y, s.act, tokens, fast),
                          "moe experts launch");
 }
