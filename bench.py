@@ -33,10 +33,11 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0                # MI355X published HBM3E peak
 MFMA_F16_PEAK_TFLOPS = 2500.0        # MI355X published dense fp16 / bf16 peak
 
-# HBM bytes per launch of the dominant kernel (q4_0_gemv_pairs<64,1,false>,
-# 4096x4096) from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by the
-# same counter on a plain copy kernel of known size; None until measured.
-MEASURED_TRAFFIC_BYTES = None
+# HBM bytes per launch of the dominant kernel (q4_0_gemv_tile<64,1,2,true>,
+# 4096x4096) from rocprofv3 --pmc FETCH_SIZE (4696 KiB x 2.000) and WRITE_SIZE
+# (16 KiB x 1.000), each scaled by what the same counter reads for a plain
+# 256 MiB copy in the same run.
+MEASURED_TRAFFIC_BYTES = 9633792
 
 
 def parse_args():
@@ -46,8 +47,8 @@ def parse_args():
     p.add_argument("--warmup", type=int, default=200)
     p.add_argument("--skip-others", action="store_true", help="headline only")
     p.add_argument("--skip-cpu", action="store_true", help="no cpu_baseline leg")
-    p.add_argument("--only", default="", help="run one kernel family only (for profiling): "
-                   "q4_0 | q6_k | q4_k | gemm | moe1 | moe64 | copy")
+    p.add_argument("--only", default="", help="comma-separated kernel families to run (for "
+                   "profiling): q4_0, q6_k, q4_k, gemm, moe1, moe64, copy")
     return p.parse_args()
 
 
@@ -139,12 +140,16 @@ def main():
     result = {}
     others = {}
     only = args.only
+    only_set = {f for f in only.split(",") if f}
+
+    def want(*families):
+        return not only_set or any(f in only_set for f in families)
 
     # ------------------------------------------------------------------ Q4_0
     rows = cols = 4096
     q4_bytes_w = rows * cols // 32 * 18
     q4_alg_bytes = q4_bytes_w + cols * 4 + rows * 4            # 9,469,952
-    if only in ("", "q4_0"):
+    if want("q4_0"):
         ncopy = 64                                             # 604 MB ring > 256 MB cache
         ring = make_q4_0(ncopy * rows * cols // 32)
         x = torch.randn(cols, device=dev, generator=gen)
@@ -209,17 +214,22 @@ def main():
 
     if not args.skip_others or only:
         # ---------------------------------------------------- streaming probe
-        if only in ("", "copy"):
+        if want("copy"):
             buf = rand_bytes(1 << 30)
             sink = torch.zeros(4, dtype=torch.int32, device=dev)
             for nbytes, label in ((q4_bytes_w, "stream_read_9MiB_same_buffer"), (1 << 30, "stream_read_1GiB")):
                 run_other(label, lambda i: must(lib.lev_hip_stream_read_probe(
                     c, buf.data_ptr(), nbytes, sink.data_ptr(), 512)), nbytes, 50, 10)
             run_other("empty_kernel_launch", lambda i: must(lib.lev_hip_empty_launch(c)), 0, 1000, 100)
-            del buf
+            # plain copy of known size: the calibration kernel for the
+            # FETCH_SIZE / WRITE_SIZE counters (reads and writes 256 MiB each)
+            src = buf[: 1 << 28].view(torch.int32)
+            dst = torch.empty_like(src)
+            run_other("copy_256MiB", lambda i: dst.copy_(src), 2 << 28, 20, 5)
+            del buf, src, dst
 
         # ---------------------------------------------- Q4_0 large streaming
-        if only in ("", "q4_0"):
+        if want("q4_0"):
             rows2 = 32768
             nb2 = rows2 * cols // 32
             ring2 = make_q4_0(8 * nb2)
@@ -231,7 +241,7 @@ def main():
             del ring2
 
         # ------------------------------------------------------ Q6_K + argmax
-        if only in ("", "q6_k"):
+        if want("q6_k"):
             r6, nb6 = 32000, 32000 * 4096 // 256
             ring6 = make_q6_k(6 * nb6)
             x = torch.randn(cols, device=dev, generator=gen)
@@ -248,11 +258,11 @@ def main():
             del ring6
 
         # ------------------------------------------- RMSNorm + Q4_K N columns
-        if only in ("", "q4_k", "gemm"):
+        if want("q4_k", "gemm"):
             r4, nb4 = 12288, 12288 * 4096 // 256
             ncopy4 = 20
             ring4 = make_q4_k(ncopy4 * nb4)
-        if only in ("", "q4_k"):
+        if want("q4_k"):
             gain = 1.0 + 0.1 * torch.randn(cols, device=dev, generator=gen)
             for n in (1, 2, 3, 4, 8):
                 xn = torch.randn(n, cols, device=dev, generator=gen)
@@ -263,7 +273,7 @@ def main():
                     nb4 * 144 + cols * 4 + n * (cols * 4 + r4 * 4), 200, 20)
 
         # --------------------------------------------------- Q4_K prefill GEMM
-        if only in ("", "gemm"):
+        if want("gemm"):
             tokens = 512
             xh = torch.randn(tokens, cols, device=dev, generator=gen).to(torch.float16)
             yg = torch.empty(tokens, r4, device=dev)
@@ -277,11 +287,11 @@ def main():
                 c, ring4.data_ptr(), ring4.numel(), (i % ncopy4) * nb4 * 144, xh.data_ptr(), xh.numel(),
                 yg.data_ptr(), yg.numel(), cols, r4, tokens)),
                 nb4 * 144 + tokens * cols * 2 + tokens * r4 * 4, 30, 5, gemm_extra)
-        if only in ("", "q4_k", "gemm"):
+        if want("q4_k", "gemm"):
             del ring4
 
         # ------------------------------------------------------------- MoE
-        if only in ("", "moe1", "moe64"):
+        if want("moe1", "moe64"):
             hidden, inter, experts, top_k = 2048, 768, 128, 8
             gu = inter * (hidden // 32) * 18
             dn = hidden * (inter // 32) * 18
@@ -292,7 +302,7 @@ def main():
                      for p in pools_t]
             import ctypes as C
             for T in (1, 64):
-                if only and only != f"moe{T}":
+                if not want(f"moe{T}"):
                     continue
                 xt = torch.randn(T, hidden, device=dev, generator=gen)
                 yt = torch.empty(T, hidden, device=dev)
@@ -342,7 +352,7 @@ def main():
                    "in_dim": cols, "out_rows": rows, "algorithmic_bytes_per_step": q4_alg_bytes},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES,
-                     "kernel": "q4_0_gemv_pairs<64,1,false>",
+                     "kernel": "q4_0_gemv_tile<64,1,2,true>",
                      "note": "achieved = 9,469,952 B / mean launch-to-launch time of the timed "
                              "region (HIP events on the launch stream)"},
         "cpu_baseline": result.get("cpu_baseline"),
