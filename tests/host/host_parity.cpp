@@ -1,0 +1,424 @@
+// Parity tests of the C++ host mirror (leviathan_amd/host/leviathan_hip.hpp)
+// against the CPU oracle, written the way the reference's own Swift tests
+// exercise the same operators (Tests/.../main.swift; line numbers per case).
+//
+// Needs a GPU.  Prints one "ok <case>" line per case, "FAIL ..." and a
+// non-zero exit status otherwise.  `--list` prints the case names and exits
+// without touching the device.
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <functional>
+#include <map>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "leviathan_hip.hpp"
+
+extern "C" {
+#include "lev_oracle.h"
+}
+
+using namespace leviathan;
+
+namespace {
+
+int g_failures = 0;
+
+#define EXPECT(cond)                                                              \
+    do {                                                                          \
+        if (!(cond)) {                                                            \
+            std::printf("FAIL %s:%d: %s\n", __FILE__, __LINE__, #cond);           \
+            std::fflush(stdout);                                                  \
+            ++g_failures;                                                         \
+        }                                                                         \
+    } while (0)
+
+template <typename E, typename F>
+bool throws_q4(E code, F &&fn) {
+    try {
+        fn();
+    } catch (const Q4Exception &e) {
+        return e.code == code;
+    } catch (...) {
+        return false;
+    }
+    return false;
+}
+
+template <typename F>
+bool throws_geometry(F &&fn) {
+    try {
+        fn();
+    } catch (const Gemma4Error &e) {
+        return e.kind == Gemma4Error::badTensorGeometry;
+    } catch (...) {
+        return false;
+    }
+    return false;
+}
+
+double rel_err(const std::vector<float> &got, const std::vector<double> &ref) {
+    return levo_max_rel_err(got.data(), got.size(), ref.data(), ref.size());
+}
+
+// ---- standalone backends ----------------------------------------------------
+
+// main.swift:727-737: two rows of one block, d = +1 and d = -1, all codes 0.
+void q4_backend_2x32() {
+    std::vector<uint8_t> w = {0x00, 0x3C};
+    w.insert(w.end(), 16, 0);
+    w.push_back(0x00);
+    w.push_back(0xBC);
+    w.insert(w.end(), 16, 0);
+    std::vector<float> x(32);
+    levo_fill_uniform(7, x.data(), 32);
+    float sum = 0.f;
+    for (float v : x) sum += v;
+    auto [y, ev] = Q4HipBackend::matvecReporting(w, 2, 32, x);
+    EXPECT(y.size() == 2);
+    EXPECT(std::fabs(y[0] - (-8.f * sum)) < 1e-3f);
+    EXPECT(std::fabs(y[1] - (8.f * sum)) < 1e-3f);
+    EXPECT(ev.outDim == 2 && ev.inDim == 32);
+    EXPECT(!ev.deviceName.empty());
+    EXPECT(ev.commandStatus == "completed");
+}
+
+// main.swift:5106-5117: codes l | (16+l)<<4 against ones gives -16 exactly.
+void q4_backend_minus_16() {
+    std::vector<uint8_t> w = {0x00, 0x3C};
+    for (int l = 0; l < 16; ++l) w.push_back((uint8_t)((l | ((16 + l) << 4)) & 0xFF));
+    std::vector<float> x(32, 1.f);
+    EXPECT(Q4HipBackend::matvec(w, 1, 32, x)[0] == -16.f);
+}
+
+// main.swift:778-796 and Q4.swift:168-196: every guard fires before the device is used.
+void q4_backend_guards() {
+    std::vector<uint8_t> none;
+    std::vector<float> nox;
+    EXPECT(throws_q4(Q4Error::badDimensions, [&] { Q4HipBackend::matvecReporting(none, 8, 33, nox); }));
+    EXPECT(throws_q4(Q4Error::badDimensions, [&] { Q4HipBackend::matvecReporting(none, 8, 32, nox); }));
+    EXPECT(throws_q4(Q4Error::badDimensions, [&] { Q4HipBackend::matvecReporting(none, 0, 32, nox); }));
+    std::vector<uint8_t> w(8 * 18, 0);
+    std::vector<float> three(3, 0.f);
+    EXPECT(throws_q4(Q4Error::wrongInputCount, [&] { Q4HipBackend::matvecReporting(w, 8, 32, three); }));
+    std::vector<float> bad(32, 0.f);
+    bad[5] = NAN;
+    EXPECT(throws_q4(Q4Error::nonFiniteInput, [&] { Q4HipBackend::matvecReporting(w, 8, 32, bad); }));
+    bad[5] = INFINITY;
+    EXPECT(throws_q4(Q4Error::nonFiniteInput, [&] { Q4HipBackend::matvecReporting(w, 8, 32, bad); }));
+}
+
+// main.swift:1091-1120: the hand-computed Q6_K row, -315 exactly.
+void q6_backend_minus_315() {
+    std::vector<uint8_t> b(210, 0);
+    b[208] = 0x00; b[209] = 0x3C;
+    b[192] = 3; b[193] = 0xFD; b[196] = 2; b[200] = 3; b[204] = 2;
+    b[0] = 0x21; b[128] = 0x03; b[64] = 0x21; b[160] = 0x01;
+    std::vector<float> x(256, 0.f);
+    x[0] = 1; x[16] = -1; x[64] = 2; x[128] = -2; x[192] = 4;
+    auto [y, ev] = Q6HipBackend::matvecReporting(b, 1, 256, x);
+    EXPECT(y.size() == 1 && y[0] == -315.f);
+    EXPECT(ev.inDim == 256);
+    std::vector<float> shortx(255, 0.f);
+    EXPECT(throws_q4(Q4Error::wrongInputCount, [&] { Q6HipBackend::matvecReporting(b, 1, 256, shortx); }));
+    EXPECT(throws_q4(Q4Error::badDimensions, [&] { Q6HipBackend::matvecReporting(b, 1, 128, x); }));
+}
+
+// Seeded 64x512 against the FP64 oracle, gate 1e-4 (Q4Lowering.swift:887-937).
+void q4_backend_seeded() {
+    const int rows = 64, cols = 512;
+    std::vector<uint8_t> w((size_t)rows * cols / 32 * 18);
+    levo_synth_q4_0(21, 0.02f, w.data(), w.size() / 18);
+    std::vector<float> x(cols);
+    levo_fill_uniform(22, x.data(), cols);
+    std::vector<double> ref(rows);
+    EXPECT(levo_q4_0_matvec_f64(w.data(), w.size(), rows, cols, x.data(), cols, ref.data()) == 0);
+    EXPECT(rel_err(Q4HipBackend::matvec(w, rows, cols, x), ref) < 1e-4);
+}
+
+// ---- runner operators --------------------------------------------------------
+
+struct Model {
+    // one weight buffer: a Q4_0 matrix, a Q6_K matrix, an F32 norm weight, an
+    // F32 router and the expert tensors of layer 0, at 256-byte aligned offsets
+    static constexpr int hidden = 256, inter = 128, experts = 8, topK = 2, vocab = 96;
+    std::vector<uint8_t> bytes;
+    std::map<std::string, TensorRef> table;
+    MoEBinding binding;
+    int64_t gu_slice, dn_slice;
+
+    int64_t add(const std::string &name, GGMLTensorType t, int64_t inDim, int64_t outDim, int64_t nexp,
+                const std::function<void(uint8_t *, size_t)> &fill) {
+        size_t start = (bytes.size() + 255) & ~(size_t)255;
+        size_t n = (size_t)(inDim / elementsPerBlock(t)) * bytesPerBlock(t) * outDim * nexp;
+        bytes.resize(start + n);
+        fill(bytes.data() + start, n);
+        TensorRef r;
+        r.type = t; r.offset = (int64_t)start; r.end = (int64_t)(start + n);
+        r.inDim = inDim; r.outDim = outDim; r.experts = nexp;
+        table[name] = r;
+        return (int64_t)start;
+    }
+
+    Model() {
+        add("blk.0.attn_q.weight", GGMLTensorType::q4_0, hidden, hidden, 1,
+            [](uint8_t *p, size_t n) { levo_synth_q4_0(31, 0.02f, p, n / 18); });
+        add("output.weight", GGMLTensorType::q6_K, hidden, vocab, 1,
+            [](uint8_t *p, size_t n) { levo_synth_q6_k(32, 0.01f, p, n / 210); });
+        add("blk.0.ffn_norm.weight", GGMLTensorType::float32, hidden, 1, 1,
+            [](uint8_t *p, size_t n) { levo_fill_normal(33, 1.f, 0.1f, reinterpret_cast<float *>(p), n / 4); });
+        add("blk.0.ffn_gate_inp.weight", GGMLTensorType::float32, hidden, experts, 1,
+            [](uint8_t *p, size_t n) { levo_fill_normal(34, 0.f, 0.02f, reinterpret_cast<float *>(p), n / 4); });
+        // fused gate|up [2I, H] per expert, as the reference stores it
+        int64_t gu = add("blk.0.ffn_gate_up_exps.weight", GGMLTensorType::q4_0, hidden, 2 * inter, experts,
+                         [](uint8_t *p, size_t n) { levo_synth_q4_0(35, 0.02f, p, n / 18); });
+        int64_t dn = add("blk.0.ffn_down_exps.weight", GGMLTensorType::q4_0, inter, hidden, experts,
+                         [](uint8_t *p, size_t n) { levo_synth_q4_0(36, 0.02f, p, n / 18); });
+        gu_slice = (int64_t)2 * inter * (hidden / 32) * 18;
+        dn_slice = (int64_t)hidden * (inter / 32) * 18;
+        binding.gateOffset = gu;
+        binding.upOffset = gu + gu_slice / 2;
+        binding.downOffset = dn;
+        binding.gateStride = binding.upStride = gu_slice;
+        binding.downStride = dn_slice;
+        binding.hidden = hidden;
+        binding.expertIntermediate = inter;
+        binding.experts = experts;
+        binding.topK = topK;
+    }
+    const uint8_t *at(const std::string &name) const { return bytes.data() + table.at(name).offset; }
+};
+
+void runner_matvec(Runner &r, const Model &m) {
+    const int H = Model::hidden;
+    std::vector<float> x(H);
+    levo_fill_normal(41, 0.f, 1.f, x.data(), H);
+    DeviceBuffer dx = r.makeBuffer(x), dy = r.makeBuffer((int64_t)H * 4 + 256);
+    r.matvec("blk.0.attn_q.weight", dx, H, dy, H + 64);
+    std::vector<double> ref(H);
+    const TensorRef &t = m.table.at("blk.0.attn_q.weight");
+    levo_q4_0_matvec_f64(m.at("blk.0.attn_q.weight"), (size_t)(t.end - t.offset), H, H, x.data(), H, ref.data());
+    EXPECT(rel_err(r.read<float>(dy, H), ref) < 1e-4);
+
+    // a row range: rows 32.. through extraOffset, written at a shifted output binding
+    const int64_t row_bytes = H / 32 * 18;
+    r.matvec("blk.0.attn_q.weight", dx, H, dy, H + 64, 32 * row_bytes, 16, 256);
+    std::vector<float> all = r.read<float>(dy, H + 64);
+    std::vector<float> part(all.begin() + 64, all.begin() + 80);
+    std::vector<double> pref(ref.begin() + 32, ref.begin() + 48);
+    EXPECT(rel_err(part, pref) < 1e-4);
+
+    // Q6_K head
+    DeviceBuffer dl = r.makeBuffer((int64_t)Model::vocab * 4);
+    r.matvec("output.weight", dx, H, dl, Model::vocab);
+    std::vector<double> lref(Model::vocab);
+    const TensorRef &o = m.table.at("output.weight");
+    levo_q6_k_matvec_f64(m.at("output.weight"), (size_t)(o.end - o.offset), Model::vocab, H, x.data(), H,
+                         lref.data());
+    EXPECT(rel_err(r.read<float>(dl, Model::vocab), lref) < 1e-4);
+
+    // guards of Gemma4.swift:2588-2627, each before any launch
+    EXPECT(throws_geometry([&] { r.matvec("missing.weight", dx, H, dy, H); }));
+    EXPECT(throws_geometry([&] { r.matvec("blk.0.attn_q.weight", dx, H - 1, dy, H); }));          // xCount
+    EXPECT(throws_geometry([&] { r.matvec("blk.0.attn_q.weight", dx, H, dy, H - 1); }));          // yCapacity
+    EXPECT(throws_geometry([&] { r.matvec("blk.0.attn_q.weight", dx, H, dy, H, 0, std::nullopt, 4); }));  // y offset % 256
+    EXPECT(throws_geometry([&] { r.matvec("blk.0.attn_q.weight", dx, H, dy, H, row_bytes, H); }));       // beyond extent
+    EXPECT(throws_geometry([&] { r.matvec("blk.0.attn_q.weight", dx, H, dy, H, -18); }));         // before the tensor
+    EXPECT(throws_geometry([&] { r.matvec("blk.0.attn_q.weight", dx, H, dy, H, 0, 0); }));        // zero rows
+    r.flushOpenSegment();   // nothing failed on the device
+}
+
+void runner_elementwise(Runner &r, const Model &m) {
+    const int H = Model::hidden, V = 3;
+    std::vector<float> x((size_t)V * H);
+    levo_fill_normal(51, 0.f, 1.f, x.data(), x.size());
+    DeviceBuffer dx = r.makeBuffer(x), dy = r.makeBuffer((int64_t)V * H * 4);
+    r.rmsnorm(dx, dy, H, V, std::string("blk.0.ffn_norm.weight"));
+    std::vector<float> y = r.read<float>(dy, (size_t)V * H);
+    const float *gain = reinterpret_cast<const float *>(m.at("blk.0.ffn_norm.weight"));
+    for (int v = 0; v < V; ++v) {
+        std::vector<double> ref(H);
+        levo_rmsnorm_f64(x.data() + (size_t)v * H, gain, 1e-6, H, ref.data());
+        std::vector<float> got(y.begin() + (size_t)v * H, y.begin() + (size_t)(v + 1) * H);
+        EXPECT(rel_err(got, ref) < 1e-5);
+    }
+    // lev-model lib.rs:431-435: x = 2, no weight -> 1 (times w = 0.5 there)
+    std::vector<float> twos(H, 2.f);
+    DeviceBuffer d2 = r.makeBuffer(twos), dn = r.makeBuffer((int64_t)H * 4);
+    r.rmsnorm(d2, dn, H, 1, std::nullopt);
+    for (float v : r.read<float>(dn, H)) EXPECT(std::fabs(v - 1.f) < 1e-5f);
+    EXPECT(throws_geometry([&] { r.rmsnorm(dx, dy, H, V + 1, std::nullopt); }));
+    EXPECT(throws_geometry([&] { r.rmsnorm(dx, dy, H / 2, 1, std::string("blk.0.ffn_norm.weight")); }));
+    EXPECT(throws_geometry([&] { r.rmsnorm(dx, dy, H, 1, std::string("blk.0.attn_q.weight")); }));
+
+    // geluUp: main.swift:8947-8950 and 6680-6690
+    std::vector<float> gu = {1.f, -20.f, 1e30f, -1e30f, 1e-30f, 1e20f, 0.5f, -0.5f,
+                             1.f, 3.f, 2.f, 2.f, 2.f, 2.f, 4.f, 4.f};
+    DeviceBuffer dgu = r.makeBuffer(gu), dact = r.makeBuffer((int64_t)8 * 4);
+    r.geluUp(dgu, dact, 8);
+    std::vector<float> act = r.read<float>(dact, 8);
+    EXPECT(std::fabs(act[0] - 0.841192f) < 1e-6f);
+    EXPECT(act[1] == 0.f || std::fabs(act[1]) < 1e-30f);
+    for (int i = 0; i < 8; ++i) {
+        EXPECT(std::isfinite(act[i]));
+        float want = levo_gelu_up_f32(gu[i], gu[8 + i]);
+        EXPECT(std::fabs(act[i] - want) <= 1e-6f * std::fmax(1.f, std::fabs(want)));
+    }
+    EXPECT(throws_geometry([&] { r.geluUp(dgu, dact, 9); }));
+
+    // axpy: Gemma4.swift:3115-3140
+    std::vector<float> a = {1, 2, 3, 4, 5, 6, 7, 8}, b = {10, 20, 30, 40};
+    DeviceBuffer da = r.makeBuffer(a), db = r.makeBuffer(b);
+    r.axpy(da, db, 0.5f, 4, 16);   // x from element 4
+    std::vector<float> got = r.read<float>(db, 4);
+    EXPECT(got[0] == 12.5f && got[1] == 23.f && got[2] == 33.5f && got[3] == 44.f);
+    EXPECT(throws_geometry([&] { r.axpy(da, db, 1.f, 0); }));
+    EXPECT(throws_geometry([&] { r.axpy(da, db, NAN, 4); }));
+    EXPECT(throws_geometry([&] { r.axpy(da, db, 1.f, 4, 2); }));     // offset % 4
+    EXPECT(throws_geometry([&] { r.axpy(da, db, 1.f, 4, 20); }));    // beyond x
+    EXPECT(throws_geometry([&] { r.axpy(da, db, 1.f, 5); }));        // beyond y
+}
+
+void runner_moe(Runner &r, const Model &m) {
+    const int H = Model::hidden, I = Model::inter, K = Model::topK;
+    std::vector<float> x(H);
+    levo_fill_normal(61, 0.f, 1.f, x.data(), H);
+    DeviceBuffer dx = r.makeBuffer(x), dy = r.makeBuffer((int64_t)H * 4);
+
+    // router: ids bit-exact, weights to 1e-6 (Gemma4.swift:3795-3810)
+    auto [topIdx, weights] = r.routeTopK("blk.0.ffn_gate_inp.weight", dx, K);
+    std::vector<float> scores(Model::experts);
+    levo_f32_matvec(reinterpret_cast<const float *>(m.at("blk.0.ffn_gate_inp.weight")), Model::experts, H,
+                    x.data(), scores.data());
+    std::vector<int32_t> rid(K);
+    std::vector<float> rw(K);
+    EXPECT(levo_router_topk(scores.data(), Model::experts, K, nullptr, rid.data(), rw.data()) == 0);
+    for (int k = 0; k < K; ++k) {
+        EXPECT(topIdx[k] == rid[k]);
+        EXPECT(std::fabs(weights[k] - rw[k]) < 1e-6f);
+    }
+
+    // routed experts against the FP64 oracle (MoESIMDLowering.swift:986-1030), gate 1e-4
+    r.runMoeBatchedRouted(dx, dy, topIdx, weights, m.binding);
+    std::vector<float> y = r.read<float>(dy, H);
+    const uint8_t *gate = m.bytes.data() + m.binding.gateOffset;
+    const uint8_t *up = m.bytes.data() + m.binding.upOffset;
+    const uint8_t *down = m.bytes.data() + m.binding.downOffset;
+    std::vector<double> yref(H), g((size_t)K * I), u((size_t)K * I), a((size_t)K * I), d((size_t)K * H);
+    EXPECT(levo_moe_experts_f64(gate, up, down, (size_t)m.gu_slice, (size_t)m.gu_slice, (size_t)m.dn_slice, H, I,
+                                K, rid.data(), rw.data(), x.data(), yref.data(), g.data(), u.data(), a.data(),
+                                d.data()) == 0);
+    EXPECT(rel_err(y, yref) < 1e-4);
+
+    // the same through the per-slot operators, as forwardLayer's serial loop does
+    // (Gemma4.swift:3856-3880): expertMatvec(gate_up) -> geluUp -> expertMatvec(down) -> axpy
+    DeviceBuffer dgu = r.makeBuffer((int64_t)2 * I * 4), dact = r.makeBuffer((int64_t)I * 4),
+                 ddn = r.makeBuffer((int64_t)H * 4);
+    DeviceBuffer dacc = r.makeBuffer(std::vector<float>(H, 0.f));
+    for (int k = 0; k < K; ++k) {
+        r.expertMatvec("blk.0.ffn_gate_up_exps.weight", 0, topIdx[k], dx, H, dgu, 2 * I);
+        r.geluUp(dgu, dact, I);
+        r.expertMatvec("blk.0.ffn_down_exps.weight", 0, topIdx[k], dact, I, ddn, H);
+        r.axpy(ddn, dacc, weights[k], H);
+    }
+    std::vector<float> yserial = r.read<float>(dacc, H);
+    EXPECT(rel_err(yserial, yref) < 1e-4);
+    std::vector<double> yd(y.begin(), y.end());
+    EXPECT(rel_err(yserial, yd) < 1e-5);   // the composite and the serial loop agree
+
+    // guards: MoEModelBinding.offsets and Gemma4.swift:2094-2110
+    EXPECT(throws_geometry([&] { r.runMoeBatchedRouted(dx, dy, {0, 0}, weights, m.binding); }));
+    EXPECT(throws_geometry([&] { r.runMoeBatchedRouted(dx, dy, {0, Model::experts}, weights, m.binding); }));
+    EXPECT(throws_geometry([&] { r.runMoeBatchedRouted(dx, dy, {0, -1}, weights, m.binding); }));
+    EXPECT(throws_geometry([&] { r.runMoeBatchedRouted(dx, dy, {0}, weights, m.binding); }));
+    EXPECT(throws_geometry([&] { r.runMoeBatchedRouted(dx, dy, topIdx, {0.5f}, m.binding); }));
+    EXPECT(throws_geometry([&] { r.runMoeBatchedRouted(dx, dy, topIdx, {0.5f, NAN}, m.binding); }));
+    EXPECT(throws_geometry([&] { r.runMoeBatchedRouted(dx, dx, topIdx, weights, m.binding); }));
+    EXPECT(throws_geometry([&] { r.expertMatvec("blk.0.attn_q.weight", 0, 0, dx, H, dgu, 2 * I); }));
+    EXPECT(throws_geometry([&] { r.expertMatvec("blk.0.ffn_gate_up_exps.weight", 1, 0, dx, H, dgu, 2 * I); }));
+    EXPECT(throws_geometry([&] { r.expertMatvec("blk.0.ffn_gate_up_exps.weight", 0, Model::experts, dx, H, dgu, 2 * I); }));
+    EXPECT(throws_geometry([&] { r.expertMatvec("blk.0.ffn_gate_up_exps.weight", 0, 0, dx, H, dgu, 2 * I - 1); }));
+    r.flushOpenSegment();
+}
+
+// main.swift:8925-8946: 32/32/top-1, gate 16, up 2, act 32, down 512 -- exact.
+void runner_moe_hand_computed(Runner &) {
+    auto rows = [](uint8_t lo, uint8_t hi, uint8_t q) {
+        std::vector<uint8_t> out;
+        for (int r = 0; r < 32; ++r) {
+            out.push_back(lo);
+            out.push_back(hi);
+            out.insert(out.end(), 16, q);
+        }
+        return out;
+    };
+    std::vector<uint8_t> bytes = rows(0x00, 0x3C, 0x98), up = rows(0x00, 0x30, 0x98), down = rows(0x00, 0x38, 0x99);
+    MoEBinding b;
+    b.gateOffset = 0;
+    b.upOffset = (int64_t)bytes.size();
+    bytes.insert(bytes.end(), up.begin(), up.end());
+    b.downOffset = (int64_t)bytes.size();
+    bytes.insert(bytes.end(), down.begin(), down.end());
+    b.gateStride = b.upStride = b.downStride = 32 * 18;
+    b.hidden = 32; b.expertIntermediate = 32; b.experts = 1; b.topK = 1;
+    Runner r2;
+    r2.bindWeights(bytes, {});
+    DeviceBuffer dx = r2.makeBuffer(std::vector<float>(32, 1.f)), dy = r2.makeBuffer((int64_t)32 * 4);
+    r2.runMoeBatchedRouted(dx, dy, {0}, {1.0f}, b);
+    for (float v : r2.read<float>(dy, 32)) EXPECT(v == 512.f);
+    r2.runMoeBatchedRouted(dx, dy, {0}, {0.5f}, b);
+    for (float v : r2.read<float>(dy, 32)) EXPECT(v == 256.f);
+}
+
+struct Case {
+    const char *name;
+    std::function<void()> run;
+};
+
+}  // namespace
+
+int main(int argc, char **argv) {
+    Model model;
+    std::unique_ptr<Runner> runner;
+    auto R = [&]() -> Runner & {
+        if (!runner) {
+            runner = std::make_unique<Runner>(0);
+            runner->bindWeights(model.bytes, model.table);
+        }
+        return *runner;
+    };
+    std::vector<Case> cases = {
+        {"q4_backend_2x32", q4_backend_2x32},
+        {"q4_backend_minus_16", q4_backend_minus_16},
+        {"q4_backend_guards", q4_backend_guards},
+        {"q6_backend_minus_315", q6_backend_minus_315},
+        {"q4_backend_seeded", q4_backend_seeded},
+        {"runner_matvec", [&] { runner_matvec(R(), model); }},
+        {"runner_elementwise", [&] { runner_elementwise(R(), model); }},
+        {"runner_moe", [&] { runner_moe(R(), model); }},
+        {"runner_moe_hand_computed", [&] { runner_moe_hand_computed(R()); }},
+    };
+    if (argc > 1 && std::strcmp(argv[1], "--list") == 0) {
+        for (auto &c : cases) std::printf("%s\n", c.name);
+        return 0;
+    }
+    for (auto &c : cases) {
+        std::printf("run %s\n", c.name);
+        std::fflush(stdout);
+        int before = g_failures;
+        try {
+            c.run();
+        } catch (const std::exception &e) {
+            std::printf("FAIL %s: unexpected exception: %s\n", c.name, e.what());
+            ++g_failures;
+        }
+        if (g_failures == before) std::printf("ok %s\n", c.name);
+        std::fflush(stdout);
+    }
+    runner.reset();
+    std::printf(g_failures ? "FAILED %d check(s)\n" : "all host parity cases passed\n", g_failures);
+    return g_failures ? 1 : 0;
+}
