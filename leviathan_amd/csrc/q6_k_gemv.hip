@@ -125,6 +125,39 @@ __device__ __forceinline__ void q6_fetch_x(const lev_f32x4 *xs, uint32_t units, 
     x.sum_hi = b;
 }
 
+// ---- argmax + margin (lev-forge/src/ops.rs:479-516) ------------------------
+
+struct top2 {
+    float best, second;
+    uint32_t idx;
+};
+
+__device__ __forceinline__ top2 top2_merge(top2 a, top2 b) {
+    // take b when strictly larger, or equal with the lower index (ops.rs:508)
+    bool take = b.best > a.best || (b.best == a.best && b.idx < a.idx);
+    top2 r;
+    r.best = take ? b.best : a.best;
+    r.idx = take ? b.idx : a.idx;
+    float other = take ? fmaxf(a.best, b.second) : fmaxf(b.best, a.second);
+    r.second = fmaxf(other, take ? a.second : b.second);
+    return r;
+}
+
+
+__device__ __forceinline__ top2 top2_wave(top2 m) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        top2 o;
+        o.best = __shfl_xor(m.best, off);
+        o.second = __shfl_xor(m.second, off);
+        o.idx = __shfl_xor(m.idx, off);
+        m = top2_merge(m, o);
+    }
+    return m;
+}
+
+constexpr float kTop2Floor = -INFINITY;
+
 template <int L, int P>
 __device__ __forceinline__ void q6_load_row(const uint8_t *__restrict__ w, uint64_t row_bytes,
                                             uint32_t row, uint32_t rows, uint32_t lu,
@@ -144,34 +177,55 @@ __device__ __forceinline__ void q6_load_row(const uint8_t *__restrict__ w, uint6
 template <int L, int P>
 __device__ __forceinline__ void q6_finish_row(float *__restrict__ y, uint32_t row, uint32_t rows,
                                               uint32_t lu, const q6_unit_w (&W)[P],
-                                              const q6_unit_x (&X)[P]) {
+                                              const q6_unit_x (&X)[P], top2 &m) {
     float acc = 0.f;
 #pragma unroll
     for (int p = 0; p < P; ++p) acc += q6_unit_dot(W[p], X[p], (lu + p * L) & 3u);
     acc = lev_group_sum<L>(acc);
-    if (lu == L - 1 && row < rows) y[row] = acc;
+    if (lu % L == L - 1 && row < rows) {
+        y[row] = acc;
+        // running top two of the rows this lane finishes (rows ascend, so a
+        // tie keeps the earlier, lower index)
+        if (acc > m.best) {
+            m.second = m.best;
+            m.best = acc;
+            m.idx = row;
+        } else if (acc > m.second) {
+            m.second = acc;
+        }
+    }
 }
 
-// L lanes per row, P passes of L units per row (units <= L*P), one row per
-// wave-group and tile; persistent workgroups, weights double-buffered.
-template <int L, int P>
+// L lanes per row-part, P passes of L units, S waves share a row (units <=
+// S*L*P; S > 1 only with L = 64): with S = 2 a 4096-wide row costs each lane
+// one unit instead of two, which brings the kernel under 128 VGPRs and five
+// waves per SIMD instead of three.  Persistent workgroups, weights
+// double-buffered.
+// partials (optional): the workgroup's top two logits and the index of the
+// best, one float4 {best, second, idx bits, 0} per workgroup, for the greedy
+// token epilogue.
+template <int L, int P, int S>
 __global__ void __launch_bounds__(kThreads)
 q6_k_gemv_units(const uint8_t *__restrict__ w, const float *__restrict__ x, float *__restrict__ y,
-                uint32_t units, uint32_t rows) {
+                uint32_t units, uint32_t rows, lev_f32x4 *__restrict__ partials) {
     extern __shared__ lev_f32x4 xs[];
     constexpr int G = LEV_WAVE / L;
-    constexpr uint32_t kRowsPerTile = kWaves * G;
+    constexpr uint32_t kRowsPerTile = kWaves * G / S;
+    static_assert(S == 1 || L == LEV_WAVE, "rows are shared by whole waves only");
+    __shared__ float part[2][S > 1 ? kWaves : 1];
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & (LEV_WAVE - 1);
     const uint32_t wave = tid / LEV_WAVE;
-    const uint32_t grp = lane / L, lu = lane % L;
+    const uint32_t grp = lane / L;
+    const uint32_t lu = (wave % S) * (L * P) + lane % L;   // first unit of this lane
     const uint64_t row_bytes = (uint64_t)(units >> 3) * 210u;
-    const uint32_t in_tile = wave * G + grp;
+    const uint32_t in_tile = (wave / S) * G + grp;
     const uint32_t step = gridDim.x * kRowsPerTile;
 
     uint32_t base = blockIdx.x * kRowsPerTile;
-    if (base >= rows) return;
+    if (base >= rows) return;   // never: the grid has at most one workgroup per tile
 
+    top2 m{kTop2Floor, kTop2Floor, 0xFFFFFFFFu};
     q6_unit_w Wa[P], Wb[P];
     q6_load_row<L, P>(w, row_bytes, base + in_tile, rows, lu, units, Wa);
     q6_stage_x(x, xs, units, tid);
@@ -190,17 +244,92 @@ q6_k_gemv_units(const uint8_t *__restrict__ w, const float *__restrict__ x, floa
         }
     }
 
+    // The prefetch is unconditional (clamped past the end): a branch around the
+    // loads would make the compiler wait for them before the current row is used.
+    uint32_t buf = 0;
+    auto finish = [&](uint32_t row0, const q6_unit_w (&W)[P]) {
+        if constexpr (S == 1) {
+            q6_finish_row<L, P>(y, row0 + in_tile, rows, lu, W, X, m);
+        } else {
+            // the S waves of a row leave their parts in LDS; one thread per row
+            // adds them in wave order.  Two part buffers: one barrier per tile.
+            float acc = 0.f;
+#pragma unroll
+            for (int p = 0; p < P; ++p) acc += q6_unit_dot(W[p], X[p], (lu + p * L) & 3u);
+            acc = lev_group_sum<L>(acc);
+            if (lane == LEV_WAVE - 1) part[buf][wave] = acc;
+            __syncthreads();
+            if (tid < kRowsPerTile && row0 + tid < rows) {
+                float sum = part[buf][tid * S];
+#pragma unroll
+                for (int k = 1; k < S; ++k) sum += part[buf][tid * S + k];
+                y[row0 + tid] = sum;
+                if (sum > m.best) {
+                    m.second = m.best;
+                    m.best = sum;
+                    m.idx = row0 + tid;
+                } else if (sum > m.second) {
+                    m.second = sum;
+                }
+            }
+            buf ^= 1u;
+        }
+    };
     while (true) {
         uint32_t next = base + step;
-        if (next < rows) q6_load_row<L, P>(w, row_bytes, next + in_tile, rows, lu, units, Wb);
-        q6_finish_row<L, P>(y, base + in_tile, rows, lu, Wa, X);
+        q6_load_row<L, P>(w, row_bytes, next + in_tile, rows, lu, units, Wb);
+        finish(base, Wa);
         if (next >= rows) break;
         base = next;
         next = base + step;
-        if (next < rows) q6_load_row<L, P>(w, row_bytes, next + in_tile, rows, lu, units, Wa);
-        q6_finish_row<L, P>(y, base + in_tile, rows, lu, Wb, X);
+        q6_load_row<L, P>(w, row_bytes, next + in_tile, rows, lu, units, Wa);
+        finish(base, Wb);
         if (next >= rows) break;
         base = next;
+    }
+    if (partials) {
+        __shared__ float s_best[kWaves], s_second[kWaves];
+        __shared__ uint32_t s_idx[kWaves];
+        m = top2_wave(m);
+        if (lane == 0) {
+            s_best[wave] = m.best;
+            s_second[wave] = m.second;
+            s_idx[wave] = m.idx;
+        }
+        __syncthreads();
+        if (tid == 0) {
+            top2 r{s_best[0], s_second[0], s_idx[0]};
+            for (int k = 1; k < kWaves; ++k) r = top2_merge(r, top2{s_best[k], s_second[k], s_idx[k]});
+            partials[blockIdx.x] = lev_f32x4{r.best, r.second, __builtin_bit_cast(float, r.idx), 0.f};
+        }
+    }
+}
+
+// One workgroup: merges the per-workgroup partials of the GEMV.
+__global__ void __launch_bounds__(256)
+argmax_partials_kernel(const lev_f32x4 *__restrict__ partials, uint32_t n,
+                       uint32_t *__restrict__ out_idx, float *__restrict__ out_margin) {
+    __shared__ float s_best[4], s_second[4];
+    __shared__ uint32_t s_idx[4];
+    const uint32_t t = threadIdx.x;
+    top2 m{kTop2Floor, kTop2Floor, 0xFFFFFFFFu};
+    for (uint32_t i = t; i < n; i += 256u) {
+        lev_f32x4 p = partials[i];
+        const float idx_bits = p.z;   // a copy: bit_cast straight from a vector element reads element 0
+        m = top2_merge(m, top2{p.x, p.y, __float_as_uint(idx_bits)});
+    }
+    m = top2_wave(m);
+    if ((t & 63u) == 0) {
+        s_best[t >> 6] = m.best;
+        s_second[t >> 6] = m.second;
+        s_idx[t >> 6] = m.idx;
+    }
+    __syncthreads();
+    if (t == 0) {
+        top2 r{s_best[0], s_second[0], s_idx[0]};
+        for (int k = 1; k < 4; ++k) r = top2_merge(r, top2{s_best[k], s_second[k], s_idx[k]});
+        if (out_idx) out_idx[0] = r.idx == 0xFFFFFFFFu ? 0u : r.idx;   // nothing above -inf: first
+        if (out_margin) out_margin[0] = r.best - r.second;
     }
 }
 
@@ -234,24 +363,6 @@ q6_k_gemv_generic(const uint8_t *__restrict__ w, const float *__restrict__ x,
     if (lane == LEV_WAVE - 1) y[row] = acc;
 }
 
-// ---- argmax + margin: one workgroup of 1024 threads per column ----------
-
-struct top2 {
-    float best, second;
-    uint32_t idx;
-};
-
-__device__ __forceinline__ top2 top2_merge(top2 a, top2 b) {
-    // take b when strictly larger, or equal with the lower index (ops.rs:508)
-    bool take = b.best > a.best || (b.best == a.best && b.idx < a.idx);
-    top2 r;
-    r.best = take ? b.best : a.best;
-    r.idx = take ? b.idx : a.idx;
-    float other = take ? fmaxf(a.best, b.second) : fmaxf(b.best, a.second);
-    r.second = fmaxf(other, take ? a.second : b.second);
-    return r;
-}
-
 __global__ void __launch_bounds__(1024)
 argmax_kernel(const float *__restrict__ logits, uint32_t vocab, uint32_t *__restrict__ out_idx,
               float *__restrict__ out_margin) {
@@ -259,7 +370,7 @@ argmax_kernel(const float *__restrict__ logits, uint32_t vocab, uint32_t *__rest
     __shared__ uint32_t s_idx[16];
     const float *l = logits + (uint64_t)blockIdx.x * vocab;
     const uint32_t t = threadIdx.x;
-    top2 m{-3.0e38f, -3.0e38f, 0u};
+    top2 m{kTop2Floor, kTop2Floor, 0xFFFFFFFFu};
     for (uint32_t i = t; i < vocab; i += 1024) {
         float v = l[i];
         if (v > m.best) {
@@ -287,28 +398,45 @@ argmax_kernel(const float *__restrict__ logits, uint32_t vocab, uint32_t *__rest
     if (t == 0) {
         top2 r{s_best[0], s_second[0], s_idx[0]};
         for (int k = 1; k < 16; ++k) r = top2_merge(r, top2{s_best[k], s_second[k], s_idx[k]});
-        if (out_idx) out_idx[blockIdx.x] = r.idx;
+        if (out_idx) out_idx[blockIdx.x] = r.idx == 0xFFFFFFFFu ? 0u : r.idx;
         if (out_margin) out_margin[blockIdx.x] = r.best - r.second;
     }
 }
 
-template <int L, int P>
+template <int L, int P, int S = 1>
 hipError_t launch_units(lev_ctx *ctx, const uint8_t *w, const float *x, float *y, uint32_t units,
-                        uint32_t rows) {
-    constexpr uint32_t rows_per_tile = kWaves * (LEV_WAVE / L);
+                        uint32_t rows, uint32_t *d_argmax, float *d_margin) {
+    constexpr uint32_t rows_per_tile = kWaves * (LEV_WAVE / L) / S;
     uint32_t blocks = (rows + rows_per_tile - 1) / rows_per_tile;
-    uint32_t cap = (uint32_t)ctx->num_cus * 4u;
-    if (blocks > cap) blocks = cap;
     size_t lds = (size_t)8 * (units + 1) * sizeof(lev_f32x4);
-    hipLaunchKernelGGL((q6_k_gemv_units<L, P>), dim3(blocks), dim3(kThreads), lds, ctx->stream, w, x,
-                       y, units, rows);
+    // persistent grid: exactly the workgroups that are resident at once, so
+    // that no workgroup waits for a slot behind another one's whole loop
+    int per_cu = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, q6_k_gemv_units<L, P, S>, kThreads, lds) !=
+            hipSuccess || per_cu < 1)
+        per_cu = 2;
+    uint32_t cap = (uint32_t)ctx->num_cus * (uint32_t)per_cu;
+    if (blocks > cap) blocks = cap;
+    lev_f32x4 *partials = nullptr;
+    if (d_argmax || d_margin) {
+        partials = static_cast<lev_f32x4 *>(lev_scratch(ctx, (size_t)blocks * sizeof(lev_f32x4)));
+        if (!partials) return hipErrorOutOfMemory;
+    }
+    hipLaunchKernelGGL((q6_k_gemv_units<L, P, S>), dim3(blocks), dim3(kThreads), lds, ctx->stream, w, x,
+                       y, units, rows, partials);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess || !partials) return e;
+    hipLaunchKernelGGL(argmax_partials_kernel, dim3(1), dim3(256), 0, ctx->stream, partials, blocks,
+                       d_argmax, d_margin);
     return hipGetLastError();
 }
 
 }  // namespace
 
-hipError_t lev_q6_k_gemv_launch(lev_ctx *ctx, const uint8_t *w, const float *x, float *y,
-                                uint32_t in_dim, uint32_t rows) {
+// GEMV with the greedy-token epilogue: d_argmax / d_margin may be NULL.
+hipError_t lev_q6_k_gemv_argmax_launch(lev_ctx *ctx, const uint8_t *w, const float *x, float *y,
+                                       uint32_t in_dim, uint32_t rows, uint32_t *d_argmax,
+                                       float *d_margin) {
     const uint32_t units = in_dim / 32u;   // 8 per superblock
     const bool fast = ((reinterpret_cast<uintptr_t>(w) & 1u) == 0u) &&
                       ((reinterpret_cast<uintptr_t>(x) & 15u) == 0u) && units <= 256u;
@@ -316,15 +444,24 @@ hipError_t lev_q6_k_gemv_launch(lev_ctx *ctx, const uint8_t *w, const float *x, 
         uint32_t blocks = (rows + kWaves - 1) / kWaves;
         hipLaunchKernelGGL(q6_k_gemv_generic, dim3(blocks), dim3(kThreads), 0, ctx->stream, w, x, y,
                            units, rows);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess || (!d_argmax && !d_margin)) return e;
+        hipLaunchKernelGGL(argmax_kernel, dim3(1), dim3(1024), 0, ctx->stream, y, rows, d_argmax,
+                           d_margin);
         return hipGetLastError();
     }
-    if (units > 192) return launch_units<64, 4>(ctx, w, x, y, units, rows);
-    if (units > 128) return launch_units<64, 3>(ctx, w, x, y, units, rows);
-    if (units > 64) return launch_units<64, 2>(ctx, w, x, y, units, rows);
-    if (units > 32) return launch_units<64, 1>(ctx, w, x, y, units, rows);
-    if (units > 16) return launch_units<32, 1>(ctx, w, x, y, units, rows);
-    if (units > 8) return launch_units<16, 1>(ctx, w, x, y, units, rows);
-    return launch_units<8, 1>(ctx, w, x, y, units, rows);
+    if (units > 192) return launch_units<64, 4>(ctx, w, x, y, units, rows, d_argmax, d_margin);
+    if (units > 128) return launch_units<64, 3>(ctx, w, x, y, units, rows, d_argmax, d_margin);
+    if (units > 64) return launch_units<64, 1, 2>(ctx, w, x, y, units, rows, d_argmax, d_margin);
+    if (units > 32) return launch_units<64, 1>(ctx, w, x, y, units, rows, d_argmax, d_margin);
+    if (units > 16) return launch_units<32, 1>(ctx, w, x, y, units, rows, d_argmax, d_margin);
+    if (units > 8) return launch_units<16, 1>(ctx, w, x, y, units, rows, d_argmax, d_margin);
+    return launch_units<8, 1>(ctx, w, x, y, units, rows, d_argmax, d_margin);
+}
+
+hipError_t lev_q6_k_gemv_launch(lev_ctx *ctx, const uint8_t *w, const float *x, float *y,
+                                uint32_t in_dim, uint32_t rows) {
+    return lev_q6_k_gemv_argmax_launch(ctx, w, x, y, in_dim, rows, nullptr, nullptr);
 }
 
 hipError_t lev_argmax_launch(lev_ctx *ctx, const float *logits, uint32_t vocab, uint32_t ncol,
@@ -344,13 +481,10 @@ extern "C" int lev_hip_q6_k_gemv(lev_ctx *ctx, const void *d_w, size_t w_bytes, 
                               d_y, y_capacity, out_rows, in_dim, out_rows, &g);
     if (st != LEV_OK) return st;
     const uint8_t *w = static_cast<const uint8_t *>(d_w) + w_off;
-    st = lev_hip_check(ctx, lev_q6_k_gemv_launch(ctx, w, d_x, d_y, in_dim, out_rows),
-                       "q6_k_gemv launch");
-    if (st != LEV_OK) return st;
-    if (d_argmax || d_margin)
-        st = lev_hip_check(ctx, lev_argmax_launch(ctx, d_y, out_rows, 1, d_argmax, d_margin),
-                           "argmax launch");
-    return st;
+    return lev_hip_check(ctx,
+                         lev_q6_k_gemv_argmax_launch(ctx, w, d_x, d_y, in_dim, out_rows, d_argmax,
+                                                     d_margin),
+                         "q6_k_gemv launch");
 }
 
 extern "C" int lev_hip_argmax(lev_ctx *ctx, const float *d_logits, uint32_t vocab, uint32_t ncol,
