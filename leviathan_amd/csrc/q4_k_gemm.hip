@@ -8,16 +8,24 @@
 // because one MFMA takes one input type; fp16 keeps X exactly as given.
 //
 // Tiling (one workgroup = 4 waves = 256 tokens x 128 rows):
-//   - wave w owns rows 32w..32w+31 of the tile for ALL 256 tokens: 8
-//     accumulator tiles of 32x32 (v_mfma_f32_32x32x16_f16), A = X, B = W^T, so
-//     lane l holds output row (l%32) -> stores of Y are contiguous along rows;
+//   - wave (wr, wm) owns rows 64wr..64wr+63 (two 32-row tiles) for tokens
+//     128wm..128wm+127 (four 32-token tiles): 8 accumulator tiles of 32x32
+//     (v_mfma_f32_32x32x16_f16), A = X, B = W^T, so lane l holds output row
+//     (l%32) -> stores of Y are contiguous along rows.  Every X fragment read
+//     from LDS feeds two MFMAs (one per row tile): with one row tile per wave
+//     the LDS reads alone take as long as the MFMAs;
 //   - W never goes through LDS: lane (r = l%32, h = l/32) loads the 16 code
-//     bytes 16h..16h+15 of each 32-byte chunk of ITS row plus the superblock
-//     header and dequantises them in registers straight into B fragments, so
-//     every weight is decoded exactly once per workgroup;
-//   - X goes through LDS in K-steps of 64 (one Q4_K chunk: sub-blocks 2c, 2c+1),
-//     double-buffered, rows padded to 144 bytes so that the 128-bit fragment
-//     reads of 8 consecutive lanes cover all 32 banks.
+//     bytes 16h..16h+15 of each 32-byte chunk of ITS two rows plus their
+//     superblock headers and dequantises them in registers straight into B
+//     fragments (the two waves that share rows both decode them);
+//   - X goes through LDS in K-steps of 64 (one Q4_K chunk) with direct
+//     global -> LDS loads (global_load_lds_dwordx4: no registers in between),
+//     four buffers, three steps in flight, which covers the load latency that a
+//     single wave per SIMD cannot hide otherwise.  A direct load places lane
+//     l's 16 bytes at base + 16*l, so padding rows is not possible; instead
+//     the 16-byte chunk c of token row t is stored at position c ^ (t & 7)
+//     (the source address is permuted), which spreads the fragment reads of
+//     consecutive rows over all banks.
 // K order inside a 64-step is permuted consistently on both operands:
 // MFMA q (0..3) of chunk c takes, for lane half h, elements
 //   q<2 : 64c + 16h + 8q .. +7        (low nibbles of code bytes 8q..8q+7)
@@ -32,10 +40,12 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 constexpr int kThreads = 256;
 constexpr int kBM = 256;          // tokens per workgroup
 constexpr int kBN = 128;          // rows per workgroup (32 per wave)
-constexpr int kMT = kBM / 32;     // accumulator tiles per wave
-constexpr int kKS = 64;           // K-step
-constexpr int kXRow = 144;        // bytes per token row in LDS (128 + 16 pad)
+constexpr int kMT = 4;            // 32-token tiles per wave
+constexpr int kRT = 2;            // 32-row tiles per wave
+constexpr int kKS = 64;           // K-step (one chunk)
+constexpr int kXRow = 128;        // bytes per token row in LDS
 constexpr int kXBuf = kBM * kXRow;
+constexpr int kXBufs = 4;         // LDS buffers: three steps in flight
 
 // (d*sc, dmin*m) of the 8 sub-blocks of a superblock (lev-cpu/src/lib.rs:64-74,
 // 117-124).
@@ -64,7 +74,7 @@ __device__ __forceinline__ void q4k_all_factors(const lev_u32x4 hdr, float d1[8]
 // the two-step rounding in about one weight in ten thousand.
 __device__ __forceinline__ _Float16 q4k_weight_f16(float d1, float code, float mm) {
     float w32 = fmaf(d1, code, -mm);   // d1*code is exact (17 + 4 bits): one rounding, as in the reference
-    asm volatile("" : "+v"(w32));
+    asm("" : "+v"(w32));
     return (_Float16)w32;
 }
 
@@ -74,6 +84,10 @@ __device__ __forceinline__ f16x8 q4k_frag(uint32_t q0, uint32_t q1, bool hi, flo
     uint32_t a = hi ? (q0 >> 4) : q0, b = hi ? (q1 >> 4) : q1;
     a &= 0x0F0F0F0Fu;
     b &= 0x0F0F0F0Fu;
+    // opaque from here: the compiler would otherwise fold the mask into four
+    // bit-field extracts per dword instead of using v_cvt_f32_ubyte0..3 directly
+    asm("" : "+v"(a));
+    asm("" : "+v"(b));
     f16x8 f;
     f[0] = q4k_weight_f16(d1, (float)(a & 0xFFu), mm);
     f[1] = q4k_weight_f16(d1, (float)((a >> 8) & 0xFFu), mm);
@@ -86,98 +100,175 @@ __device__ __forceinline__ f16x8 q4k_frag(uint32_t q0, uint32_t q1, bool hi, flo
     return f;
 }
 
-// grid (ceil(rows/128), ceil(tokens/256)); LDS 2*kXBuf bytes.
+// grid (ceil(rows/128), ceil(tokens/256)); LDS kXBufs*kXBuf bytes.
 __global__ void __launch_bounds__(kThreads)
 q4_k_gemm_kernel(const uint8_t *__restrict__ w, const uint16_t *__restrict__ x,
                  float *__restrict__ y, uint32_t in_dim, uint32_t rows, uint32_t tokens) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t lr = lane & 31u, lh = lane >> 5;
-    const uint32_t row0 = blockIdx.x * kBN + wave * 32u;
+    const uint32_t wr = wave & 1u, wm = wave >> 1;
+    const uint32_t row0 = blockIdx.x * kBN + wr * 64u;
     const uint32_t tok0 = blockIdx.y * kBM;
     const uint32_t nsb = in_dim / 256u;
-    const uint32_t my_row = row0 + lr;
-    const uint8_t *wrow = w + (uint64_t)(my_row < rows ? my_row : rows - 1u) * nsb * 144u;
+    const uint8_t *wrow[kRT];
+#pragma unroll
+    for (int r = 0; r < kRT; ++r) {
+        const uint32_t row = row0 + 32u * r + lr;
+        wrow[r] = w + (uint64_t)(row < rows ? row : rows - 1u) * nsb * 144u;
+    }
 
-    // X staging: thread covers 16 bytes of 8 token rows per K-step.
-    const uint32_t xs_tok = tid >> 3;          // 0..31, + 32*i
-    const uint32_t xs_col = (tid & 7u) * 16u;  // byte offset inside the 128-byte K-step row
-    lev_u32x4 xr[8];
-    auto x_load = [&](uint32_t kstep) {
+    // X staging: per K-step a thread requests 16 bytes of 8 token rows, sent
+    // straight to LDS.  Thread (token = tid/8 + 32i, position p = tid%8) fetches
+    // source chunk p ^ (token & 7).  Token rows past the end repeat the last
+    // one (their outputs are never stored).
+    const uint32_t xs_tok = tid >> 3, xs_pos = tid & 7u;
+    const uint8_t *xsrc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const uint32_t tl = xs_tok + 32u * i;
+        const uint32_t t = tok0 + tl < tokens ? tok0 + tl : tokens - 1u;
+        xsrc[i] = reinterpret_cast<const uint8_t *>(x) + (uint64_t)t * in_dim * 2u + 16u * (xs_pos ^ (tl & 7u));
+    }
+    auto x_request = [&](uint32_t kstep, uint32_t buf) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            uint32_t t = tok0 + xs_tok + 32u * i;
-            if (t < tokens)
-                xr[i] = *reinterpret_cast<const lev_u32x4 *>(
-                    reinterpret_cast<const uint8_t *>(x) + ((uint64_t)t * in_dim + kstep * kKS) * 2u + xs_col);
-            else
-                xr[i] = lev_u32x4{0u, 0u, 0u, 0u};
+            const uint8_t *src = xsrc[i] + (uint64_t)kstep * (kKS * 2u);
+            // lane l of the wave lands at base + 16*l: base = this wave's 1 KB of pass i
+            uint8_t *dst = lds + buf * kXBuf + i * 4096 + wave * 1024u;
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
+                                             (__attribute__((address_space(3))) void *)dst, 16, 0, 0);
         }
     };
-    auto x_store = [&](uint32_t buf) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i)
-            *reinterpret_cast<lev_u32x4 *>(lds + buf * kXBuf + (xs_tok + 32u * i) * kXRow + xs_col) = xr[i];
-    };
+    // s_waitcnt vmcnt(n) leaves at most n loads outstanding; loads complete in
+    // issue order, so everything older than the n newest has landed.  Encoding:
+    // vmcnt in bits 3:0 and 15:14, expcnt (6:4) and lgkmcnt (11:8) left at "any".
+#define LEV_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xF) | (((n) >> 4) << 14) | (7 << 4) | (15 << 8))
 
-    f32x16 acc[kMT];
+    f32x16 acc[kRT][kMT];
 #pragma unroll
-    for (int m = 0; m < kMT; ++m)
+    for (int r = 0; r < kRT; ++r)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) acc[m][i] = 0.f;
+        for (int m = 0; m < kMT; ++m)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[r][m][i] = 0.f;
 
     const uint32_t nsteps = nsb * 4u;
-    x_load(0);
-    x_store(0);
-    __syncthreads();
+    // steps 0, 1, 2 in flight (clamped for very short K)
+    x_request(0, 0);
+    x_request(1 < nsteps ? 1 : nsteps - 1, 1);
+    x_request(2 < nsteps ? 2 : nsteps - 1, 2);
 
-    for (uint32_t sb = 0; sb < nsb; ++sb) {
-        const uint8_t *blk = wrow + (uint64_t)sb * 144u;
-        lev_u32x4 hdr = *reinterpret_cast<const lev_u32x4 *>(blk);
-        lev_u32x4 qs[4];
+    // The weights of superblock sb+1 are requested while sb is multiplied: with
+    // one wave per SIMD nothing else hides their latency.  Loads are
+    // unconditional (clamped at the end) so that no branch forces a wait.
+    lev_u32x4 hdr_n[kRT], qs_n[kRT][4];
+    auto w_load = [&](uint32_t sb) {
+        const uint32_t sbc = sb < nsb ? sb : nsb - 1u;
 #pragma unroll
-        for (int cc = 0; cc < 4; ++cc)
-            qs[cc] = *reinterpret_cast<const lev_u32x4 *>(blk + 16u + 32u * cc + 16u * lh);
-        float d1[8], mm[8];
-        q4k_all_factors(hdr, d1, mm);
+        for (int r = 0; r < kRT; ++r) {
+            const uint8_t *blk = wrow[r] + (uint64_t)sbc * 144u;
+            hdr_n[r] = *reinterpret_cast<const lev_u32x4 *>(blk);
+#pragma unroll
+            for (int cc = 0; cc < 4; ++cc)
+                qs_n[r][cc] = *reinterpret_cast<const lev_u32x4 *>(blk + 16u + 32u * cc + 16u * lh);
+        }
+    };
+    lev_u32x4 qs[kRT][4];
+    float d1[kRT][8], mm[kRT][8];
+    auto take = [&]() {   // the prefetched superblock becomes the current one
+#pragma unroll
+        for (int r = 0; r < kRT; ++r) {
+#pragma unroll
+            for (int cc = 0; cc < 4; ++cc) qs[r][cc] = qs_n[r][cc];
+            q4k_all_factors(hdr_n[r], d1[r], mm[r]);
+        }
+    };
+    // this lane's 32 weights of chunk c of each of its two rows -> B fragments
+    auto dequant = [&](int c, f16x8 (&f)[kRT][4]) {
+#pragma unroll
+        for (int r = 0; r < kRT; ++r) {
+            const lev_u32x4 q = qs[r][c];
+            f[r][0] = q4k_frag(q.x, q.y, false, d1[r][2 * c], mm[r][2 * c]);
+            f[r][1] = q4k_frag(q.z, q.w, false, d1[r][2 * c], mm[r][2 * c]);
+            f[r][2] = q4k_frag(q.x, q.y, true, d1[r][2 * c + 1], mm[r][2 * c + 1]);
+            f[r][3] = q4k_frag(q.z, q.w, true, d1[r][2 * c + 1], mm[r][2 * c + 1]);
+        }
+    };
+    w_load(0);
+    take();
+    w_load(1);
+    f16x8 bf[kRT][4];
+    dequant(0, bf);
+    for (uint32_t sb = 0; sb < nsb; ++sb) {
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             const uint32_t ks = sb * 4u + c;
-            if (ks + 1 < nsteps) x_load(ks + 1);
-
-            // this lane's 32 weights of chunk c -> four B fragments
-            const lev_u32x4 q = qs[c];
-            f16x8 bf[4];
-            bf[0] = q4k_frag(q.x, q.y, false, d1[2 * c], mm[2 * c]);
-            bf[1] = q4k_frag(q.z, q.w, false, d1[2 * c], mm[2 * c]);
-            bf[2] = q4k_frag(q.x, q.y, true, d1[2 * c + 1], mm[2 * c + 1]);
-            bf[3] = q4k_frag(q.z, q.w, true, d1[2 * c + 1], mm[2 * c + 1]);
-
-            const uint8_t *xb = lds + (ks & 1u) * kXBuf + lr * kXRow + 32u * lh;
-#pragma unroll
-            for (int qq = 0; qq < 4; ++qq) {
-                // byte offset of this MFMA's 8 activations inside the 128-byte row
-                const uint32_t koff = (qq < 2 ? 16u * qq : 64u + 16u * (qq - 2));
-#pragma unroll
-                for (int m = 0; m < kMT; ++m) {
-                    f16x8 a = *reinterpret_cast<const f16x8 *>(xb + m * 32 * kXRow + koff);
-                    acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bf[qq], acc[m], 0, 0, 0);
-                }
-            }
-            if (ks + 1 < nsteps) x_store((ks + 1) & 1u);
+            // Step ks+3 goes into the buffer that step ks-1 used: every wave is
+            // past the barrier that ended that step.  Then wait for step ks: its
+            // 8 loads are older than the 24 of steps ks+1..ks+3 (any weight load
+            // issued in between only makes the wait stricter).
+            x_request(ks + 3 < nsteps ? ks + 3 : nsteps - 1, (ks + 3) & 3u);
+            LEV_WAIT_VMCNT(24);
             __syncthreads();
+
+            // The fragments of the NEXT chunk are decoded while this chunk is
+            // multiplied.  A wave issues in order, so with one wave per SIMD the
+            // vector ALU and the matrix core only work together if the two
+            // streams alternate in program order: eight groups of { decode one
+            // fragment (about 30 vector instructions), two LDS reads, four MFMAs },
+            // fenced so that the scheduler keeps them apart.  The MFMAs of a group
+            // run while the next group's decode issues.
+            f16x8 bn[kRT][4];
+            if (c == 3) {
+                take();
+                w_load(sb + 2u);
+            }
+            const int cn = c == 3 ? 0 : c + 1;
+            const uint8_t *xb = lds + (ks & 3u) * kXBuf + (wm * 128u + lr) * kXRow;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                {
+                    const int r = j >> 2, q = j & 3;
+                    const lev_u32x4 w4 = qs[r][cn];
+                    const int sub = 2 * cn + (q >> 1);
+                    bn[r][q] = q4k_frag((q & 1) ? w4.z : w4.x, (q & 1) ? w4.w : w4.y, q >= 2, d1[r][sub], mm[r][sub]);
+                }
+                const int qq = j >> 1;
+                // 16-byte chunk of this MFMA's 8 activations inside the 128-byte row,
+                // at its swizzled position (rows 32m + lr: same low bits as lr)
+                const uint32_t chunk = 2u * lh + (qq < 2 ? qq : 2u + qq);
+                const uint32_t koff = 16u * (chunk ^ (lr & 7u));
+#pragma unroll
+                for (int mm2 = 0; mm2 < 2; ++mm2) {
+                    const int m = 2 * (j & 1) + mm2;
+                    f16x8 a = *reinterpret_cast<const f16x8 *>(xb + m * 32 * kXRow + koff);
+#pragma unroll
+                    for (int r = 0; r < kRT; ++r)
+                        acc[r][m] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bf[r][qq], acc[r][m], 0, 0, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int r = 0; r < kRT; ++r)
+#pragma unroll
+                for (int qq = 0; qq < 4; ++qq) bf[r][qq] = bn[r][qq];
+            __syncthreads();   // all reads of this step's buffer done before it is requested again
         }
     }
 
     // D layout of the 32x32 tile: lane -> column n = l%32 (our row), register
     // i -> line m = 8*(i/4) + 4*(l/32) + i%4 (our token).
-    if (my_row < rows) {
+#pragma unroll
+    for (int r = 0; r < kRT; ++r) {
+        const uint32_t my_row = row0 + 32u * r + lr;
+        if (my_row >= rows) continue;
 #pragma unroll
         for (int m = 0; m < kMT; ++m)
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
-                uint32_t t = tok0 + m * 32 + 8 * (i / 4) + 4 * lh + (i % 4);
-                if (t < tokens) y[(uint64_t)t * rows + my_row] = acc[m][i];
+                uint32_t t = tok0 + wm * 128u + m * 32 + 8 * (i / 4) + 4 * lh + (i % 4);
+                if (t < tokens) y[(uint64_t)t * rows + my_row] = acc[r][m][i];
             }
     }
 }
@@ -187,7 +278,7 @@ q4_k_gemm_kernel(const uint8_t *__restrict__ w, const uint16_t *__restrict__ x,
 hipError_t lev_q4_k_gemm_launch(lev_ctx *ctx, const uint8_t *w, const uint16_t *x, float *y,
                                 uint32_t in_dim, uint32_t rows, uint32_t tokens) {
     static bool attr_set = false;
-    const size_t lds = 2 * (size_t)kXBuf;
+    const size_t lds = (size_t)kXBufs * kXBuf;
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&q4_k_gemm_kernel),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
