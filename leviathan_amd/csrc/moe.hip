@@ -17,6 +17,7 @@
 //   3. down: wave s of a workgroup streams the rows of slot s for the
 //      workgroup's tile of outputs; partial results meet in LDS and are merged
 //      IN SLOT ORDER in f32, as the reference's axpy chain does.
+#include "moe_grouped.hpp"
 #include "q4_0_device.hpp"
 
 namespace {
@@ -254,7 +255,7 @@ moe_scores_kernel(const float *__restrict__ wr, const float *__restrict__ x,
     double acc[K] = {};
     if (vec) {
         const lev_f32x4 *r4 = reinterpret_cast<const lev_f32x4 *>(row);
-#pragma unroll 2
+#pragma unroll 4
         for (uint32_t i = lane; i < hidden / 4u; i += 64u) {
             const lev_f32x4 a = r4[i];
 #pragma unroll
@@ -764,17 +765,38 @@ hipError_t run_experts(lev_ctx *ctx, const moe_args &a, const float *x, const gu
 struct moe_scratch {
     float *scores;
     float *act;
+    void *grouped;   // work area of the many-token path (grouped_bytes > 0)
 };
 
 int get_scratch(lev_ctx *ctx, uint32_t tokens, uint32_t experts, uint32_t top_k, uint32_t inter,
-                moe_scratch *s) {
+                moe_scratch *s, size_t grouped_bytes = 0) {
     size_t s_bytes = ((size_t)tokens * experts * 4 + 255) & ~(size_t)255;
-    size_t a_bytes = (size_t)tokens * top_k * inter * 4;
-    char *p = static_cast<char *>(lev_scratch(ctx, s_bytes + a_bytes));
+    size_t a_bytes = ((size_t)tokens * top_k * inter * 4 + 255) & ~(size_t)255;
+    char *p = static_cast<char *>(lev_scratch(ctx, s_bytes + a_bytes + grouped_bytes));
     if (!p) return lev_fail(ctx, LEV_ERR_EXCEEDS_WORKING_SET, "moe: scratch allocation failed");
     s->scores = reinterpret_cast<float *>(p);
     s->act = reinterpret_cast<float *>(p + s_bytes);
+    s->grouped = p + s_bytes + a_bytes;
     return LEV_OK;
+}
+
+// Tokens from which pairs are grouped by expert and multiplied on the matrix
+// cores; below, every (token, slot) streams its expert by itself.
+constexpr uint32_t kGroupedMinTokens = 5;
+
+lev_moe_grouped_args grouped_args(const moe_args &a, uint32_t tokens) {
+    return lev_moe_grouped_args{a.base,        a.gate_off,  a.up_off, a.down_off, a.gate_stride,
+                                a.up_stride,   a.down_stride, a.hidden, a.inter,   a.experts,
+                                a.top_k,       tokens};
+}
+
+bool use_grouped(const lev_ctx *ctx, const moe_args &a, const float *x, uint32_t tokens) {
+    static const bool enabled = [] {
+        const char *e = getenv("LEV_MOE_GROUPED");   // LEV_MOE_GROUPED=0: per-pair kernels, for comparison
+        return !(e && e[0] == '0');
+    }();
+    return enabled && tokens >= kGroupedMinTokens && experts_fast(a, x) &&
+           lev_moe_grouped_usable(ctx, grouped_args(a, tokens));
 }
 
 hipError_t run_scores(lev_ctx *ctx, const float *wr, const float *x, float *scores, uint32_t hidden,
@@ -844,13 +866,20 @@ extern "C" int lev_hip_moe_experts_q4_0(lev_ctx *ctx, const lev_moe_experts *poo
     moe_args a;
     int st = check_pools(ctx, pools, top_k, tokens, &a);
     if (st != LEV_OK) return st;
+    const bool grouped = use_grouped(ctx, a, d_x, tokens) && (reinterpret_cast<uintptr_t>(d_act) & 15u) == 0u;
     float *act = d_act;
-    if (!act) {
-        moe_scratch s;
-        st = get_scratch(ctx, tokens, a.experts, top_k, a.inter, &s);
+    moe_scratch s{nullptr, nullptr, nullptr};
+    if (!act || grouped) {
+        st = get_scratch(ctx, tokens, a.experts, top_k, a.inter, &s,
+                         grouped ? lev_moe_grouped_scratch_bytes(grouped_args(a, tokens)) : 0);
         if (st != LEV_OK) return st;
-        act = s.act;
+        if (!act) act = s.act;
     }
+    if (grouped)
+        return lev_hip_check(ctx,
+                             lev_moe_grouped_launch(ctx, grouped_args(a, tokens), d_x, d_ids, d_weights,
+                                                    d_y, act, s.grouped),
+                             "moe grouped experts launch");
     const bool fast = experts_fast(a, d_x) && (reinterpret_cast<uintptr_t>(act) & 15u) == 0u;
     gu_route rt{d_ids, nullptr, nullptr, nullptr, nullptr};
     return lev_hip_check(ctx, run_experts(ctx, a, d_x, rt, d_ids, d_weights, d_y, act, tokens, fast),
@@ -868,8 +897,10 @@ extern "C" int lev_hip_moe_layer_q4_0(lev_ctx *ctx, const lev_moe_experts *pools
     int st = check_pools(ctx, pools, top_k, tokens, &a);
     if (st != LEV_OK) return st;
     if (a.experts > 4096u) return lev_fail(ctx, LEV_ERR_BAD_DIMENSIONS, "moe_layer: %u experts", a.experts);
+    const bool grouped = use_grouped(ctx, a, d_x, tokens);
     moe_scratch s;
-    st = get_scratch(ctx, tokens, a.experts, top_k, a.inter, &s);
+    st = get_scratch(ctx, tokens, a.experts, top_k, a.inter, &s,
+                     grouped ? lev_moe_grouped_scratch_bytes(grouped_args(a, tokens)) : 0);
     if (st != LEV_OK) return st;
     st = lev_hip_check(ctx, run_scores(ctx, d_router_w, d_x, s.scores, a.hidden, a.experts, tokens),
                        "moe router scores launch");
@@ -886,6 +917,11 @@ extern "C" int lev_hip_moe_layer_q4_0(lev_ctx *ctx, const lev_moe_experts *pools
                            "moe router top-k launch");
         if (st != LEV_OK) return st;
     }
+    if (grouped)
+        return lev_hip_check(ctx,
+                             lev_moe_grouped_launch(ctx, grouped_args(a, tokens), d_x, d_ids, d_weights,
+                                                    d_y, s.act, s.grouped),
+                             "moe grouped experts launch");
     return lev_hip_check(ctx, run_experts(ctx, a, d_x, rt, d_ids, d_weights, d_y, s.act, tokens, fast),
                          "moe experts launch");
 }

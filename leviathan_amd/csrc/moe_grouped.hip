@@ -1,0 +1,444 @@
+// Routed Q4_0 experts for MANY tokens on gfx950: (token, slot) pairs are
+// grouped by expert, and each expert's weights are streamed once and applied
+// to all of its tokens on the matrix cores.
+//
+// Stands in for runMoeBatchedRouted applied token after token
+// (Sources/LeviathanCore/Gemma4.swift:2073, per-slot loop :3856-3880;
+// moegen_gu/act/dn, MoELowering.swift:749-835): same results per pair, same
+// slot-ordered f32 merge; only the order in which pairs are visited changes.
+// With one launch per (token, slot) every pair streams its expert's 2.65 MB
+// again (64 tokens x top-8 = 512 x 2.65 MB against 126 distinct experts).
+//
+// Pipeline (all on the context's stream):
+//   1. group:  histogram of expert ids -> offsets; list of pairs per expert.
+//   2. prep:   rows of f32 activations -> two fp16 planes (high + low half,
+//              after a power-of-two row scale), in the k-slot order of step 3.
+//   3. gate/up on MFMA -> act = gelu_tanh(g)*u (f32, [pair][inter]).
+//   4. prep(act), down on MFMA -> dn (f32, [pair][hidden]).
+//   5. merge:  y[t] = sum over slots, IN SLOT ORDER, fmaf(w_slot, dn_slot, acc).
+//
+// MFMA formulation (v_mfma_f32_16x16x32_f16), per Q4_0 block of 32 weights:
+//   B = 16 weight rows x the block's 32 codes as exact fp16 integers n-8
+//       (mask, OR in 1024's exponent, subtract 1032: two instructions per two
+//       weights, no conversion);
+//   A = up to 8 tokens' activations of that block, fp16 high and low halves
+//       (two MFMAs), x = hi + lo to 2^-22;
+//   the output lane of weight row n is the lane that holds row n's block scale
+//   d, so y += d * (A.B) needs no exchange.
+// A lane fetches a PAIR of blocks (36 bytes, as in the decode GEMV: wide loads,
+// whole rows contiguous per wave) and the four lanes of a row swap code bytes
+// through a small wave-private LDS area so that each MFMA sees one block.
+#include "moe_grouped.hpp"
+
+namespace {
+
+constexpr int kGrpThreads = 1024;
+constexpr int kGrpWaves = kGrpThreads / LEV_WAVE;
+constexpr int kNC = 8;                 // token columns per pass
+constexpr int kFlagBadExpertId = 1;    // same bit as the per-token kernels
+
+typedef _Float16 g_h8 __attribute__((ext_vector_type(8)));
+typedef uint32_t g_u4 __attribute__((ext_vector_type(4)));
+typedef uint32_t g_u2 __attribute__((ext_vector_type(2)));
+
+// ---------------------------------------------------------------------------
+// 1. group pairs by expert.  One workgroup.  A pair is dropped (and flagged)
+// when its id is out of range or repeats an earlier slot of the same token,
+// as MoEModelBinding.offsets requires (MoEModelBinding.swift:174-214).
+// goff[e] .. goff[e+1]: expert e's pairs in glist; valid[p]: pair p takes part.
+// ---------------------------------------------------------------------------
+__global__ void __launch_bounds__(1024)
+moe_group_kernel(const int32_t *__restrict__ ids, uint32_t pairs, uint32_t experts, uint32_t top_k,
+                 int32_t *__restrict__ goff, int32_t *__restrict__ glist,
+                 uint8_t *__restrict__ valid, int *__restrict__ flag) {
+    extern __shared__ int32_t s_cnt[];          // [experts] counts, then [experts] cursors
+    int32_t *s_cur = s_cnt + experts;
+    const uint32_t tid = threadIdx.x;
+    for (uint32_t e = tid; e < experts; e += 1024u) s_cnt[e] = 0;
+    __syncthreads();
+    bool bad_seen = false;
+    for (uint32_t p = tid; p < pairs; p += 1024u) {
+        const int32_t e = ids[p];
+        bool ok = e >= 0 && (uint32_t)e < experts;
+        const uint32_t slot = p % top_k, first = p - slot;
+        for (uint32_t k = 0; k < top_k && ok; ++k)
+            if (k != slot && ids[first + k] == e) ok = false;   // both copies of a duplicate are dropped
+        valid[p] = ok ? 1 : 0;
+        if (ok) atomicAdd(&s_cnt[e], 1);
+        bad_seen = bad_seen || !ok;
+    }
+    if (bad_seen) atomicOr(flag, kFlagBadExpertId);
+    __syncthreads();
+    // exclusive scan, every thread for its own experts (broadcast LDS reads;
+    // experts <= 4096, so at most a few thousand short iterations)
+    for (uint32_t e = tid; e <= experts; e += 1024u) {
+        int32_t run = 0;
+        for (uint32_t j = 0; j < e; ++j) run += s_cnt[j];
+        goff[e] = run;
+        if (e < experts) s_cur[e] = run;
+    }
+    __syncthreads();
+    // The order of an expert's pairs in the list depends on the atomics; no
+    // result does: every pair is computed independently and owns its outputs.
+    for (uint32_t p = tid; p < pairs; p += 1024u)
+        if (valid[p]) glist[atomicAdd(&s_cur[ids[p]], 1)] = (int32_t)p;
+}
+
+// ---------------------------------------------------------------------------
+// 2. prep: one workgroup of 256 threads per row of `len` floats (len % 32 == 0).
+// hi/lo planes keep the row order except inside each run of 8 elements, which
+// is stored as elements 0,2,1,3,4,6,5,7: the order in which the masks of step 3
+// deliver the code bytes of a dword pair.  unscale[row] undoes the row scale.
+// ---------------------------------------------------------------------------
+__global__ void __launch_bounds__(256)
+moe_prep_kernel(const float *__restrict__ src, uint32_t len, _Float16 *__restrict__ hi,
+                _Float16 *__restrict__ lo, float *__restrict__ unscale) {
+    __shared__ float s_max[4];
+    __shared__ float s_scale;
+    const uint32_t row = blockIdx.x, tid = threadIdx.x;
+    const lev_f32x4 *s4 = reinterpret_cast<const lev_f32x4 *>(src + (uint64_t)row * len);
+    const uint32_t runs = len >> 3;
+    float mx = 0.f;
+    for (uint32_t q = tid; q < runs; q += 256u) {
+        const lev_f32x4 a = s4[2u * q], b = s4[2u * q + 1u];
+        mx = fmaxf(mx, fmaxf(fmaxf(fabsf(a.x), fabsf(a.y)), fmaxf(fabsf(a.z), fabsf(a.w))));
+        mx = fmaxf(mx, fmaxf(fmaxf(fabsf(b.x), fabsf(b.y)), fmaxf(fabsf(b.z), fabsf(b.w))));
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
+    if ((tid & 63u) == 0u) s_max[tid >> 6] = mx;
+    __syncthreads();
+    if (tid == 0) {
+        const float m = fmaxf(fmaxf(s_max[0], s_max[1]), fmaxf(s_max[2], s_max[3]));
+        // power-of-two scale that brings the row maximum into [1, 2)
+        uint32_t ex = (__float_as_uint(m) >> 23) & 0xFFu;
+        if (ex == 0u || ex >= 254u) ex = 127u;      // zero / denormal / non-finite row: no scaling
+        s_scale = __uint_as_float((254u - ex) << 23);
+        unscale[row] = __uint_as_float(ex << 23);
+    }
+    __syncthreads();
+    const float scale = s_scale;
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+    for (uint32_t q = tid; q < runs; q += 256u) {
+        const lev_f32x4 a = s4[2u * q] * scale, b = s4[2u * q + 1u] * scale;
+        const float m[8] = {a.x, a.z, a.y, a.w, b.x, b.z, b.y, b.w};
+        g_h8 h, l;
+#pragma unroll
+        for (int k = 0; k < 8; k += 2) {
+            const f32x2 pair = {m[k], m[k + 1]};
+            const f16x2 hp = __builtin_convertvector(pair, f16x2);
+            const f32x2 rest = {pair.x - (float)hp.x, pair.y - (float)hp.y};
+            const f16x2 lp = __builtin_convertvector(rest, f16x2);
+            h[k] = hp.x; h[k + 1] = hp.y;
+            l[k] = lp.x; l[k + 1] = lp.y;
+        }
+        *reinterpret_cast<g_h8 *>(hi + (uint64_t)row * len + 8u * q) = h;
+        *reinterpret_cast<g_h8 *>(lo + (uint64_t)row * len + 8u * q) = l;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// 3./4. grouped matrix-core kernel, 16 waves.  Down: grid (row tiles of 256,
+// experts), wave w owns rows 16w..16w+15 of the tile.  PAIRED (gate/up): grid
+// (row tiles of 128, experts), waves 0..7 own the tile's gate rows, waves 8..15
+// the same rows of the up matrix; gate values meet the up waves in LDS.
+// Column j of a pass is pair glist[goff[e] + pass*8 + j]; its activation row is
+// the pair's token (PAIRED: gate/up read x) or the pair itself (down reads act).
+// ---------------------------------------------------------------------------
+
+// the 8 code bytes a lane needs of one block -> B operand: fp16 integers n - 8.
+// sh = 0 for the lanes that take the low nibbles, 4 for the high nibbles; mask
+// and magic arrive in registers so that (v & mask) | magic is ONE v_and_or_b32.
+__device__ __forceinline__ g_h8 q4_0_operand(g_u2 codes, uint32_t sh, uint32_t mask, uint32_t magic) {
+    typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+    const f16x2 bias = {(_Float16)1032.0f, (_Float16)1032.0f};
+    auto two = [&](uint32_t v) {
+        // 0x6400 | n is the fp16 number 1024 + n
+        const f16x2 h = __builtin_bit_cast(f16x2, (v & mask) | magic);
+        return __builtin_bit_cast(uint32_t, h - bias);
+    };
+    g_u4 bits;
+    bits.x = two(codes.x >> sh);
+    bits.y = two(codes.x >> (sh + 8u));
+    bits.z = two(codes.y >> sh);
+    bits.w = two(codes.y >> (sh + 8u));
+    return __builtin_bit_cast(g_h8, bits);
+}
+
+template <bool PAIRED>
+__global__ void __launch_bounds__(kGrpThreads)
+moe_grouped_kernel(lev_moe_grouped_args a, const _Float16 *__restrict__ xh,
+                   const _Float16 *__restrict__ xl, const float *__restrict__ unscale,
+                   const int32_t *__restrict__ goff, const int32_t *__restrict__ glist,
+                   float *__restrict__ out) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const uint32_t in_len = PAIRED ? a.hidden : a.inter;
+    const uint32_t out_rows = PAIRED ? a.inter : a.hidden;
+    const uint32_t nblk = in_len >> 5, runs = in_len >> 3;
+    const uint32_t e = blockIdx.y;
+    const int32_t first = goff[e];
+    const uint32_t n = (uint32_t)(goff[e + 1] - first);
+    if (n == 0u) return;
+
+    constexpr int NM = 1;   // matrices per wave
+    const uint32_t plane = runs * kNC * 8u;                      // halfs
+    _Float16 *sxh = reinterpret_cast<_Float16 *>(smem);           // [run][col][8]
+    _Float16 *sxl = sxh + plane;
+    // wave-private exchange area: per matrix 16 rows x (8 blocks x 4 dwords + 4 pad), then 16 x 8 scales
+    uint32_t *xch = reinterpret_cast<uint32_t *>(sxl + plane);
+    constexpr uint32_t kRowDw = 36, kXchDw = 16 * kRowDw + 16 * 8;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    uint32_t *my = xch + wave * (NM * kXchDw);
+    __shared__ int32_t s_pair[kNC];
+    __shared__ float s_us[kNC];
+    __shared__ float s_gate[PAIRED ? (kGrpWaves / 2) * 16 * kNC : 1];   // [tile row][col]
+
+    const uint32_t r = lane & 15u, g = lane >> 4;
+    const uint32_t is_up = PAIRED ? wave / (kGrpWaves / 2) : 0u;
+    const uint32_t wv = PAIRED ? wave % (kGrpWaves / 2) : wave;          // 16-row slice of the tile
+    const uint32_t tile_rows = PAIRED ? (kGrpWaves / 2) * 16 : kGrpWaves * 16;
+    const uint32_t row = blockIdx.x * tile_rows + wv * 16u + r;
+    const uint32_t rowc = row < out_rows ? row : out_rows - 1u;
+    const uint64_t row_bytes = (uint64_t)nblk * 18u;
+    const uint8_t *wrow[NM];
+    if (PAIRED)
+        wrow[0] = a.base + (is_up ? a.up_off + e * a.up_stride : a.gate_off + e * a.gate_stride) +
+                  rowc * row_bytes;
+    else
+        wrow[0] = a.base + a.down_off + e * a.down_stride + rowc * row_bytes;
+
+    for (uint32_t pass = 0; pass * kNC < n; ++pass) {
+        const uint32_t ncols = n - pass * kNC < (uint32_t)kNC ? n - pass * kNC : (uint32_t)kNC;
+        __syncthreads();   // previous pass done with the planes and s_pair
+        if (tid < (uint32_t)kNC) {
+            // columns past the end repeat the last pair (never stored)
+            const int32_t p = glist[first + pass * kNC + (tid < ncols ? tid : ncols - 1u)];
+            s_pair[tid] = p;
+            s_us[tid] = unscale[PAIRED ? p / (int32_t)a.top_k : p];
+        }
+        __syncthreads();
+        // stage the columns: 16-byte runs, global rows are contiguous
+        for (uint32_t i = tid; i < runs * kNC; i += kGrpThreads) {
+            const uint32_t c = i / runs, q = i - c * runs;
+            const int32_t p = s_pair[c];
+            const uint64_t src = (uint64_t)(PAIRED ? p / (int32_t)a.top_k : p) * in_len + 8u * q;
+            *reinterpret_cast<g_h8 *>(sxh + (q * kNC + c) * 8u) = *reinterpret_cast<const g_h8 *>(xh + src);
+            *reinterpret_cast<g_h8 *>(sxl + (q * kNC + c) * 8u) = *reinterpret_cast<const g_h8 *>(xl + src);
+        }
+        __syncthreads();
+
+        lev_f32x4 y[NM];
+#pragma unroll
+        for (int m = 0; m < NM; ++m) y[m] = lev_f32x4{0.f, 0.f, 0.f, 0.f};
+        const uint32_t colc = r < (uint32_t)kNC ? r : (uint32_t)kNC - 1u;   // A rows past kNC: any valid address
+
+        // groups of 8 blocks = 4 pairs; lane (r, g) fetches pair g of row r
+        const uint32_t ngrp = nblk >> 3;
+        auto fetch = [&](uint32_t grp, uint32_t (&D)[NM][9]) {
+            const uint32_t gc = grp < ngrp ? grp : ngrp - 1u;
+#pragma unroll
+            for (int m = 0; m < NM; ++m) {
+                const uint8_t *p = wrow[m] + (uint64_t)(gc * 4u + g) * 36u;
+                lev_u32x4_a4 v0 = *reinterpret_cast<const lev_u32x4_a4 *>(p);
+                lev_u32x4_a4 v1 = *reinterpret_cast<const lev_u32x4_a4 *>(p + 16);
+                lev_u32_a4 v2 = *reinterpret_cast<const lev_u32_a4 *>(p + 32);
+                D[m][0] = v0.v[0]; D[m][1] = v0.v[1]; D[m][2] = v0.v[2]; D[m][3] = v0.v[3];
+                D[m][4] = v1.v[0]; D[m][5] = v1.v[1]; D[m][6] = v1.v[2]; D[m][7] = v1.v[3];
+                D[m][8] = v2.v;
+            }
+        };
+        const uint32_t nib_shift = 4u * (g >> 1);
+        uint32_t k_mask = 0x000F000Fu, k_magic = 0x64006400u;
+        asm("" : "+v"(k_mask), "+v"(k_magic));   // keep both in registers (see q4_0_operand)
+        auto process = [&](uint32_t grp, const uint32_t (&Dcur)[NM][9]) {
+            // hand the pair's two blocks to the lanes that need them
+#pragma unroll
+            for (int m = 0; m < NM; ++m) {
+                const uint32_t *D = Dcur[m];
+                uint32_t *area = my + m * kXchDw;
+                g_u4 qa, qb;
+                qa.x = __builtin_amdgcn_alignbit(D[1], D[0], 16);
+                qa.y = __builtin_amdgcn_alignbit(D[2], D[1], 16);
+                qa.z = __builtin_amdgcn_alignbit(D[3], D[2], 16);
+                qa.w = __builtin_amdgcn_alignbit(D[4], D[3], 16);
+                qb.x = D[5]; qb.y = D[6]; qb.z = D[7]; qb.w = D[8];
+                *reinterpret_cast<g_u4 *>(area + r * kRowDw + (2u * g) * 4u) = qa;
+                *reinterpret_cast<g_u4 *>(area + r * kRowDw + (2u * g + 1u) * 4u) = qb;
+                float *sc = reinterpret_cast<float *>(area + 16 * kRowDw) + r * 8u + 2u * g;
+                sc[0] = lev_f16_bits_to_f32(D[0] & 0xFFFFu);
+                sc[1] = lev_f16_bits_to_f32(D[4] >> 16);
+            }
+            // wave-private area: the hardware runs one wave's LDS accesses in order
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+            for (uint32_t b = 0; b < 8u; ++b) {
+                const uint32_t at = (((grp * 8u + b) * 4u + g) * kNC + colc) * 8u;
+                const g_h8 Ah = *reinterpret_cast<const g_h8 *>(sxh + at);
+                const g_h8 Al = *reinterpret_cast<const g_h8 *>(sxl + at);
+#pragma unroll
+                for (int m = 0; m < NM; ++m) {
+                    const uint32_t *area = my + m * kXchDw;
+                    const g_u2 codes = *reinterpret_cast<const g_u2 *>(area + r * kRowDw + b * 4u + 2u * (g & 1u));
+                    const float d = reinterpret_cast<const float *>(area + 16 * kRowDw)[r * 8u + b];
+                    const g_h8 B = q4_0_operand(codes, nib_shift, k_mask, k_magic);
+                    lev_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ah, B, acc, 0, 0, 0);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(Al, B, acc, 0, 0, 0);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) y[m][i] = fmaf(d, acc[i], y[m][i]);
+                }
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();   // reads done before the next group's writes
+        };
+        // the next group is requested before the current one is multiplied
+        // (a third group in flight costs more in registers than it gains)
+        uint32_t Dc[NM][9], Dn[NM][9];
+        fetch(0, Dc);
+        for (uint32_t grp = 0; grp < ngrp; ++grp) {
+            fetch(grp + 1u, Dn);   // unconditional (clamped): no branch around loads
+            process(grp, Dc);
+#pragma unroll
+            for (int m = 0; m < NM; ++m)
+#pragma unroll
+                for (int k = 0; k < 9; ++k) Dc[m][k] = Dn[m][k];
+        }
+
+        // output lane (r, g): weight row r, columns 4g..4g+3
+        if (PAIRED) {
+            if (!is_up) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (4u * g + i < (uint32_t)kNC) s_gate[(wv * 16u + r) * kNC + 4u * g + i] = y[0][i] * s_us[4u * g + i];
+            }
+            __syncthreads();
+        }
+        if (row < out_rows && (!PAIRED || is_up)) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t col = 4u * g + i;
+                if (col < ncols) {
+                    const int32_t p = s_pair[col];
+                    const float us = s_us[col];
+                    float v = y[0][i] * us;
+                    if (PAIRED) v = lev_gelu_up_value(s_gate[(wv * 16u + r) * kNC + col], v);
+                    out[(uint64_t)p * out_rows + row] = v;
+                }
+            }
+        }
+    }
+}
+
+// 5. merge in slot order (g4_axpy chain, Gemma4.swift:2171-2175); dropped pairs add nothing.
+__global__ void __launch_bounds__(256)
+moe_merge_kernel(const float *__restrict__ dn, const float *__restrict__ weights,
+                 const uint8_t *__restrict__ valid, float *__restrict__ y, uint32_t hidden,
+                 uint32_t top_k) {
+    const uint32_t t = blockIdx.y, h = blockIdx.x * 256u + threadIdx.x;
+    if (h >= hidden) return;
+    float acc = 0.f;
+    for (uint32_t k = 0; k < top_k; ++k) {
+        const uint32_t p = t * top_k + k;
+        const float v = valid[p] ? dn[(uint64_t)p * hidden + h] : 0.f;
+        acc = fmaf(weights[p], v, acc);
+    }
+    y[(uint64_t)t * hidden + h] = acc;
+}
+
+size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+struct grouped_layout {
+    size_t goff, glist, valid, xh, xl, xus, ah, al, aus, dn, total;
+};
+
+grouped_layout layout_of(const lev_moe_grouped_args &a) {
+    const size_t pairs = (size_t)a.tokens * a.top_k;
+    grouped_layout L;
+    size_t o = 0;
+    L.goff = o; o += align256((a.experts + 1) * 4);
+    L.glist = o; o += align256(pairs * 4);
+    L.valid = o; o += align256(pairs);
+    L.xh = o; o += align256((size_t)a.tokens * a.hidden * 2);
+    L.xl = o; o += align256((size_t)a.tokens * a.hidden * 2);
+    L.xus = o; o += align256((size_t)a.tokens * 4);
+    L.ah = o; o += align256(pairs * a.inter * 2);
+    L.al = o; o += align256(pairs * a.inter * 2);
+    L.aus = o; o += align256(pairs * 4);
+    L.dn = o; o += align256(pairs * a.hidden * 4);
+    L.total = o;
+    return L;
+}
+
+size_t grouped_lds(uint32_t in_len, bool paired) {
+    (void)paired;
+    return (size_t)2 * (in_len / 8) * kNC * 16 + (size_t)kGrpWaves * (16 * 36 + 16 * 8) * 4;
+}
+
+}  // namespace
+
+size_t lev_moe_grouped_scratch_bytes(const lev_moe_grouped_args &a) { return layout_of(a).total; }
+
+// Geometry the grouped path serves (the caller also checks 4-byte aligned pools).
+bool lev_moe_grouped_usable(const lev_ctx *ctx, const lev_moe_grouped_args &a) {
+    const size_t limit = ctx->props.sharedMemPerBlockOptin > ctx->props.sharedMemPerBlock
+                             ? ctx->props.sharedMemPerBlockOptin
+                             : ctx->props.sharedMemPerBlock;
+    return a.hidden % 256u == 0u && a.inter % 256u == 0u && a.experts <= 4096u &&
+           (uint64_t)a.tokens * a.top_k <= (1u << 20) && grouped_lds(a.hidden, true) <= limit &&
+           grouped_lds(a.inter, false) <= limit;
+}
+
+// act: f32 [tokens*top_k][inter] (written here, read by the down stage).
+hipError_t lev_moe_grouped_launch(lev_ctx *ctx, const lev_moe_grouped_args &a, const float *x,
+                                  const int32_t *ids, const float *weights, float *y, float *act,
+                                  void *scratch) {
+    const grouped_layout L = layout_of(a);
+    char *s = static_cast<char *>(scratch);
+    int32_t *goff = reinterpret_cast<int32_t *>(s + L.goff);
+    int32_t *glist = reinterpret_cast<int32_t *>(s + L.glist);
+    uint8_t *valid = reinterpret_cast<uint8_t *>(s + L.valid);
+    _Float16 *xh = reinterpret_cast<_Float16 *>(s + L.xh), *xl = reinterpret_cast<_Float16 *>(s + L.xl);
+    _Float16 *ah = reinterpret_cast<_Float16 *>(s + L.ah), *al = reinterpret_cast<_Float16 *>(s + L.al);
+    float *xus = reinterpret_cast<float *>(s + L.xus), *aus = reinterpret_cast<float *>(s + L.aus);
+    float *dn = reinterpret_cast<float *>(s + L.dn);
+    const uint32_t pairs = a.tokens * a.top_k;
+    hipError_t e;
+
+    hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), (size_t)2 * a.experts * 4, ctx->stream, ids,
+                       pairs, a.experts, a.top_k, goff, glist, valid, ctx->d_flag);
+    if ((e = hipGetLastError()) != hipSuccess) return e;
+    hipLaunchKernelGGL(moe_prep_kernel, dim3(a.tokens), dim3(256), 0, ctx->stream, x, a.hidden, xh, xl, xus);
+    if ((e = hipGetLastError()) != hipSuccess) return e;
+
+    static size_t lds_set[2] = {0, 0};
+    const size_t lds_gu = grouped_lds(a.hidden, true), lds_dn = grouped_lds(a.inter, false);
+    if (lds_gu > 48 * 1024 && lds_gu > lds_set[0]) {
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&moe_grouped_kernel<true>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_gu);
+        if (e != hipSuccess) return e;
+        lds_set[0] = lds_gu;
+    }
+    if (lds_dn > 48 * 1024 && lds_dn > lds_set[1]) {
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&moe_grouped_kernel<false>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dn);
+        if (e != hipSuccess) return e;
+        lds_set[1] = lds_dn;
+    }
+    const uint32_t rows_per_wg = kGrpWaves * 16, rows_per_wg_gu = rows_per_wg / 2;
+    hipLaunchKernelGGL((moe_grouped_kernel<true>), dim3((a.inter + rows_per_wg_gu - 1) / rows_per_wg_gu, a.experts),
+                       dim3(kGrpThreads), lds_gu, ctx->stream, a, xh, xl, xus, goff, glist, act);
+    if ((e = hipGetLastError()) != hipSuccess) return e;
+    // rows of act that belong to dropped pairs are never written; prep reads
+    // them all the same (any finite or non-finite value: they are never used)
+    hipLaunchKernelGGL(moe_prep_kernel, dim3(pairs), dim3(256), 0, ctx->stream, act, a.inter, ah, al, aus);
+    if ((e = hipGetLastError()) != hipSuccess) return e;
+    hipLaunchKernelGGL((moe_grouped_kernel<false>), dim3((a.hidden + rows_per_wg - 1) / rows_per_wg, a.experts),
+                       dim3(kGrpThreads), lds_dn, ctx->stream, a, ah, al, aus, goff, glist, dn);
+    if ((e = hipGetLastError()) != hipSuccess) return e;
+    hipLaunchKernelGGL(moe_merge_kernel, dim3((a.hidden + 255) / 256, a.tokens), dim3(256), 0, ctx->stream,
+                       dn, weights, valid, y, a.hidden, a.top_k);
+    return hipGetLastError();
+}

@@ -1,0 +1,20 @@
+// Interface between the MoE entry points and the many-token (grouped,
+// matrix-core) expert path.
+#pragma once
+
+#include "lev_common.hpp"
+
+struct lev_moe_grouped_args {
+    const uint8_t *base;
+    uint64_t gate_off, up_off, down_off;
+    uint64_t gate_stride, up_stride, down_stride;
+    uint32_t hidden, inter, experts, top_k, tokens;
+};
+
+size_t lev_moe_grouped_scratch_bytes(const lev_moe_grouped_args &a);
+// Geometry the grouped path serves (the caller also checks 4-byte aligned pools).
+bool lev_moe_grouped_usable(const lev_ctx *ctx, const lev_moe_grouped_args &a);
+// act: f32 [tokens*top_k][inter] (written here, read by the down stage).
+hipError_t lev_moe_grouped_launch(lev_ctx *ctx, const lev_moe_grouped_args &a, const float *x,
+                                  const int32_t *ids, const float *weights, float *y, float *act,
+                                  void *scratch);
