@@ -271,6 +271,27 @@ def main():
                     c, ring4.data_ptr(), ring4.numel(), (i % ncopy4) * nb4 * 144, xn.data_ptr(),
                     xn.numel(), gain.data_ptr(), 1e-6, yn.data_ptr(), yn.numel(), cols, r4, n)),
                     nb4 * 144 + cols * 4 + n * (cols * 4 + r4 * 4), 200, 20)
+            # int8-activation path: RMSNorm+quantise, then the integer-dot GEMV
+            # (timed together, as the reference's vk-q8 command times quantize + matvec)
+            for n in (1, 2, 4, 8, 16):
+                xn = torch.randn(n, cols, device=dev, generator=gen)
+                yn = torch.empty(n, r4, device=dev)
+                xq = torch.empty(n, cols, dtype=torch.int8, device=dev)
+                xs = torch.empty(n, cols // 32, 2, device=dev)
+
+                def q8_step(i, n=n, xn=xn, yn=yn, xq=xq, xs=xs):
+                    must(lib.lev_hip_norm_quant_q8(c, xn.data_ptr(), xn.numel(), None, gain.data_ptr(),
+                                                   1e-6, xq.data_ptr(), xs.data_ptr(), None, cols, n))
+                    must(lib.lev_hip_q4_k_gemv_q8(c, ring4.data_ptr(), ring4.numel(),
+                                                  (i % ncopy4) * nb4 * 144, xq.data_ptr(), xs.data_ptr(),
+                                                  xq.numel(), yn.data_ptr(), yn.numel(), cols, r4, n))
+                run_other(f"norm_quant_q8_q4_k_gemv_12288x4096_N{n}", q8_step,
+                          nb4 * 144 + cols * 4 + n * (cols * 4 + cols + cols // 4 + r4 * 4), 200, 20)
+                if n in (1, 8):
+                    run_other(f"q4_k_gemv_q8_only_12288x4096_N{n}", lambda i: must(lib.lev_hip_q4_k_gemv_q8(
+                        c, ring4.data_ptr(), ring4.numel(), (i % ncopy4) * nb4 * 144, xq.data_ptr(),
+                        xs.data_ptr(), xq.numel(), yn.data_ptr(), yn.numel(), cols, r4, n)),
+                        nb4 * 144 + n * (cols + cols // 4 + r4 * 4), 200, 20)
 
         # --------------------------------------------------- Q4_K prefill GEMM
         if want("gemm"):

@@ -159,6 +159,31 @@ int lev_hip_q4_k_gemv_ncol(lev_ctx *ctx, const void *d_w, size_t w_bytes, uint64
                            float *d_y, size_t y_capacity, uint32_t in_dim, uint32_t rows,
                            uint32_t ncol);
 
+/* ---- int8-activation decode path ----
+ * Activation quantiser: groups of 32, d = amax/127, q = roundEven(v * 127/amax),
+ * s = d * sum(q) (quantize_q8, lev-cpu/src/lib.rs:295-322; emit_quantize,
+ * lev-forge/src/q8.rs:20-51), optionally behind the residual add and the
+ * RMSNorm of the block input (emit_norm_quant, q8.rs:127-164; Builder::norm_quant,
+ * lev-model/src/gpu.rs:295):
+ *   d_add  != NULL: x += add first, written back to d_x (read-write then);
+ *   d_gain != NULL: v = rmsnorm(x, eps) * gain (f64 mean of squares as the
+ *                   reference CPU path, lev-model/src/lib.rs:110-114), else v = x;
+ *   d_y    != NULL: v is also stored as f32.
+ * x is [ncol][n], n a multiple of 32.  d_xq: int8 [ncol][n] (4-byte aligned),
+ * d_xs: f32 pairs (d, s) [ncol][n/32]. */
+int lev_hip_norm_quant_q8(lev_ctx *ctx, float *d_x, size_t x_count, const float *d_add,
+                          const float *d_gain, float eps, int8_t *d_xq, float *d_xs, float *d_y,
+                          uint32_t n, uint32_t ncol);
+
+/* Q4_K GEMV on the int8 activations above, ncol columns per weight read
+ * (q4k.q8.matvec, emit_q4k_q8, lev-forge/src/q8.rs:191-326; oracle
+ * matvec_q4k_q8_f64, lev-cpu/src/lib.rs:324-331).  Integer dot products per
+ * sub-block are exact; y[col*rows + row].  x_count counts int8 codes
+ * (in_dim * ncol); weights, d_xq and d_xs 16-byte aligned. */
+int lev_hip_q4_k_gemv_q8(lev_ctx *ctx, const void *d_w, size_t w_bytes, uint64_t w_off,
+                         const int8_t *d_xq, const float *d_xs, size_t x_count, float *d_y,
+                         size_t y_capacity, uint32_t in_dim, uint32_t rows, uint32_t ncol);
+
 /* ---- prefill GEMM (Builder::matvec_rows with gemm, gpu.rs:345-355;
  * q4k gemm blocked, lev-forge/src/coopmat.rs:236-323) ----
  * x is fp16 [tokens][in_dim], y is f32 [tokens][rows]; W is dequantised to

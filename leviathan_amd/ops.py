@@ -137,6 +137,32 @@ class Context:
                                                     in_dim, rows, ncol))
         return y
 
+    def norm_quant_q8(self, x, n: int, ncol: int, gain=None, eps: float = 1e-6, add=None,
+                      want_y: bool = False):
+        """Int8 activations of ``x`` [ncol][n]: returns (xq int8, xs (d, s) pairs[, y f32])."""
+        _dev(x, torch.float32, "x")
+        if gain is not None:
+            _dev(gain, torch.float32, "gain")
+        if add is not None:
+            _dev(add, torch.float32, "add")
+        xq = torch.empty((max(ncol, 1), max(n, 1)), dtype=torch.int8, device=x.device)
+        xs = torch.empty((max(ncol, 1), max(n // 32, 1), 2), dtype=torch.float32, device=x.device)
+        y = torch.empty_like(x) if want_y else None
+        self._check(self.lib.lev_hip_norm_quant_q8(self.ctx, _ptr(x), x.numel(), _ptr(add), _ptr(gain),
+                                                   eps, _ptr(xq), _ptr(xs), _ptr(y), n, ncol))
+        return (xq, xs, y) if want_y else (xq, xs)
+
+    def q4_k_gemv_q8(self, w, xq, xs, in_dim: int, rows: int, ncol: int, y=None, w_off: int = 0):
+        _dev(w, torch.uint8, "w")
+        _dev(xq, torch.int8, "xq")
+        _dev(xs, torch.float32, "xs")
+        if y is None:
+            y = torch.empty((max(ncol, 1), max(rows, 1)), dtype=torch.float32, device=w.device)
+        self._check(self.lib.lev_hip_q4_k_gemv_q8(self.ctx, _ptr(w), w.numel(), w_off, _ptr(xq),
+                                                  _ptr(xs), xq.numel(), _ptr(y), y.numel(), in_dim,
+                                                  rows, ncol))
+        return y
+
     def q4_k_gemm_prefill(self, w, x_f16, in_dim: int, rows: int, tokens: int, y=None, w_off: int = 0):
         _dev(w, torch.uint8, "w")
         _dev(x_f16, torch.float16, "x")

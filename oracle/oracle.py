@@ -351,6 +351,23 @@ def quantize_q8(x):
     return q, d, s
 
 
+def dequantize_q8(q, d) -> np.ndarray:
+    """xd = q as f32 * d[group], one f32 product per element (lev-cpu/src/lib.rs:327)."""
+    q = np.asarray(q, dtype=np.int8).reshape(-1)
+    d = np.asarray(d, dtype=np.float32).reshape(-1)
+    return (q.astype(np.float32) * np.repeat(d, 32)).astype(np.float32)
+
+
+def q4_k_matvec_q8_f64(w, rows, cols, q, d) -> np.ndarray:
+    """matvec_q4k_q8_f64, lev-cpu/src/lib.rs:324-331."""
+    return q4_k_matvec_f64(w, rows, cols, dequantize_q8(q, d))
+
+
+def q6_k_matvec_q8_f64(w, rows, cols, q, d) -> np.ndarray:
+    """matvec_q6k_q8_f64, lev-cpu/src/lib.rs:333-337."""
+    return q6_k_matvec_f64(w, rows, cols, dequantize_q8(q, d))
+
+
 # ---- RMSNorm ----
 _rms = _sig("levo_rmsnorm", None, _f32p, _f32p, C.c_float, C.c_size_t, _f32p)
 _rms_serial = _sig("levo_rmsnorm_f32_serial", None, _f32p, _f32p, C.c_float, C.c_size_t, _f32p)

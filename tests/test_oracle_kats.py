@@ -392,6 +392,27 @@ def test_q8_round_trip():
     assert not q.any() and d[0] == 0.0
 
 
+def test_q8_matvec_oracle_reduces_to_the_float_oracle_on_exact_codes():
+    """matvec_q4k_q8_f64 / matvec_q6k_q8_f64 (lev-cpu lib.rs:324-337) are the f64
+    matvec over q*d.  With integer activations whose group maximum is 127 the
+    scale is exactly 1 and q*d == x, so both oracles must give the float oracle's
+    answer bit for bit; halving x halves d (a power of two) and the answer."""
+    rng = np.random.default_rng(5)
+    x = rng.integers(-127, 128, size=512).astype(np.float32)
+    x[::32] = 127.0
+    q, d, s = O.quantize_q8(x)
+    assert (d == 1.0).all() and np.array_equal(q.astype(np.float32), x)
+    assert np.array_equal(s, x.reshape(-1, 32).sum(axis=1))
+    assert np.array_equal(O.dequantize_q8(q, d), x)
+    w4 = O.synth_q4_k(3, 6 * 2)
+    w6 = O.synth_q6_k(4, 6 * 2)
+    assert np.array_equal(O.q4_k_matvec_q8_f64(w4, 6, 512, q, d), O.q4_k_matvec_f64(w4, 6, 512, x))
+    assert np.array_equal(O.q6_k_matvec_q8_f64(w6, 6, 512, q, d), O.q6_k_matvec_f64(w6, 6, 512, x))
+    qh, dh, _ = O.quantize_q8(x * np.float32(0.5))
+    assert np.array_equal(qh, q) and (dh == 0.5).all()
+    assert np.array_equal(O.q4_k_matvec_q8_f64(w4, 6, 512, qh, dh), 0.5 * O.q4_k_matvec_f64(w4, 6, 512, x))
+
+
 # --------------------------------------------------------------------------
 # RMSNorm -- lev-model lib.rs:431-435; closed form; torch cross-check
 # --------------------------------------------------------------------------
