@@ -22,6 +22,8 @@
 // for the column counts of speculative verify.
 #include "lev_common.hpp"
 
+#include <cstdlib>
+
 #pragma clang fp contract(off)
 
 namespace {
@@ -263,6 +265,276 @@ hipError_t launch_q8(lev_ctx *ctx, const uint8_t *w, const uint32_t *xq, const f
     return hipGetLastError();
 }
 
+// ---------------------------------------------------------------------------
+// Q4_K x int8 GEMV on the matrix cores, up to 16 columns per weight read.
+//
+// v_mfma_i32_16x16x32_i8, one per sub-block of 32 weights: A = the activation
+// codes (16 "rows" = columns of x), B = 16 weight rows x 32 nibbles unpacked to
+// bytes, exact int32 out.  Lane (r, g) = (l % 16, l / 16) loads row r's header
+// and bytes 8g..8g+7 of each 32-byte chunk: their low nibbles are its 8 k-slots
+// of sub-block 2c, their high nibbles those of sub-block 2c+1 (one AND per four
+// weights, no permutation: the activations keep their natural order).  The
+// output lane of weight row n is the lane that loaded row n's header, so
+// d*sc_j and dmin are applied in place:
+//   y[col] += d*sc_j * (dx_j[col] * idot)      per sub-block, 12 vector ops for 4 columns
+//   y[col] -= dmin * sum_j m_j * s_j[col]      two v_mfma_f32_16x16x4_f32
+// Workgroup = 16 waves, one per CU; the waves share 16 weight rows, one
+// superblock column each, and their partial sums meet in LDS in wave order.
+// LDS: codes [sub-block][NCL columns][32 B] (a wave's A read is 512 contiguous
+// bytes), d and s as [sub-block][NCL] floats.
+// ---------------------------------------------------------------------------
+constexpr uint32_t kQ8MfmaMinCols = 9;   // measured on 12288x4096: the dot4 kernel wins up to 8 columns
+constexpr int kMThreads = 1024;
+constexpr int kMWaves = kMThreads / LEV_WAVE;
+typedef int lev_i32x4 __attribute__((ext_vector_type(4)));
+constexpr int kQ8mPieces = 6;   // 16-byte pieces of a column's codes a thread stages without a loop
+
+struct q8m_regs {
+    lev_u32x4 hdr;
+    lev_u32x2 c[4];
+};
+
+__device__ __forceinline__ void q8m_issue(const uint8_t *__restrict__ w, uint64_t row_bytes, uint32_t row,
+                                          uint32_t sb, uint32_t g, q8m_regs &R) {
+    const uint8_t *p = w + (uint64_t)row * row_bytes + (uint64_t)sb * 144u;
+    R.hdr = *reinterpret_cast<const lev_u32x4 *>(p);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) R.c[c] = *reinterpret_cast<const lev_u32x2 *>(p + 16u + 32u * c + 8u * g);
+}
+
+// NCL: columns the LDS layout holds (>= ncol).  SHORT: no wave has more than
+// three tasks and a column's codes fit the unrolled staging; the kernel is then
+// straight-line code (no loop holds a load), so every wait covers exactly the
+// loads it needs and the first task is multiplied while the others stream in.
+template <int NCL, bool SHORT>
+__global__ void __launch_bounds__(kMThreads)
+q4_k_q8_mfma(const uint8_t *__restrict__ w, const uint8_t *__restrict__ xq, const float *__restrict__ xs,
+             float *__restrict__ y, uint32_t cols, uint32_t rows, uint32_t ncol, uint32_t lognp) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const uint32_t SB = cols >> 8, subs = cols >> 5;
+    uint8_t *xa = smem;                                                  // [subs][NCL][32]
+    float *sd = reinterpret_cast<float *>(smem + (size_t)cols * NCL);    // [subs][NCL]
+    float *ssum = sd + (size_t)subs * NCL;                               // [subs][NCL]
+    float *part = ssum + (size_t)subs * NCL;                             // [2][wave][row][NCL]
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t r = lane & 15u, g = lane >> 4;
+
+    // ---- activations: 16 >> lognp waves per column, 16-byte pieces ----
+    const uint32_t np = 1u << lognp;
+    const uint32_t ac = wave & (np - 1u), apart = wave >> lognp, astride = 64u * (kMWaves >> lognp);
+    const bool acol = ac < ncol;
+    const uint32_t P = cols >> 4;                 // pieces per column
+    const lev_u32x4 *xsrc = reinterpret_cast<const lev_u32x4 *>(xq + (uint64_t)(acol ? ac : 0u) * cols);
+    const lev_u32x2 *ssrc = reinterpret_cast<const lev_u32x2 *>(xs) + (uint64_t)(acol ? ac : 0u) * subs;
+    constexpr int CHX = kQ8mPieces, CHS = kQ8mPieces / 2;
+    lev_u32x4 xv[CHX];
+    lev_u32x2 sv[CHS];
+    const uint32_t p0 = apart * 64u + lane;
+#pragma unroll
+    for (int i = 0; i < CHX; ++i) {
+        const uint32_t p = p0 + (uint32_t)i * astride;
+        xv[i] = xsrc[p < P ? p : 0u];
+    }
+#pragma unroll
+    for (int i = 0; i < CHS; ++i) {
+        const uint32_t k = p0 + (uint32_t)i * astride;
+        sv[i] = ssrc[k < subs ? k : 0u];
+    }
+
+    // ---- geometry of the weight stream: task = superblock wave + 16*t of the
+    // 16 rows of group rg (stride gridDim.x); a cursor walks them, no divisions.
+    // A task past the end reads the first bytes of the matrix. ----
+    const uint64_t row_bytes = (uint64_t)SB * 144u;
+    const uint32_t ngroups = (rows + 15u) >> 4;
+    const uint32_t tpr = (SB + kMWaves - 1u) / kMWaves;
+    const uint32_t ntasks = ((ngroups - blockIdx.x + gridDim.x - 1u) / gridDim.x) * tpr;
+    struct cursor {
+        uint32_t k, rg, t;
+    };
+    auto advance = [&](cursor &c) {
+        ++c.k;
+        if (++c.t == tpr) {
+            c.t = 0;
+            c.rg += gridDim.x;
+        }
+    };
+    auto issue = [&](cursor &c, q8m_regs &W) {
+        const uint32_t sbw = wave + kMWaves * c.t;
+        const bool real = c.k < ntasks && sbw < SB;
+        uint32_t row = c.rg * 16u + r;
+        row = row < rows ? row : rows - 1u;
+        q8m_issue(w, row_bytes, real ? row : 0u, real ? sbw : 0u, real ? g : 0u, W);
+        advance(c);
+    };
+    cursor ci{0u, blockIdx.x, 0u}, cc{0u, blockIdx.x, 0u};
+    q8m_regs W0, W1, W2;
+    issue(ci, W0);
+    issue(ci, W1);
+    issue(ci, W2);
+
+    // the activation loads were issued first and return first
+#pragma unroll
+    for (int i = 0; i < CHX; ++i) {
+        const uint32_t p = p0 + (uint32_t)i * astride;
+        if (acol && p < P) *reinterpret_cast<lev_u32x4 *>(xa + ((size_t)(p >> 1) * NCL + ac) * 32u + (p & 1u) * 16u) = xv[i];
+    }
+#pragma unroll
+    for (int i = 0; i < CHS; ++i) {
+        const uint32_t k = p0 + (uint32_t)i * astride;
+        if (acol && k < subs) {
+            sd[(size_t)k * NCL + ac] = __uint_as_float(sv[i].x);
+            ssum[(size_t)k * NCL + ac] = __uint_as_float(sv[i].y);
+        }
+    }
+    if constexpr (!SHORT) if (acol) {   // columns longer than the unrolled part
+        for (uint32_t p = p0 + CHX * astride; p < P; p += astride)
+            *reinterpret_cast<lev_u32x4 *>(xa + ((size_t)(p >> 1) * NCL + ac) * 32u + (p & 1u) * 16u) = xsrc[p];
+        for (uint32_t k = p0 + CHS * astride; k < subs; k += astride) {
+            const lev_u32x2 v = ssrc[k];
+            sd[(size_t)k * NCL + ac] = __uint_as_float(v.x);
+            ssum[(size_t)k * NCL + ac] = __uint_as_float(v.y);
+        }
+    }
+    __syncthreads();
+
+    // ---- stream the weights ----
+    const uint32_t colc = r < (uint32_t)NCL ? r : (uint32_t)NCL - 1u;    // A rows past NCL: any valid address
+    const uint32_t gq = 4u * g < (uint32_t)NCL ? 4u * g : 0u;            // first of the lane's four output columns
+    const uint32_t gm8 = 8u * g;
+    lev_f32x4 yacc = {0.f, 0.f, 0.f, 0.f};
+    uint32_t parity = 0;
+    auto compute = [&](cursor &c, const q8m_regs &W) {
+        const uint32_t rg = c.rg, t = c.t;
+        const uint32_t sbw = wave + kMWaves * t;
+        const bool live = sbw < SB;
+        const uint32_t sb = live ? sbw : SB - 1u;
+        const uint32_t S0 = W.hdr.y, S1 = W.hdr.z, S2 = W.hdr.w;
+        const float d = live ? lev_f16_bits_to_f32(W.hdr.x & 0xFFFFu) : 0.f;
+        const float dmin = live ? lev_f16_bits_to_f32(W.hdr.x >> 16) : 0.f;
+        const uint8_t *xrow = xa + ((size_t)sb * 8u * NCL + colc) * 32u + gm8;
+        const float *drow = sd + (size_t)sb * 8u * NCL + gq;
+        lev_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            // unpack_scale_min, lev-cpu/src/lib.rs:64-74
+            const uint32_t sc = j < 4 ? (S0 >> (8 * j)) & 63u
+                                      : ((S2 >> (8 * (j - 4))) & 0xFu) | (((S0 >> (8 * (j - 4) + 6)) & 3u) << 4);
+            const float scl = d * (float)sc;
+            lev_u32x2 wv = W.c[j >> 1];
+            if (j & 1) wv >>= 4;
+            wv &= 0x0F0F0F0Fu;
+            const long B = __builtin_bit_cast(long, wv);
+            const long A = *reinterpret_cast<const long *>(xrow + (size_t)j * NCL * 32u);
+            const lev_i32x4 D = __builtin_amdgcn_mfma_i32_16x16x32_i8(A, B, lev_i32x4{0, 0, 0, 0}, 0, 0, 0);
+            const lev_f32x4 dx = *reinterpret_cast<const lev_f32x4 *>(drow + (size_t)j * NCL);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[i] = fmaf(scl, dx[i] * (float)D[i], acc[i]);
+        }
+        // mins: two 16x16x4 f32 products, k = lane group: m_g and m_{4+g} of the lane's row
+        const float mA = (float)((S1 >> gm8) & 63u);
+        const float mB = (float)(((S2 >> (gm8 + 4u)) & 0xFu) | (((S1 >> (gm8 + 6u)) & 3u) << 4));
+        const float sA = ssum[((size_t)sb * 8u + g) * NCL + colc];
+        const float sB = ssum[((size_t)sb * 8u + 4u + g) * NCL + colc];
+        lev_f32x4 acc2 = {0.f, 0.f, 0.f, 0.f};
+        acc2 = __builtin_amdgcn_mfma_f32_16x16x4f32(sA, mA, acc2, 0, 0, 0);
+        acc2 = __builtin_amdgcn_mfma_f32_16x16x4f32(sB, mB, acc2, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) yacc[i] += fmaf(-dmin, acc2[i], acc[i]);
+
+        if (t + 1u == tpr) {   // workgroup-uniform
+            float *pp = part + parity * (kMWaves * 16 * NCL);   // two buffers: one barrier per group
+            parity ^= 1u;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (4u * g + (uint32_t)i < (uint32_t)NCL) pp[(wave * 16u + r) * NCL + 4u * g + i] = yacc[i];
+            yacc = lev_f32x4{0.f, 0.f, 0.f, 0.f};
+            __syncthreads();
+            if (tid < 16u * NCL) {
+                const uint32_t col = tid >> 4, rr = tid & 15u, row = rg * 16u + rr;
+                float sum = 0.f;
+#pragma unroll
+                for (int kk = 0; kk < kMWaves; ++kk) sum += pp[((uint32_t)kk * 16u + rr) * NCL + col];
+                if (col < ncol && row < rows) y[(uint64_t)col * rows + row] = sum;
+            }
+        }
+        advance(c);
+    };
+
+    if constexpr (SHORT) {
+        compute(cc, W0);
+        if (ntasks > 1u) compute(cc, W1);
+        if (ntasks > 2u) compute(cc, W2);
+        return;
+    }
+    // The scheduling barriers keep a refill's loads behind the compute that
+    // frees its registers.
+    while (true) {
+        compute(cc, W0);
+        __builtin_amdgcn_sched_barrier(0);
+        issue(ci, W0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (cc.k >= ntasks) break;
+        compute(cc, W1);
+        __builtin_amdgcn_sched_barrier(0);
+        issue(ci, W1);
+        __builtin_amdgcn_sched_barrier(0);
+        if (cc.k >= ntasks) break;
+        compute(cc, W2);
+        __builtin_amdgcn_sched_barrier(0);
+        issue(ci, W2);
+        __builtin_amdgcn_sched_barrier(0);
+        if (cc.k >= ntasks) break;
+    }
+}
+
+size_t q8m_lds_bytes(uint32_t cols, uint32_t ncl) {
+    return (size_t)cols * ncl + (size_t)2 * (cols >> 5) * ncl * 4 + (size_t)2 * kMWaves * 16 * ncl * 4;
+}
+
+template <int NCL, bool SHORT>
+hipError_t launch_q8m_variant(lev_ctx *ctx, const uint8_t *w, const uint8_t *xq, const float *xs, float *y,
+                              uint32_t cols, uint32_t rows, uint32_t ncol, uint32_t blocks) {
+    const size_t lds = q8m_lds_bytes(cols, NCL);
+    static size_t configured = 0;   // per instantiation: raise the dynamic LDS limit once per size
+    if (lds > 48 * 1024 && lds > configured) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&q4_k_q8_mfma<NCL, SHORT>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        configured = lds;
+    }
+    uint32_t lognp = 0;
+    while ((1u << lognp) < ncol) ++lognp;
+    hipLaunchKernelGGL((q4_k_q8_mfma<NCL, SHORT>), dim3(blocks), dim3(kMThreads), lds, ctx->stream, w, xq,
+                       xs, y, cols, rows, ncol, lognp);
+    return hipGetLastError();
+}
+
+template <int NCL>
+hipError_t launch_q8m(lev_ctx *ctx, const uint8_t *w, const uint8_t *xq, const float *xs, float *y,
+                      uint32_t cols, uint32_t rows, uint32_t ncol) {
+    const uint32_t groups = (rows + 15u) / 16u;
+    const uint32_t blocks = groups < (uint32_t)ctx->num_cus ? groups : (uint32_t)ctx->num_cus;
+    const uint32_t tpr = ((cols >> 8) + kMWaves - 1u) / kMWaves;
+    const uint32_t most = ((groups + blocks - 1u) / blocks) * tpr;   // tasks of the busiest wave
+    uint32_t lognp = 0;
+    while ((1u << lognp) < ncol) ++lognp;
+    const bool staged = (cols >> 4) <= kQ8mPieces * 64u * ((uint32_t)kMWaves >> lognp);
+    if (most <= 3u && staged)
+        return launch_q8m_variant<NCL, true>(ctx, w, xq, xs, y, cols, rows, ncol, blocks);
+    return launch_q8m_variant<NCL, false>(ctx, w, xq, xs, y, cols, rows, ncol, blocks);
+}
+
+// Columns one launch of the matrix-core kernel takes for this in_dim (0: none).
+uint32_t q8m_cols(const lev_ctx *ctx, uint32_t in_dim) {
+    const size_t limit = ctx->props.sharedMemPerBlockOptin > ctx->props.sharedMemPerBlock
+                             ? ctx->props.sharedMemPerBlockOptin
+                             : ctx->props.sharedMemPerBlock;
+    for (uint32_t ncl = 16; ncl >= 4u; ncl >>= 1)
+        if (q8m_lds_bytes(in_dim, ncl) <= limit) return ncl;
+    return 0;
+}
+
 }  // namespace
 
 extern "C" int lev_hip_norm_quant_q8(lev_ctx *ctx, float *d_x, size_t x_count, const float *d_add,
@@ -307,23 +579,36 @@ extern "C" int lev_hip_q4_k_gemv_q8(lev_ctx *ctx, const void *d_w, size_t w_byte
                              ? ctx->props.sharedMemPerBlockOptin
                              : ctx->props.sharedMemPerBlock;
     const uint32_t *xq = reinterpret_cast<const uint32_t *>(d_xq);
+    // Matrix-core kernel from kQ8MfmaMinCols columns up (LEV_Q8_MFMA=0 / 1 forces
+    // the choice, for measurements); the dot4 kernel otherwise.
+    const uint32_t mcols = q8m_cols(ctx, in_dim);
+    const char *force = getenv("LEV_Q8_MFMA");
+    const bool mfma = mcols != 0u && (force ? force[0] != '0' : ncol >= kQ8MfmaMinCols);
     uint32_t done = 0;
     while (done < ncol) {
         uint32_t nc = ncol - done;
-        // columns per launch: 8, 4, 2 or 1, within the LDS budget
-        uint32_t fit = 8;
-        while (fit > 1u && (size_t)fit * (in_dim >> 8) * (kCodeStride + kPairStride) > limit) fit >>= 1;
-        if ((size_t)(in_dim >> 8) * (kCodeStride + kPairStride) > limit)
-            return lev_fail(ctx, LEV_ERR_EXCEEDS_MODEL_WORKLOAD, "q4_k_gemv_q8: inDim %u does not fit the staging", in_dim);
-        if (nc > fit) nc = fit;
         const uint32_t *xqc = xq + ((uint64_t)done * in_dim >> 2);
         const float *xsc = d_xs + (uint64_t)done * (in_dim >> 5) * 2u;
         float *yc = d_y + (uint64_t)done * rows;
         hipError_t e;
-        if (nc > 4) e = launch_q8<8>(ctx, w, xqc, xsc, yc, in_dim, rows, nc);
-        else if (nc > 2) e = launch_q8<4>(ctx, w, xqc, xsc, yc, in_dim, rows, nc);
-        else if (nc > 1) e = launch_q8<2>(ctx, w, xqc, xsc, yc, in_dim, rows, nc);
-        else e = launch_q8<1>(ctx, w, xqc, xsc, yc, in_dim, rows, nc);
+        if (mfma) {
+            if (nc > mcols) nc = mcols;
+            const uint8_t *xb = reinterpret_cast<const uint8_t *>(xqc);
+            if (mcols == 16u) e = launch_q8m<16>(ctx, w, xb, xsc, yc, in_dim, rows, nc);
+            else if (mcols == 8u) e = launch_q8m<8>(ctx, w, xb, xsc, yc, in_dim, rows, nc);
+            else e = launch_q8m<4>(ctx, w, xb, xsc, yc, in_dim, rows, nc);
+        } else {
+            // columns per launch: 8, 4, 2 or 1, within the LDS budget
+            uint32_t fit = 8;
+            while (fit > 1u && (size_t)fit * (in_dim >> 8) * (kCodeStride + kPairStride) > limit) fit >>= 1;
+            if ((size_t)(in_dim >> 8) * (kCodeStride + kPairStride) > limit)
+                return lev_fail(ctx, LEV_ERR_EXCEEDS_MODEL_WORKLOAD, "q4_k_gemv_q8: inDim %u does not fit the staging", in_dim);
+            if (nc > fit) nc = fit;
+            if (nc > 4) e = launch_q8<8>(ctx, w, xqc, xsc, yc, in_dim, rows, nc);
+            else if (nc > 2) e = launch_q8<4>(ctx, w, xqc, xsc, yc, in_dim, rows, nc);
+            else if (nc > 1) e = launch_q8<2>(ctx, w, xqc, xsc, yc, in_dim, rows, nc);
+            else e = launch_q8<1>(ctx, w, xqc, xsc, yc, in_dim, rows, nc);
+        }
         if (e != hipSuccess) return lev_hip_check(ctx, e, "q4_k_gemv_q8 launch");
         done += nc;
     }
