@@ -13,6 +13,7 @@
 //   Runner::matvec / matvecDispatch      Gemma4.swift:2583, 2638
 //   Runner::expertMatvec                 Gemma4.swift:2805 (slice addressing; the slot cache is not mirrored)
 //   Runner::rmsnorm / geluUp / axpy      Gemma4.swift:3014, 3103, 3115
+//   Runner::normQuant / matvecQ8         Builder::norm_quant / matvec, rust/crates/lev-model/src/gpu.rs:295, 334
 //   Runner::routeTopK                    Gemma4.swift:3795-3810 (router matvec + softmax/top-k)
 //   Runner::runMoeBatchedRouted          Gemma4.swift:2073
 //   Runner::flushOpenSegment             Gemma4.swift:2313
@@ -22,6 +23,7 @@
 // Header-only; link with -lleviathan_hip.
 #pragma once
 
+#include <algorithm>
 #include <cmath>
 #include <cstdint>
 #include <cstring>
@@ -349,6 +351,57 @@ public:
             geometry("rmsnorm buffers too small");
         check(lev_hip_rmsnorm(ctx_, x.floats(), y.floats(), (uint32_t)n, (uint32_t)vectors, w, eps_),
               "rmsnorm");
+    }
+
+    // ---- Builder::norm_quant, rust/crates/lev-model/src/gpu.rs:295-320 ----
+    // x [nb][ne] += add (if given, written back), RMS norm with the weight
+    // tensor (if given; otherwise the plain quantiser, gpu.rs:282-290), int8
+    // codes into xq [nb][ne], (d, s) pairs into xs [nb][ne/32]; y (if given)
+    // also receives the f32 result.
+    void normQuant(DeviceBuffer &x, int64_t ne, int64_t nb, const std::optional<std::string> &weightTensor,
+                   DeviceBuffer &xq, DeviceBuffer &xs, const DeviceBuffer *add = nullptr,
+                   DeviceBuffer *y = nullptr) {
+        const float *w = nullptr;
+        if (weightTensor) {
+            auto it = ref_.find(*weightTensor);
+            if (it == ref_.end() || it->second.type != GGMLTensorType::float32 ||
+                it->second.inDim != ne || it->second.end - it->second.offset != ne * 4)
+                geometry("bad norm weight " + *weightTensor);
+            w = reinterpret_cast<const float *>(static_cast<const char *>(weights_.contents()) +
+                                                it->second.offset);
+        }
+        int64_t count;
+        if (ne <= 0 || nb <= 0 || ne % 32 != 0 || __builtin_mul_overflow(ne, nb, &count) ||
+            x.length < count * 4 || xq.length < count || xs.length < count / 32 * 8 ||
+            (add && add->length < count * 4) || (y && y->length < count * 4))
+            geometry("norm_quant buffers too small");
+        check(lev_hip_norm_quant_q8(ctx_, x.floats(), (size_t)count, add ? add->floats() : nullptr, w, eps_,
+                                    static_cast<int8_t *>(xq.contents()), xs.floats(),
+                                    y ? y->floats() : nullptr, (uint32_t)ne, (uint32_t)nb),
+              "norm_quant");
+    }
+
+    // ---- Builder::matvec / matvec_rows on int8 activations, gpu.rs:334-370 ----
+    // y[nb][rows] (from float index yOffset) = W x for a Q4_K tensor; reads the
+    // activations quantised by normQuant; maxRows takes a prefix of the rows.
+    void matvecQ8(const std::string &tensor, const DeviceBuffer &xq, const DeviceBuffer &xs, int64_t nb,
+                  DeviceBuffer &y, int64_t yOffset = 0, std::optional<int64_t> maxRows = std::nullopt) {
+        const TensorRef &r = lookup(tensor);
+        if (r.type != GGMLTensorType::q4_K) geometry(tensor + ": unsupported type for the int8 matvec");
+        const int64_t rows = std::min(r.outDim, maxRows.value_or(r.outDim));
+        int64_t count, outs, weightBytes, wEnd;
+        if (!(rows > 0 && r.inDim > 0 && r.inDim % 256 == 0 && nb > 0 && yOffset >= 0) ||
+            __builtin_mul_overflow(r.inDim, nb, &count) || __builtin_mul_overflow(rows, nb, &outs) ||
+            xq.length < count || xs.length < count / 32 * 8 || y.length < (yOffset + outs) * 4)
+            geometry("buffer extents violated for " + tensor);
+        if (__builtin_mul_overflow(rows, r.inDim / 256 * 144, &weightBytes) ||
+            __builtin_add_overflow(r.offset, weightBytes, &wEnd) || wEnd > r.end || wEnd > mapEnd_)
+            geometry(tensor + ": weight bytes beyond tensor extent");
+        check(lev_hip_q4_k_gemv_q8(ctx_, weights_.contents(), (size_t)weights_.length, (uint64_t)r.offset,
+                                   static_cast<const int8_t *>(xq.contents()), xs.floats(), (size_t)count,
+                                   y.floats() + yOffset, (size_t)(y.length / 4 - yOffset), (uint32_t)r.inDim,
+                                   (uint32_t)rows, (uint32_t)nb),
+              tensor);
     }
 
     // ---- Gemma4.swift:3103 ----

@@ -172,6 +172,8 @@ struct Model {
             [](uint8_t *p, size_t n) { levo_fill_normal(33, 1.f, 0.1f, reinterpret_cast<float *>(p), n / 4); });
         add("blk.0.ffn_gate_inp.weight", GGMLTensorType::float32, hidden, experts, 1,
             [](uint8_t *p, size_t n) { levo_fill_normal(34, 0.f, 0.02f, reinterpret_cast<float *>(p), n / 4); });
+        add("blk.0.ffn_up.weight", GGMLTensorType::q4_K, hidden, 64, 1,
+            [](uint8_t *p, size_t n) { levo_synth_q4_k(37, 0.01f, p, n / 144); });
         // fused gate|up [2I, H] per expert, as the reference stores it
         int64_t gu = add("blk.0.ffn_gate_up_exps.weight", GGMLTensorType::q4_0, hidden, 2 * inter, experts,
                          [](uint8_t *p, size_t n) { levo_synth_q4_0(35, 0.02f, p, n / 18); });
@@ -229,6 +231,59 @@ void runner_matvec(Runner &r, const Model &m) {
     EXPECT(throws_geometry([&] { r.matvec("blk.0.attn_q.weight", dx, H, dy, H, -18); }));         // before the tensor
     EXPECT(throws_geometry([&] { r.matvec("blk.0.attn_q.weight", dx, H, dy, H, 0, 0); }));        // zero rows
     r.flushOpenSegment();   // nothing failed on the device
+}
+
+// Int8-activation decode path: Builder::norm_quant then Builder::matvec
+// (rust/crates/lev-model/src/gpu.rs:295-370), gated as vk_q8 does
+// (lev-cli/src/main.rs:1788-1868): codes bit-exact with quantize_q8 of the CPU
+// rmsnorm, product within 1e-4 of the f64 oracle on those codes.
+void runner_int8_path(Runner &r, const Model &m) {
+    const int H = Model::hidden, NB = 2, ROWS = 64;
+    std::vector<float> x((size_t)NB * H), delta((size_t)NB * H);
+    levo_fill_normal(71, 0.f, 1.f, x.data(), x.size());
+    levo_fill_normal(72, 0.f, 0.5f, delta.data(), delta.size());
+    DeviceBuffer dx = r.makeBuffer(x), dd = r.makeBuffer(delta);
+    DeviceBuffer xq = r.makeBuffer((int64_t)NB * H), xs = r.makeBuffer((int64_t)NB * H / 32 * 8);
+    DeviceBuffer dyn = r.makeBuffer((int64_t)NB * H * 4), dy = r.makeBuffer((int64_t)NB * ROWS * 4);
+    r.normQuant(dx, H, NB, std::string("blk.0.ffn_norm.weight"), xq, xs, &dd, &dyn);
+    r.matvecQ8("blk.0.ffn_up.weight", xq, xs, NB, dy);
+    std::vector<float> xsum = r.read<float>(dx, x.size()), yn = r.read<float>(dyn, x.size());
+    std::vector<int8_t> q = r.read<int8_t>(xq, x.size());
+    std::vector<float> pairs = r.read<float>(xs, (size_t)NB * H / 32 * 2), y = r.read<float>(dy, (size_t)NB * ROWS);
+    const float *gain = reinterpret_cast<const float *>(m.at("blk.0.ffn_norm.weight"));
+    const TensorRef &t = m.table.at("blk.0.ffn_up.weight");
+    for (int c = 0; c < NB; ++c) {
+        std::vector<float> sum(H), want(H), wd(H / 32), ws(H / 32), xd(H);
+        std::vector<int8_t> wq(H);
+        for (int i = 0; i < H; ++i) sum[i] = x[(size_t)c * H + i] + delta[(size_t)c * H + i];
+        levo_rmsnorm(sum.data(), gain, 1e-6f, H, want.data());
+        EXPECT(levo_quantize_q8(want.data(), H, wq.data(), wd.data(), ws.data()) == 0);
+        EXPECT(std::memcmp(xsum.data() + (size_t)c * H, sum.data(), H * 4) == 0);      // x += add, written back
+        EXPECT(std::memcmp(yn.data() + (size_t)c * H, want.data(), H * 4) == 0);      // f32 result
+        EXPECT(std::memcmp(q.data() + (size_t)c * H, wq.data(), H) == 0);
+        for (int g = 0; g < H / 32; ++g) {
+            EXPECT(pairs[((size_t)c * (H / 32) + g) * 2] == wd[g]);
+            EXPECT(pairs[((size_t)c * (H / 32) + g) * 2 + 1] == ws[g]);
+        }
+        for (int i = 0; i < H; ++i) xd[i] = (float)wq[i] * wd[i / 32];                 // lev-cpu/src/lib.rs:327
+        std::vector<double> ref(ROWS);
+        EXPECT(levo_q4_k_matvec_f64(m.at("blk.0.ffn_up.weight"), (size_t)(t.end - t.offset), ROWS, H, xd.data(), H,
+                                    ref.data()) == 0);
+        std::vector<float> got(y.begin() + (size_t)c * ROWS, y.begin() + (size_t)(c + 1) * ROWS);
+        EXPECT(rel_err(got, ref) < 1e-4);
+    }
+    // a prefix of the rows (matvec_rows), and the guards before any launch
+    r.matvecQ8("blk.0.ffn_up.weight", xq, xs, NB, dy, 0, 16);
+    std::vector<float> y16 = r.read<float>(dy, (size_t)NB * 16);
+    for (int c = 0; c < NB; ++c)
+        for (int i = 0; i < 16; ++i) EXPECT(y16[(size_t)c * 16 + i] == y[(size_t)c * ROWS + i]);
+    EXPECT(throws_geometry([&] { r.matvecQ8("blk.0.attn_q.weight", xq, xs, NB, dy); }));        // not Q4_K
+    EXPECT(throws_geometry([&] { r.matvecQ8("blk.0.ffn_up.weight", xq, xs, NB + 1, dy); }));    // xq too small
+    EXPECT(throws_geometry([&] { r.matvecQ8("blk.0.ffn_up.weight", xq, xs, NB, dy, 8); }));     // y too small
+    EXPECT(throws_geometry([&] { r.normQuant(dx, H - 32 + 1, 1, std::nullopt, xq, xs); }));     // not a multiple of 32
+    EXPECT(throws_geometry([&] { r.normQuant(dx, H, NB + 1, std::nullopt, xq, xs); }));
+    EXPECT(throws_geometry([&] { r.normQuant(dx, H, NB, std::string("blk.0.attn_q.weight"), xq, xs); }));
+    r.flushOpenSegment();
 }
 
 void runner_elementwise(Runner &r, const Model &m) {
@@ -398,6 +453,7 @@ int main(int argc, char **argv) {
         {"q4_backend_seeded", q4_backend_seeded},
         {"runner_matvec", [&] { runner_matvec(R(), model); }},
         {"runner_elementwise", [&] { runner_elementwise(R(), model); }},
+        {"runner_int8_path", [&] { runner_int8_path(R(), model); }},
         {"runner_moe", [&] { runner_moe(R(), model); }},
         {"runner_moe_hand_computed", [&] { runner_moe_hand_computed(R()); }},
     };
