@@ -255,6 +255,18 @@ def main():
             run_other("q6_k_gemv_32000x4096_no_argmax", lambda i: must(lib.lev_hip_q6_k_gemv(
                 c, ring6.data_ptr(), ring6.numel(), (i % 6) * nb6 * 210, x.data_ptr(), cols,
                 y6.data_ptr(), r6, cols, r6, None, None)), nb6 * 210 + cols * 4 + r6 * 4, 100, 20)
+            # the head on int8 activations, N columns per weight read (MTP verify)
+            for n in (1, 4, 8):
+                xn = torch.randn(n, cols, device=dev, generator=gen)
+                yn = torch.empty(n, r6, device=dev)
+                xq = torch.empty(n, cols, dtype=torch.int8, device=dev)
+                xs = torch.empty(n, cols // 32, 2, device=dev)
+                must(lib.lev_hip_norm_quant_q8(c, xn.data_ptr(), xn.numel(), None, None, 0.0,
+                                               xq.data_ptr(), xs.data_ptr(), None, cols, n))
+                run_other(f"q6_k_gemv_q8_32000x4096_N{n}", lambda i: must(lib.lev_hip_q6_k_gemv_q8(
+                    c, ring6.data_ptr(), ring6.numel(), (i % 6) * nb6 * 210, xq.data_ptr(), xs.data_ptr(),
+                    xq.numel(), yn.data_ptr(), yn.numel(), cols, r6, n)),
+                    nb6 * 210 + n * (cols + cols // 4 + r6 * 4), 50, 10)
             del ring6
 
         # ------------------------------------------- RMSNorm + Q4_K N columns

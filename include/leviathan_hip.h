@@ -184,6 +184,19 @@ int lev_hip_q4_k_gemv_q8(lev_ctx *ctx, const void *d_w, size_t w_bytes, uint64_t
                          const int8_t *d_xq, const float *d_xs, size_t x_count, float *d_y,
                          size_t y_capacity, uint32_t in_dim, uint32_t rows, uint32_t ncol);
 
+/* Q6_K GEMV on the same int8 activations (q6k.q8.matvec, emit_q6k_q8,
+ * lev-forge/src/q8.rs:330-447; oracle matvec_q6k_q8_f64, lev-cpu/src/lib.rs:333-337):
+ * the LM head of a multi-column verify step.  Weights 2-byte aligned (GGUF). */
+int lev_hip_q6_k_gemv_q8(lev_ctx *ctx, const void *d_w, size_t w_bytes, uint64_t w_off,
+                         const int8_t *d_xq, const float *d_xs, size_t x_count, float *d_y,
+                         size_t y_capacity, uint32_t in_dim, uint32_t rows, uint32_t ncol);
+
+/* act = silu(gate) * up fused with the quantiser (emit_swiglu_quant,
+ * lev-forge/src/q8.rs:166-177; Builder::swiglu_quant, lev-model/src/gpu.rs:322-330).
+ * count values (a multiple of 32); d_act (optional) also receives act as f32. */
+int lev_hip_swiglu_quant_q8(lev_ctx *ctx, const float *d_gate, const float *d_up, size_t count,
+                            int8_t *d_xq, float *d_xs, float *d_act);
+
 /* ---- prefill GEMM (Builder::matvec_rows with gemm, gpu.rs:345-355;
  * q4k gemm blocked, lev-forge/src/coopmat.rs:236-323) ----
  * x is fp16 [tokens][in_dim], y is f32 [tokens][rows]; W is dequantised to

@@ -266,6 +266,190 @@ hipError_t launch_q8(lev_ctx *ctx, const uint8_t *w, const uint32_t *xq, const f
 }
 
 // ---------------------------------------------------------------------------
+// Q6_K x int8 GEMV, NC columns (q6k.q8.matvec, emit_q6k_q8, lev-forge/src/q8.rs:330-447;
+// oracle matvec_q6k_q8_f64, lev-cpu/src/lib.rs:333-337).
+//
+// A lane owns half a superblock: 64 ql bytes, the 32 qh bytes they pair with,
+// 8 sub-scales and d (q6k_unpack, lev-cpu/src/lib.rs:203-216).  Its 128 weights
+// are four activation groups of 32 (k = 0..3): byte l of the assembled dwords
+//   k=0: (qlA & 15) | (qh     & 3) << 4      k=1: (qlB & 15) | (qh >> 2 & 3) << 4
+//   k=2: (qlA >> 4) | (qh >> 4 & 3) << 4     k=3: (qlB >> 4) | (qh >> 6 & 3) << 4
+// is element 32k + l, in the order of the activation codes, so every dword goes
+// straight into v_dot4.  The codes stay unsigned (0..63); the -32 is applied
+// through the sum of the activation codes over each 16 weights, formed once
+// per column while staging:  sc * dx * (sum q*xq - 32 * sum xq).
+// 32 lanes per row (4096 columns = 32 halves), a wave covers two rows.
+// LDS per (column, superblock): 272 B of codes, 8 group scales, 16 code sums.
+// ---------------------------------------------------------------------------
+constexpr uint32_t kQ6Stride = 272 + 32 + 64;
+struct __attribute__((packed, aligned(2))) q8_u32x4_a2 { uint32_t v[4]; };
+struct __attribute__((packed, aligned(2))) q8_u32x2_a2 { uint32_t v[2]; };
+
+template <int NC>
+__global__ void __launch_bounds__(kQThreads)
+q6_k_gemv_q8_kernel(const uint8_t *__restrict__ w, const uint32_t *__restrict__ xq,
+                    const float *__restrict__ xs, float *__restrict__ y, uint32_t in_dim,
+                    uint32_t rows, uint32_t ncol) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const uint32_t SB = in_dim >> 8;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+
+    // stage: 16-byte pieces of codes and their sums; group scales
+    for (uint32_t i = tid; i < (uint32_t)NC * SB * 16u; i += kQThreads) {
+        const uint32_t c = i / (SB * 16u), rem = i - c * (SB * 16u), sb = rem >> 4, k = rem & 15u;
+        lev_u32x4 v = {0u, 0u, 0u, 0u};
+        if (c < ncol) v = *reinterpret_cast<const lev_u32x4 *>(xq + ((uint64_t)c * in_dim >> 2) + sb * 64u + k * 4u);
+        uint8_t *base = smem + ((size_t)c * SB + sb) * kQ6Stride;
+        *reinterpret_cast<lev_u32x4 *>(base + k * 16u) = v;
+        int sum = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) sum = __builtin_amdgcn_sdot4(0x01010101, (int)v[j], sum, false);
+        reinterpret_cast<int *>(base + 304u)[k] = sum;
+    }
+    for (uint32_t i = tid; i < (uint32_t)NC * SB * 8u; i += kQThreads) {
+        const uint32_t c = i / (SB * 8u), rem = i - c * (SB * 8u), sb = rem >> 3, k = rem & 7u;
+        float d = 0.f;
+        if (c < ncol) d = xs[((uint64_t)c * (in_dim >> 5) + sb * 8u + k) * 2u];
+        reinterpret_cast<float *>(smem + ((size_t)c * SB + sb) * kQ6Stride + 272u)[k] = d;
+    }
+    __syncthreads();
+
+    const uint32_t grp = lane >> 5, lp = lane & 31u;
+    const uint32_t halves = SB * 2u;
+    const uint64_t row_bytes = (uint64_t)SB * 210u;
+    const uint32_t tiles = (rows + 7u) >> 3;            // 8 rows per workgroup tile
+    for (uint32_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+        const uint32_t row = tile * 8u + wave * 2u + grp;
+        const uint32_t rowc = row < rows ? row : rows - 1u;
+        float acc[NC];
+#pragma unroll
+        for (int c = 0; c < NC; ++c) acc[c] = 0.f;
+        for (uint32_t h0 = 0; h0 < halves; h0 += 32u) {
+            const uint32_t hh = h0 + lp;
+            const bool live = hh < halves;
+            const uint32_t hc = live ? hh : halves - 1u;
+            const uint32_t sb = hc >> 1, half = hc & 1u;
+            const uint8_t *blk = w + rowc * row_bytes + (uint64_t)sb * 210u;
+            uint32_t qa[8], qb[8], qh[8];
+#pragma unroll
+            for (int k = 0; k < 2; ++k) {
+                const q8_u32x4_a2 a = *reinterpret_cast<const q8_u32x4_a2 *>(blk + 64u * half + 16u * k);
+                const q8_u32x4_a2 b = *reinterpret_cast<const q8_u32x4_a2 *>(blk + 64u * half + 32u + 16u * k);
+                const q8_u32x4_a2 t = *reinterpret_cast<const q8_u32x4_a2 *>(blk + 128u + 32u * half + 16u * k);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) qa[4 * k + j] = a.v[j], qb[4 * k + j] = b.v[j], qh[4 * k + j] = t.v[j];
+            }
+            const q8_u32x2_a2 scb = *reinterpret_cast<const q8_u32x2_a2 *>(blk + 192u + 8u * half);
+            const float d = live ? lev_f16_bits_to_f32(*reinterpret_cast<const uint16_t *>(blk + 208u)) : 0.f;
+            float scl[8];   // d * sub-scale: index 2k + p for group k, 16-weight part p
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                scl[j] = d * (float)(int)__builtin_amdgcn_sbfe((int)scb.v[j >> 2], 8 * (j & 3), 8);
+            // the four code planes, eight dwords each
+            uint32_t cw[4][8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                cw[0][i] = (qa[i] & 0x0F0F0F0Fu) | ((qh[i] << 4) & 0x30303030u);
+                cw[1][i] = (qb[i] & 0x0F0F0F0Fu) | ((qh[i] << 2) & 0x30303030u);
+                cw[2][i] = ((qa[i] >> 4) & 0x0F0F0F0Fu) | (qh[i] & 0x30303030u);
+                cw[3][i] = ((qb[i] >> 4) & 0x0F0F0F0Fu) | ((qh[i] >> 2) & 0x30303030u);
+            }
+#pragma unroll
+            for (int c = 0; c < NC; ++c) {
+                const uint8_t *base = smem + ((size_t)c * SB + sb) * kQ6Stride;
+                const lev_f32x4 dx = *reinterpret_cast<const lev_f32x4 *>(base + 272u + 16u * half);
+                float a = 0.f;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const lev_u32x4 x0 = *reinterpret_cast<const lev_u32x4 *>(base + 128u * half + 32u * k);
+                    const lev_u32x4 x1 = *reinterpret_cast<const lev_u32x4 *>(base + 128u * half + 32u * k + 16u);
+                    const lev_u32x2 sums = *reinterpret_cast<const lev_u32x2 *>(base + 304u + 32u * half + 8u * k);
+                    int lo = 0, hi = 0;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        lo = __builtin_amdgcn_sdot4((int)cw[k][j], (int)x0[j], lo, false);
+                        hi = __builtin_amdgcn_sdot4((int)cw[k][4 + j], (int)x1[j], hi, false);
+                    }
+                    lo -= 32 * (int)sums.x;
+                    hi -= 32 * (int)sums.y;
+                    a = fmaf(scl[2 * k] * dx[k], (float)lo, a);
+                    a = fmaf(scl[2 * k + 1] * dx[k], (float)hi, a);
+                }
+                acc[c] += a;
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            const float sum = lev_group_sum<32>(acc[c]);
+            if (lp == 31u && row < rows && (uint32_t)c < ncol) y[(uint64_t)c * rows + row] = sum;
+        }
+    }
+}
+
+template <int NC>
+hipError_t launch_q6_q8(lev_ctx *ctx, const uint8_t *w, const uint32_t *xq, const float *xs, float *y,
+                        uint32_t in_dim, uint32_t rows, uint32_t ncol) {
+    const size_t lds = (size_t)NC * (in_dim >> 8) * kQ6Stride;
+    static size_t configured = 0;
+    if (lds > 48 * 1024 && lds > configured) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&q6_k_gemv_q8_kernel<NC>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        configured = lds;
+    }
+    int per_cu = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, q6_k_gemv_q8_kernel<NC>, kQThreads, lds) !=
+            hipSuccess || per_cu < 1)
+        per_cu = 1;
+    const uint32_t tiles = (rows + 7u) / 8u;
+    uint32_t blocks = (uint32_t)ctx->num_cus * (uint32_t)per_cu;
+    if (blocks > tiles) blocks = tiles;
+    hipLaunchKernelGGL((q6_k_gemv_q8_kernel<NC>), dim3(blocks), dim3(kQThreads), lds, ctx->stream, w, xq,
+                       xs, y, in_dim, rows, ncol);
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// act = silu(gate) * up fused with the quantiser (emit_swiglu_quant,
+// lev-forge/src/q8.rs:166-177; silu, lev-model/src/lib.rs:120).  Eight lanes of
+// four values form a group of 32.
+// ---------------------------------------------------------------------------
+__global__ void __launch_bounds__(256)
+swiglu_quant_kernel(const float *__restrict__ gate, const float *__restrict__ up, uint32_t *__restrict__ xq,
+                    float *__restrict__ xs, float *__restrict__ act, uint32_t n4) {
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    const bool live = i < n4;                  // count % 32 == 0: eight lanes live or not together
+    lev_f32x4 v = {0.f, 0.f, 0.f, 0.f};
+    if (live) {
+        const lev_f32x4 g = reinterpret_cast<const lev_f32x4 *>(gate)[i];
+        const lev_f32x4 u = reinterpret_cast<const lev_f32x4 *>(up)[i];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) v[k] = g[k] / (1.0f + expf(-g[k])) * u[k];
+        if (act) reinterpret_cast<lev_f32x4 *>(act)[i] = v;
+    }
+    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    amax = dpp_max<0xB1>(amax);
+    amax = dpp_max<0x4E>(amax);
+    amax = dpp_max<0x141>(amax);
+    const float dq = amax / 127.0f;
+    const float idq = amax > 0.0f ? 127.0f / amax : 0.0f;
+    const int q0 = (int)rintf(v.x * idq), q1 = (int)rintf(v.y * idq);
+    const int q2 = (int)rintf(v.z * idq), q3 = (int)rintf(v.w * idq);
+    int qsum = (q0 + q1) + (q2 + q3);
+    qsum = dpp_addi<0xB1>(qsum);
+    qsum = dpp_addi<0x4E>(qsum);
+    qsum = dpp_addi<0x141>(qsum);
+    if (live) {
+        xq[i] = ((uint32_t)q0 & 255u) | (((uint32_t)q1 & 255u) << 8) | (((uint32_t)q2 & 255u) << 16) |
+                ((uint32_t)q3 << 24);
+        if ((threadIdx.x & 7u) == 0u) {
+            lev_f32x2 pair = {dq, dq * (float)qsum};
+            reinterpret_cast<lev_f32x2 *>(xs)[i >> 3] = pair;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
 // Q4_K x int8 GEMV on the matrix cores, up to 16 columns per weight read.
 //
 // v_mfma_i32_16x16x32_i8, one per sub-block of 32 weights: A = the activation
@@ -613,4 +797,67 @@ extern "C" int lev_hip_q4_k_gemv_q8(lev_ctx *ctx, const void *d_w, size_t w_byte
         done += nc;
     }
     return LEV_OK;
+}
+
+extern "C" int lev_hip_q6_k_gemv_q8(lev_ctx *ctx, const void *d_w, size_t w_bytes, uint64_t w_off,
+                                    const int8_t *d_xq, const float *d_xs, size_t x_count, float *d_y,
+                                    size_t y_capacity, uint32_t in_dim, uint32_t rows, uint32_t ncol) {
+    LEV_REQUIRE_CTX(ctx);
+    if (ncol == 0 || ncol > LEV_MAX_GEMV_COLUMNS)
+        return lev_fail(ctx, LEV_ERR_BAD_DIMENSIONS, "q6_k_gemv_q8: %u columns (1..%d)", ncol,
+                        LEV_MAX_GEMV_COLUMNS);
+    if (!d_xs) return lev_fail(ctx, LEV_ERR_INVALID_ARGUMENT, "q6_k_gemv_q8: null pointer");
+    lev_geom g;
+    int st = lev_check_matvec(ctx, "q6_k_gemv_q8", 256, 210, d_w, w_bytes, w_off, d_xq, x_count,
+                              (uint64_t)in_dim * ncol, d_y, y_capacity, (uint64_t)rows * ncol, in_dim, rows,
+                              &g);
+    if (st != LEV_OK) return st;
+    const uint8_t *w = static_cast<const uint8_t *>(d_w) + w_off;
+    if ((reinterpret_cast<uintptr_t>(w) & 1u) || (reinterpret_cast<uintptr_t>(d_xq) & 15u) ||
+        (reinterpret_cast<uintptr_t>(d_xs) & 7u))
+        return lev_fail(ctx, LEV_ERR_BAD_DIMENSIONS,
+                        "q6_k_gemv_q8: weights must be 2-byte, xq 16-byte, xs 8-byte aligned");
+    const size_t limit = ctx->props.sharedMemPerBlockOptin > ctx->props.sharedMemPerBlock
+                             ? ctx->props.sharedMemPerBlockOptin
+                             : ctx->props.sharedMemPerBlock;
+    const size_t per_col = (size_t)(in_dim >> 8) * kQ6Stride;
+    if (per_col > limit)
+        return lev_fail(ctx, LEV_ERR_EXCEEDS_MODEL_WORKLOAD, "q6_k_gemv_q8: inDim %u does not fit the staging", in_dim);
+    uint32_t fit = 8;
+    while (fit > 1u && fit * per_col > limit) fit >>= 1;
+    const uint32_t *xq = reinterpret_cast<const uint32_t *>(d_xq);
+    uint32_t done = 0;
+    while (done < ncol) {
+        uint32_t nc = ncol - done;
+        if (nc > fit) nc = fit;
+        const uint32_t *xqc = xq + ((uint64_t)done * in_dim >> 2);
+        const float *xsc = d_xs + (uint64_t)done * (in_dim >> 5) * 2u;
+        float *yc = d_y + (uint64_t)done * rows;
+        hipError_t e;
+        if (nc > 4) e = launch_q6_q8<8>(ctx, w, xqc, xsc, yc, in_dim, rows, nc);
+        else if (nc > 2) e = launch_q6_q8<4>(ctx, w, xqc, xsc, yc, in_dim, rows, nc);
+        else if (nc > 1) e = launch_q6_q8<2>(ctx, w, xqc, xsc, yc, in_dim, rows, nc);
+        else e = launch_q6_q8<1>(ctx, w, xqc, xsc, yc, in_dim, rows, nc);
+        if (e != hipSuccess) return lev_hip_check(ctx, e, "q6_k_gemv_q8 launch");
+        done += nc;
+    }
+    return LEV_OK;
+}
+
+extern "C" int lev_hip_swiglu_quant_q8(lev_ctx *ctx, const float *d_gate, const float *d_up, size_t count,
+                                       int8_t *d_xq, float *d_xs, float *d_act) {
+    LEV_REQUIRE_CTX(ctx);
+    if (!d_gate || !d_up || !d_xq || !d_xs)
+        return lev_fail(ctx, LEV_ERR_INVALID_ARGUMENT, "swiglu_quant_q8: null pointer");
+    if (count == 0 || count % 32u != 0u || count > ((size_t)1 << 31))
+        return lev_fail(ctx, LEV_ERR_BAD_DIMENSIONS, "swiglu_quant_q8: %zu values (a multiple of 32)", count);
+    if (((reinterpret_cast<uintptr_t>(d_gate) | reinterpret_cast<uintptr_t>(d_up) |
+          reinterpret_cast<uintptr_t>(d_act)) & 15u) ||
+        (reinterpret_cast<uintptr_t>(d_xq) & 3u) || (reinterpret_cast<uintptr_t>(d_xs) & 7u))
+        return lev_fail(ctx, LEV_ERR_BAD_DIMENSIONS,
+                        "swiglu_quant_q8: gate, up and act must be 16-byte, xq 4-byte, xs 8-byte aligned");
+    const uint32_t n4 = (uint32_t)(count >> 2);
+    hipLaunchKernelGGL(swiglu_quant_kernel, dim3((n4 + 255u) / 256u), dim3(256), 0, ctx->stream, d_gate, d_up,
+                       reinterpret_cast<uint32_t *>(d_xq), d_xs, d_act, n4);
+    return lev_hip_check(ctx, hipGetLastError(), "swiglu_quant_q8 launch");
 }

@@ -382,25 +382,28 @@ public:
     }
 
     // ---- Builder::matvec / matvec_rows on int8 activations, gpu.rs:334-370 ----
-    // y[nb][rows] (from float index yOffset) = W x for a Q4_K tensor; reads the
+    // y[nb][rows] (from float index yOffset) = W x for a Q4_K or Q6_K tensor; reads the
     // activations quantised by normQuant; maxRows takes a prefix of the rows.
     void matvecQ8(const std::string &tensor, const DeviceBuffer &xq, const DeviceBuffer &xs, int64_t nb,
                   DeviceBuffer &y, int64_t yOffset = 0, std::optional<int64_t> maxRows = std::nullopt) {
         const TensorRef &r = lookup(tensor);
-        if (r.type != GGMLTensorType::q4_K) geometry(tensor + ": unsupported type for the int8 matvec");
+        if (r.type != GGMLTensorType::q4_K && r.type != GGMLTensorType::q6_K)
+            geometry(tensor + ": unsupported type for the int8 matvec");
+        const int64_t blockBytes = bytesPerBlock(r.type);
         const int64_t rows = std::min(r.outDim, maxRows.value_or(r.outDim));
         int64_t count, outs, weightBytes, wEnd;
         if (!(rows > 0 && r.inDim > 0 && r.inDim % 256 == 0 && nb > 0 && yOffset >= 0) ||
             __builtin_mul_overflow(r.inDim, nb, &count) || __builtin_mul_overflow(rows, nb, &outs) ||
             xq.length < count || xs.length < count / 32 * 8 || y.length < (yOffset + outs) * 4)
             geometry("buffer extents violated for " + tensor);
-        if (__builtin_mul_overflow(rows, r.inDim / 256 * 144, &weightBytes) ||
+        if (__builtin_mul_overflow(rows, r.inDim / 256 * blockBytes, &weightBytes) ||
             __builtin_add_overflow(r.offset, weightBytes, &wEnd) || wEnd > r.end || wEnd > mapEnd_)
             geometry(tensor + ": weight bytes beyond tensor extent");
-        check(lev_hip_q4_k_gemv_q8(ctx_, weights_.contents(), (size_t)weights_.length, (uint64_t)r.offset,
-                                   static_cast<const int8_t *>(xq.contents()), xs.floats(), (size_t)count,
-                                   y.floats() + yOffset, (size_t)(y.length / 4 - yOffset), (uint32_t)r.inDim,
-                                   (uint32_t)rows, (uint32_t)nb),
+        auto *kernel = r.type == GGMLTensorType::q4_K ? lev_hip_q4_k_gemv_q8 : lev_hip_q6_k_gemv_q8;
+        check(kernel(ctx_, weights_.contents(), (size_t)weights_.length, (uint64_t)r.offset,
+                     static_cast<const int8_t *>(xq.contents()), xs.floats(), (size_t)count,
+                     y.floats() + yOffset, (size_t)(y.length / 4 - yOffset), (uint32_t)r.inDim, (uint32_t)rows,
+                     (uint32_t)nb),
               tensor);
     }
 

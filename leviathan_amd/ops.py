@@ -163,6 +163,29 @@ class Context:
                                                   rows, ncol))
         return y
 
+    def q6_k_gemv_q8(self, w, xq, xs, in_dim: int, rows: int, ncol: int, y=None, w_off: int = 0):
+        _dev(w, torch.uint8, "w")
+        _dev(xq, torch.int8, "xq")
+        _dev(xs, torch.float32, "xs")
+        if y is None:
+            y = torch.empty((max(ncol, 1), max(rows, 1)), dtype=torch.float32, device=w.device)
+        self._check(self.lib.lev_hip_q6_k_gemv_q8(self.ctx, _ptr(w), w.numel(), w_off, _ptr(xq),
+                                                  _ptr(xs), xq.numel(), _ptr(y), y.numel(), in_dim,
+                                                  rows, ncol))
+        return y
+
+    def swiglu_quant_q8(self, gate, up, want_act: bool = False):
+        """Int8 activations of silu(gate) * up: returns (xq, xs (d, s) pairs[, act f32])."""
+        _dev(gate, torch.float32, "gate")
+        _dev(up, torch.float32, "up")
+        n = gate.numel()
+        xq = torch.empty(max(n, 1), dtype=torch.int8, device=gate.device)
+        xs = torch.empty((max(n // 32, 1), 2), dtype=torch.float32, device=gate.device)
+        act = torch.empty_like(gate) if want_act else None
+        self._check(self.lib.lev_hip_swiglu_quant_q8(self.ctx, _ptr(gate), _ptr(up), n, _ptr(xq),
+                                                     _ptr(xs), _ptr(act)))
+        return (xq, xs, act) if want_act else (xq, xs)
+
     def q4_k_gemm_prefill(self, w, x_f16, in_dim: int, rows: int, tokens: int, y=None, w_off: int = 0):
         _dev(w, torch.uint8, "w")
         _dev(x_f16, torch.float16, "x")

@@ -272,6 +272,20 @@ void runner_int8_path(Runner &r, const Model &m) {
         std::vector<float> got(y.begin() + (size_t)c * ROWS, y.begin() + (size_t)(c + 1) * ROWS);
         EXPECT(rel_err(got, ref) < 1e-4);
     }
+    // the Q6_K head on the same activations
+    DeviceBuffer dl = r.makeBuffer((int64_t)NB * Model::vocab * 4);
+    r.matvecQ8("output.weight", xq, xs, NB, dl);
+    std::vector<float> logits = r.read<float>(dl, (size_t)NB * Model::vocab);
+    const TensorRef &o = m.table.at("output.weight");
+    for (int c = 0; c < NB; ++c) {
+        std::vector<float> xd(H);
+        for (int i = 0; i < H; ++i) xd[i] = (float)q[(size_t)c * H + i] * pairs[((size_t)c * (H / 32) + i / 32) * 2];
+        std::vector<double> ref(Model::vocab);
+        EXPECT(levo_q6_k_matvec_f64(m.at("output.weight"), (size_t)(o.end - o.offset), Model::vocab, H, xd.data(), H,
+                                    ref.data()) == 0);
+        std::vector<float> got(logits.begin() + (size_t)c * Model::vocab, logits.begin() + (size_t)(c + 1) * Model::vocab);
+        EXPECT(rel_err(got, ref) < 1e-4);
+    }
     // a prefix of the rows (matvec_rows), and the guards before any launch
     r.matvecQ8("blk.0.ffn_up.weight", xq, xs, NB, dy, 0, 16);
     std::vector<float> y16 = r.read<float>(dy, (size_t)NB * 16);

@@ -240,6 +240,84 @@ def test_q4_k_q8_weight_offset(ctx):
     assert torch.equal(base, shifted)
 
 
+# ------------------------------------------------------------ Q6_K x int8 ----
+
+def q6_q8_gemv(ctx, w, x2d, rows, cols):
+    ncol = x2d.shape[0]
+    xq, xs = ctx.norm_quant_q8(dev(x2d), cols, ncol)
+    y = torch.full((ncol, rows), float("nan"), device="cuda")
+    ctx.q6_k_gemv_q8(dev(w), xq, xs, cols, rows, ncol, y=y)
+    ctx.sync()
+    return y.cpu().numpy(), xq.cpu().numpy(), xs.cpu().numpy()
+
+
+def check_q6(got, w, rows, cols, xq, xs):
+    for c in range(got.shape[0]):
+        ref = O.q6_k_matvec_q8_f64(w, rows, cols, xq[c], xs[c, :, 0])
+        assert O.max_rel_err(got[c], ref) < GATE, c
+
+
+@pytest.mark.parametrize("nb", [1, 2, 3, 4, 8, 16])
+def test_q6_k_q8_reference_gate_protocol(ctx, nb):
+    """vk_q8 on a Q6_K tensor (lev-cli/src/main.rs:1788-1868), seed and gate as above."""
+    rows, cols = 200, 4096
+    w = O.synth_q6_k(6, rows * cols // 256)
+    x = O.signed_units(nb * cols, 0x4C455649).reshape(nb, cols)
+    got, xq, xs = q6_q8_gemv(ctx, w, x, rows, cols)
+    check_q6(got, w, rows, cols, xq, xs)
+    for c in range(nb):
+        ref = O.q6_k_matvec_f64(w, rows, cols, x[c])
+        assert np.linalg.norm(got[c] - ref) < 0.02 * np.linalg.norm(ref)
+
+
+@pytest.mark.parametrize("rows,cols,ncol", [(37, 1024, 1), (9, 256, 3), (20, 12288, 8), (130, 4352, 5),
+                                            (11, 8192, 16)])
+def test_q6_k_q8_shapes(ctx, rows, cols, ncol):
+    w = O.synth_q6_k(rows + ncol, rows * cols // 256)
+    x = O.normal(ncol * cols, 7 + rows).reshape(ncol, cols)
+    got, xq, xs = q6_q8_gemv(ctx, w, x, rows, cols)
+    check_q6(got, w, rows, cols, xq, xs)
+
+
+def test_q6_k_q8_hand_block_and_saturated_codes(ctx):
+    """The hand-computed -315 block of main.swift:1091-1112 (its activations are
+    powers of two times +-1: every code is +-127 and q*d is x to one rounding),
+    and blocks of all-ones bytes (codes 63, scales -1)."""
+    blk, x = H.minus_315_block()
+    got, xq, xs = q6_q8_gemv(ctx, blk, x[None], 1, 256)
+    assert abs(got[0, 0] + 315.0) <= 1e-4 * 315.0
+    check_q6(got, blk, 1, 256, xq, xs)
+    sat = np.full(210 * 4, 0xFF, np.uint8)
+    sat[208::210], sat[209::210] = 0x00, 0x3C          # d = 1.0
+    x = O.signed_units(2 * 512, 3).reshape(2, 512)
+    got, xq, xs = q6_q8_gemv(ctx, sat, x, 2, 512)
+    check_q6(got, sat, 2, 512, xq, xs)
+
+
+def test_q6_k_q8_lm_head_full_size(ctx):
+    w, x = H.config2()
+    x2 = np.stack([x, x[::-1].copy()])
+    got, xq, xs = q6_q8_gemv(ctx, w, x2, 32000, 4096)
+    check_q6(got, w, 32000, 4096, xq, xs)
+
+
+# ------------------------------------------------------- SwiGLU + quantise ----
+
+@pytest.mark.parametrize("n", [32, 4096, 3 * 11008 - 3 * 11008 % 32])
+def test_swiglu_quant(ctx, n):
+    g = O.normal(n, 21, sigma=2.0)
+    u = O.normal(n, 22)
+    g[:4] = [0.0, -100.0, 100.0, -0.0]
+    xq, xs, act = ctx.swiglu_quant_q8(dev(g), dev(u), want_act=True)
+    ctx.sync()
+    act = act.cpu().numpy()
+    g64, u64 = g.astype(np.float64), u.astype(np.float64)
+    want = g64 / (1.0 + np.exp(-g64)) * u64               # silu(g) * u, lev-model/src/lib.rs:120, 240
+    assert np.all(np.abs(act - want) <= 1e-6 * np.maximum(1.0, np.abs(want)))
+    # the codes are the quantiser's, bit for bit, on the f32 activations the kernel formed
+    check_quant((xq.cpu().numpy()[None], xs.cpu().numpy()[None]), act[None])
+
+
 def test_q8_guards(ctx):
     from leviathan_amd import capi
     from leviathan_amd.ops import LevError
