@@ -220,6 +220,11 @@ def main():
             for nbytes, label in ((q4_bytes_w, "stream_read_9MiB_same_buffer"), (1 << 30, "stream_read_1GiB")):
                 run_other(label, lambda i: must(lib.lev_hip_stream_read_probe(
                     c, buf.data_ptr(), nbytes, sink.data_ptr(), 512)), nbytes, 50, 10)
+            # the same 9 MiB read from a different part of the 1 GiB buffer every launch: what HBM
+            # (not the memory-side cache) delivers to a launch of the headline kernel's size
+            nrot = (1 << 30) // q4_bytes_w
+            run_other("stream_read_9MiB_rotating", lambda i: must(lib.lev_hip_stream_read_probe(
+                c, buf.data_ptr() + (i % nrot) * q4_bytes_w, q4_bytes_w, sink.data_ptr(), 512)), q4_bytes_w, 200, 20)
             run_other("empty_kernel_launch", lambda i: must(lib.lev_hip_empty_launch(c)), 0, 1000, 100)
             # plain copy of known size: the calibration kernel for the
             # FETCH_SIZE / WRITE_SIZE counters (reads and writes 256 MiB each)

@@ -20,8 +20,8 @@
 //     fragments (the two waves that share rows both decode them);
 //   - X goes through LDS in K-steps of 64 (one Q4_K chunk) with direct
 //     global -> LDS loads (global_load_lds_dwordx4: no registers in between),
-//     four buffers, three steps in flight, which covers the load latency that a
-//     single wave per SIMD cannot hide otherwise.  A direct load places lane
+//     four buffers, two steps in flight and one barrier per step, which covers
+//     the load latency that a single wave per SIMD cannot hide otherwise.  A direct load places lane
 //     l's 16 bytes at base + 16*l, so padding rows is not possible; instead
 //     the 16-byte chunk c of token row t is stored at position c ^ (t & 7)
 //     (the source address is permuted), which spreads the fragment reads of
@@ -45,7 +45,7 @@ constexpr int kRT = 2;            // 32-row tiles per wave
 constexpr int kKS = 64;           // K-step (one chunk)
 constexpr int kXRow = 128;        // bytes per token row in LDS
 constexpr int kXBuf = kBM * kXRow;
-constexpr int kXBufs = 4;         // LDS buffers: three steps in flight
+constexpr int kXBufs = 4;         // LDS buffers: the step in use, the one before it (still being read by late waves), two in flight
 
 // (d*sc, dmin*m) of the 8 sub-blocks of a superblock (lev-cpu/src/lib.rs:64-74,
 // 117-124).
@@ -157,7 +157,6 @@ q4_k_gemm_kernel(const uint8_t *__restrict__ w, const uint16_t *__restrict__ x,
     // steps 0, 1, 2 in flight (clamped for very short K)
     x_request(0, 0);
     x_request(1 < nsteps ? 1 : nsteps - 1, 1);
-    x_request(2 < nsteps ? 2 : nsteps - 1, 2);
 
     // The weights of superblock sb+1 are requested while sb is multiplied: with
     // one wave per SIMD nothing else hides their latency.  Loads are
@@ -204,12 +203,14 @@ q4_k_gemm_kernel(const uint8_t *__restrict__ w, const uint16_t *__restrict__ x,
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             const uint32_t ks = sb * 4u + c;
-            // Step ks+3 goes into the buffer that step ks-1 used: every wave is
-            // past the barrier that ended that step.  Then wait for step ks: its
-            // 8 loads are older than the 24 of steps ks+1..ks+3 (any weight load
-            // issued in between only makes the wait stricter).
-            x_request(ks + 3 < nsteps ? ks + 3 : nsteps - 1, (ks + 3) & 3u);
-            LEV_WAIT_VMCNT(24);
+            // Step ks+2 goes into the buffer that step ks-2 used: a wave that gets
+            // here has passed the barrier of step ks-1, which every wave reaches
+            // only after its reads of step ks-2, so one barrier per step suffices.
+            // Then wait for step ks: its 8 loads are older than the 16 of steps
+            // ks+1 and ks+2 (a weight load issued in between only makes the wait
+            // stricter).
+            x_request(ks + 2 < nsteps ? ks + 2 : nsteps - 1, (ks + 2) & 3u);
+            LEV_WAIT_VMCNT(16);
             __syncthreads();
 
             // The fragments of the NEXT chunk are decoded while this chunk is
@@ -226,8 +227,23 @@ q4_k_gemm_kernel(const uint8_t *__restrict__ w, const uint16_t *__restrict__ x,
             }
             const int cn = c == 3 ? 0 : c + 1;
             const uint8_t *xb = lds + (ks & 3u) * kXBuf + (wm * 128u + lr) * kXRow;
+            // fragment reads run one group ahead of the MFMAs that use them, so
+            // that their LDS latency passes behind the decode of the group
+            auto a_read = [&](int j, f16x8 (&a)[2]) {
+                const int qq = j >> 1;
+                // 16-byte chunk of this MFMA's 8 activations inside the 128-byte row,
+                // at its swizzled position (rows 32m + lr: same low bits as lr)
+                const uint32_t chunk = 2u * lh + (qq < 2 ? qq : 2u + qq);
+                const uint32_t koff = 16u * (chunk ^ (lr & 7u));
+#pragma unroll
+                for (int mm2 = 0; mm2 < 2; ++mm2)
+                    a[mm2] = *reinterpret_cast<const f16x8 *>(xb + (2 * (j & 1) + mm2) * 32 * kXRow + koff);
+            };
+            f16x8 a_cur[2], a_nxt[2];
+            a_read(0, a_cur);
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
+                if (j < 7) a_read(j + 1, a_nxt);
                 {
                     const int r = j >> 2, q = j & 3;
                     const lev_u32x4 w4 = qs[r][cn];
@@ -235,25 +251,21 @@ q4_k_gemm_kernel(const uint8_t *__restrict__ w, const uint16_t *__restrict__ x,
                     bn[r][q] = q4k_frag((q & 1) ? w4.z : w4.x, (q & 1) ? w4.w : w4.y, q >= 2, d1[r][sub], mm[r][sub]);
                 }
                 const int qq = j >> 1;
-                // 16-byte chunk of this MFMA's 8 activations inside the 128-byte row,
-                // at its swizzled position (rows 32m + lr: same low bits as lr)
-                const uint32_t chunk = 2u * lh + (qq < 2 ? qq : 2u + qq);
-                const uint32_t koff = 16u * (chunk ^ (lr & 7u));
 #pragma unroll
                 for (int mm2 = 0; mm2 < 2; ++mm2) {
                     const int m = 2 * (j & 1) + mm2;
-                    f16x8 a = *reinterpret_cast<const f16x8 *>(xb + m * 32 * kXRow + koff);
 #pragma unroll
                     for (int r = 0; r < kRT; ++r)
-                        acc[r][m] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bf[r][qq], acc[r][m], 0, 0, 0);
+                        acc[r][m] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_cur[mm2], bf[r][qq], acc[r][m], 0, 0, 0);
                 }
+                a_cur[0] = a_nxt[0];
+                a_cur[1] = a_nxt[1];
                 __builtin_amdgcn_sched_barrier(0);
             }
 #pragma unroll
             for (int r = 0; r < kRT; ++r)
 #pragma unroll
                 for (int qq = 0; qq < 4; ++qq) bf[r][qq] = bn[r][qq];
-            __syncthreads();   // all reads of this step's buffer done before it is requested again
         }
     }
 
