@@ -179,7 +179,13 @@ q4_k_gemm_kernel(const uint8_t *__restrict__ w, const uint16_t *__restrict__ x,
 #pragma unroll
         for (int r = 0; r < kRT; ++r) {
 #pragma unroll
-            for (int cc = 0; cc < 4; ++cc) qs[r][cc] = qs_n[r][cc];
+            for (int cc = 0; cc < 4; ++cc) {
+                qs[r][cc] = qs_n[r][cc];
+                // touched here so that the wait for these loads is placed HERE, where
+                // the compiler can count the loads issued since; left to the first
+                // use, in the next trip of the loop, it waits for everything
+                asm volatile("" : "+v"(qs[r][cc].x), "+v"(qs[r][cc].y), "+v"(qs[r][cc].z), "+v"(qs[r][cc].w));
+            }
             q4k_all_factors(hdr_n[r], d1[r], mm[r]);
         }
     };
@@ -196,7 +202,6 @@ q4_k_gemm_kernel(const uint8_t *__restrict__ w, const uint16_t *__restrict__ x,
     };
     w_load(0);
     take();
-    w_load(1);
     f16x8 bf[kRT][4];
     dequant(0, bf);
     for (uint32_t sb = 0; sb < nsb; ++sb) {
@@ -211,7 +216,11 @@ q4_k_gemm_kernel(const uint8_t *__restrict__ w, const uint16_t *__restrict__ x,
             // stricter).
             x_request(ks + 2 < nsteps ? ks + 2 : nsteps - 1, (ks + 2) & 3u);
             LEV_WAIT_VMCNT(16);
-            __syncthreads();
+            // A bare barrier: __syncthreads() carries a workgroup fence, for which
+            // the compiler waits for EVERY outstanding load (the two steps just
+            // requested included).  LDS is coherent within the CU; each wave has
+            // waited for its own part of step ks above.
+            asm volatile("s_barrier" ::: "memory");
 
             // The fragments of the NEXT chunk are decoded while this chunk is
             // multiplied.  A wave issues in order, so with one wave per SIMD the
@@ -221,10 +230,12 @@ q4_k_gemm_kernel(const uint8_t *__restrict__ w, const uint16_t *__restrict__ x,
             // fenced so that the scheduler keeps them apart.  The MFMAs of a group
             // run while the next group's decode issues.
             f16x8 bn[kRT][4];
-            if (c == 3) {
-                take();
-                w_load(sb + 2u);
-            }
+            // The next superblock's weights are requested in step 0 and taken over
+            // in step 3 of the SAME trip of the loop: the compiler then knows how
+            // many loads were issued in between and waits for exactly those (over
+            // the loop's back edge it would wait for everything in flight).
+            if (c == 0) w_load(sb + 1u);
+            if (c == 3) take();
             const int cn = c == 3 ? 0 : c + 1;
             const uint8_t *xb = lds + (ks & 3u) * kXBuf + (wm * 128u + lr) * kXRow;
             // fragment reads run one group ahead of the MFMAs that use them, so
