@@ -25,6 +25,7 @@
 
 #include <algorithm>
 #include <cmath>
+#include <cstdio>
 #include <cstdint>
 #include <cstring>
 #include <map>
@@ -35,6 +36,7 @@
 #include <utility>
 #include <vector>
 
+#include "leviathan_gguf.hpp"
 #include "leviathan_hip.h"
 
 namespace leviathan {
@@ -251,6 +253,63 @@ public:
         weights_ = makeBuffer(bytes);
         mapEnd_ = (int64_t)bytes.size();
         ref_ = std::move(table);
+    }
+
+    // Makes a GGUF file resident from offset 0 (buffer offset == file offset, as
+    // the reference's mapped file, Gemma4.swift:543-566; uploaded here, since
+    // registering mapped host memory is not available) and builds the tensor
+    // table from its directory.  Tensors of types this path has no kernel for
+    // stay in the buffer but get no table entry.
+    GGUFFile bindGGUF(const std::string &path) {
+        GGUFFile g = GGUFFile::open(path);
+        std::vector<uint8_t> bytes((size_t)g.fileLen);
+        FILE *f = std::fopen(path.c_str(), "rb");
+        if (!f || std::fread(bytes.data(), 1, bytes.size(), f) != bytes.size()) {
+            if (f) std::fclose(f);
+            throw GGUFError("cannot read " + path);
+        }
+        std::fclose(f);
+        std::map<std::string, TensorRef> table;
+        for (const GGUFTensorInfo &t : g.tensors) {
+            TensorRef r;
+            switch (t.ggmlType) {
+            case LEV_TYPE_F32: r.type = GGMLTensorType::float32; break;
+            case LEV_TYPE_F16: r.type = GGMLTensorType::float16; break;
+            case LEV_TYPE_Q4_0: r.type = GGMLTensorType::q4_0; break;
+            case LEV_TYPE_Q4_K: r.type = GGMLTensorType::q4_K; break;
+            case LEV_TYPE_Q6_K: r.type = GGMLTensorType::q6_K; break;
+            default: continue;
+            }
+            uint64_t start, end;
+            g.tensorRange(t, start, end);
+            r.offset = (int64_t)start;
+            r.end = (int64_t)end;
+            r.inDim = (int64_t)t.dims[0];
+            r.outDim = t.dims.size() > 1 ? (int64_t)t.dims[1] : 1;
+            r.experts = t.dims.size() > 2 ? (int64_t)t.dims[2] : 1;
+            if (t.dims.size() > 3) continue;
+            table[t.name] = r;
+        }
+        bindWeights(bytes, std::move(table));
+        return g;
+    }
+
+    // The routed-expert pools of one layer, from the checked file binding
+    // (fused gate|up rows [2I, H] per expert: up follows gate inside a slice).
+    static MoEBinding moeBinding(const MoEModelBinding &b, int64_t layer) {
+        if (layer < 0 || layer >= b.layerCount)
+            throw Gemma4Error(Gemma4Error::badTensorGeometry, "layer outside the model");
+        MoEBinding m;
+        m.gateOffset = b.guTensorStarts[(size_t)layer];
+        m.upOffset = m.gateOffset + b.guStride / 2;
+        m.downOffset = b.dnTensorStarts[(size_t)layer];
+        m.gateStride = m.upStride = b.guStride;
+        m.downStride = b.dnStride;
+        m.hidden = (int)b.hidden;
+        m.expertIntermediate = (int)b.inter;
+        m.experts = (int)b.expertCount;
+        m.topK = (int)b.topK;
+        return m;
     }
 
     // ---- Gemma4.swift:2583 ----

@@ -6,6 +6,8 @@ oracle and the HIP path.
 """
 from __future__ import annotations
 
+import struct
+
 import numpy as np
 
 import oracle as O
@@ -137,3 +139,47 @@ def config5(hidden=2048, inter=768, experts=128, tokens=1, seed=5):
 def rmsnorm_rows(x, gain, eps=1e-6):
     """Reference RMSNorm (lev-model/src/lib.rs:110-114) applied per row."""
     return np.stack([O.rmsnorm(r, gain, eps) for r in np.atleast_2d(x)])
+
+
+# ---- GGUF files for the reader tests (the container format of the weights) ----
+
+def gguf_str(s) -> bytes:
+    raw = s if isinstance(s, bytes) else s.encode("utf-8")
+    return struct.pack("<Q", len(raw)) + raw
+
+
+_GGUF_FMT = {0: "<B", 1: "<b", 2: "<H", 3: "<h", 4: "<I", 5: "<i", 6: "<f", 7: "<B", 10: "<Q", 11: "<q", 12: "<d"}
+
+
+def gguf_value(ty: int, v) -> bytes:
+    if ty == 8:
+        return gguf_str(v)
+    if ty == 9:
+        et, items = v
+        return struct.pack("<IQ", et, len(items)) + b"".join(gguf_value(et, x) for x in items)
+    return struct.pack(_GGUF_FMT[ty], v)
+
+
+def write_gguf(kvs, tensors, version=3, alignment=None, pad_data_to=None) -> bytes:
+    """kvs: [(key, type id, value)]; tensors: [(name, dims, type id, data bytes)].
+    Tensor data is laid out in order, each at the next multiple of the alignment."""
+    align = alignment or 32
+    out = b"GGUF" + struct.pack("<IQQ", version, len(tensors), len(kvs))
+    for key, ty, v in kvs:
+        out += gguf_str(key) + struct.pack("<I", ty) + gguf_value(ty, v)
+    offsets, off = [], 0
+    for name, dims, ty, data in tensors:
+        off = -(-off // align) * align
+        offsets.append(off)
+        off += len(data)
+    for (name, dims, ty, data), o in zip(tensors, offsets):
+        out += gguf_str(name) + struct.pack("<I", len(dims)) + b"".join(struct.pack("<Q", d) for d in dims)
+        out += struct.pack("<IQ", ty, o)
+    out += b"\0" * (-len(out) % align)
+    body = b""
+    for (name, dims, ty, data), o in zip(tensors, offsets):
+        body += b"\0" * (o - len(body)) + bytes(data)
+    out += body
+    if pad_data_to is not None:
+        out += b"\0" * max(0, pad_data_to - len(out))
+    return out

@@ -449,6 +449,126 @@ struct Case {
 
 }  // namespace
 
+// ---- model file -> resident buffer -> kernels ----------------------------------
+// The Model's tensors written as a GGUF v3 file (gemma4 metadata, 32-byte
+// alignment), read back through GGUFFile / MoEModelBinding / Runner::bindGGUF:
+// the same operators must give the same bits as on the memory-bound weights.
+static void put_u32(std::vector<uint8_t> &o, uint32_t v) { o.insert(o.end(), (uint8_t *)&v, (uint8_t *)&v + 4); }
+static void put_u64(std::vector<uint8_t> &o, uint64_t v) { o.insert(o.end(), (uint8_t *)&v, (uint8_t *)&v + 8); }
+static void put_str(std::vector<uint8_t> &o, const std::string &s) {
+    put_u64(o, s.size());
+    o.insert(o.end(), s.begin(), s.end());
+}
+
+std::string write_model_gguf(const Model &m) {
+    std::vector<uint8_t> o = {'G', 'G', 'U', 'F'};
+    put_u32(o, 3);
+    put_u64(o, m.table.size());
+    put_u64(o, 6);
+    put_str(o, "general.architecture"); put_u32(o, 8); put_str(o, "gemma4");
+    const std::pair<const char *, uint32_t> ints[] = {
+        {"gemma4.block_count", 1}, {"gemma4.expert_count", Model::experts}, {"gemma4.expert_used_count", Model::topK},
+        {"gemma4.embedding_length", Model::hidden}, {"gemma4.expert_feed_forward_length", Model::inter}};
+    for (auto &kv : ints) {
+        put_str(o, kv.first);
+        put_u32(o, 4);
+        put_u32(o, kv.second);
+    }
+    uint64_t off = 0;
+    std::vector<std::pair<const TensorRef *, uint64_t>> placed;
+    for (auto &kv : m.table) {
+        const TensorRef &t = kv.second;
+        put_str(o, kv.first);
+        const bool three = t.experts > 1, one = t.outDim == 1 && !three;
+        put_u32(o, three ? 3 : one ? 1 : 2);
+        put_u64(o, (uint64_t)t.inDim);
+        if (!one) put_u64(o, (uint64_t)t.outDim);
+        if (three) put_u64(o, (uint64_t)t.experts);
+        put_u32(o, (uint32_t)t.type);
+        off = (off + 31) / 32 * 32;
+        put_u64(o, off);
+        placed.push_back({&t, off});
+        off += (uint64_t)(t.end - t.offset);
+    }
+    while (o.size() % 32) o.push_back(0);
+    const size_t data0 = o.size();
+    o.resize(data0 + off);
+    for (auto &pl : placed)
+        std::memcpy(o.data() + data0 + pl.second, m.bytes.data() + pl.first->offset, (size_t)(pl.first->end - pl.first->offset));
+    char path[] = "/tmp/lev_host_parity_XXXXXX";
+    const int fd = mkstemp(path);
+    EXPECT(fd >= 0);
+    FILE *f = fdopen(fd, "wb");
+    EXPECT(f && std::fwrite(o.data(), 1, o.size(), f) == o.size());
+    if (f) std::fclose(f);
+    return path;
+}
+
+void runner_gguf_file(Runner &mem, const Model &m) {
+    const std::string path = write_model_gguf(m);
+    Runner r(0);
+    GGUFFile g = r.bindGGUF(path);
+    EXPECT(g.version == 3 && g.tensors.size() == m.table.size() && g.alignment == 32);
+    MoEModelBinding mb = MoEModelBinding::bind(g);
+    EXPECT(mb.layerCount == 1 && mb.expertCount == Model::experts && mb.topK == Model::topK);
+    EXPECT(mb.guStride == m.gu_slice && mb.dnStride == m.dn_slice);
+    const MoEBinding bind = Runner::moeBinding(mb, 0);
+    std::remove(path.c_str());
+
+    const int H = Model::hidden, K = Model::topK;
+    std::vector<float> x(H);
+    levo_fill_normal(91, 0.f, 1.f, x.data(), H);
+    auto both = [&](auto &&fn) {   // the file-bound and the memory-bound runner, same operator
+        std::vector<float> a = fn(r), b = fn(mem);
+        EXPECT(a.size() == b.size() && std::memcmp(a.data(), b.data(), a.size() * 4) == 0);
+        return a;
+    };
+    std::vector<float> y = both([&](Runner &rr) {
+        DeviceBuffer dx = rr.makeBuffer(x), dy = rr.makeBuffer((int64_t)H * 4);
+        rr.matvec("blk.0.attn_q.weight", dx, H, dy, H);
+        return rr.read<float>(dy, H);
+    });
+    std::vector<double> ref(H);
+    const TensorRef &t = m.table.at("blk.0.attn_q.weight");
+    levo_q4_0_matvec_f64(m.at("blk.0.attn_q.weight"), (size_t)(t.end - t.offset), H, H, x.data(), H, ref.data());
+    EXPECT(rel_err(y, ref) < 1e-4);
+    both([&](Runner &rr) {
+        DeviceBuffer dx = rr.makeBuffer(x), dl = rr.makeBuffer((int64_t)Model::vocab * 4);
+        rr.matvec("output.weight", dx, H, dl, Model::vocab);
+        return rr.read<float>(dl, Model::vocab);
+    });
+    // the MoE block through the binding taken from the file
+    std::vector<int32_t> ids;
+    std::vector<float> wts;
+    std::vector<float> ym = both([&](Runner &rr) {
+        DeviceBuffer dx = rr.makeBuffer(x), dy = rr.makeBuffer((int64_t)H * 4);
+        auto [topIdx, weights] = rr.routeTopK("blk.0.ffn_gate_inp.weight", dx, K);
+        ids.assign(topIdx.begin(), topIdx.end());
+        wts = weights;
+        rr.runMoeBatchedRouted(dx, dy, topIdx, weights, &rr == &r ? bind : m.binding);
+        return rr.read<float>(dy, H);
+    });
+    std::vector<double> yref(H), gg((size_t)K * Model::inter), uu(gg.size()), aa(gg.size()), dd((size_t)K * H);
+    EXPECT(levo_moe_experts_f64(m.bytes.data() + m.binding.gateOffset, m.bytes.data() + m.binding.upOffset,
+                                m.bytes.data() + m.binding.downOffset, (size_t)m.gu_slice, (size_t)m.gu_slice,
+                                (size_t)m.dn_slice, H, Model::inter, K, ids.data(), wts.data(), x.data(), yref.data(),
+                                gg.data(), uu.data(), aa.data(), dd.data()) == 0);
+    EXPECT(rel_err(ym, yref) < 1e-4);
+    // slice offsets of a route: exactly the operator's own addressing
+    std::vector<uint64_t> gu, dn;
+    mb.offsets(0, {Model::experts - 1, 0}, gu, dn);
+    EXPECT(gu[0] == (uint64_t)(bind.gateOffset + (Model::experts - 1) * bind.gateStride) && gu[1] == (uint64_t)bind.gateOffset);
+    EXPECT(dn[1] == (uint64_t)bind.downOffset);
+    bool threw = false;
+    try {
+        mb.offsets(0, {0, 0}, gu, dn);
+    } catch (const GGUFError &) {
+        threw = true;
+    }
+    EXPECT(threw);
+}
+
+
 int main(int argc, char **argv) {
     Model model;
     std::unique_ptr<Runner> runner;
@@ -470,6 +590,7 @@ int main(int argc, char **argv) {
         {"runner_int8_path", [&] { runner_int8_path(R(), model); }},
         {"runner_moe", [&] { runner_moe(R(), model); }},
         {"runner_moe_hand_computed", [&] { runner_moe_hand_computed(R()); }},
+        {"runner_gguf_file", [&] { runner_gguf_file(R(), model); }},
     };
     if (argc > 1 && std::strcmp(argv[1], "--list") == 0) {
         for (auto &c : cases) std::printf("%s\n", c.name);
