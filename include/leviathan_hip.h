@@ -208,6 +208,14 @@ int lev_hip_q4_k_gemm_prefill(lev_ctx *ctx, const void *d_w, size_t w_bytes, uin
 /* act_f16 (lev-forge/src/coopmat.rs:49): f32 -> f16, round to nearest even. */
 int lev_hip_f32_to_f16(lev_ctx *ctx, const float *d_x, uint16_t *d_out, size_t n);
 
+/* Embedding lookup from a Q4_K table (embed_q4k, lev-forge/src/ops.rs:523-555; Builder step
+ * "embed", lev-model/src/gpu.rs:457): column c of out (dim floats) is row d_tokens[c] of the
+ * [vocab][dim] table, dequantised bit-exactly as lev_hip_dequant does.  A token id >= vocab
+ * writes nothing and is reported by the next lev_hip_sync as LEV_ERR_BAD_DIMENSIONS. */
+int lev_hip_embed_q4_k(lev_ctx *ctx, const void *d_w, size_t w_bytes, uint64_t w_off,
+                       const uint32_t *d_tokens, uint32_t ntokens, float *d_out, size_t out_capacity,
+                       uint32_t dim, uint32_t vocab);
+
 /* ---- elementwise operators of the runner ---- */
 /* rmsnorm(x:y:n:vectors:weightTensor:) (Gemma4.swift:3014; kernel :4247);
  * d_weight may be NULL (scale-free). */

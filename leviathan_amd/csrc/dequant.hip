@@ -67,7 +67,61 @@ dequant_q4_k(const uint8_t *__restrict__ w, float *__restrict__ out, uint64_t nv
     out[i] = d1 * n - mm;
 }
 
+// Embedding lookup from a Q4_K table (embed_q4k, lev-forge/src/ops.rs:523-555):
+// column c of out is row tok[c], one workgroup per 256-weight block, the
+// arithmetic of dequant_q4_k above.  A token id beyond the table raises the
+// context's flag (bit 2) and writes nothing.
+constexpr int kFlagBadToken = 4;
+
+__global__ void __launch_bounds__(256)
+embed_q4_k(const uint8_t *__restrict__ w, const uint32_t *__restrict__ tok, float *__restrict__ out,
+           uint32_t blocks_per_row, uint32_t vocab, int *__restrict__ flag) {
+    const uint32_t col = blockIdx.x / blocks_per_row, b = blockIdx.x - col * blocks_per_row;
+    const uint32_t token = tok[col];
+    if (token >= vocab) {
+        if (threadIdx.x == 0 && b == 0) atomicOr(flag, kFlagBadToken);
+        return;
+    }
+    const uint8_t *blk = w + ((uint64_t)token * blocks_per_row + b) * 144u;
+    const uint32_t e = threadIdx.x, j = e >> 5, l = e & 31u;
+    float d = lev_f16_bits_to_f32((uint32_t)blk[0] | ((uint32_t)blk[1] << 8));
+    float dmin = lev_f16_bits_to_f32((uint32_t)blk[2] | ((uint32_t)blk[3] << 8));
+    uint32_t sc, mn;
+    q4_k_scale_min(j, blk + 4, sc, mn);
+    uint8_t q = blk[16 + (j >> 1) * 32 + l];
+    float n = (float)((j & 1u) ? (q >> 4) : (q & 0xF));
+    float d1 = d * (float)sc;
+    float mm = dmin * (float)mn;
+    out[((uint64_t)col * blocks_per_row + b) * 256u + e] = d1 * n - mm;
+}
+
 }  // namespace
+
+extern "C" int lev_hip_embed_q4_k(lev_ctx *ctx, const void *d_w, size_t w_bytes, uint64_t w_off,
+                                  const uint32_t *d_tokens, uint32_t ntokens, float *d_out,
+                                  size_t out_capacity, uint32_t dim, uint32_t vocab) {
+    LEV_REQUIRE_CTX(ctx);
+    if (!d_w || !d_tokens || !d_out) return lev_fail(ctx, LEV_ERR_INVALID_ARGUMENT, "embed_q4_k: null pointer");
+    if (dim == 0 || dim % 256u != 0u || dim > LEV_MAX_Q4_INPUT_DIM || vocab == 0 || ntokens == 0 ||
+        ntokens > (1u << 20))
+        return lev_fail(ctx, LEV_ERR_BAD_DIMENSIONS, "embed_q4_k: dim %u (multiple of 256), vocab %u, %u tokens",
+                        dim, vocab, ntokens);
+    uint64_t need, end;
+    if (__builtin_mul_overflow((uint64_t)vocab, (uint64_t)(dim / 256u) * 144u, &need) ||
+        __builtin_add_overflow(w_off, need, &end))
+        return lev_fail(ctx, LEV_ERR_INTEGER_OVERFLOW, "embed_q4_k: extent overflows");
+    if (end > w_bytes || need > LEV_MAX_Q4_WEIGHT_BYTES)
+        return lev_fail(ctx, LEV_ERR_BAD_DIMENSIONS, "embed_q4_k: table [%llu, %llu) beyond %zu bytes",
+                        (unsigned long long)w_off, (unsigned long long)end, w_bytes);
+    if (out_capacity < (uint64_t)ntokens * dim)
+        return lev_fail(ctx, LEV_ERR_BAD_DIMENSIONS, "embed_q4_k: out holds %zu, needs %llu", out_capacity,
+                        (unsigned long long)ntokens * dim);
+    const uint64_t groups = (uint64_t)ntokens * (dim / 256u);
+    if (groups > 0x7FFFFFFFull) return lev_fail(ctx, LEV_ERR_EXCEEDS_MODEL_WORKLOAD, "embed_q4_k: grid");
+    hipLaunchKernelGGL(embed_q4_k, dim3((unsigned)groups), dim3(256), 0, ctx->stream,
+                       static_cast<const uint8_t *>(d_w) + w_off, d_tokens, d_out, dim / 256u, vocab, ctx->d_flag);
+    return lev_hip_check(ctx, hipGetLastError(), "embed_q4_k launch");
+}
 
 extern "C" int lev_hip_dequant(lev_ctx *ctx, int type, const void *d_w, size_t w_bytes,
                                uint64_t w_off, uint64_t nblocks, float *d_out,

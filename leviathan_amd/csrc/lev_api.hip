@@ -155,8 +155,9 @@ extern "C" int lev_hip_sync(lev_ctx *ctx) {
         LEV_HIP(ctx, lev_zero_async(ctx, ctx->d_flag, sizeof(int)));
         LEV_HIP(ctx, hipStreamSynchronize(ctx->stream));
         return lev_fail(ctx, LEV_ERR_BAD_DIMENSIONS,
-                        "a kernel rejected device-resident arguments (code %d: expert ids must be "
-                        "distinct and below the expert count)",
+                        "a kernel rejected device-resident arguments (code %d; bit 0: expert ids must be "
+                        "distinct and below the expert count, bit 1: non-finite router score, bit 2: token id "
+                        "beyond the embedding table)",
                         flag);
     }
     return LEV_OK;

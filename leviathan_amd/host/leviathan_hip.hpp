@@ -14,6 +14,8 @@
 //   Runner::expertMatvec                 Gemma4.swift:2805 (slice addressing; the slot cache is not mirrored)
 //   Runner::rmsnorm / geluUp / axpy      Gemma4.swift:3014, 3103, 3115
 //   Runner::normQuant / matvecQ8         Builder::norm_quant / matvec, rust/crates/lev-model/src/gpu.rs:295, 334
+//   Runner::embed                        Builder step "embed", gpu.rs:457
+//   Runner::bindGGUF / moeBinding        Gemma4.swift:543-566 (resident file), MoEModelBinding.swift:95-214
 //   Runner::routeTopK                    Gemma4.swift:3795-3810 (router matvec + softmax/top-k)
 //   Runner::runMoeBatchedRouted          Gemma4.swift:2073
 //   Runner::flushOpenSegment             Gemma4.swift:2313
@@ -410,6 +412,20 @@ public:
             geometry("rmsnorm buffers too small");
         check(lev_hip_rmsnorm(ctx_, x.floats(), y.floats(), (uint32_t)n, (uint32_t)vectors, w, eps_),
               "rmsnorm");
+    }
+
+    // ---- Builder step "embed", rust/crates/lev-model/src/gpu.rs:457 (embed_q4k, lev-forge/src/ops.rs:523) ----
+    // out[nb][dim] = rows tokens[0..nb) of a Q4_K table [vocab][dim]; tokens are u32 on the device.
+    void embed(const std::string &tensor, const DeviceBuffer &tokens, int64_t nb, DeviceBuffer &out) {
+        const TensorRef &r = lookup(tensor);
+        int64_t count;
+        if (r.type != GGMLTensorType::q4_K || r.inDim <= 0 || r.inDim % 256 != 0 || r.outDim <= 0 || nb <= 0 ||
+            __builtin_mul_overflow(r.inDim, nb, &count) || tokens.length < nb * 4 || out.length < count * 4)
+            geometry("embed: " + tensor + " is not a Q4_K table or the buffers are too small");
+        check(lev_hip_embed_q4_k(ctx_, weights_.contents(), (size_t)weights_.length, (uint64_t)r.offset,
+                                 static_cast<const uint32_t *>(tokens.contents()), (uint32_t)nb, out.floats(),
+                                 (size_t)(out.length / 4), (uint32_t)r.inDim, (uint32_t)r.outDim),
+              tensor);
     }
 
     // ---- Builder::norm_quant, rust/crates/lev-model/src/gpu.rs:295-320 ----

@@ -186,6 +186,16 @@ class Context:
                                                      _ptr(xs), _ptr(act)))
         return (xq, xs, act) if want_act else (xq, xs)
 
+    def embed_q4_k(self, w, tokens, dim: int, vocab: int, out=None, w_off: int = 0):
+        _dev(w, torch.uint8, "w")
+        _dev(tokens, torch.int32, "tokens")
+        n = tokens.numel()
+        if out is None:
+            out = torch.empty((max(n, 1), dim), dtype=torch.float32, device=w.device)
+        self._check(self.lib.lev_hip_embed_q4_k(self.ctx, _ptr(w), w.numel(), w_off, _ptr(tokens), n,
+                                                _ptr(out), out.numel(), dim, vocab))
+        return out
+
     def q4_k_gemm_prefill(self, w, x_f16, in_dim: int, rows: int, tokens: int, y=None, w_off: int = 0):
         _dev(w, torch.uint8, "w")
         _dev(x_f16, torch.float16, "x")

@@ -286,6 +286,19 @@ void runner_int8_path(Runner &r, const Model &m) {
         std::vector<float> got(logits.begin() + (size_t)c * Model::vocab, logits.begin() + (size_t)(c + 1) * Model::vocab);
         EXPECT(rel_err(got, ref) < 1e-4);
     }
+    // embedding gather from the same Q4_K tensor used as a [64][256] table: rows 63, 0, 5
+    {
+        std::vector<uint32_t> tok = {63, 0, 5};
+        DeviceBuffer dt = r.makeBuffer(tok), de = r.makeBuffer((int64_t)3 * H * 4);
+        r.embed("blk.0.ffn_up.weight", dt, 3, de);
+        std::vector<float> e = r.read<float>(de, (size_t)3 * H), want(H);
+        for (int c = 0; c < 3; ++c) {
+            levo_q4_k_dequant_block_f32(m.at("blk.0.ffn_up.weight") + (size_t)tok[c] * 144, want.data());
+            EXPECT(std::memcmp(e.data() + (size_t)c * H, want.data(), H * 4) == 0);
+        }
+        EXPECT(throws_geometry([&] { r.embed("blk.0.attn_q.weight", dt, 3, de); }));
+        EXPECT(throws_geometry([&] { r.embed("blk.0.ffn_up.weight", dt, 4, de); }));
+    }
     // a prefix of the rows (matvec_rows), and the guards before any launch
     r.matvecQ8("blk.0.ffn_up.weight", xq, xs, NB, dy, 0, 16);
     std::vector<float> y16 = r.read<float>(dy, (size_t)NB * 16);

@@ -402,6 +402,34 @@ def test_q4_k_config3_full_size(ctx, ncol):
         assert O.max_rel_err(alone[0], got[0].astype(np.float64)) < 1e-5
 
 
+def test_q4_k_embedding_gather_bit_exact(ctx):
+    """embed_q4k (lev-forge/src/ops.rs:523-555): out[c] is row tok[c] of the table, dequantised."""
+    from leviathan_amd.ops import LevError
+    vocab, dim = 300, 1024
+    w = O.synth_q4_k(77, vocab * dim // 256)
+    table = O.q4_k_dequant(w).reshape(vocab, dim)
+    tok = np.array([0, 299, 7, 7, 123, 1], np.int32)
+    got = ctx.embed_q4_k(dev(w), dev(tok), dim, vocab)
+    ctx.sync()
+    assert np.array_equal(bits(got.cpu().numpy()), bits(table[tok]))
+    # a tensor inside a larger buffer
+    pad = np.zeros(144 * 5, np.uint8)
+    got = ctx.embed_q4_k(dev(np.concatenate([pad, w])), dev(tok), dim, vocab, w_off=pad.size)
+    ctx.sync()
+    assert np.array_equal(bits(got.cpu().numpy()), bits(table[tok]))
+    # a token beyond the table writes nothing and surfaces at the next sync
+    out = torch.full((2, dim), float("nan"), device="cuda")
+    ctx.embed_q4_k(dev(w), dev(np.array([5, 300], np.int32)), dim, vocab, out=out)
+    with pytest.raises(LevError):
+        ctx.sync()
+    res = out.cpu().numpy()
+    assert np.array_equal(bits(res[0]), bits(table[5])) and np.isnan(res[1]).all()
+    ctx.sync()                                   # the flag is cleared
+    for kw in (dict(dim=100, vocab=vocab), dict(dim=dim, vocab=vocab + 1), dict(dim=dim, vocab=0)):
+        with pytest.raises(LevError):
+            ctx.embed_q4_k(dev(w), dev(tok), **kw)
+
+
 def test_q4_k_guards(ctx):
     from leviathan_amd import capi
     from leviathan_amd.ops import LevError
