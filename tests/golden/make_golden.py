@@ -57,6 +57,16 @@ def main():
     xh = O.normal(5 * cols, 3104).astype(np.float16).reshape(5, cols)
     v.update(gemm_x_f16_bits=xh.view(np.uint16),
              gemm_y_f64=O.q4_k_gemm_f16_oracle(w, rows, cols, xh.view(np.uint16), 5, 0, 1))
+    # int8-activation path: quantiser behind the RMSNorm of the Q4_K case's activations, the Q4_K
+    # product on those codes, and the Q6_K product on the plainly quantised Q6_K activation
+    q8 = [O.quantize_q8(O.rmsnorm(x[c], gain, 1e-6)) for c in range(ncol)]
+    v.update(q8_codes=np.stack([q for q, d, s in q8]), q8_d_bits=np.stack([d for q, d, s in q8]).view(np.uint32),
+             q8_s_bits=np.stack([s for q, d, s in q8]).view(np.uint32),
+             q8_q4_k_y_f64=np.stack([O.q4_k_matvec_q8_f64(w, rows, cols, q, d) for q, d, s in q8]))
+    q6, d6, s6 = O.quantize_q8(v["q6_k_x"])
+    r6, c6 = (int(t) for t in v["q6_k_dims"])
+    v.update(q8_q6_k_codes=q6, q8_q6_k_d_bits=d6.view(np.uint32),
+             q8_q6_k_y_f64=O.q6_k_matvec_q8_f64(v["q6_k_w"], r6, c6, q6, d6))
     # elementwise
     g = np.array([1.0, -20.0, 1e30, -1e30, 1e-30, 1e20, 0.5, -0.5, 3.25, -7.5], dtype=np.float32)
     u = np.array([1.0, 3.0, 2.0, 2.0, 2.0, 2.0, 4.0, 4.0, -1.5, 0.25], dtype=np.float32)

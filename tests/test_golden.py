@@ -47,6 +47,20 @@ def test_oracle_reproduces_golden_k_quants():
     assert np.array_equal(O.q4_k_gemm_f16_oracle(w, rows, cols, G["gemm_x_f16_bits"], 5, 0, 1), G["gemm_y_f64"])
 
 
+def test_oracle_reproduces_golden_int8_path():
+    rows, cols, ncol = (int(v) for v in G["q4_k_dims"])
+    w, x, gain = G["q4_k_w"], G["q4_k_x"], G["q4_k_gain"]
+    for c in range(ncol):
+        q, d, s = O.quantize_q8(O.rmsnorm(x[c], gain, 1e-6))
+        assert np.array_equal(q, G["q8_codes"][c]) and np.array_equal(d.view(np.uint32), G["q8_d_bits"][c])
+        assert np.array_equal(s.view(np.uint32), G["q8_s_bits"][c])
+        assert np.array_equal(O.q4_k_matvec_q8_f64(w, rows, cols, q, d), G["q8_q4_k_y_f64"][c])
+    r6, c6 = (int(v) for v in G["q6_k_dims"])
+    q, d, s = O.quantize_q8(G["q6_k_x"])
+    assert np.array_equal(q, G["q8_q6_k_codes"]) and np.array_equal(d.view(np.uint32), G["q8_q6_k_d_bits"])
+    assert np.array_equal(O.q6_k_matvec_q8_f64(G["q6_k_w"], r6, c6, q, d), G["q8_q6_k_y_f64"])
+
+
 def test_oracle_reproduces_golden_moe_and_elementwise():
     got = np.array([O.gelu_up_f32(float(a), float(b)) for a, b in zip(G["gelu_g"], G["gelu_u"])],
                    dtype=np.float32)
@@ -132,6 +146,26 @@ def test_gpu_golden_q4_k(ctx):
         assert O.max_rel_err(host(yp)[c], G["q4_k_y_plain_f64"][c]) < TOL
     for t in range(5):
         assert O.max_rel_err(host(yg)[t], G["gemm_y_f64"][t]) < 1e-3      # fp16 inputs: 1e-3
+
+
+@pytest.mark.gpu
+def test_gpu_golden_int8_path(ctx):
+    rows, cols, ncol = (int(v) for v in G["q4_k_dims"])
+    w, x, gain = dev(G["q4_k_w"]), dev(G["q4_k_x"].copy()), dev(G["q4_k_gain"])
+    xq, xs = ctx.norm_quant_q8(x, cols, ncol, gain=gain)
+    y = ctx.q4_k_gemv_q8(w, xq, xs, cols, rows, ncol)
+    r6, c6 = (int(v) for v in G["q6_k_dims"])
+    xq6, xs6 = ctx.norm_quant_q8(dev(G["q6_k_x"].copy()), c6, 1)
+    y6 = ctx.q6_k_gemv_q8(dev(G["q6_k_w"]), xq6, xs6, c6, r6, 1)
+    ctx.sync()
+    assert np.array_equal(host(xq), G["q8_codes"])                       # codes, scales, sums: bit-exact
+    assert np.array_equal(host(xs)[..., 0].view(np.uint32), G["q8_d_bits"])
+    assert np.array_equal(host(xs)[..., 1].view(np.uint32), G["q8_s_bits"])
+    assert np.array_equal(host(xq6)[0], G["q8_q6_k_codes"])
+    assert np.array_equal(host(xs6)[0, :, 0].view(np.uint32), G["q8_q6_k_d_bits"])
+    for c in range(ncol):
+        assert O.max_rel_err(host(y)[c], G["q8_q4_k_y_f64"][c]) < TOL
+    assert O.max_rel_err(host(y6)[0], G["q8_q6_k_y_f64"]) < TOL
 
 
 @pytest.mark.gpu
