@@ -181,11 +181,12 @@ def test_q4_k_q8_shapes(ctx, rows, cols, ncol):
 
 @pytest.mark.parametrize("force", ["0", "1"])
 @pytest.mark.parametrize("rows,cols,ncol", [(37, 1024, 1), (130, 4352, 3), (20, 12288, 8), (64, 4096, 16),
-                                            (5000, 4096, 12), (16, 16384, 5)])
+                                            (5000, 4096, 12), (16, 16384, 5), (40, 28672, 4)])
 def test_q4_k_q8_both_kernels_every_column_count(ctx, monkeypatch, rows, cols, ncol, force):
     """LEV_Q8_MFMA pins the kernel: 1 the matrix-core kernel (default from 9
     columns), 0 the dot4 kernel (default below); both meet the gate everywhere.
-    5000 rows give a wave more than three tasks (the looping variant)."""
+    5000 rows give a wave more than three tasks (the looping variant); 28672
+    columns exceed the unrolled staging of the matrix-core kernel (its tail loops)."""
     monkeypatch.setenv("LEV_Q8_MFMA", force)
     w, x, gain = H.config3(rows, cols, ncol, seed=rows + ncol)
     got, xq, xs = q8_gemv(ctx, w, x, rows, cols, gain)
