@@ -24,6 +24,7 @@ namespace {
 
 constexpr int kFlagBadExpertId = 1;
 constexpr int kFlagNonFiniteScore = 2;
+constexpr uint32_t kScoresMfmaMinTokens = 16;   // from here the router scores run on the f64 matrix cores
 
 // ---------------------------------------------------------------------------
 // router
@@ -277,6 +278,55 @@ moe_scores_kernel(const float *__restrict__ wr, const float *__restrict__ x,
     for (uint32_t k = 0; k < K; ++k) {
         const double total = wave_sum_f64(acc[k]);
         if (lane == 0 && t0 + k < tokens) scores[(uint64_t)(t0 + k) * experts + e] = (float)total;
+    }
+}
+
+// Many tokens: scores as a small f64 matrix product on the matrix cores
+// (v_mfma_f64_16x16x4_f64: exact products of f32 inputs, f64 sums, rounded to
+// f32 once).  Workgroup = a 16-token x 16-expert tile, its sixteen waves split
+// the hidden dimension (the loop is latency-bound: a short share per wave keeps
+// all of its loads in flight at once) and their partial tiles are added in
+// wave order.  The router
+// and the activations are each read (tokens/16) resp. (experts/16) times instead
+// of once per (expert, 16 tokens).
+// Lane (i, kq) = (l % 16, l / 16) loads four consecutive floats of token row i
+// and of router row i; MFMA m of a step takes element m of both, i.e. the 16
+// k's of a step are spread as k = 4*kq + m: the same permutation on both
+// operands.  hidden % 256 == 0, rows 16-byte aligned.
+typedef double moe_f64x4 __attribute__((ext_vector_type(4)));
+
+__global__ void __launch_bounds__(1024)
+moe_scores_mfma_kernel(const float *__restrict__ wr, const float *__restrict__ x, float *__restrict__ scores,
+                       uint32_t hidden, uint32_t experts, uint32_t tokens) {
+    __shared__ double part[16][256];
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t i = lane & 15u, kq = lane >> 4;
+    const uint32_t e0 = blockIdx.x * 16u, t0 = blockIdx.y * 16u;
+    const uint32_t tok = t0 + i < tokens ? t0 + i : tokens - 1u;       // rows past the end repeat the last one
+    const uint32_t exp = e0 + i < experts ? e0 + i : experts - 1u;
+    const uint32_t span = hidden >> 4;                                  // this wave's share of the hidden dimension
+    const lev_f32x4 *xa = reinterpret_cast<const lev_f32x4 *>(x + (uint64_t)tok * hidden + wave * span) + kq;
+    const lev_f32x4 *wb = reinterpret_cast<const lev_f32x4 *>(wr + (uint64_t)exp * hidden + wave * span) + kq;
+    moe_f64x4 acc = {0.0, 0.0, 0.0, 0.0};
+    const uint32_t steps = span >> 4;
+#pragma unroll 8
+    for (uint32_t s = 0; s < steps; ++s) {
+        const lev_f32x4 a = xa[4u * s], b = wb[4u * s];
+        acc = __builtin_amdgcn_mfma_f64_16x16x4f64((double)a.x, (double)b.x, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f64_16x16x4f64((double)a.y, (double)b.y, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f64_16x16x4f64((double)a.z, (double)b.z, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f64_16x16x4f64((double)a.w, (double)b.w, acc, 0, 0, 0);
+    }
+    // D of the f64 16x16x4 product: register r of lane (i, kq) is row (token) 4*r + kq of column (expert) i
+#pragma unroll
+    for (int r = 0; r < 4; ++r) part[wave][(4u * (uint32_t)r + kq) * 16u + i] = acc[r];
+    __syncthreads();
+    const uint32_t tt = (threadIdx.x >> 4) & 15u, ee = threadIdx.x & 15u;
+    if (threadIdx.x < 256u && t0 + tt < tokens && e0 + ee < experts) {
+        double total = part[0][threadIdx.x];
+#pragma unroll
+        for (int w = 1; w < 16; ++w) total += part[w][threadIdx.x];
+        scores[(uint64_t)(t0 + tt) * experts + e0 + ee] = (float)total;
     }
 }
 
@@ -801,6 +851,12 @@ bool use_grouped(const lev_ctx *ctx, const moe_args &a, const float *x, uint32_t
 
 hipError_t run_scores(lev_ctx *ctx, const float *wr, const float *x, float *scores, uint32_t hidden,
                       uint32_t experts, uint32_t tokens) {
+    if (tokens >= kScoresMfmaMinTokens && hidden % 256u == 0u &&
+        ((reinterpret_cast<uintptr_t>(wr) | reinterpret_cast<uintptr_t>(x)) & 15u) == 0u) {
+        hipLaunchKernelGGL(moe_scores_mfma_kernel, dim3((experts + 15u) / 16u, (tokens + 15u) / 16u), dim3(1024), 0,
+                           ctx->stream, wr, x, scores, hidden, experts, tokens);
+        return hipGetLastError();
+    }
     const int split = tokens <= 4u;
     const uint32_t per_group = 4u * kScoreTokensPerWave;
     const uint32_t groups = split ? 1u : (tokens + per_group - 1u) / per_group;

@@ -46,7 +46,8 @@ def cpu_route(wr, x, top_k, scale=None):
 
 @pytest.mark.parametrize("hidden,experts,top_k,tokens", [(2048, 128, 8, 1), (2048, 128, 8, 64),
                                                          (256, 16, 3, 5), (2816, 128, 8, 3),
-                                                         (96, 8, 8, 2), (130, 200, 64, 2)])
+                                                         (96, 8, 8, 2), (130, 200, 64, 2),
+                                                         (512, 20, 4, 33), (768, 130, 8, 16), (2080, 64, 8, 40)])
 def test_router_ids_bit_exact_weights_close(ctx, hidden, experts, top_k, tokens):
     wr = O.normal(experts * hidden, 7 + hidden, 0.0, 0.02).reshape(experts, hidden)
     x = O.normal(tokens * hidden, 8 + experts).reshape(tokens, hidden)
