@@ -85,10 +85,12 @@ __device__ __forceinline__ void wave_lds_fence() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-// LDS the selection needs: a table of probabilities (experts rounded up to a
-// multiple of 64), as many rank counters, then 64 selected probabilities and ids.
-__host__ __device__ constexpr size_t router_lds_bytes(uint32_t experts) {
-    return (size_t)((experts + 63u) & ~63u) * 12u + 64u * 8u + 64u * 4u;
+// LDS the selection needs: a table of probabilities with 64*J entries (J as the
+// selection is instantiated, not the expert count: the layout below is laid
+// out for the whole table), as many rank counters, then 64 selected
+// probabilities and ids.
+__host__ __device__ constexpr size_t router_lds_bytes(uint32_t j) {
+    return (size_t)(64u * j) * 12u + 64u * 8u + 64u * 4u;
 }
 
 struct router_sel {
@@ -700,7 +702,7 @@ hipError_t launch_gate_up(lev_ctx *ctx, const moe_args &a, const float *x, const
                            a, x, rt.ids, nullptr, nullptr, nullptr, nullptr, act, ctx->d_flag,
                            rows_per_block);
     } else {
-        lds += 8 + router_lds_bytes(a.experts);
+        lds += 8 + router_lds_bytes(a.experts <= 128u ? 2u : 4u);
         if (a.experts <= 128u)
             hipLaunchKernelGGL((moe_gate_up_kernel<P, R, NS, 2>), grid, dim3(kGuThreads), lds, ctx->stream,
                                a, x, nullptr, rt.scores, rt.expert_scale, rt.ids_out, rt.weights_out,
@@ -867,16 +869,16 @@ hipError_t run_scores(lev_ctx *ctx, const float *wr, const float *x, float *scor
 
 hipError_t run_topk(lev_ctx *ctx, const float *scores, const float *scale, int32_t *ids,
                     float *weights, uint32_t experts, uint32_t top_k, uint32_t tokens) {
-    const size_t lds = router_lds_bytes(experts);
 #define LEV_TOPK(J)                                                                               \
-    hipLaunchKernelGGL((moe_topk_kernel<J>), dim3(tokens), dim3(256), lds, ctx->stream, scores,   \
-                       scale, ids, weights, ctx->d_flag, experts, top_k)
+    hipLaunchKernelGGL((moe_topk_kernel<J>), dim3(tokens), dim3(256), router_lds_bytes(J), ctx->stream, \
+                       scores, scale, ids, weights, ctx->d_flag, experts, top_k)
     if (experts <= 128u) LEV_TOPK(2);
     else if (experts <= 256u) LEV_TOPK(4);
     else if (experts <= 1024u) LEV_TOPK(16);
     else {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&moe_topk_kernel<64>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+                                           hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           (int)router_lds_bytes(64));
         if (e != hipSuccess) return e;
         LEV_TOPK(64);
     }

@@ -246,6 +246,29 @@ def test_moe_layer_config5(ctx, tokens):
         assert O.max_rel_err(y1.cpu().numpy()[0], y[0].astype(np.float64)) < TOL
 
 
+@pytest.mark.parametrize("hidden,inter,experts,top_k,tokens", [(1024, 256, 8, 2, 1), (256, 256, 16, 3, 4),
+                                                             (512, 256, 70, 5, 2), (256, 256, 200, 8, 3),
+                                                             (1024, 256, 8, 2, 9), (256, 256, 40, 4, 20)])
+def test_moe_layer_small_and_odd_expert_counts(ctx, hidden, inter, experts, top_k, tokens):
+    """The whole block (router in the gate/up kernel up to four tokens, separate
+    selection kernel above) for expert counts well below and between the table
+    sizes the selection is instantiated for."""
+    from leviathan_amd import ops
+    wr, pool, offs, x = H.config5(hidden, inter, experts, tokens, seed=experts + tokens)
+    pools = ops.Context.moe_pools(dev(pool), hidden, inter, experts, offs["gate_off"], offs["up_off"],
+                                  offs["down_off"])
+    y, ids, wts = ctx.moe_layer_q4_0(pools, dev(wr), dev(x), top_k, tokens)
+    ctx.sync()
+    y, ids, wts = y.cpu().numpy(), ids.cpu().numpy(), wts.cpu().numpy()
+    g, u, d = (pool[offs["gate_off"]:], pool[offs["up_off"]:], pool[offs["down_off"]:])
+    for t in range(tokens):
+        _, ref_ids, ref_w = cpu_route(wr, x[t], top_k)
+        assert ids[t].tolist() == ref_ids.tolist()
+        assert np.allclose(wts[t], ref_w, rtol=2e-5)
+        ref = O.moe_experts_f64(g, u, d, hidden, inter, ref_ids, ref_w, x[t])
+        assert O.max_rel_err(y[t], ref["y"]) < TOL_WIDE
+
+
 # ---------------------------------------------------------- prefill GEMM ----
 
 def gemm(ctx, w, x16, rows, cols, tokens):

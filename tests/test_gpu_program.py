@@ -1,0 +1,112 @@
+"""A recorded decode-like step (record once, replay; Program / Step,
+rust/crates/lev-vulkan/src/engine.rs:94-141; deferred segments,
+Sources/LeviathanCore/Gemma4.swift:2313-2376) over the int8 path and the MoE
+layer: every replay, with new device-resident inputs and eager work and
+synchronisations in between, must reproduce the eager step bit for bit.
+
+The step: embed(token) -> rmsnorm+quantise -> Q4_K x int8 (gate|up) ->
+swiglu+quantise -> Q4_K x int8 (down) -> residual add + rmsnorm + quantise ->
+MoE layer on the f32 stream -> Q6_K x int8 head -> argmax.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+DIM, FF, VOCAB, HEAD = 1024, 1024, 64, 96
+EXPERTS, TOPK, INTER = 8, 2, 256
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def p(t):
+    return C.c_void_p(t.data_ptr()) if t is not None else C.c_void_p(0)
+
+
+def test_recorded_step_replays_bit_exact():
+    from leviathan_amd import ops
+    stream = torch.cuda.Stream()
+    ctx = ops.Context(0, stream=stream)
+    lib, c = ctx.lib, ctx.ctx
+
+    def must(st):
+        if st:
+            raise RuntimeError(lib.lev_hip_last_error(c).decode())
+
+    table = dev(O.synth_q4_k(1, VOCAB * DIM // 256))
+    w_gu = dev(O.synth_q4_k(2, 2 * FF * DIM // 256))
+    w_dn = dev(O.synth_q4_k(3, DIM * FF // 256))
+    w_head = dev(O.synth_q6_k(4, HEAD * DIM // 256))
+    gain = dev((1.0 + 0.1 * O.normal(DIM, 5)).astype(np.float32))
+    gu_bytes, dn_bytes = INTER * (DIM // 32) * 18, DIM * (INTER // 32) * 18
+    pool = dev(np.concatenate([O.synth_q4_0(6, EXPERTS * gu_bytes // 18), O.synth_q4_0(7, EXPERTS * gu_bytes // 18),
+                               O.synth_q4_0(8, EXPERTS * dn_bytes // 18)]))
+    pools = ops.Context.moe_pools(pool, DIM, INTER, EXPERTS, 0, EXPERTS * gu_bytes, 2 * EXPERTS * gu_bytes)
+    router = dev(O.normal(EXPERTS * DIM, 9, 0.0, 0.02).reshape(EXPERTS, DIM))
+
+    with torch.cuda.stream(stream):
+        tok = torch.zeros(1, dtype=torch.int32, device="cuda")
+        x = torch.empty(1, DIM, device="cuda")
+        xq = torch.empty(1, max(DIM, FF), dtype=torch.int8, device="cuda")
+        xs = torch.empty(1, max(DIM, FF) // 32, 2, device="cuda")
+        gu = torch.empty(2 * FF, device="cuda")
+        dn = torch.empty(1, DIM, device="cuda")
+        ymoe = torch.empty(1, DIM, device="cuda")
+        ids = torch.empty(1, TOPK, dtype=torch.int32, device="cuda")
+        wts = torch.empty(1, TOPK, device="cuda")
+        logits = torch.empty(1, HEAD, device="cuda")
+        best = torch.empty(1, dtype=torch.int32, device="cuda")
+        margin = torch.empty(1, device="cuda")
+
+    def step():
+        must(lib.lev_hip_embed_q4_k(c, p(table), table.numel(), 0, p(tok), 1, p(x), x.numel(), DIM, VOCAB))
+        must(lib.lev_hip_norm_quant_q8(c, p(x), DIM, None, p(gain), 1e-6, p(xq), p(xs), None, DIM, 1))
+        must(lib.lev_hip_q4_k_gemv_q8(c, p(w_gu), w_gu.numel(), 0, p(xq), p(xs), DIM, p(gu), gu.numel(), DIM, 2 * FF, 1))
+        must(lib.lev_hip_swiglu_quant_q8(c, p(gu), C.c_void_p(gu.data_ptr() + 4 * FF), FF, p(xq), p(xs), None))
+        must(lib.lev_hip_q4_k_gemv_q8(c, p(w_dn), w_dn.numel(), 0, p(xq), p(xs), FF, p(dn), dn.numel(), FF, DIM, 1))
+        must(lib.lev_hip_norm_quant_q8(c, p(x), DIM, p(dn), p(gain), 1e-6, p(xq), p(xs), None, DIM, 1))   # x += dn
+        must(lib.lev_hip_moe_layer_q4_0(c, C.byref(pools), p(router), None, p(x), p(ymoe), p(ids), p(wts), TOPK, 1))
+        must(lib.lev_hip_axpy(c, p(ymoe), p(x), 1.0, DIM))
+        must(lib.lev_hip_q6_k_gemv_q8(c, p(w_head), w_head.numel(), 0, p(xq), p(xs), DIM, p(logits), logits.numel(),
+                                      DIM, HEAD, 1))
+        must(lib.lev_hip_argmax(c, p(logits), HEAD, 1, p(best), p(margin)))
+
+    def snapshot():
+        ctx.sync()
+        return [t.clone() for t in (x, xq, xs, gu, dn, ymoe, ids, wts, logits, best, margin)]
+
+    def set_token(t):
+        with torch.cuda.stream(stream):
+            tok.fill_(t)
+
+    # eager runs (the first also sizes the MoE scratch, which may not grow while recording)
+    eager = {}
+    for t in (3, 41, 17, 63):
+        set_token(t)
+        step()
+        eager[t] = snapshot()
+    assert not torch.equal(eager[3][8], eager[41][8])           # the step depends on its token
+
+    ctx.program_begin()
+    step()
+    prog = ctx.program_end()
+    assert prog.node_count() >= 10
+    for t in (41, 3, 63, 17, 41):
+        set_token(t)
+        prog.run()
+        got = snapshot()
+        for a, b in zip(got, eager[t]):
+            assert torch.equal(a, b), t
+        # the program's own eager work between replays
+        set_token((t * 7) % VOCAB)
+        step()
+        ctx.sync()
+    prog.destroy()
+    ctx.close()
