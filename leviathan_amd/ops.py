@@ -247,9 +247,11 @@ class Context:
                   up_off: int, down_off: int, gate_stride=None, up_stride=None, down_stride=None):
         gu = inter * (hidden // 32) * 18
         dn = hidden * (inter // 32) * 18
-        return capi.MoEExperts(C.c_void_p(base.data_ptr()), base.numel(), gate_off, up_off, down_off,
-                               gate_stride or gu, up_stride or gu, down_stride or dn, hidden, inter,
-                               experts)
+        pools = capi.MoEExperts(C.c_void_p(base.data_ptr()), base.numel(), gate_off, up_off, down_off,
+                                gate_stride or gu, up_stride or gu, down_stride or dn, hidden, inter,
+                                experts)
+        pools.keepalive = base      # the struct holds a raw pointer: the tensor lives as long as it
+        return pools
 
     def moe_route_topk(self, router_w, x, hidden: int, experts: int, top_k: int, tokens: int,
                        expert_scale=None, want_scores: bool = False):

@@ -47,7 +47,9 @@ def cpu_route(wr, x, top_k, scale=None):
 @pytest.mark.parametrize("hidden,experts,top_k,tokens", [(2048, 128, 8, 1), (2048, 128, 8, 64),
                                                          (256, 16, 3, 5), (2816, 128, 8, 3),
                                                          (96, 8, 8, 2), (130, 200, 64, 2),
-                                                         (512, 20, 4, 33), (768, 130, 8, 16), (2080, 64, 8, 40)])
+                                                         (512, 20, 4, 33), (768, 130, 8, 16), (2080, 64, 8, 40),
+                                                         (256, 600, 16, 2), (128, 2000, 64, 3), (256, 1024, 8, 17),
+                                                         (64, 4096, 32, 1)])
 def test_router_ids_bit_exact_weights_close(ctx, hidden, experts, top_k, tokens):
     wr = O.normal(experts * hidden, 7 + hidden, 0.0, 0.02).reshape(experts, hidden)
     x = O.normal(tokens * hidden, 8 + experts).reshape(tokens, hidden)
@@ -248,11 +250,13 @@ def test_moe_layer_config5(ctx, tokens):
 
 @pytest.mark.parametrize("hidden,inter,experts,top_k,tokens", [(1024, 256, 8, 2, 1), (256, 256, 16, 3, 4),
                                                              (512, 256, 70, 5, 2), (256, 256, 200, 8, 3),
-                                                             (1024, 256, 8, 2, 9), (256, 256, 40, 4, 20)])
+                                                             (1024, 256, 8, 2, 9), (256, 256, 40, 4, 20),
+                                                             (256, 256, 4, 2, 40), (512, 512, 3, 1, 30)])
 def test_moe_layer_small_and_odd_expert_counts(ctx, hidden, inter, experts, top_k, tokens):
     """The whole block (router in the gate/up kernel up to four tokens, separate
     selection kernel above) for expert counts well below and between the table
-    sizes the selection is instantiated for."""
+    sizes the selection is instantiated for; the last two give every expert more
+    tokens than one pass of the grouped kernel takes."""
     from leviathan_amd import ops
     wr, pool, offs, x = H.config5(hidden, inter, experts, tokens, seed=experts + tokens)
     pools = ops.Context.moe_pools(dev(pool), hidden, inter, experts, offs["gate_off"], offs["up_off"],
