@@ -314,21 +314,230 @@ q4_k_gemm_kernel(const uint8_t *__restrict__ w, const uint16_t *__restrict__ x,
     }
 }
 
+
+// ---- variant with the weight fragments shared through LDS --------------------
+// One workgroup = 256 tokens x 96 rows (so 512 x 12288 makes 256 workgroups, one
+// per CU).  Wave w multiplies tokens 64w..64w+63 (two 32-token tiles) with all
+// 96 rows (three 32-row tiles): 6 accumulator tiles.  Waves 0..2 each decode ONE
+// row tile per K-step (lane = row l%32, half l/32 of the 32 code bytes) and
+// write the four fp16 B fragments to LDS, where all four waves read them: a
+// weight is decoded once per workgroup.  Wave 3 runs the same instruction stream
+// on wave 2's rows (and stores the same values).  X is staged as above.
+constexpr int kSBN = 96;
+constexpr int kSRT = 3;
+constexpr int kSMT = 2;
+constexpr int kBFrag = 64 * 16;                 // one B fragment: 16 bytes per lane
+constexpr int kBBuf = 4 * kSRT * kBFrag;        // [q][row tile][lane], one K-step
+constexpr int kSThreads = 512;                  // four multiplying waves and four that load X
+
+__global__ void __launch_bounds__(kSThreads)
+q4_k_gemm_shared_kernel(const uint8_t *__restrict__ w, const uint16_t *__restrict__ x,
+                        float *__restrict__ y, uint32_t in_dim, uint32_t rows, uint32_t tokens) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    uint8_t *const ldsb = lds + kXBufs * kXBuf;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t lr = lane & 31u, lh = lane >> 5;
+    const uint32_t row0 = blockIdx.x * kSBN;
+    const uint32_t tok0 = blockIdx.y * kBM;
+    const uint32_t nsb = in_dim / 256u;
+    const uint32_t drt = wave < 3u ? wave : 2u;          // row tile this wave decodes
+    const uint32_t drow = row0 + 32u * drt + lr;
+    const uint8_t *const wrow = w + (uint64_t)(drow < rows ? drow : rows - 1u) * nsb * 144u;
+
+    const uint32_t nsteps = nsb * 4u;
+
+    // Waves 4..7 only move X, one on each SIMD: per K-step each issues 8 direct
+    // global -> LDS loads (eight token rows of 128 bytes per load).  The path from
+    // L1 takes 64 bytes a cycle, so the 32 KB of a step keep it busy for most of
+    // the step; a wave that multiplies would stall at every request until the path
+    // accepts it, these have nothing else to do.  Step ks+2 goes into the buffer
+    // step ks-2 used (every wave has passed barrier ks-1, hence finished reading
+    // it); vmcnt(8) before barrier ks leaves only the loads of step ks+1
+    // outstanding.  Addresses are a uniform base plus a 32-bit lane offset fixed
+    // for the whole kernel, so a request costs no vector instruction.
+    if (wave >= 4u) {
+        const uint32_t lw = __builtin_amdgcn_readfirstlane(wave) - 4u, ltok = lane >> 3, lpos = lane & 7u;
+        const uint8_t *const xtile = reinterpret_cast<const uint8_t *>(x) + (uint64_t)tok0 * in_dim * 2u;
+        uint32_t voff[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const uint32_t tl = 8u * (8u * lw + j) + ltok;
+            const uint32_t t = tok0 + tl < tokens ? tl : tokens - 1u - tok0;
+            voff[j] = t * in_dim * 2u + 16u * (lpos ^ (ltok & 7u));
+        }
+        auto x_request = [&](uint32_t kstep, uint32_t buf) {
+            const uint8_t *const xk = xtile + (uint64_t)kstep * (kKS * 2u);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                uint8_t *dst = lds + buf * kXBuf + (8u * lw + j) * 1024u;
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(xk + voff[j]),
+                                                 (__attribute__((address_space(3))) void *)dst, 16, 0, 0);
+            }
+        };
+        x_request(0, 0);
+        x_request(1 < nsteps ? 1 : nsteps - 1, 1);
+        for (uint32_t ks = 0; ks < nsteps; ++ks) {
+            LEV_WAIT_VMCNT(8);
+            asm volatile("s_barrier" ::: "memory");
+            x_request(ks + 2 < nsteps ? ks + 2 : nsteps - 1, (ks + 2) & 3u);
+        }
+        LEV_WAIT_VMCNT(0);
+        return;
+    }
+
+    f32x16 acc[kSRT][kSMT];
+#pragma unroll
+    for (int r = 0; r < kSRT; ++r)
+#pragma unroll
+        for (int m = 0; m < kSMT; ++m)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[r][m][i] = 0.f;
+
+    lev_u32x4 hdr_n, qs_n[4];
+    auto w_load = [&](uint32_t sb) {
+        const uint32_t sbc = sb < nsb ? sb : nsb - 1u;
+        const uint8_t *blk = wrow + (uint64_t)sbc * 144u;
+        hdr_n = *reinterpret_cast<const lev_u32x4 *>(blk);
+#pragma unroll
+        for (int cc = 0; cc < 4; ++cc)
+            qs_n[cc] = *reinterpret_cast<const lev_u32x4 *>(blk + 16u + 32u * cc + 16u * lh);
+    };
+    lev_u32x4 qs[4];
+    float d1[8], mm[8];
+    auto take = [&]() {
+#pragma unroll
+        for (int cc = 0; cc < 4; ++cc) {
+            qs[cc] = qs_n[cc];
+            asm volatile("" : "+v"(qs[cc].x), "+v"(qs[cc].y), "+v"(qs[cc].z), "+v"(qs[cc].w));
+        }
+        q4k_all_factors(hdr_n, d1, mm);
+    };
+    w_load(0);
+    take();
+    {   // chunk 0 of superblock 0 -> B buffer 0
+        const lev_u32x4 q = qs[0];
+        f16x8 f[4];
+        f[0] = q4k_frag(q.x, q.y, false, d1[0], mm[0]);
+        f[1] = q4k_frag(q.z, q.w, false, d1[0], mm[0]);
+        f[2] = q4k_frag(q.x, q.y, true, d1[1], mm[1]);
+        f[3] = q4k_frag(q.z, q.w, true, d1[1], mm[1]);
+#pragma unroll
+        for (int qq = 0; qq < 4; ++qq)
+            *reinterpret_cast<f16x8 *>(ldsb + (qq * kSRT + drt) * kBFrag + lane * 16u) = f[qq];
+    }
+    for (uint32_t sb = 0; sb < nsb; ++sb) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const uint32_t ks = sb * 4u + c;
+            // this wave's B fragments of step ks have left for LDS (the bare
+            // barrier does not wait for them); wave 4 has waited for X of step ks
+            __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0), vmcnt and expcnt left open
+            asm volatile("s_barrier" ::: "memory");
+
+            const int cn = c == 3 ? 0 : c + 1;
+            const uint8_t *xb = lds + (ks & 3u) * kXBuf + (wave * 64u + lr) * kXRow;
+            const uint8_t *bb = ldsb + (ks & 1u) * kBBuf + lane * 16u;
+            uint8_t *bw = ldsb + ((ks + 1u) & 1u) * kBBuf + drt * kBFrag + lane * 16u;
+            // fragment `which` (use order a0 b0 b1 b2 a1) of MFMA group qq
+            f16x8 a_buf[2][kSMT], b_buf[2][kSRT];
+            auto frag_read_one = [&](int qq, int which) {
+                if (which == 0 || which == 4) {
+                    const int m = which == 0 ? 0 : 1;
+                    const uint32_t chunk = 2u * lh + (qq < 2 ? qq : 2u + qq);
+                    const uint32_t koff = 16u * (chunk ^ (lr & 7u));
+                    a_buf[qq & 1][m] = *reinterpret_cast<const f16x8 *>(xb + m * 32 * kXRow + koff);
+                } else {
+                    const int r = which - 1;
+                    b_buf[qq & 1][r] = *reinterpret_cast<const f16x8 *>(bb + (qq * kSRT + r) * kBFrag);
+                }
+            };
+            // The step opens with everything that does not depend on the first
+            // fragments, issued behind their reads so that it fills their latency.
+#pragma unroll
+            for (int f = 0; f < 5; ++f) frag_read_one(0, f);
+            if (c == 0) w_load(sb + 1u);
+            if (c == 3) take();
+#pragma unroll
+            for (int qq = 0; qq < 4; ++qq) {
+                // fragment qq of the NEXT chunk is decoded behind this group's MFMAs
+                const lev_u32x4 w4 = qs[cn];
+                uint32_t c0 = (qq & 1) ? w4.z : w4.x, c1 = (qq & 1) ? w4.w : w4.y;
+                if (qq >= 2) {
+                    c0 >>= 4;
+                    c1 >>= 4;
+                }
+                c0 &= 0x0F0F0F0Fu;
+                c1 &= 0x0F0F0F0Fu;
+                asm("" : "+v"(c0));
+                asm("" : "+v"(c1));
+                const float fd = d1[2 * cn + (qq >> 1)], fm = mm[2 * cn + (qq >> 1)];
+                f16x8 nf;
+                // Six slots of { one MFMA, a few other instructions }: a wave issues in
+                // order and an MFMA holds the matrix pipe for 32 cycles, so what is
+                // issued behind it within that time is free.  Five slots take one
+                // fragment read of the next group, four take two weights of the decode.
+#pragma unroll
+                for (int i = 0; i < 6; ++i) {
+                    const int r = i % 3, m = i / 3;
+                    acc[r][m] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_buf[qq & 1][m], b_buf[qq & 1][r], acc[r][m], 0, 0, 0);
+                    if (qq < 3 && i < 5) frag_read_one(qq + 1, i);
+                    if (r != 2) {
+                        const int s4 = 2 * m + r;
+                        const uint32_t cw = s4 < 2 ? c0 : c1;
+                        const float e0 = (s4 & 1) ? (float)((cw >> 16) & 0xFFu) : (float)(cw & 0xFFu);
+                        const float e1 = (s4 & 1) ? (float)(cw >> 24) : (float)((cw >> 8) & 0xFFu);
+                        nf[2 * s4] = q4k_weight_f16(fd, e0, fm);
+                        nf[2 * s4 + 1] = q4k_weight_f16(fd, e1, fm);
+                    }
+                    // wave 3 decoded wave 2's rows: it stores the same values to the same place,
+                    // which keeps the stream free of branches (a branch makes the compiler wait
+                    // for every LDS operation at the join)
+                    if (i == 5) *reinterpret_cast<f16x8 *>(bw + qq * kSRT * kBFrag) = nf;
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        }
+    }
+
+#pragma unroll
+    for (int r = 0; r < kSRT; ++r) {
+        const uint32_t my_row = row0 + 32u * r + lr;
+        if (my_row >= rows) continue;
+#pragma unroll
+        for (int m = 0; m < kSMT; ++m)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                uint32_t t = tok0 + wave * 64u + m * 32 + 8 * (i / 4) + 4 * lh + (i % 4);
+                if (t < tokens) y[(uint64_t)t * rows + my_row] = acc[r][m][i];
+            }
+    }
+}
+
 }  // namespace
 
 hipError_t lev_q4_k_gemm_launch(lev_ctx *ctx, const uint8_t *w, const uint16_t *x, float *y,
                                 uint32_t in_dim, uint32_t rows, uint32_t tokens) {
-    static bool attr_set = false;
-    const size_t lds = (size_t)kXBufs * kXBuf;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&q4_k_gemm_kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return e;
-        attr_set = true;
+    static int shared = -1;
+    if (shared < 0) {
+        const char *e = getenv("LEV_GEMM_SHARED");
+        const size_t lds = (size_t)kXBufs * kXBuf, lds_s = lds + 2 * kBBuf;
+        hipError_t st = hipFuncSetAttribute(reinterpret_cast<const void *>(&q4_k_gemm_kernel),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (st != hipSuccess) return st;
+        st = hipFuncSetAttribute(reinterpret_cast<const void *>(&q4_k_gemm_shared_kernel),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_s);
+        if (st != hipSuccess) return st;
+        shared = (e && e[0] == '0') ? 0 : 1;
     }
-    dim3 grid((rows + kBN - 1) / kBN, (tokens + kBM - 1) / kBM);
-    hipLaunchKernelGGL(q4_k_gemm_kernel, grid, dim3(kThreads), lds, ctx->stream, w, x, y, in_dim,
-                       rows, tokens);
+    if (shared) {
+        dim3 grid((rows + kSBN - 1) / kSBN, (tokens + kBM - 1) / kBM);
+        hipLaunchKernelGGL(q4_k_gemm_shared_kernel, grid, dim3(kSThreads), (size_t)kXBufs * kXBuf + 2 * kBBuf,
+                           ctx->stream, w, x, y, in_dim, rows, tokens);
+    } else {
+        dim3 grid((rows + kBN - 1) / kBN, (tokens + kBM - 1) / kBM);
+        hipLaunchKernelGGL(q4_k_gemm_kernel, grid, dim3(kThreads), (size_t)kXBufs * kXBuf, ctx->stream, w, x, y,
+                           in_dim, rows, tokens);
+    }
     return hipGetLastError();
 }
 
