@@ -7,28 +7,28 @@
 // as fp16; products accumulate in f32.  Both operands use the same 16-bit type
 // because one MFMA takes one input type; fp16 keeps X exactly as given.
 //
-// Tiling (one workgroup = 4 waves = 256 tokens x 128 rows):
-//   - wave (wr, wm) owns rows 64wr..64wr+63 (two 32-row tiles) for tokens
-//     128wm..128wm+127 (four 32-token tiles): 8 accumulator tiles of 32x32
+// One workgroup = 256 tokens x 96 rows, so that 512 x 12288 makes 256 workgroups,
+// one per CU.  Eight waves:
+//   - waves 0..3 multiply.  Wave w owns tokens 64w..64w+63 (two 32-token tiles)
+//     times all 96 rows (three 32-row tiles): 6 accumulator tiles of 32x32
 //     (v_mfma_f32_32x32x16_f16), A = X, B = W^T, so lane l holds output row
-//     (l%32) -> stores of Y are contiguous along rows.  Every X fragment read
-//     from LDS feeds two MFMAs (one per row tile): with one row tile per wave
-//     the LDS reads alone take as long as the MFMAs;
-//   - W never goes through LDS: lane (r = l%32, h = l/32) loads the 16 code
-//     bytes 16h..16h+15 of each 32-byte chunk of ITS two rows plus their
-//     superblock headers and dequantises them in registers straight into B
-//     fragments (the two waves that share rows both decode them);
-//   - X goes through LDS in K-steps of 64 (one Q4_K chunk) with direct
-//     global -> LDS loads (global_load_lds_dwordx4: no registers in between),
-//     four buffers, two steps in flight and one barrier per step, which covers
-//     the load latency that a single wave per SIMD cannot hide otherwise.  A direct load places lane
-//     l's 16 bytes at base + 16*l, so padding rows is not possible; instead
-//     the 16-byte chunk c of token row t is stored at position c ^ (t & 7)
-//     (the source address is permuted), which spreads the fragment reads of
-//     consecutive rows over all banks.
-// One wave per SIMD: a variant with two waves per SIMD (a pair of waves splitting
-// each K-step, half of the decode and half of the MFMAs each, partial sums
-// added through LDS) measured 13 % slower on 512 x 12288 x 4096.
+//     (l%32) and stores of Y are contiguous along rows;
+//   - W is decoded ONCE per workgroup: per K-step of 64 (one Q4_K chunk) waves
+//     0..2 each decode one row tile (lane = row l%32, half l/32 of the chunk's
+//     32 code bytes, loaded straight from global memory with the superblock
+//     header) into four fp16 B fragments and write them to LDS, where all four
+//     multiplying waves read them.  Wave 3 runs the same instruction stream on
+//     wave 2's rows and stores the same values: no branch in the stream.  The
+//     fragments of step ks+1 are decoded between the MFMAs of step ks;
+//   - waves 4..7 only move X, with direct global -> LDS loads
+//     (global_load_lds_dwordx4: no registers in between), four buffers, two
+//     steps in flight.  A direct load places lane l's 16 bytes at base + 16*l,
+//     so padding rows is not possible; instead the 16-byte chunk c of token row
+//     t is stored at position c ^ (t & 7) (the source address is permuted),
+//     which spreads the fragment reads of consecutive rows over all banks;
+//   - one barrier per K-step.  It is a bare s_barrier behind counted waits:
+//     __syncthreads() carries a workgroup fence for which the compiler waits for
+//     every outstanding load, the steps in flight included.
 // K order inside a 64-step is permuted consistently on both operands:
 // MFMA q (0..3) of chunk c takes, for lane half h, elements
 //   q<2 : 64c + 16h + 8q .. +7        (low nibbles of code bytes 8q..8q+7)
@@ -40,15 +40,17 @@ namespace {
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-constexpr int kThreads = 256;
 constexpr int kBM = 256;          // tokens per workgroup
-constexpr int kBN = 128;          // rows per workgroup (32 per wave)
-constexpr int kMT = 4;            // 32-token tiles per wave
-constexpr int kRT = 2;            // 32-row tiles per wave
+constexpr int kSBN = 96;          // rows per workgroup
+constexpr int kSRT = 3;           // 32-row tiles per wave
+constexpr int kSMT = 2;           // 32-token tiles per wave
 constexpr int kKS = 64;           // K-step (one chunk)
 constexpr int kXRow = 128;        // bytes per token row in LDS
 constexpr int kXBuf = kBM * kXRow;
-constexpr int kXBufs = 4;         // LDS buffers: the step in use, the one before it (still being read by late waves), two in flight
+constexpr int kXBufs = 4;         // X buffers in LDS: the step in use, the next (landed), two in flight
+constexpr int kBFrag = 64 * 16;                 // one B fragment: 16 bytes per lane
+constexpr int kBBuf = 4 * kSRT * kBFrag;        // [q][row tile][lane], one K-step; two of them
+constexpr int kSThreads = 512;                  // four multiplying waves and four that load X
 
 // (d*sc, dmin*m) of the 8 sub-blocks of a superblock (lev-cpu/src/lib.rs:64-74,
 // 117-124).
@@ -103,235 +105,14 @@ __device__ __forceinline__ f16x8 q4k_frag(uint32_t q0, uint32_t q1, bool hi, flo
     return f;
 }
 
-// grid (ceil(rows/128), ceil(tokens/256)); LDS kXBufs*kXBuf bytes.
-__global__ void __launch_bounds__(kThreads)
-q4_k_gemm_kernel(const uint8_t *__restrict__ w, const uint16_t *__restrict__ x,
-                 float *__restrict__ y, uint32_t in_dim, uint32_t rows, uint32_t tokens) {
-    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-    const uint32_t lr = lane & 31u, lh = lane >> 5;
-    const uint32_t wr = wave & 1u, wm = wave >> 1;
-    const uint32_t row0 = blockIdx.x * kBN + wr * 64u;
-    const uint32_t tok0 = blockIdx.y * kBM;
-    const uint32_t nsb = in_dim / 256u;
-    const uint8_t *wrow[kRT];
-#pragma unroll
-    for (int r = 0; r < kRT; ++r) {
-        const uint32_t row = row0 + 32u * r + lr;
-        wrow[r] = w + (uint64_t)(row < rows ? row : rows - 1u) * nsb * 144u;
-    }
-
-    // X staging: per K-step a thread requests 16 bytes of 8 token rows, sent
-    // straight to LDS.  Thread (token = tid/8 + 32i, position p = tid%8) fetches
-    // source chunk p ^ (token & 7).  Token rows past the end repeat the last
-    // one (their outputs are never stored).
-    const uint32_t xs_tok = tid >> 3, xs_pos = tid & 7u;
-    const uint8_t *xsrc[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const uint32_t tl = xs_tok + 32u * i;
-        const uint32_t t = tok0 + tl < tokens ? tok0 + tl : tokens - 1u;
-        xsrc[i] = reinterpret_cast<const uint8_t *>(x) + (uint64_t)t * in_dim * 2u + 16u * (xs_pos ^ (tl & 7u));
-    }
-    auto x_request = [&](uint32_t kstep, uint32_t buf) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const uint8_t *src = xsrc[i] + (uint64_t)kstep * (kKS * 2u);
-            // lane l of the wave lands at base + 16*l: base = this wave's 1 KB of pass i
-            uint8_t *dst = lds + buf * kXBuf + i * 4096 + wave * 1024u;
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
-                                             (__attribute__((address_space(3))) void *)dst, 16, 0, 0);
-        }
-    };
-    // s_waitcnt vmcnt(n) leaves at most n loads outstanding; loads complete in
-    // issue order, so everything older than the n newest has landed.  Encoding:
-    // vmcnt in bits 3:0 and 15:14, expcnt (6:4) and lgkmcnt (11:8) left at "any".
+// s_waitcnt vmcnt(n) leaves at most n loads outstanding; loads complete in
+// issue order, so everything older than the n newest has landed.  Encoding:
+// vmcnt in bits 3:0 and 15:14, expcnt (6:4) and lgkmcnt (11:8) left at "any".
 #define LEV_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xF) | (((n) >> 4) << 14) | (7 << 4) | (15 << 8))
 
-    f32x16 acc[kRT][kMT];
-#pragma unroll
-    for (int r = 0; r < kRT; ++r)
-#pragma unroll
-        for (int m = 0; m < kMT; ++m)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) acc[r][m][i] = 0.f;
-
-    const uint32_t nsteps = nsb * 4u;
-    // steps 0, 1, 2 in flight (clamped for very short K)
-    x_request(0, 0);
-    x_request(1 < nsteps ? 1 : nsteps - 1, 1);
-
-    // The weights of superblock sb+1 are requested while sb is multiplied: with
-    // one wave per SIMD nothing else hides their latency.  Loads are
-    // unconditional (clamped at the end) so that no branch forces a wait.
-    lev_u32x4 hdr_n[kRT], qs_n[kRT][4];
-    auto w_load = [&](uint32_t sb) {
-        const uint32_t sbc = sb < nsb ? sb : nsb - 1u;
-#pragma unroll
-        for (int r = 0; r < kRT; ++r) {
-            const uint8_t *blk = wrow[r] + (uint64_t)sbc * 144u;
-            hdr_n[r] = *reinterpret_cast<const lev_u32x4 *>(blk);
-#pragma unroll
-            for (int cc = 0; cc < 4; ++cc)
-                qs_n[r][cc] = *reinterpret_cast<const lev_u32x4 *>(blk + 16u + 32u * cc + 16u * lh);
-        }
-    };
-    lev_u32x4 qs[kRT][4];
-    float d1[kRT][8], mm[kRT][8];
-    auto take = [&]() {   // the prefetched superblock becomes the current one
-#pragma unroll
-        for (int r = 0; r < kRT; ++r) {
-#pragma unroll
-            for (int cc = 0; cc < 4; ++cc) {
-                qs[r][cc] = qs_n[r][cc];
-                // touched here so that the wait for these loads is placed HERE, where
-                // the compiler can count the loads issued since; left to the first
-                // use, in the next trip of the loop, it waits for everything
-                asm volatile("" : "+v"(qs[r][cc].x), "+v"(qs[r][cc].y), "+v"(qs[r][cc].z), "+v"(qs[r][cc].w));
-            }
-            q4k_all_factors(hdr_n[r], d1[r], mm[r]);
-        }
-    };
-    // this lane's 32 weights of chunk c of each of its two rows -> B fragments
-    auto dequant = [&](int c, f16x8 (&f)[kRT][4]) {
-#pragma unroll
-        for (int r = 0; r < kRT; ++r) {
-            const lev_u32x4 q = qs[r][c];
-            f[r][0] = q4k_frag(q.x, q.y, false, d1[r][2 * c], mm[r][2 * c]);
-            f[r][1] = q4k_frag(q.z, q.w, false, d1[r][2 * c], mm[r][2 * c]);
-            f[r][2] = q4k_frag(q.x, q.y, true, d1[r][2 * c + 1], mm[r][2 * c + 1]);
-            f[r][3] = q4k_frag(q.z, q.w, true, d1[r][2 * c + 1], mm[r][2 * c + 1]);
-        }
-    };
-    w_load(0);
-    take();
-    f16x8 bf[kRT][4];
-    dequant(0, bf);
-    for (uint32_t sb = 0; sb < nsb; ++sb) {
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            const uint32_t ks = sb * 4u + c;
-            // Step ks+2 goes into the buffer that step ks-2 used: a wave that gets
-            // here has passed the barrier of step ks-1, which every wave reaches
-            // only after its reads of step ks-2, so one barrier per step suffices.
-            // Then wait for step ks: its 8 loads are older than the 16 of steps
-            // ks+1 and ks+2 (a weight load issued in between only makes the wait
-            // stricter).
-            x_request(ks + 2 < nsteps ? ks + 2 : nsteps - 1, (ks + 2) & 3u);
-            LEV_WAIT_VMCNT(16);
-            // A bare barrier: __syncthreads() carries a workgroup fence, for which
-            // the compiler waits for EVERY outstanding load (the two steps just
-            // requested included).  LDS is coherent within the CU; each wave has
-            // waited for its own part of step ks above.
-            asm volatile("s_barrier" ::: "memory");
-
-            // The fragments of the NEXT chunk are decoded while this chunk is
-            // multiplied.  A wave issues in order, so with one wave per SIMD the
-            // vector ALU and the matrix core only work together if the two
-            // streams alternate in program order: eight groups of { decode one
-            // fragment (about 30 vector instructions), two LDS reads, four MFMAs },
-            // fenced so that the scheduler keeps them apart.  The MFMAs of a group
-            // run while the next group's decode issues.
-            f16x8 bn[kRT][4];
-            // The next superblock's weights are requested in step 0 and taken over
-            // in step 3 of the SAME trip of the loop: the compiler then knows how
-            // many loads were issued in between and waits for exactly those (over
-            // the loop's back edge it would wait for everything in flight).
-            if (c == 0) w_load(sb + 1u);
-            if (c == 3) take();
-            const int cn = c == 3 ? 0 : c + 1;
-            const uint8_t *xb = lds + (ks & 3u) * kXBuf + (wm * 128u + lr) * kXRow;
-            // fragment reads run one group ahead of the MFMAs that use them, so
-            // that their LDS latency passes behind the decode of the group
-            auto a_read = [&](int j, f16x8 (&a)[2]) {
-                const int qq = j >> 1;
-                // 16-byte chunk of this MFMA's 8 activations inside the 128-byte row,
-                // at its swizzled position (rows 32m + lr: same low bits as lr)
-                const uint32_t chunk = 2u * lh + (qq < 2 ? qq : 2u + qq);
-                const uint32_t koff = 16u * (chunk ^ (lr & 7u));
-#pragma unroll
-                for (int mm2 = 0; mm2 < 2; ++mm2)
-                    a[mm2] = *reinterpret_cast<const f16x8 *>(xb + (2 * (j & 1) + mm2) * 32 * kXRow + koff);
-            };
-            f16x8 a_buf[2][2];
-            a_read(0, a_buf[0]);
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                f16x8 (&a_cur)[2] = a_buf[j & 1];
-                if (j < 7) a_read(j + 1, a_buf[(j + 1) & 1]);
-                // One fragment of the next chunk per group, decoded in four slices
-                // of two weights, one slice behind each MFMA: a wave issues in
-                // order and an MFMA holds the matrix pipe for 8 passes, so the
-                // slice's vector instructions issue while it runs.  A whole
-                // fragment decoded in front of four back-to-back MFMAs would wait
-                // for the pipe instead.
-                const int fr = j >> 2, fq = j & 3;
-                const int sub = 2 * cn + (fq >> 1);
-                const lev_u32x4 w4 = qs[fr][cn];
-                uint32_t c0 = (fq & 1) ? w4.z : w4.x, c1 = (fq & 1) ? w4.w : w4.y;
-                if (fq >= 2) {
-                    c0 >>= 4;
-                    c1 >>= 4;
-                }
-                c0 &= 0x0F0F0F0Fu;
-                c1 &= 0x0F0F0F0Fu;
-                asm("" : "+v"(c0));
-                asm("" : "+v"(c1));
-                const float fd = d1[fr][sub], fm = mm[fr][sub];
-                const int qq = j >> 1;
-#pragma unroll
-                for (int s4 = 0; s4 < 4; ++s4) {
-                    const int mm2 = s4 >> 1, r = s4 & 1, m = 2 * (j & 1) + mm2;
-                    acc[r][m] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_cur[mm2], bf[r][qq], acc[r][m], 0, 0, 0);
-                    const uint32_t cw = s4 < 2 ? c0 : c1;
-                    const float e0 = (s4 & 1) ? (float)((cw >> 16) & 0xFFu) : (float)(cw & 0xFFu);
-                    const float e1 = (s4 & 1) ? (float)(cw >> 24) : (float)((cw >> 8) & 0xFFu);
-                    bn[fr][fq][2 * s4] = q4k_weight_f16(fd, e0, fm);
-                    bn[fr][fq][2 * s4 + 1] = q4k_weight_f16(fd, e1, fm);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-            }
-#pragma unroll
-            for (int r = 0; r < kRT; ++r)
-#pragma unroll
-                for (int qq = 0; qq < 4; ++qq) bf[r][qq] = bn[r][qq];
-        }
-    }
-
-    // D layout of the 32x32 tile: lane -> column n = l%32 (our row), register
-    // i -> line m = 8*(i/4) + 4*(l/32) + i%4 (our token).
-#pragma unroll
-    for (int r = 0; r < kRT; ++r) {
-        const uint32_t my_row = row0 + 32u * r + lr;
-        if (my_row >= rows) continue;
-#pragma unroll
-        for (int m = 0; m < kMT; ++m)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                uint32_t t = tok0 + wm * 128u + m * 32 + 8 * (i / 4) + 4 * lh + (i % 4);
-                if (t < tokens) y[(uint64_t)t * rows + my_row] = acc[r][m][i];
-            }
-    }
-}
-
-
-// ---- variant with the weight fragments shared through LDS --------------------
-// One workgroup = 256 tokens x 96 rows (so 512 x 12288 makes 256 workgroups, one
-// per CU).  Wave w multiplies tokens 64w..64w+63 (two 32-token tiles) with all
-// 96 rows (three 32-row tiles): 6 accumulator tiles.  Waves 0..2 each decode ONE
-// row tile per K-step (lane = row l%32, half l/32 of the 32 code bytes) and
-// write the four fp16 B fragments to LDS, where all four waves read them: a
-// weight is decoded once per workgroup.  Wave 3 runs the same instruction stream
-// on wave 2's rows (and stores the same values).  X is staged as above.
-constexpr int kSBN = 96;
-constexpr int kSRT = 3;
-constexpr int kSMT = 2;
-constexpr int kBFrag = 64 * 16;                 // one B fragment: 16 bytes per lane
-constexpr int kBBuf = 4 * kSRT * kBFrag;        // [q][row tile][lane], one K-step
-constexpr int kSThreads = 512;                  // four multiplying waves and four that load X
-
+// grid (ceil(rows/96), ceil(tokens/256)); LDS kXBufs*kXBuf + 2*kBBuf bytes.
 __global__ void __launch_bounds__(kSThreads)
-q4_k_gemm_shared_kernel(const uint8_t *__restrict__ w, const uint16_t *__restrict__ x,
+q4_k_gemm_kernel(const uint8_t *__restrict__ w, const uint16_t *__restrict__ x,
                         float *__restrict__ y, uint32_t in_dim, uint32_t rows, uint32_t tokens) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     uint8_t *const ldsb = lds + kXBufs * kXBuf;
@@ -517,27 +298,17 @@ q4_k_gemm_shared_kernel(const uint8_t *__restrict__ w, const uint16_t *__restric
 
 hipError_t lev_q4_k_gemm_launch(lev_ctx *ctx, const uint8_t *w, const uint16_t *x, float *y,
                                 uint32_t in_dim, uint32_t rows, uint32_t tokens) {
-    static int shared = -1;
-    if (shared < 0) {
-        const char *e = getenv("LEV_GEMM_SHARED");
-        const size_t lds = (size_t)kXBufs * kXBuf, lds_s = lds + 2 * kBBuf;
-        hipError_t st = hipFuncSetAttribute(reinterpret_cast<const void *>(&q4_k_gemm_kernel),
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (st != hipSuccess) return st;
-        st = hipFuncSetAttribute(reinterpret_cast<const void *>(&q4_k_gemm_shared_kernel),
-                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_s);
-        if (st != hipSuccess) return st;
-        shared = (e && e[0] == '0') ? 0 : 1;
+    static bool attr_set = false;
+    const size_t lds = (size_t)kXBufs * kXBuf + 2 * kBBuf;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&q4_k_gemm_kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        attr_set = true;
     }
-    if (shared) {
-        dim3 grid((rows + kSBN - 1) / kSBN, (tokens + kBM - 1) / kBM);
-        hipLaunchKernelGGL(q4_k_gemm_shared_kernel, grid, dim3(kSThreads), (size_t)kXBufs * kXBuf + 2 * kBBuf,
-                           ctx->stream, w, x, y, in_dim, rows, tokens);
-    } else {
-        dim3 grid((rows + kBN - 1) / kBN, (tokens + kBM - 1) / kBM);
-        hipLaunchKernelGGL(q4_k_gemm_kernel, grid, dim3(kThreads), (size_t)kXBufs * kXBuf, ctx->stream, w, x, y,
-                           in_dim, rows, tokens);
-    }
+    dim3 grid((rows + kSBN - 1) / kSBN, (tokens + kBM - 1) / kBM);
+    hipLaunchKernelGGL(q4_k_gemm_kernel, grid, dim3(kSThreads), lds, ctx->stream, w, x, y, in_dim,
+                       rows, tokens);
     return hipGetLastError();
 }
 
@@ -548,6 +319,8 @@ extern "C" int lev_hip_q4_k_gemm_prefill(lev_ctx *ctx, const void *d_w, size_t w
     LEV_REQUIRE_CTX(ctx);
     if (tokens == 0 || tokens > (1u << 20))
         return lev_fail(ctx, LEV_ERR_BAD_DIMENSIONS, "q4_k_gemm_prefill: %u tokens", tokens);
+    if (in_dim > (1u << 22))   // the X loaders keep 32-bit byte offsets inside a 256-token tile
+        return lev_fail(ctx, LEV_ERR_BAD_DIMENSIONS, "q4_k_gemm_prefill: in_dim %u above 4194304", in_dim);
     lev_geom g;
     int st = lev_check_matvec(ctx, "q4_k_gemm_prefill", 256, 144, d_w, w_bytes, w_off, d_x_f16,
                               x_count, (uint64_t)in_dim * tokens, d_y, y_capacity,

@@ -283,7 +283,9 @@ def gemm(ctx, w, x16, rows, cols, tokens):
 
 
 @pytest.mark.parametrize("rows,cols,tokens", [(128, 256, 32), (96, 512, 64), (200, 1024, 37),
-                                              (33, 256, 1), (256, 4096, 300)])
+                                              (33, 256, 1), (256, 4096, 300),
+                                              # either side of the 96-row x 256-token workgroup tile
+                                              (97, 256, 257), (95, 512, 255), (192, 256, 256), (289, 768, 511)])
 def test_gemm_small_shapes_every_row(ctx, rows, cols, tokens):
     w, x = H.config4(rows, cols, tokens, seed=rows + tokens)
     got = gemm(ctx, w, x, rows, cols, tokens)
