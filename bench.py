@@ -324,7 +324,7 @@ def main():
             run_other("q4_k_prefill_gemm_512x12288x4096", lambda i: must(lib.lev_hip_q4_k_gemm_prefill(
                 c, ring4.data_ptr(), ring4.numel(), (i % ncopy4) * nb4 * 144, xh.data_ptr(), xh.numel(),
                 yg.data_ptr(), yg.numel(), cols, r4, tokens)),
-                nb4 * 144 + tokens * cols * 2 + tokens * r4 * 4, 500, 1500, gemm_extra)
+                nb4 * 144 + tokens * cols * 2 + tokens * r4 * 4, int(os.environ.get("LEV_BENCH_GEMM_STEPS", "500")), int(os.environ.get("LEV_BENCH_GEMM_WARMUP", "1500")), gemm_extra)
             # 1500 warm-up launches (about 0.1 s): this kernel is bound by the matrix
             # cores, whose clock takes tens of milliseconds of load to reach its
             # sustained level (launch 40 of a cold sequence runs 25 % slower than

@@ -206,12 +206,35 @@ q4_k_gemm_kernel(const uint8_t *__restrict__ w, const uint16_t *__restrict__ x,
         for (int qq = 0; qq < 4; ++qq)
             *reinterpret_cast<f16x8 *>(ldsb + (qq * kSRT + drt) * kBFrag + lane * 16u) = f[qq];
     }
+    // The loop is rotated by two MFMA groups: groups 2 and 3 of a step are
+    // multiplied AFTER the barrier of the next step, from fragments read before
+    // it, so that the matrix cores have work while the first fragments of the
+    // new step come in from LDS (with X landing in LDS at the same time such a
+    // read takes several hundred cycles).  A trip is therefore
+    //   barrier(ks) | read group 0 | MFMA 2, 3 of ks-1 (reading group 1) |
+    //   MFMA 0, 1 of ks (reading groups 2, 3)
+    // with fragment p of chunk ks+1 decoded in phase p, so the B fragments of
+    // step ks+1 are complete (and the reads of step ks done) before barrier(ks+1).
+    // The first trip multiplies zero fragments in its phases 0 and 1.
+    f16x8 a_buf[4][kSMT], b_buf[4][kSRT];
+#pragma unroll
+    for (int g = 2; g < 4; ++g) {
+#pragma unroll
+        for (int m = 0; m < kSMT; ++m)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) a_buf[g][m][i] = (_Float16)0.f;
+#pragma unroll
+        for (int r = 0; r < kSRT; ++r)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) b_buf[g][r][i] = (_Float16)0.f;
+    }
     for (uint32_t sb = 0; sb < nsb; ++sb) {
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             const uint32_t ks = sb * 4u + c;
-            // this wave's B fragments of step ks have left for LDS (the bare
-            // barrier does not wait for them); wave 4 has waited for X of step ks
+            // this wave's B fragments of step ks have left for LDS and its reads of
+            // step ks-1 have arrived (the bare barrier waits for neither); the
+            // loader waves have waited for X of step ks
             __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0), vmcnt and expcnt left open
             asm volatile("s_barrier" ::: "memory");
 
@@ -220,30 +243,29 @@ q4_k_gemm_kernel(const uint8_t *__restrict__ w, const uint16_t *__restrict__ x,
             const uint8_t *bb = ldsb + (ks & 1u) * kBBuf + lane * 16u;
             uint8_t *bw = ldsb + ((ks + 1u) & 1u) * kBBuf + drt * kBFrag + lane * 16u;
             // fragment `which` (use order a0 b0 b1 b2 a1) of MFMA group qq
-            f16x8 a_buf[2][kSMT], b_buf[2][kSRT];
             auto frag_read_one = [&](int qq, int which) {
                 if (which == 0 || which == 4) {
                     const int m = which == 0 ? 0 : 1;
                     const uint32_t chunk = 2u * lh + (qq < 2 ? qq : 2u + qq);
                     const uint32_t koff = 16u * (chunk ^ (lr & 7u));
-                    a_buf[qq & 1][m] = *reinterpret_cast<const f16x8 *>(xb + m * 32 * kXRow + koff);
+                    a_buf[qq][m] = *reinterpret_cast<const f16x8 *>(xb + m * 32 * kXRow + koff);
                 } else {
                     const int r = which - 1;
-                    b_buf[qq & 1][r] = *reinterpret_cast<const f16x8 *>(bb + (qq * kSRT + r) * kBFrag);
+                    b_buf[qq][r] = *reinterpret_cast<const f16x8 *>(bb + (qq * kSRT + r) * kBFrag);
                 }
             };
-            // The step opens with everything that does not depend on the first
-            // fragments, issued behind their reads so that it fills their latency.
 #pragma unroll
             for (int f = 0; f < 5; ++f) frag_read_one(0, f);
             if (c == 0) w_load(sb + 1u);
             if (c == 3) take();
 #pragma unroll
-            for (int qq = 0; qq < 4; ++qq) {
-                // fragment qq of the NEXT chunk is decoded behind this group's MFMAs
+            for (int ph = 0; ph < 4; ++ph) {
+                const int qq = (ph + 2) & 3;   // the MFMA group of this phase
+                const int rg = ph == 0 ? 1 : ph;   // the group read in this phase (none in phase 1)
+                // fragment ph of the NEXT chunk is decoded behind this phase's MFMAs
                 const lev_u32x4 w4 = qs[cn];
-                uint32_t c0 = (qq & 1) ? w4.z : w4.x, c1 = (qq & 1) ? w4.w : w4.y;
-                if (qq >= 2) {
+                uint32_t c0 = (ph & 1) ? w4.z : w4.x, c1 = (ph & 1) ? w4.w : w4.y;
+                if (ph >= 2) {
                     c0 >>= 4;
                     c1 >>= 4;
                 }
@@ -251,17 +273,18 @@ q4_k_gemm_kernel(const uint8_t *__restrict__ w, const uint16_t *__restrict__ x,
                 c1 &= 0x0F0F0F0Fu;
                 asm("" : "+v"(c0));
                 asm("" : "+v"(c1));
-                const float fd = d1[2 * cn + (qq >> 1)], fm = mm[2 * cn + (qq >> 1)];
+                const float fd = d1[2 * cn + (ph >> 1)], fm = mm[2 * cn + (ph >> 1)];
                 f16x8 nf;
                 // Six slots of { one MFMA, a few other instructions }: a wave issues in
                 // order and an MFMA holds the matrix pipe for 32 cycles, so what is
                 // issued behind it within that time is free.  Five slots take one
-                // fragment read of the next group, four take two weights of the decode.
+                // fragment read (two groups ahead of its use), four take two weights
+                // of the decode.
 #pragma unroll
                 for (int i = 0; i < 6; ++i) {
                     const int r = i % 3, m = i / 3;
-                    acc[r][m] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_buf[qq & 1][m], b_buf[qq & 1][r], acc[r][m], 0, 0, 0);
-                    if (qq < 3 && i < 5) frag_read_one(qq + 1, i);
+                    acc[r][m] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_buf[qq][m], b_buf[qq][r], acc[r][m], 0, 0, 0);
+                    if (ph != 1 && i < 5) frag_read_one(rg, i);
                     if (r != 2) {
                         const int s4 = 2 * m + r;
                         const uint32_t cw = s4 < 2 ? c0 : c1;
@@ -273,12 +296,20 @@ q4_k_gemm_kernel(const uint8_t *__restrict__ w, const uint16_t *__restrict__ x,
                     // wave 3 decoded wave 2's rows: it stores the same values to the same place,
                     // which keeps the stream free of branches (a branch makes the compiler wait
                     // for every LDS operation at the join)
-                    if (i == 5) *reinterpret_cast<f16x8 *>(bw + qq * kSRT * kBFrag) = nf;
+                    if (i == 5) *reinterpret_cast<f16x8 *>(bw + ph * kSRT * kBFrag) = nf;
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
         }
     }
+    // groups 2 and 3 of the last step
+#pragma unroll
+    for (int g = 2; g < 4; ++g)
+#pragma unroll
+        for (int i = 0; i < 6; ++i) {
+            const int r = i % 3, m = i / 3;
+            acc[r][m] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_buf[g][m], b_buf[g][r], acc[r][m], 0, 0, 0);
+        }
 
 #pragma unroll
     for (int r = 0; r < kSRT; ++r) {
@@ -293,6 +324,7 @@ q4_k_gemm_kernel(const uint8_t *__restrict__ w, const uint16_t *__restrict__ x,
             }
     }
 }
+
 
 }  // namespace
 
