@@ -283,6 +283,33 @@ int lev_hip_q6_k_matvec_reporting(const uint8_t *blocks, size_t blocks_count, in
                                   int64_t in_dim, const float *x, size_t x_count, float *y_out,
                                   lev_evidence *evidence);
 
+/* ---- schedule candidates and per-shape selection (the library side of the
+ * forge loop: schedule::derive, lev-forge/src/schedule.rs:83-105;
+ * Q4ScheduleDeriver.derive, Q4Lowering.swift:283-362; the measured selection
+ * of lev-cli/src/main.rs:1977-2022 runs above this ABI) ----
+ * The reference derives schedules and emits a shader per candidate; here a
+ * schedule names one of the precompiled kernel variants.  Candidate 0 is
+ * always the built-in choice (the reference's BASELINE).  A selection applies
+ * to exactly one (op, in_dim, rows, ncol) on this context and is consulted by
+ * lev_hip_q4_0_gemv / lev_hip_q4_k_gemv_ncol before their built-in choice. */
+#define LEV_OP_Q4_0_GEMV 1u
+#define LEV_OP_Q4_K_GEMV 2u
+typedef struct lev_schedule {
+    uint32_t op;             /* LEV_OP_* */
+    uint32_t family;         /* Q4_K: 1 = matrix-core kernel, 0 = vector-ALU kernel; Q4_0: 0 */
+    uint32_t rows_in_flight; /* Q4_0: rows a wave keeps in flight (1, 2, 4; 0 = no variants for the shape) */
+    uint32_t persistent;     /* Q4_0: 0 = one workgroup per row tile, 1 = resident grid walking the tiles */
+} lev_schedule;
+/* Writes min(*count, capacity) candidates; *count is the full number. */
+int lev_hip_forge_candidates(lev_ctx *ctx, uint32_t op, uint32_t in_dim, uint32_t rows,
+                             uint32_t ncol, lev_schedule *out, uint32_t capacity, uint32_t *count);
+/* Installs `schedule` (which must be one of the shape's candidates, else
+ * LEV_ERR_INVALID_ARGUMENT) for the shape; replaces an earlier selection. */
+int lev_hip_forge_select(lev_ctx *ctx, uint32_t in_dim, uint32_t rows, uint32_t ncol,
+                         const lev_schedule *schedule);
+/* Back to the built-in choice for the shape. */
+int lev_hip_forge_clear(lev_ctx *ctx, uint32_t op, uint32_t in_dim, uint32_t rows, uint32_t ncol);
+
 #ifdef __cplusplus
 }
 #endif

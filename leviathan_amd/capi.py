@@ -48,6 +48,16 @@ class MoEExperts(C.Structure):
                 ("hidden", C.c_uint32), ("inter", C.c_uint32), ("experts", C.c_uint32)]
 
 
+class Schedule(C.Structure):
+    _fields_ = [("op", C.c_uint32), ("family", C.c_uint32), ("rows_in_flight", C.c_uint32),
+                ("persistent", C.c_uint32)]
+
+    def key(self):
+        return (self.op, self.family, self.rows_in_flight, self.persistent)
+
+
+OP_Q4_0_GEMV, OP_Q4_K_GEMV = 1, 2
+
 _vp, _sz, _u64, _u32, _f32, _i64, _int = (C.c_void_p, C.c_size_t, C.c_uint64, C.c_uint32, C.c_float,
                                           C.c_int64, C.c_int)
 
@@ -92,6 +102,10 @@ SIGNATURES = {
                                         _u32]),
     "lev_hip_moe_layer_q4_0": (_int, [_vp, C.POINTER(MoEExperts), _vp, _vp, _vp, _vp, _vp, _vp,
                                       _u32, _u32]),
+    "lev_hip_forge_candidates": (_int, [_vp, _u32, _u32, _u32, _u32, C.POINTER(Schedule), _u32,
+                                        C.POINTER(_u32)]),
+    "lev_hip_forge_select": (_int, [_vp, _u32, _u32, _u32, C.POINTER(Schedule)]),
+    "lev_hip_forge_clear": (_int, [_vp, _u32, _u32, _u32, _u32]),
     "lev_hip_q4_0_matvec_reporting": (_int, [_vp, _sz, _i64, _i64, _vp, _sz, _vp,
                                              C.POINTER(Evidence)]),
     "lev_hip_q6_k_matvec_reporting": (_int, [_vp, _sz, _i64, _i64, _vp, _sz, _vp,

@@ -9,6 +9,7 @@
 #include <cstdio>
 #include <cstring>
 #include <string>
+#include <vector>
 
 #include "../../include/leviathan_hip.h"
 
@@ -34,7 +35,17 @@ struct lev_ctx {
     // True between lev_hip_program_begin and lev_hip_program_end: the stream
     // is being captured, so nothing may allocate or synchronise.
     bool recording = false;
+    // Schedules installed per (op, shape) by lev_hip_forge_select; the matvec
+    // entry points look their shape up here before their built-in choice.
+    struct selection {
+        uint32_t in_dim, rows, ncol;
+        lev_schedule schedule;
+    };
+    std::vector<selection> selections;
 };
+
+// The schedule installed for this op and shape, or nullptr.
+const lev_schedule *lev_selected(const lev_ctx *ctx, uint32_t op, uint32_t in_dim, uint32_t rows, uint32_t ncol);
 
 int lev_fail(lev_ctx *ctx, int status, const char *fmt, ...);
 int lev_hip_check(lev_ctx *ctx, hipError_t err, const char *what);

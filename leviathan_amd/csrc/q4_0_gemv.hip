@@ -236,10 +236,12 @@ q4_0_gemv_generic(const uint8_t *__restrict__ w, const float *__restrict__ x,
 // NS = float4 of the activation vector each thread stages from registers.
 template <int L, int R, bool MULTI = false, int NS = 1>
 hipError_t launch_pairs(lev_ctx *ctx, const uint8_t *w, const float *x, float *y, uint32_t pairs,
-                        uint32_t rows) {
+                        uint32_t rows, int persistent = -1) {
     constexpr uint32_t rows_per_tile = kWaves * (LEV_WAVE / L) * R;
     uint32_t blocks = (rows + rows_per_tile - 1) / rows_per_tile;
-    if (!MULTI && blocks <= (uint32_t)ctx->num_cus * 4u) {
+    // built-in choice (persistent < 0): one workgroup per tile while every tile is resident at once
+    const bool tiles = persistent < 0 ? blocks <= (uint32_t)ctx->num_cus * 4u : persistent == 0;
+    if (!MULTI && tiles) {
         // every tile is resident at once: one straight-line tile per workgroup
         size_t lds1 = (size_t)16 * (pairs + 1) * sizeof(lev_f32x4) + (size_t)2 * pairs * sizeof(float);
         const bool exact = pairs == (uint32_t)L && pairs * 16u == (uint32_t)NS * kThreads;
@@ -280,24 +282,61 @@ hipError_t lev_q4_0_gemv_launch(lev_ctx *ctx, const uint8_t *w, const float *x, 
         return hipGetLastError();
     }
     const uint32_t pairs = nb / 2u;
+    // a schedule installed for this shape (lev_hip_forge_select) overrides the built-in choice
+    const lev_schedule *sel = lev_selected(ctx, LEV_OP_Q4_0_GEMV, in_dim, rows, 1);
+    if (sel && pairs > 16 && pairs <= 64) {
+        const int pm = (int)sel->persistent;
+        if (pairs > 32) {
+            if (sel->rows_in_flight == 1) return launch_pairs<64, 1, false, 2>(ctx, w, x, y, pairs, rows, pm);
+            if (sel->rows_in_flight == 2) return launch_pairs<64, 2, false, 2>(ctx, w, x, y, pairs, rows, pm);
+            return launch_pairs<64, 4, false, 2>(ctx, w, x, y, pairs, rows, pm);
+        }
+        if (sel->rows_in_flight == 1) return launch_pairs<32, 1>(ctx, w, x, y, pairs, rows, pm);
+        if (sel->rows_in_flight == 2) return launch_pairs<32, 2>(ctx, w, x, y, pairs, rows, pm);
+        return launch_pairs<32, 4>(ctx, w, x, y, pairs, rows, pm);
+    }
     if (pairs > 32) {
-        static const int forced = [] {
-            const char *e = getenv("LEV_Q4_R");
-            return e ? atoi(e) : 0;
-        }();
         if (pairs > 64) return launch_pairs<64, 2, true, 4>(ctx, w, x, y, pairs, rows);
-        int r = forced;
         // One row per wave and pass measured fastest at 4096 and 32768 rows:
         // 100 VGPRs leave five waves per SIMD to hide the HBM latency.
-        if (r == 0) r = 1;
-        if (r == 1) return launch_pairs<64, 1, false, 2>(ctx, w, x, y, pairs, rows);
-        if (r == 2) return launch_pairs<64, 2, false, 2>(ctx, w, x, y, pairs, rows);
-        return launch_pairs<64, 4, false, 2>(ctx, w, x, y, pairs, rows);
+        return launch_pairs<64, 1, false, 2>(ctx, w, x, y, pairs, rows);
     }
     if (pairs > 16) return launch_pairs<32, 4>(ctx, w, x, y, pairs, rows);
     if (pairs > 8) return launch_pairs<16, 4>(ctx, w, x, y, pairs, rows);
     if (pairs > 4) return launch_pairs<8, 4>(ctx, w, x, y, pairs, rows);
     return launch_pairs<4, 4>(ctx, w, x, y, pairs, rows);
+}
+
+// The candidate schedules of a Q4_0 GEMV shape, the built-in choice first
+// (Q4ScheduleDeriver.derive, Q4Lowering.swift:283-362: baseline first, then the
+// legal variants, bounded).  Shapes outside the two widest kernel families have
+// the built-in choice only.
+uint32_t lev_q4_0_gemv_candidates(const lev_ctx *ctx, uint32_t in_dim, uint32_t rows, lev_schedule *out,
+                                  uint32_t capacity) {
+    const uint32_t nb = in_dim / 32u, pairs = nb / 2u;
+    const bool family = (nb % 2u == 0u) && in_dim <= 32768u && pairs > 16 && pairs <= 64;
+    const uint32_t base_r = pairs > 32 ? 1u : 4u;
+    const uint32_t lanes = pairs > 32 ? 64u : 32u;
+    auto is_persistent = [&](uint32_t r) {
+        const uint32_t rows_per_tile = kWaves * (LEV_WAVE / lanes) * r;
+        return (rows + rows_per_tile - 1) / rows_per_tile > (uint32_t)ctx->num_cus * 4u ? 1u : 0u;
+    };
+    lev_schedule all[8];
+    uint32_t n = 0;
+    auto push = [&](uint32_t r, uint32_t p) {
+        for (uint32_t i = 0; i < n; ++i)
+            if (all[i].rows_in_flight == r && all[i].persistent == p) return;
+        all[n++] = lev_schedule{LEV_OP_Q4_0_GEMV, 0u, r, p};
+    };
+    if (!family) {
+        push(0u, 0u);   // the built-in choice, which has no parameters here
+    } else {
+        push(base_r, is_persistent(base_r));
+        for (uint32_t r : {1u, 2u, 4u})
+            for (uint32_t p : {0u, 1u}) push(r, p);
+    }
+    for (uint32_t i = 0; i < n && i < capacity; ++i) out[i] = all[i];
+    return n;
 }
 
 extern "C" int lev_hip_q4_0_gemv(lev_ctx *ctx, const void *d_w, size_t w_bytes, uint64_t w_off,

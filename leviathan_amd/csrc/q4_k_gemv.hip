@@ -332,13 +332,11 @@ hipError_t lev_q4_k_gemv_launch(lev_ctx *ctx, const uint8_t *w, const float *x, 
                                 uint32_t ncol) {
     const uint32_t units = in_dim / 64u;
     uint32_t done = 0;
-    // matrix-core kernel wherever its activation staging fits (LEV_Q4K_MFMA=0
-    // keeps the vector-ALU kernels, for comparison)
-    static const bool use_mfma = [] {
-        const char *e = getenv("LEV_Q4K_MFMA");
-        return !(e && e[0] == '0');
-    }();
-    const uint32_t mfma_cols = use_mfma ? lev_q4_k_mfma_cols(ctx, in_dim) : 0u;
+    // built-in choice: the matrix-core kernel wherever its activation staging fits
+    // a schedule installed for this shape (lev_hip_forge_select) overrides the built-in choice
+    const lev_schedule *sel = lev_selected(ctx, LEV_OP_Q4_K_GEMV, in_dim, rows, ncol);
+    const bool mfma = sel ? sel->family == 1u : true;
+    const uint32_t mfma_cols = mfma ? lev_q4_k_mfma_cols(ctx, in_dim) : 0u;
     while (mfma_cols && done < ncol) {
         uint32_t nc = ncol - done < mfma_cols ? ncol - done : mfma_cols;
         hipError_t e = lev_q4_k_mfma_gemv_launch(ctx, w, x + (uint64_t)done * in_dim, gain, eps,
@@ -363,6 +361,24 @@ hipError_t lev_q4_k_gemv_launch(lev_ctx *ctx, const uint8_t *w, const float *x, 
         done += nc;
     }
     return hipSuccess;
+}
+
+// Candidate schedules of a Q4_K GEMV shape, the built-in choice first
+// (schedule::derive, lev-forge/src/schedule.rs:83-105: baseline first, then the
+// legal alternatives): the matrix-core kernel where its staging fits, and the
+// vector-ALU kernel.
+uint32_t lev_q4_k_gemv_candidates(const lev_ctx *ctx, uint32_t in_dim, uint32_t rows, uint32_t ncol,
+                                  lev_schedule *out, uint32_t capacity) {
+    (void)rows;
+    (void)ncol;
+    uint32_t n = 0;
+    if (lev_q4_k_mfma_cols(ctx, in_dim) != 0u) {
+        if (n < capacity) out[n] = lev_schedule{LEV_OP_Q4_K_GEMV, 1u, 0u, 0u};
+        ++n;
+    }
+    if (n < capacity) out[n] = lev_schedule{LEV_OP_Q4_K_GEMV, 0u, 0u, 0u};
+    ++n;
+    return n;
 }
 
 extern "C" int lev_hip_q4_k_gemv_ncol(lev_ctx *ctx, const void *d_w, size_t w_bytes, uint64_t w_off,

@@ -196,6 +196,19 @@ class Context:
                                                 _ptr(out), out.numel(), dim, vocab))
         return out
 
+    # ---- schedule candidates and per-shape selection ----
+    def forge_candidates(self, op: int, in_dim: int, rows: int, ncol: int = 1):
+        buf = (capi.Schedule * 16)()
+        n = C.c_uint32(0)
+        self._check(self.lib.lev_hip_forge_candidates(self.ctx, op, in_dim, rows, ncol, buf, 16, C.byref(n)))
+        return [capi.Schedule(*buf[i].key()) for i in range(min(n.value, 16))]
+
+    def forge_select(self, in_dim: int, rows: int, schedule, ncol: int = 1):
+        self._check(self.lib.lev_hip_forge_select(self.ctx, in_dim, rows, ncol, C.byref(schedule)))
+
+    def forge_clear(self, op: int, in_dim: int, rows: int, ncol: int = 1):
+        self._check(self.lib.lev_hip_forge_clear(self.ctx, op, in_dim, rows, ncol))
+
     def q4_k_gemm_prefill(self, w, x_f16, in_dim: int, rows: int, tokens: int, y=None, w_off: int = 0):
         _dev(w, torch.uint8, "w")
         _dev(x_f16, torch.float16, "x")

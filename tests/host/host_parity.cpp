@@ -16,6 +16,7 @@
 #include <vector>
 
 #include "leviathan_hip.hpp"
+#include "leviathan_forge.hpp"
 
 extern "C" {
 #include "lev_oracle.h"
@@ -582,6 +583,78 @@ void runner_gguf_file(Runner &mem, const Model &m) {
 }
 
 
+// Forge loop (lev-cli/src/main.rs:1941-2024): baseline first, every candidate
+// gated against the FP64 oracle, the 2 % rule, the cache, and a gate nobody passes.
+void forge_matvec(Runner &r) {
+    struct Shape { GGMLTensorType type; int rows, cols, ncol; };
+    const Shape shapes[] = {{GGMLTensorType::q4_0, 512, 4096, 1}, {GGMLTensorType::q4_0, 300, 2048, 1},
+                            {GGMLTensorType::q4_0, 64, 256, 1}, {GGMLTensorType::q4_K, 256, 1024, 1},
+                            {GGMLTensorType::q4_K, 128, 512, 3}};
+    const std::string cache = "/tmp/leviathan_forge_test_cache.txt";
+    std::remove(cache.c_str());
+    for (const Shape &sh : shapes) {
+        const bool q40 = sh.type == GGMLTensorType::q4_0;
+        std::vector<uint8_t> w((size_t)sh.rows * sh.cols / (q40 ? 32 : 256) * (q40 ? 18 : 144));
+        if (q40) levo_synth_q4_0(51, 0.02f, w.data(), w.size() / 18);
+        else levo_synth_q4_k(52, 0.01f, w.data(), w.size() / 144);
+        ForgeOptions opt;
+        opt.launchesPerSample = 5;
+        opt.cachePath = cache;
+        ForgeReport rep = MatvecForge::forge(r, sh.type, w, sh.rows, sh.cols, sh.ncol, opt);
+        EXPECT(!rep.fromCache);
+        EXPECT(!rep.candidates.empty());
+        EXPECT(q40 || rep.candidates.size() == 2);                       // matrix-core and vector-ALU kernel
+        EXPECT(!q40 || sh.cols < 1024 || rep.candidates.size() == 6);      // 3 depths x 2 grids, baseline first
+        EXPECT(!q40 || sh.cols >= 1024 || rep.candidates.size() == 1);     // narrow rows: the built-in choice only
+        for (const ForgeCandidate &c : rep.candidates) {
+            EXPECT(c.pass);
+            EXPECT(c.maxRelErr >= 0 && c.maxRelErr < 1e-4);
+            EXPECT(c.medianUs > 0);
+        }
+        EXPECT(rep.selected >= 0 && rep.selected < (int)rep.candidates.size());
+        if (rep.selected > 0)
+            EXPECT(rep.candidates[(size_t)rep.selected].medianUs < 0.98 * rep.candidates[0].medianUs);
+        // the oracle inside the forge agrees with the test oracle on the same inputs
+        std::vector<float> x((size_t)sh.cols);
+        levo_fill_signed_unit(0x4C455649ull, x.data(), x.size());
+        std::vector<double> ref((size_t)sh.rows), mine((size_t)sh.rows, 0.0);
+        if (q40) levo_q4_0_matvec_f64(w.data(), w.size(), sh.rows, sh.cols, x.data(), sh.cols, ref.data());
+        else levo_q4_k_matvec_f64(w.data(), w.size(), sh.rows, sh.cols, x.data(), sh.cols, ref.data());
+        const size_t row_bytes = w.size() / (size_t)sh.rows;
+        double worst = 0;
+        for (int i = 0; i < sh.rows; ++i) {
+            if (q40) forge_detail::q4_0RowF64(w.data() + i * row_bytes, sh.cols, x.data(), mine[(size_t)i]);
+            else forge_detail::q4_kRowF64(w.data() + i * row_bytes, sh.cols, x.data(), mine[(size_t)i]);
+            worst = std::max(worst, std::fabs(mine[(size_t)i] - ref[(size_t)i]) / std::max(1.0, std::fabs(ref[(size_t)i])));
+        }
+        EXPECT(worst < 1e-12);
+        // second call: served from the cache, same schedule
+        ForgeReport again = MatvecForge::forge(r, sh.type, w, sh.rows, sh.cols, sh.ncol, opt);
+        EXPECT(again.fromCache && again.candidates.size() == 1);
+        const lev_schedule &a = again.candidates[0].schedule, &b = rep.candidates[(size_t)rep.selected].schedule;
+        EXPECT(a.family == b.family && a.rows_in_flight == b.rows_in_flight && a.persistent == b.persistent);
+        // a gate nobody passes selects nothing and leaves the built-in choice
+        ForgeOptions strict;
+        strict.launchesPerSample = 1;
+        strict.timed = 1;
+        strict.warm = 0;
+        strict.gate = 0.0;
+        ForgeReport none = MatvecForge::forge(r, sh.type, w, sh.rows, sh.cols, sh.ncol, strict);
+        EXPECT(none.selected == -1);
+    }
+    std::remove(cache.c_str());
+    // misuse of the selection ABI
+    lev_ctx *ctx = r.context();
+    lev_schedule bogus{LEV_OP_Q4_0_GEMV, 0u, 3u, 0u};
+    EXPECT(lev_hip_forge_select(ctx, 4096, 512, 1, &bogus) == LEV_ERR_INVALID_ARGUMENT);
+    lev_schedule wrong_op{7u, 0u, 1u, 0u};
+    EXPECT(lev_hip_forge_select(ctx, 4096, 512, 1, &wrong_op) == LEV_ERR_INVALID_ARGUMENT);
+    uint32_t n = 0;
+    EXPECT(lev_hip_forge_candidates(ctx, LEV_OP_Q4_K_GEMV, 100, 8, 1, nullptr, 0, &n) == LEV_ERR_BAD_DIMENSIONS);
+    EXPECT(lev_hip_forge_candidates(ctx, LEV_OP_Q4_0_GEMV, 4096, 8, 2, nullptr, 0, &n) == LEV_ERR_BAD_DIMENSIONS);
+    EXPECT(lev_hip_forge_candidates(ctx, LEV_OP_Q4_0_GEMV, 4096, 512, 1, nullptr, 0, &n) == LEV_OK && n == 6);
+}
+
 int main(int argc, char **argv) {
     Model model;
     std::unique_ptr<Runner> runner;
@@ -604,6 +677,7 @@ int main(int argc, char **argv) {
         {"runner_moe", [&] { runner_moe(R(), model); }},
         {"runner_moe_hand_computed", [&] { runner_moe_hand_computed(R()); }},
         {"runner_gguf_file", [&] { runner_gguf_file(R(), model); }},
+        {"forge_matvec", [&] { forge_matvec(R()); }},
     };
     if (argc > 1 && std::strcmp(argv[1], "--list") == 0) {
         for (auto &c : cases) std::printf("%s\n", c.name);

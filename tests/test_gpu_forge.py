@@ -1,0 +1,118 @@
+"""GPU: schedule candidates and per-shape selection behind the matvec entry points.
+
+The library side of the forge loop (schedule::derive, lev-forge/src/schedule.rs:83-105;
+selection rule lev-cli/src/main.rs:1977-2022).  Every candidate must pass the
+reference's gate max|y - oracle| / max(1, |oracle|) < 1e-4 on the forge's own
+input (SplitMix64(0x4C455649) signed units); candidate 0 is the built-in choice;
+a selection changes which kernel runs for exactly one shape and nothing else.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+GATE = 1e-4
+FORGE_SEED = 0x4C455649
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    from leviathan_amd import ops
+    c = ops.Context(0)
+    yield c
+    c.close()
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+@pytest.mark.parametrize("rows,cols,expected", [(4096, 4096, 6), (300, 2048, 6), (40000, 4096, 6),
+                                                (512, 1088, 6), (64, 256, 1), (16, 8192, 1)])
+def test_q4_0_candidates_pass_the_gate_and_agree_bitwise(ctx, rows, cols, expected):
+    from leviathan_amd import capi
+    w = O.synth_q4_0(rows + cols, rows * cols // 32, 0.02)
+    x = O.signed_units(cols, FORGE_SEED)
+    ref = O.q4_0_matvec_f64(w, rows, cols, x)
+    dw, dx = dev(w), dev(x)
+    cands = ctx.forge_candidates(capi.OP_Q4_0_GEMV, cols, rows)
+    assert len(cands) == expected
+    assert len({c.key() for c in cands}) == len(cands)
+    builtin = ctx.q4_0_gemv(dw, dx, cols, rows).cpu().numpy()
+    ctx.sync()
+    assert O.max_rel_err(builtin, ref) < GATE
+    try:
+        for i, s in enumerate(cands):
+            ctx.forge_select(cols, rows, s)
+            y = torch.full((rows,), float("nan"), device="cuda")
+            ctx.q4_0_gemv(dw, dx, cols, rows, y=y)
+            ctx.sync()
+            got = y.cpu().numpy()
+            assert O.max_rel_err(got, ref) < GATE, s.key()
+            # a row is summed by the same lanes in the same order whatever the tiling
+            assert np.array_equal(got.view(np.uint32), builtin.view(np.uint32)), s.key()
+    finally:
+        ctx.forge_clear(capi.OP_Q4_0_GEMV, cols, rows)
+
+
+@pytest.mark.parametrize("rows,cols,ncol", [(1024, 4096, 1), (512, 1024, 3), (96, 256, 8), (256, 4096, 16)])
+def test_q4_k_candidates_pass_the_gate(ctx, rows, cols, ncol):
+    from leviathan_amd import capi
+    w = O.synth_q4_k(rows + ncol, rows * cols // 256, 0.01)
+    x = O.signed_units(cols * ncol, FORGE_SEED).reshape(ncol, cols)
+    ref = np.stack([O.q4_k_matvec_f64(w, rows, cols, x[c]) for c in range(ncol)])
+    dw, dx = dev(w), dev(x)
+    cands = ctx.forge_candidates(capi.OP_Q4_K_GEMV, cols, rows, ncol)
+    assert [c.family for c in cands] == [1, 0]        # matrix-core kernel is the built-in choice
+    outs = []
+    try:
+        for s in cands:
+            ctx.forge_select(cols, rows, s, ncol)
+            y = torch.full((ncol, rows), float("nan"), device="cuda")
+            ctx.q4_k_gemv_ncol(dw, dx, cols, rows, ncol, y=y)
+            ctx.sync()
+            outs.append(y.cpu().numpy())
+            assert O.max_rel_err(outs[-1], ref) < GATE, s.key()
+    finally:
+        ctx.forge_clear(capi.OP_Q4_K_GEMV, cols, rows, ncol)
+    # the two families are different kernels: a selection really switches
+    assert not np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
+    again = ctx.q4_k_gemv_ncol(dw, dx, cols, rows, ncol).cpu().numpy()
+    assert np.array_equal(again.view(np.uint32), outs[0].view(np.uint32))   # cleared: built-in again
+
+
+def test_selection_applies_to_one_shape_only(ctx):
+    from leviathan_amd import capi
+    cols, ncol = 1024, 1
+    w = O.synth_q4_k(9, 512 * cols // 256, 0.01)
+    x = O.signed_units(cols, 3)
+    dw, dx = dev(w), dev(x)
+    base_256 = ctx.q4_k_gemv_ncol(dw, dx, cols, 256, ncol).cpu().numpy()
+    base_512 = ctx.q4_k_gemv_ncol(dw, dx, cols, 512, ncol).cpu().numpy()
+    valu = [c for c in ctx.forge_candidates(capi.OP_Q4_K_GEMV, cols, 256) if c.family == 0][0]
+    ctx.forge_select(cols, 256, valu)
+    try:
+        sel_256 = ctx.q4_k_gemv_ncol(dw, dx, cols, 256, ncol).cpu().numpy()
+        sel_512 = ctx.q4_k_gemv_ncol(dw, dx, cols, 512, ncol).cpu().numpy()
+    finally:
+        ctx.forge_clear(capi.OP_Q4_K_GEMV, cols, 256)
+    assert not np.array_equal(sel_256.view(np.uint32), base_256.view(np.uint32))
+    assert np.array_equal(sel_512.view(np.uint32), base_512.view(np.uint32))
+
+
+def test_selection_misuse_is_rejected(ctx):
+    from leviathan_amd import capi, ops
+    with pytest.raises(ops.LevError):
+        ctx.forge_select(4096, 512, capi.Schedule(capi.OP_Q4_0_GEMV, 0, 3, 0))       # no such depth
+    with pytest.raises(ops.LevError):
+        ctx.forge_select(4096, 512, capi.Schedule(capi.OP_Q4_0_GEMV, 1, 1, 0))       # no such family
+    with pytest.raises(ops.LevError):
+        ctx.forge_select(4096, 512, capi.Schedule(9, 0, 1, 0))                       # no such op
+    with pytest.raises(ops.LevError):
+        ctx.forge_candidates(capi.OP_Q4_K_GEMV, 100, 8)                              # not a Q4_K row
+    with pytest.raises(ops.LevError):
+        ctx.forge_candidates(capi.OP_Q4_0_GEMV, 4096, 8, 2)                          # Q4_0 GEMV is single-column
+    ctx.forge_clear(capi.OP_Q4_0_GEMV, 4096, 512)                                    # clearing nothing is fine
