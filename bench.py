@@ -56,7 +56,7 @@ def main():
     args = parse_args()
     if args.gpus != 1:
         print(f"bench.py: this build runs on ONE GPU (got --gpus {args.gpus}); "
-              "multi-GPU sharding is described in DESIGN.md and not built.", file=sys.stderr)
+              "the path is built and measured on one GPU only; nothing here shards across GPUs.", file=sys.stderr)
         sys.exit(2)
 
     import numpy as np
