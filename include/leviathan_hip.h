@@ -291,12 +291,14 @@ int lev_hip_q6_k_matvec_reporting(const uint8_t *blocks, size_t blocks_count, in
  * schedule names one of the precompiled kernel variants.  Candidate 0 is
  * always the built-in choice (the reference's BASELINE).  A selection applies
  * to exactly one (op, in_dim, rows, ncol) on this context and is consulted by
- * lev_hip_q4_0_gemv / lev_hip_q4_k_gemv_ncol before their built-in choice. */
+ * lev_hip_q4_0_gemv / lev_hip_q4_k_gemv_ncol / lev_hip_q4_k_gemv_q8 before their
+ * built-in choice. */
 #define LEV_OP_Q4_0_GEMV 1u
 #define LEV_OP_Q4_K_GEMV 2u
+#define LEV_OP_Q4_K_GEMV_Q8 3u
 typedef struct lev_schedule {
     uint32_t op;             /* LEV_OP_* */
-    uint32_t family;         /* Q4_K: 1 = matrix-core kernel, 0 = vector-ALU kernel; Q4_0: 0 */
+    uint32_t family;         /* Q4_K: 1 = matrix-core kernel, 0 = vector-ALU (int8: dot4) kernel; Q4_0: 0 */
     uint32_t rows_in_flight; /* Q4_0: rows a wave keeps in flight (1, 2, 4; 0 = no variants for the shape) */
     uint32_t persistent;     /* Q4_0: 0 = one workgroup per row tile, 1 = resident grid walking the tiles */
 } lev_schedule;

@@ -14,6 +14,8 @@ uint32_t lev_q4_0_gemv_candidates(const lev_ctx *ctx, uint32_t in_dim, uint32_t 
                                   uint32_t capacity);
 uint32_t lev_q4_k_gemv_candidates(const lev_ctx *ctx, uint32_t in_dim, uint32_t rows, uint32_t ncol,
                                   lev_schedule *out, uint32_t capacity);
+uint32_t lev_q4_k_gemv_q8_candidates(const lev_ctx *ctx, uint32_t in_dim, uint32_t rows, uint32_t ncol,
+                                     lev_schedule *out, uint32_t capacity);
 
 const lev_schedule *lev_selected(const lev_ctx *ctx, uint32_t op, uint32_t in_dim, uint32_t rows, uint32_t ncol) {
     for (const lev_ctx::selection &s : ctx->selections)
@@ -27,7 +29,7 @@ constexpr uint32_t kMaxCandidates = 16;
 
 int shape_ok(lev_ctx *ctx, uint32_t op, uint32_t in_dim, uint32_t rows, uint32_t ncol) {
     const uint32_t block = op == LEV_OP_Q4_0_GEMV ? 32u : 256u;
-    if (op != LEV_OP_Q4_0_GEMV && op != LEV_OP_Q4_K_GEMV)
+    if (op != LEV_OP_Q4_0_GEMV && op != LEV_OP_Q4_K_GEMV && op != LEV_OP_Q4_K_GEMV_Q8)
         return lev_fail(ctx, LEV_ERR_INVALID_ARGUMENT, "forge: unknown op %u", op);
     if (in_dim == 0 || rows == 0 || in_dim % block != 0 || in_dim > LEV_MAX_Q4_INPUT_DIM ||
         rows > LEV_MAX_Q4_OUTPUT_DIM)
@@ -39,8 +41,9 @@ int shape_ok(lev_ctx *ctx, uint32_t op, uint32_t in_dim, uint32_t rows, uint32_t
 
 uint32_t candidates(const lev_ctx *ctx, uint32_t op, uint32_t in_dim, uint32_t rows, uint32_t ncol,
                     lev_schedule *out, uint32_t capacity) {
-    return op == LEV_OP_Q4_0_GEMV ? lev_q4_0_gemv_candidates(ctx, in_dim, rows, out, capacity)
-                                  : lev_q4_k_gemv_candidates(ctx, in_dim, rows, ncol, out, capacity);
+    if (op == LEV_OP_Q4_0_GEMV) return lev_q4_0_gemv_candidates(ctx, in_dim, rows, out, capacity);
+    if (op == LEV_OP_Q4_K_GEMV) return lev_q4_k_gemv_candidates(ctx, in_dim, rows, ncol, out, capacity);
+    return lev_q4_k_gemv_q8_candidates(ctx, in_dim, rows, ncol, out, capacity);
 }
 
 }  // namespace

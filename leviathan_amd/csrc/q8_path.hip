@@ -742,6 +742,23 @@ extern "C" int lev_hip_norm_quant_q8(lev_ctx *ctx, float *d_x, size_t x_count, c
     return lev_hip_check(ctx, hipGetLastError(), "norm_quant_q8 launch");
 }
 
+// Candidate schedules of a Q4_K x int8 GEMV shape, the built-in choice first:
+// the dot4 kernel and, where its staging fits, the integer matrix-core kernel.
+uint32_t lev_q4_k_gemv_q8_candidates(const lev_ctx *ctx, uint32_t in_dim, uint32_t rows, uint32_t ncol,
+                                     lev_schedule *out, uint32_t capacity) {
+    (void)rows;
+    const bool has_mfma = q8m_cols(ctx, in_dim) != 0u;
+    const uint32_t first = has_mfma && ncol >= kQ8MfmaMinCols ? 1u : 0u;
+    uint32_t n = 0;
+    if (n < capacity) out[n] = lev_schedule{LEV_OP_Q4_K_GEMV_Q8, first, 0u, 0u};
+    ++n;
+    if (has_mfma) {
+        if (n < capacity) out[n] = lev_schedule{LEV_OP_Q4_K_GEMV_Q8, 1u - first, 0u, 0u};
+        ++n;
+    }
+    return n;
+}
+
 extern "C" int lev_hip_q4_k_gemv_q8(lev_ctx *ctx, const void *d_w, size_t w_bytes, uint64_t w_off,
                                     const int8_t *d_xq, const float *d_xs, size_t x_count, float *d_y,
                                     size_t y_capacity, uint32_t in_dim, uint32_t rows, uint32_t ncol) {
@@ -763,11 +780,12 @@ extern "C" int lev_hip_q4_k_gemv_q8(lev_ctx *ctx, const void *d_w, size_t w_byte
                              ? ctx->props.sharedMemPerBlockOptin
                              : ctx->props.sharedMemPerBlock;
     const uint32_t *xq = reinterpret_cast<const uint32_t *>(d_xq);
-    // Matrix-core kernel from kQ8MfmaMinCols columns up (LEV_Q8_MFMA=0 / 1 forces
-    // the choice, for measurements); the dot4 kernel otherwise.
+    // Built-in choice: the matrix-core kernel from kQ8MfmaMinCols columns up, the
+    // dot4 kernel below; a schedule installed for the shape (lev_hip_forge_select)
+    // overrides it.
     const uint32_t mcols = q8m_cols(ctx, in_dim);
-    const char *force = getenv("LEV_Q8_MFMA");
-    const bool mfma = mcols != 0u && (force ? force[0] != '0' : ncol >= kQ8MfmaMinCols);
+    const lev_schedule *sel = lev_selected(ctx, LEV_OP_Q4_K_GEMV_Q8, in_dim, rows, ncol);
+    const bool mfma = mcols != 0u && (sel ? sel->family == 1u : ncol >= kQ8MfmaMinCols);
     uint32_t done = 0;
     while (done < ncol) {
         uint32_t nc = ncol - done;

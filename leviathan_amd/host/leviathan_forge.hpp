@@ -59,6 +59,11 @@ struct ForgeOptions {
     double margin = 0.02;         // a non-baseline candidate must be more than this much faster
     uint64_t seed = 0x4C455649ull;
     std::string cachePath;        // empty: no cache
+    // Q4_K only: forge the int8-activation GEMV (lev_hip_q4_k_gemv_q8) instead of the
+    // f32 one.  The activations are quantised on the device and the oracle is the FP64
+    // product over those same codes (q * d), as `lev vk-q8` gates it
+    // (lev-cli/src/main.rs:1788-1868).
+    bool int8Activations = false;
 };
 
 namespace forge_detail {
@@ -152,7 +157,11 @@ public:
         using namespace forge_detail;
         if (type != GGMLTensorType::q4_0 && type != GGMLTensorType::q4_K)
             throw Gemma4Error(Gemma4Error::badTensorGeometry, "forge: only Q4_0 and Q4_K matvecs have schedules");
-        const uint32_t op = type == GGMLTensorType::q4_0 ? LEV_OP_Q4_0_GEMV : LEV_OP_Q4_K_GEMV;
+        if (opt.int8Activations && type != GGMLTensorType::q4_K)
+            throw Gemma4Error(Gemma4Error::badTensorGeometry, "forge: the int8-activation GEMV is Q4_K");
+        const uint32_t op = type == GGMLTensorType::q4_0 ? LEV_OP_Q4_0_GEMV
+                            : opt.int8Activations       ? LEV_OP_Q4_K_GEMV_Q8
+                                                        : LEV_OP_Q4_K_GEMV;
         const int64_t per = elementsPerBlock(type), bpb = bytesPerBlock(type);
         if (rows <= 0 || inDim <= 0 || ncol <= 0 || inDim % per != 0 ||
             (int64_t)weights.size() != rows * (inDim / per) * bpb)
@@ -206,6 +215,20 @@ public:
         for (float &v : x) v = rng.nextSignedUnit();
         std::vector<double> ref((size_t)(rows * ncol), 0.0);
         const int64_t rowBytes = inDim / per * bpb;
+        DeviceBuffer dw = r.makeBuffer(weights), dx = r.makeBuffer(x), dy = r.makeBuffer(rows * ncol * 4);
+        DeviceBuffer dxq, dxs;
+        if (opt.int8Activations) {
+            // quantise on the device, then continue with the values the codes stand for
+            dxq = r.makeBuffer(inDim * ncol);
+            dxs = r.makeBuffer(inDim / 32 * ncol * 8);
+            check(ctx, lev_hip_norm_quant_q8(ctx, dx.floats(), x.size(), nullptr, nullptr, 0.f,
+                                             static_cast<int8_t *>(dxq.contents()), dxs.floats(), nullptr,
+                                             (uint32_t)inDim, (uint32_t)ncol));
+            check(ctx, lev_hip_sync(ctx));
+            const std::vector<int8_t> q = r.read<int8_t>(dxq, (size_t)(inDim * ncol));
+            const std::vector<float> ds = r.read<float>(dxs, (size_t)(inDim / 32 * ncol * 2));
+            for (size_t i = 0; i < x.size(); ++i) x[i] = (float)q[i] * ds[(i / 32) * 2];
+        }
         for (int64_t c = 0; c < ncol; ++c)
             for (int64_t i = 0; i < rows; ++i) {
                 double s = 0;
@@ -214,8 +237,12 @@ public:
                 ref[(size_t)(c * rows + i)] = s;
             }
 
-        DeviceBuffer dw = r.makeBuffer(weights), dx = r.makeBuffer(x), dy = r.makeBuffer(rows * ncol * 4);
         auto launch = [&]() {
+            if (op == LEV_OP_Q4_K_GEMV_Q8)
+                return lev_hip_q4_k_gemv_q8(ctx, dw.contents(), weights.size(), 0,
+                                            static_cast<const int8_t *>(dxq.contents()), dxs.floats(), x.size(),
+                                            dy.floats(), (size_t)(rows * ncol), (uint32_t)inDim, (uint32_t)rows,
+                                            (uint32_t)ncol);
             if (op == LEV_OP_Q4_0_GEMV)
                 return lev_hip_q4_0_gemv(ctx, dw.contents(), weights.size(), 0, dx.floats(), (size_t)inDim,
                                          dy.floats(), (size_t)rows, (uint32_t)inDim, (uint32_t)rows);

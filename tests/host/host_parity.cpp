@@ -643,6 +643,20 @@ void forge_matvec(Runner &r) {
         EXPECT(none.selected == -1);
     }
     std::remove(cache.c_str());
+    // the int8-activation GEMV: dot4 kernel and integer matrix-core kernel, gated on the device's own codes
+    for (int ncol : {1, 12}) {
+        const int rows = 192, cols = 1024;
+        std::vector<uint8_t> w((size_t)rows * cols / 256 * 144);
+        levo_synth_q4_k(53, 0.01f, w.data(), w.size() / 144);
+        ForgeOptions opt;
+        opt.launchesPerSample = 5;
+        opt.int8Activations = true;
+        ForgeReport rep = MatvecForge::forge(r, GGMLTensorType::q4_K, w, rows, cols, ncol, opt);
+        EXPECT(rep.op == LEV_OP_Q4_K_GEMV_Q8 && rep.candidates.size() == 2);
+        EXPECT(rep.candidates[0].schedule.family == (ncol >= 9 ? 1u : 0u));   // the built-in choice first
+        for (const ForgeCandidate &c : rep.candidates) EXPECT(c.pass && c.maxRelErr < 1e-4);
+        EXPECT(rep.selected >= 0);
+    }
     // misuse of the selection ABI
     lev_ctx *ctx = r.context();
     lev_schedule bogus{LEV_OP_Q4_0_GEMV, 0u, 3u, 0u};

@@ -179,18 +179,26 @@ def test_q4_k_q8_shapes(ctx, rows, cols, ncol):
     check_gemv(got, w, rows, cols, xq, xs)
 
 
-@pytest.mark.parametrize("force", ["0", "1"])
+@pytest.mark.parametrize("family", [0, 1])
 @pytest.mark.parametrize("rows,cols,ncol", [(37, 1024, 1), (130, 4352, 3), (20, 12288, 8), (64, 4096, 16),
                                             (5000, 4096, 12), (16, 16384, 5), (40, 28672, 4)])
-def test_q4_k_q8_both_kernels_every_column_count(ctx, monkeypatch, rows, cols, ncol, force):
-    """LEV_Q8_MFMA pins the kernel: 1 the matrix-core kernel (default from 9
-    columns), 0 the dot4 kernel (default below); both meet the gate everywhere.
-    5000 rows give a wave more than three tasks (the looping variant); 28672
-    columns exceed the unrolled staging of the matrix-core kernel (its tail loops)."""
-    monkeypatch.setenv("LEV_Q8_MFMA", force)
-    w, x, gain = H.config3(rows, cols, ncol, seed=rows + ncol)
-    got, xq, xs = q8_gemv(ctx, w, x, rows, cols, gain)
-    check_gemv(got, w, rows, cols, xq, xs)
+def test_q4_k_q8_both_kernels_every_column_count(ctx, rows, cols, ncol, family):
+    """A forge selection pins the kernel: family 1 the integer matrix-core kernel
+    (built-in choice from 9 columns), 0 the dot4 kernel (built-in below); both meet
+    the gate everywhere.  5000 rows give a wave more than three tasks (the looping
+    variant); 28672 columns exceed the unrolled staging of the matrix-core kernel
+    (its tail loops)."""
+    from leviathan_amd import capi
+    cands = ctx.forge_candidates(capi.OP_Q4_K_GEMV_Q8, cols, rows, ncol)
+    assert sorted(c.family for c in cands) == [0, 1]
+    assert cands[0].family == (1 if ncol >= 9 else 0)          # candidate 0 is the built-in choice
+    ctx.forge_select(cols, rows, [c for c in cands if c.family == family][0], ncol)
+    try:
+        w, x, gain = H.config3(rows, cols, ncol, seed=rows + ncol)
+        got, xq, xs = q8_gemv(ctx, w, x, rows, cols, gain)
+        check_gemv(got, w, rows, cols, xq, xs)
+    finally:
+        ctx.forge_clear(capi.OP_Q4_K_GEMV_Q8, cols, rows, ncol)
 
 
 def test_q4_k_q8_hand_block(ctx):
