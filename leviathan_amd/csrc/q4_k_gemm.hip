@@ -113,7 +113,7 @@ __device__ __forceinline__ f16x8 q4k_frag(uint32_t q0, uint32_t q1, bool hi, flo
 // grid (ceil(rows/96), ceil(tokens/256)); LDS kXBufs*kXBuf + 2*kBBuf bytes.
 __global__ void __launch_bounds__(kSThreads)
 q4_k_gemm_kernel(const uint8_t *__restrict__ w, const uint16_t *__restrict__ x,
-                        float *__restrict__ y, uint32_t in_dim, uint32_t rows, uint32_t tokens) {
+                 float *__restrict__ y, uint32_t in_dim, uint32_t rows, uint32_t tokens) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     uint8_t *const ldsb = lds + kXBufs * kXBuf;
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
@@ -174,6 +174,12 @@ q4_k_gemm_kernel(const uint8_t *__restrict__ w, const uint16_t *__restrict__ x,
 #pragma unroll
             for (int i = 0; i < 16; ++i) acc[r][m][i] = 0.f;
 
+    // The weights of superblock sb+1 are requested in the first K-step of
+    // superblock sb and taken over in its last: with request and first use in one
+    // trip of the loop the compiler knows how many loads were issued in between
+    // and waits for exactly those (over the loop's back edge it would wait for
+    // everything in flight).  Loads are unconditional (clamped at the end) so
+    // that no branch forces a wait.
     lev_u32x4 hdr_n, qs_n[4];
     auto w_load = [&](uint32_t sb) {
         const uint32_t sbc = sb < nsb ? sb : nsb - 1u;
@@ -189,6 +195,7 @@ q4_k_gemm_kernel(const uint8_t *__restrict__ w, const uint16_t *__restrict__ x,
 #pragma unroll
         for (int cc = 0; cc < 4; ++cc) {
             qs[cc] = qs_n[cc];
+            // touched here so that the wait for these loads sits here and not at their first use
             asm volatile("" : "+v"(qs[cc].x), "+v"(qs[cc].y), "+v"(qs[cc].z), "+v"(qs[cc].w));
         }
         q4k_all_factors(hdr_n, d1, mm);
