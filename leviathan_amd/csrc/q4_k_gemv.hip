@@ -138,8 +138,9 @@ __device__ __forceinline__ void q4k_fetch_x(const lev_f32x4 *xs, uint32_t units,
 // NC columns, L lanes per row.  LDS: NC vectors in the unit-major transposed
 // layout (float4 slot q*(U+1)+u of column c at c*16*(U+1)), then NC floats of
 // 1/rms.  One row per wave-group and tile, persistent, double-buffered.
+// One column fits in 128 registers: four waves per SIMD, i.e. four workgroups per CU.
 template <int NC, int L, bool RESIDENT>
-__global__ void __launch_bounds__(kThreads)
+__global__ void __launch_bounds__(kThreads, (NC == 1 && RESIDENT) ? 4 : 1)
 q4_k_gemv_ncol(const uint8_t *__restrict__ w, const float *__restrict__ x,
                const float *__restrict__ gain, float eps, float *__restrict__ y, uint32_t units,
                uint32_t rows) {
@@ -253,9 +254,12 @@ q4_k_gemv_ncol(const uint8_t *__restrict__ w, const float *__restrict__ x,
         }
     };
 
+    // the next tile is requested unconditionally (clamped past the end): a branch
+    // around the loads would make the compiler wait for them before the current
+    // tile is used
     while (true) {
         uint32_t next = base + step;
-        if (next < rows) {
+        {
             uint32_t row = next + in_tile;
             q4k_load_unit(w + (uint64_t)(row < rows ? row : rows - 1u) * row_bytes, u0, Wb);
         }
@@ -263,7 +267,7 @@ q4_k_gemv_ncol(const uint8_t *__restrict__ w, const float *__restrict__ x,
         if (next >= rows) break;
         base = next;
         next = base + step;
-        if (next < rows) {
+        {
             uint32_t row = next + in_tile;
             q4k_load_unit(w + (uint64_t)(row < rows ? row : rows - 1u) * row_bytes, u0, Wa);
         }
@@ -279,18 +283,22 @@ hipError_t launch_ncol(lev_ctx *ctx, const uint8_t *w, const float *x, const flo
     constexpr uint32_t rows_per_tile = kWaves * (LEV_WAVE / L);
     uint32_t blocks = (rows + rows_per_tile - 1) / rows_per_tile;
     size_t lds = (size_t)NC * 16 * (units + 1) * sizeof(lev_f32x4);
-    // resident workgroups per CU: bounded by LDS (160 KB per CU) and registers
-    uint32_t per_cu = (uint32_t)((160u * 1024u) / (lds + 1024));
-    if (per_cu > 4u) per_cu = 4u;
-    if (per_cu < 1u) per_cu = 1u;
-    uint32_t cap = (uint32_t)ctx->num_cus * per_cu;
-    if (blocks > cap) blocks = cap;
     if (lds > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(
             reinterpret_cast<const void *>(&q4_k_gemv_ncol<NC, L, RESIDENT>),
             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
     }
+    // persistent grid: exactly the workgroups that are resident at once (a grid
+    // larger than that runs its surplus as a second, mostly idle round)
+    int resident = 0;
+    hipError_t oe = hipOccupancyMaxActiveBlocksPerMultiprocessor(
+        &resident, reinterpret_cast<const void *>(&q4_k_gemv_ncol<NC, L, RESIDENT>), kThreads, lds);
+    if (oe != hipSuccess) return oe;
+    uint32_t per_cu = resident < 1 ? 1u : (uint32_t)resident;
+    if (per_cu > 4u) per_cu = 4u;
+    uint32_t cap = (uint32_t)ctx->num_cus * per_cu;
+    if (blocks > cap) blocks = cap;
     hipLaunchKernelGGL((q4_k_gemv_ncol<NC, L, RESIDENT>), dim3(blocks), dim3(kThreads), lds,
                        ctx->stream, w, x, gain, eps, y, units, rows);
     return hipGetLastError();
@@ -327,15 +335,27 @@ hipError_t lev_q4_k_mfma_gemv_launch(lev_ctx *ctx, const uint8_t *w, const float
                                      float eps, float *y, uint32_t in_dim, uint32_t rows,
                                      uint32_t ncol);
 
+// Built-in kernel family (1 = matrix cores, 0 = vector ALU), from measurements on
+// MI355X: a single column of rows up to 4096 wide runs fastest on the vector-ALU
+// kernel (12288x4096: 8.5 against 10.7 us; it also starts faster: 2.5 against 4.6 us
+// for a small matrix), two columns only for rows up to 2048 wide or small matrices;
+// everything else on the matrix cores, where their activation staging fits.
+static uint32_t q4k_builtin_family(const lev_ctx *ctx, uint32_t in_dim, uint32_t rows, uint32_t ncol) {
+    if (lev_q4_k_mfma_cols(ctx, in_dim) == 0u) return 0u;
+    const uint32_t units = in_dim / 64u;
+    if (ncol == 1u && units <= 64u) return 0u;
+    if (ncol == 2u && (units <= 32u || (uint64_t)rows * in_dim <= (8u << 20))) return 0u;
+    return 1u;
+}
+
 hipError_t lev_q4_k_gemv_launch(lev_ctx *ctx, const uint8_t *w, const float *x, const float *gain,
                                 float eps, float *y, uint32_t in_dim, uint32_t rows,
                                 uint32_t ncol) {
     const uint32_t units = in_dim / 64u;
     uint32_t done = 0;
-    // built-in choice: the matrix-core kernel wherever its activation staging fits
     // a schedule installed for this shape (lev_hip_forge_select) overrides the built-in choice
     const lev_schedule *sel = lev_selected(ctx, LEV_OP_Q4_K_GEMV, in_dim, rows, ncol);
-    const bool mfma = sel ? sel->family == 1u : true;
+    const bool mfma = (sel ? sel->family : q4k_builtin_family(ctx, in_dim, rows, ncol)) == 1u;
     const uint32_t mfma_cols = mfma ? lev_q4_k_mfma_cols(ctx, in_dim) : 0u;
     while (mfma_cols && done < ncol) {
         uint32_t nc = ncol - done < mfma_cols ? ncol - done : mfma_cols;
@@ -369,15 +389,14 @@ hipError_t lev_q4_k_gemv_launch(lev_ctx *ctx, const uint8_t *w, const float *x, 
 // vector-ALU kernel.
 uint32_t lev_q4_k_gemv_candidates(const lev_ctx *ctx, uint32_t in_dim, uint32_t rows, uint32_t ncol,
                                   lev_schedule *out, uint32_t capacity) {
-    (void)rows;
-    (void)ncol;
+    const uint32_t first = q4k_builtin_family(ctx, in_dim, rows, ncol);
     uint32_t n = 0;
+    if (n < capacity) out[n] = lev_schedule{LEV_OP_Q4_K_GEMV, first, 0u, 0u};
+    ++n;
     if (lev_q4_k_mfma_cols(ctx, in_dim) != 0u) {
-        if (n < capacity) out[n] = lev_schedule{LEV_OP_Q4_K_GEMV, 1u, 0u, 0u};
+        if (n < capacity) out[n] = lev_schedule{LEV_OP_Q4_K_GEMV, 1u - first, 0u, 0u};
         ++n;
     }
-    if (n < capacity) out[n] = lev_schedule{LEV_OP_Q4_K_GEMV, 0u, 0u, 0u};
-    ++n;
     return n;
 }
 
