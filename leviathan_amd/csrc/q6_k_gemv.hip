@@ -23,7 +23,7 @@
 
 namespace {
 
-constexpr int kThreads = 256;
+constexpr int kThreads = 512;
 constexpr int kWaves = kThreads / LEV_WAVE;
 
 struct __attribute__((packed, aligned(2))) u32x4_a2 { uint32_t v[4]; };
