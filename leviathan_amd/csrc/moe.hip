@@ -353,13 +353,18 @@ moe_topk_kernel(const float *__restrict__ scores, const float *__restrict__ expe
 // expert ids: bounds + distinctness (MoEModelBinding.offsets requires both)
 // ---------------------------------------------------------------------------
 
+// The token's selection is usable for `slot` when its id is an expert and no
+// other slot names the same one.  Run by a whole wave (top_k <= 64): lane k
+// reads ids[k], so the check costs one memory round trip however many slots
+// there are.
 __device__ __forceinline__ bool expert_ids_ok(const int32_t *ids, uint32_t top_k, uint32_t slot,
-                                              uint32_t experts) {
-    int32_t me = ids[slot];
-    if (me < 0 || (uint32_t)me >= experts) return false;
-    for (uint32_t k = 0; k < top_k; ++k)
-        if (k != slot && ids[k] == me) return false;
-    return true;
+                                              uint32_t experts, uint32_t *expert) {
+    const uint32_t lane = threadIdx.x & 63u;
+    const int32_t mine = ids[lane < top_k ? lane : top_k - 1u];
+    const int32_t me = __builtin_amdgcn_readlane(mine, slot);
+    const unsigned long long same = __ballot(lane < top_k && mine == me);
+    *expert = (uint32_t)me;
+    return me >= 0 && (uint32_t)me < experts && __popcll(same) == 1;
 }
 
 // ---------------------------------------------------------------------------
@@ -439,27 +444,18 @@ moe_gate_up_kernel(moe_args a, const float *__restrict__ x, const int32_t *ids,
     lev_q4_stage_x_load<NS>(xt, pairs, tid, kGuThreads, xv);
 
     uint32_t e;
+    router_sel r{nullptr, nullptr, true};
     if constexpr (ROUTE > 0) {
         void *rl = reinterpret_cast<void *>(bsum + 2u * pairs);
         rl = reinterpret_cast<void *>((reinterpret_cast<uintptr_t>(rl) + 7u) & ~(uintptr_t)7u);
-        const router_sel r = router_select_block<ROUTE>(scores + (uint64_t)t * a.experts, rl,
-                                                        a.experts, a.top_k);
+        r = router_select_block<ROUTE>(scores + (uint64_t)t * a.experts, rl, a.experts, a.top_k);
         e = r.ok ? r.sel_id[slot] : slot;
-        if (blockIdx.x == 0 && slot == 0) {   // first workgroup of the token publishes the selection
-            if (!r.ok && tid == 0) atomicOr(flag, kFlagNonFiniteScore);
-            if (tid < a.top_k) {
-                ids_out[(uint64_t)t * a.top_k + tid] = r.ok ? (int32_t)r.sel_id[tid] : (int32_t)tid;
-                weights_out[(uint64_t)t * a.top_k + tid] =
-                    r.ok ? router_weight(r, expert_scale, a.top_k, tid) : 0.f;
-            }
-        }
     } else {
         const int32_t *tids = ids + (uint64_t)t * a.top_k;
-        if (!expert_ids_ok(tids, a.top_k, slot, a.experts)) {
+        if (!expert_ids_ok(tids, a.top_k, slot, a.experts, &e)) {
             if (tid == 0) atomicOr(flag, kFlagBadExpertId);
             return;
         }
-        e = (uint32_t)tids[slot];
     }
     const uint64_t row_bytes = (uint64_t)pairs * 36u;
     const uint8_t *wbase = a.base + (half ? a.up_off + e * a.up_stride : a.gate_off + e * a.gate_stride);
@@ -472,6 +468,18 @@ moe_gate_up_kernel(moe_args a, const float *__restrict__ x, const int32_t *ids,
     gu_load_rows<P, R>(wbase, row_bytes, i0, a.inter, pairs, lp, Da);
     lev_q4_stage_x_store_sums<NS>(xt, xs, bsum, pairs, tid, kGuThreads, xv);
     __syncthreads();
+    if constexpr (ROUTE > 0) {
+        // the first workgroup of a token publishes the selection while its
+        // weights are on their way
+        if (blockIdx.x == 0 && slot == 0) {
+            if (!r.ok && tid == 0) atomicOr(flag, kFlagNonFiniteScore);
+            if (tid < a.top_k) {
+                ids_out[(uint64_t)t * a.top_k + tid] = r.ok ? (int32_t)r.sel_id[tid] : (int32_t)tid;
+                weights_out[(uint64_t)t * a.top_k + tid] =
+                    r.ok ? router_weight(r, expert_scale, a.top_k, tid) : 0.f;
+            }
+        }
+    }
 
     lev_q4_pair_x X[P];
 #pragma unroll
@@ -515,7 +523,7 @@ constexpr int kDnThreads = kDnWaves * LEV_WAVE;
 // grid (row_tiles, tokens).  L lanes per row (pairs <= L), G = 64/L rows per
 // wave-step, `steps` wave-steps per tile: tile = G*steps rows.
 // LDS: per wave a transposed copy of its slot's activations, then
-// top_k*tile partial sums.
+// top_k*tile partial sums, then the top_k routing weights.
 template <int L>
 __global__ void __launch_bounds__(kDnThreads)
 moe_down_kernel(moe_args a, const float *__restrict__ act, const int32_t *__restrict__ ids,
@@ -535,15 +543,19 @@ moe_down_kernel(moe_args a, const float *__restrict__ act, const int32_t *__rest
     float *partial = reinterpret_cast<float *>(lds + kDnWaves * x_slots);   // [top_k][tile]
     const int32_t *tids = ids + (uint64_t)t * a.top_k;
     const uint32_t pc = lp < pairs ? lp : pairs - 1u;
+    // the routing weights are requested now and parked in LDS for the merge at
+    // the end (top_k <= 64: one lane each)
+    float *w_slot = partial + a.top_k * tile;
+    const float w_mine = weights[(uint64_t)t * a.top_k + (lane < a.top_k ? lane : a.top_k - 1u)];
 
     bool bad = false;
     for (uint32_t slot = wave; slot < a.top_k; slot += kDnWaves) {
-        if (!expert_ids_ok(tids, a.top_k, slot, a.experts)) {
+        uint32_t e;
+        if (!expert_ids_ok(tids, a.top_k, slot, a.experts, &e)) {
             bad = true;
             for (uint32_t r = lane; r < tile; r += 64u) partial[slot * tile + r] = 0.f;
             continue;
         }
-        const uint32_t e = (uint32_t)tids[slot];
         const uint8_t *wbase = a.base + a.down_off + e * a.down_stride;
         // first rows' weights go out before the activations are touched
         uint32_t Da[9], Db[9];
@@ -585,6 +597,7 @@ moe_down_kernel(moe_args a, const float *__restrict__ act, const int32_t *__rest
         __builtin_amdgcn_wave_barrier();   // X reads done before the next slot restages xs
     }
     if (bad && lane == 0) atomicOr(flag, kFlagBadExpertId);
+    if (wave == 0 && lane < a.top_k) w_slot[lane] = w_mine;
     __syncthreads();
     // ordered merge: y = sum over slots, in slot order, of w_slot * dn[slot]
     for (uint32_t r = tid; r < tile; r += kDnThreads) {
@@ -592,7 +605,7 @@ moe_down_kernel(moe_args a, const float *__restrict__ act, const int32_t *__rest
         if (row >= a.hidden) continue;
         float accum = 0.f;
         for (uint32_t slot = 0; slot < a.top_k; ++slot)
-            accum = fmaf(weights[(uint64_t)t * a.top_k + slot], partial[slot * tile + r], accum);
+            accum = fmaf(w_slot[slot], partial[slot * tile + r], accum);
         y[(uint64_t)t * a.hidden + row] = accum;
     }
 }
@@ -633,12 +646,13 @@ moe_gate_up_generic(moe_args a, const float *__restrict__ x, const int32_t *__re
     const uint32_t lane = threadIdx.x & 63u, i = blockIdx.x * 4u + (threadIdx.x >> 6);
     const uint32_t slot = blockIdx.y, t = blockIdx.z;
     const int32_t *tids = ids + (uint64_t)t * a.top_k;
-    if (!expert_ids_ok(tids, a.top_k, slot, a.experts)) {
+    uint32_t e;
+    if (!expert_ids_ok(tids, a.top_k, slot, a.experts, &e)) {
         if (threadIdx.x == 0) atomicOr(flag, kFlagBadExpertId);
         return;
     }
     if (i >= a.inter) return;
-    const uint32_t e = (uint32_t)tids[slot], blocks = a.hidden / 32u;
+    const uint32_t blocks = a.hidden / 32u;
     const float *xt = x + (uint64_t)t * a.hidden;
     float g = q4_0_row_dot_generic(a.base + a.gate_off + e * a.gate_stride + (uint64_t)i * blocks * 18u,
                                    xt, blocks, lane);
@@ -659,11 +673,11 @@ moe_down_generic(moe_args a, const float *__restrict__ act, const int32_t *__res
     const uint32_t blocks = a.inter / 32u;
     float accum = 0.f;
     for (uint32_t slot = 0; slot < a.top_k; ++slot) {
-        if (!expert_ids_ok(tids, a.top_k, slot, a.experts)) {
+        uint32_t e;
+        if (!expert_ids_ok(tids, a.top_k, slot, a.experts, &e)) {
             if (lane == 0) atomicOr(flag, kFlagBadExpertId);
             continue;
         }
-        const uint32_t e = (uint32_t)tids[slot];
         float d = q4_0_row_dot_generic(
             a.base + a.down_off + e * a.down_stride + (uint64_t)row * blocks * 18u,
             act + ((uint64_t)t * a.top_k + slot) * a.inter, blocks, lane);
@@ -729,7 +743,7 @@ hipError_t launch_down(lev_ctx *ctx, const moe_args &a, const float *act, const 
     tile = steps * G;
     uint32_t tiles = (a.hidden + tile - 1) / tile;
     size_t lds = (size_t)kDnWaves * 16 * (a.inter / 64u + 1u) * sizeof(lev_f32x4) +
-                 (size_t)a.top_k * tile * sizeof(float);
+                 (size_t)a.top_k * (tile + 1u) * sizeof(float);
     if (lds > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&moe_down_kernel<L>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
