@@ -114,12 +114,14 @@ struct router_sel {
 // J: each lane of a wave keeps experts j*64+lane, j < J, in registers, and
 // every wave computes the whole softmax for itself (same values, same order,
 // same result), so the only exchanges are the table, the ranks and the winners.
+// need_p = false (uniform over the workgroup): the caller only wants the ids;
+// sel_p is then not meaningful.
 template <int J>
 __device__ router_sel router_select_block(const float *__restrict__ srow, void *lds,
-                                          uint32_t experts, uint32_t top_k) {
+                                          uint32_t experts, uint32_t top_k, bool need_p = true) {
     constexpr uint32_t padded = 64u * J;
-    double *p_lds = static_cast<double *>(lds);
-    double *sel_p = p_lds + padded;
+    uint64_t *table = static_cast<uint64_t *>(lds);   // probabilities (f64) or order keys
+    double *sel_p = reinterpret_cast<double *>(table + padded);
     uint32_t *rank = reinterpret_cast<uint32_t *>(sel_p + 64);
     uint32_t *sel_id = rank + padded;
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
@@ -141,30 +143,63 @@ __device__ router_sel router_select_block(const float *__restrict__ srow, void *
         out.ok = false;
         return out;
     }
-    double p[J], sum = 0.0;
+    // The probabilities are exp(d)/sum with d = score - max <= 0 (f32).  While
+    // every d is 0 or lies in [-690, -1e-6], two different d are at least 1e-13
+    // apart relative to exp's value and every quotient is a normal number, so the
+    // probabilities order exactly as the d do and equal d give equal
+    // probabilities: the order "p larger, ties to the lower index" is then the
+    // ascending order of the integer (|d| bits, index).  Outside that range
+    // (exp saturating at 1 or running into denormals) the probabilities
+    // themselves are compared.
+    uint64_t key[J];
+    bool plain = true;
 #pragma unroll
     for (int j = 0; j < J; ++j) {
-        const bool valid = lane + 64u * j < experts;
-        p[j] = valid ? exp((double)(sc[j] - mx)) : 0.0;   // subtraction in f32, exp in f64
-        sum += p[j];
+        const uint32_t i = lane + 64u * j;
+        const bool valid = i < experts;
+        const float d = sc[j] - mx;
+        plain = plain && (!valid || d == 0.f || (d <= -1e-6f && d >= -690.f));
+        key[j] = valid ? ((uint64_t)(__float_as_uint(d) & 0x7FFFFFFFu) << 32) | i : ~0ull;
     }
-    sum = wave_sum_f64(sum);
+    const bool by_key = !__any(!plain);   // every wave holds the same scores: uniform
+    const bool with_p = need_p || !by_key;
+    double p[J];
+    if (with_p) {
+        double sum = 0.0;
+#pragma unroll
+        for (int j = 0; j < J; ++j) {
+            const bool valid = lane + 64u * j < experts;
+            p[j] = valid ? exp((double)(sc[j] - mx)) : 0.0;   // subtraction in f32, exp in f64
+            sum += p[j];
+        }
+        sum = wave_sum_f64(sum);
+#pragma unroll
+        for (int j = 0; j < J; ++j) p[j] = lane + 64u * j < experts ? p[j] / sum : 0.0;
+    }
     if (wave == 0) {
 #pragma unroll
         for (int j = 0; j < J; ++j) {
-            // padding entries hold 0 at indices above every real one: they rank last
-            p_lds[lane + 64u * j] = lane + 64u * j < experts ? p[j] / sum : 0.0;
+            // padding entries (probability 0, or the largest key) sit at indices
+            // above every real one: they rank last
+            table[lane + 64u * j] = by_key ? key[j] : (uint64_t)__double_as_longlong(p[j]);
             rank[lane + 64u * j] = 0u;
         }
     }
     __syncthreads();
     auto count_before = [&](uint32_t i, uint32_t j0, uint32_t j1) {
-        const double pi = p_lds[i];
         uint32_t before = 0;
+        if (by_key) {
+            const uint64_t ki = table[i];
 #pragma unroll 8
-        for (uint32_t j = j0; j < j1; ++j) {
-            const double pj = p_lds[j];   // same address across the wave: a broadcast read
-            before += (pj > pi || (pj == pi && j < i)) ? 1u : 0u;
+            for (uint32_t j = j0; j < j1; ++j) before += table[j] < ki ? 1u : 0u;
+        } else {
+            const double pi = __longlong_as_double((long long)table[i]);
+#pragma unroll 8
+            for (uint32_t j = j0; j < j1; ++j) {
+                // same address across the wave: a broadcast read
+                const double pj = __longlong_as_double((long long)table[j]);
+                before += (pj > pi || (pj == pi && j < i)) ? 1u : 0u;
+            }
         }
         return before;
     };
@@ -176,11 +211,15 @@ __device__ router_sel router_select_block(const float *__restrict__ srow, void *
         for (uint32_t i = tid; i < padded; i += blockDim.x) rank[i] = count_before(i, 0u, padded);
     }
     __syncthreads();
-    for (uint32_t i = tid; i < experts; i += blockDim.x) {
-        const uint32_t r = rank[i];
-        if (r < top_k) {
-            sel_id[r] = i;
-            sel_p[r] = p_lds[i];
+    if (wave == 0) {
+#pragma unroll
+        for (int j = 0; j < J; ++j) {
+            const uint32_t i = lane + 64u * j;
+            const uint32_t r = rank[i];
+            if (i < experts && r < top_k) {
+                sel_id[r] = i;
+                sel_p[r] = with_p ? p[j] : 0.0;
+            }
         }
     }
     __syncthreads();
@@ -448,7 +487,9 @@ moe_gate_up_kernel(moe_args a, const float *__restrict__ x, const int32_t *ids,
     if constexpr (ROUTE > 0) {
         void *rl = reinterpret_cast<void *>(bsum + 2u * pairs);
         rl = reinterpret_cast<void *>((reinterpret_cast<uintptr_t>(rl) + 7u) & ~(uintptr_t)7u);
-        r = router_select_block<ROUTE>(scores + (uint64_t)t * a.experts, rl, a.experts, a.top_k);
+        // only the workgroup that publishes the selection needs the probabilities
+        r = router_select_block<ROUTE>(scores + (uint64_t)t * a.experts, rl, a.experts, a.top_k,
+                                       blockIdx.x == 0 && slot == 0);
         e = r.ok ? r.sel_id[slot] : slot;
     } else {
         const int32_t *tids = ids + (uint64_t)t * a.top_k;

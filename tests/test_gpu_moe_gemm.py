@@ -97,6 +97,52 @@ def test_router_topk_is_exact_on_its_own_scores(ctx):
     assert np.allclose(wts.cpu().numpy()[0], ref_w, rtol=1e-6)
 
 
+ORDER_CASES = {
+    # exp() saturates at 1.0 for every score: all probabilities tie, index order wins
+    "saturating_exp": [3e-20, 1e-20, 2e-20, 0.0, 5e-21, 4e-20, 0.0, 1e-21],
+    # exp() underflows to 0 below about -745: those tie at 0, index order wins
+    "underflow": [0.0, -800.0, -900.0, -1000.0, -750.0, -700.0, -2000.0, -760.0],
+    # the ordinary range, with exact ties and a negative maximum
+    "plain": [-3.0, -1.5, -3.0, -1.5, -7.25, -1.5, -20.0, -3.0],
+    # one score just below the maximum (the gap is smaller than 1e-6), the rest ordinary
+    "near_max": [1.0, 1.0 - 2.0 ** -24, -1.0, 1.0 - 2.0 ** -23, 0.5, 1.0, -4.0, 0.25],
+}
+
+
+@pytest.mark.parametrize("case", sorted(ORDER_CASES))
+@pytest.mark.parametrize("experts", [8, 128, 200])
+def test_router_selection_order_edge_cases(ctx, case, experts):
+    """Selection order where the probabilities tie although the scores differ,
+    and where they do not: one-hot x makes the scores exactly the chosen values,
+    so ids are compared bit for bit, from the stand-alone router and from the
+    selection the single-token layer runs inside its gate/up kernel."""
+    from leviathan_amd import ops
+    hidden, inter, top_k = 64, 64, 5
+    vals = np.array(ORDER_CASES[case], np.float32)
+    rng = np.random.default_rng(experts)
+    scores = np.resize(vals, experts).astype(np.float32)
+    scores[8:] = rng.permutation(scores[8:])
+    wr = np.zeros((experts, hidden), np.float32)
+    wr[:, 3] = scores
+    x = np.zeros((1, hidden), np.float32)
+    x[0, 3] = 1.0
+    ref_ids, ref_w = O.router_topk(scores, top_k)
+    ids, wts, got = ctx.moe_route_topk(dev(wr), dev(x), hidden, experts, top_k, 1, want_scores=True)
+    ctx.sync()
+    assert np.array_equal(got.cpu().numpy()[0], scores)
+    assert ids.cpu().numpy()[0].tolist() == ref_ids.tolist()
+    assert np.allclose(wts.cpu().numpy()[0], ref_w, rtol=1e-6, atol=0)
+
+    gu, dn = inter * (hidden // 32) * 18, hidden * (inter // 32) * 18
+    pool = rng.integers(0, 256, experts * (2 * gu + dn), dtype=np.uint8)
+    pool.reshape(-1, 18)[:, 1] = 0x20          # fp16 scales of ordinary size
+    pools = ops.Context.moe_pools(dev(pool), hidden, inter, experts, 0, experts * gu, 2 * experts * gu)
+    _, ids2, wts2 = ctx.moe_layer_q4_0(pools, dev(wr), dev(x), top_k, 1)
+    ctx.sync()
+    assert ids2.cpu().numpy()[0].tolist() == ref_ids.tolist()
+    assert np.allclose(wts2.cpu().numpy()[0], ref_w, rtol=1e-6, atol=0)
+
+
 # ------------------------------------------------------------- experts ----
 
 def run_experts(ctx, pool, offs, hidden, inter, experts, x, ids, wts):
