@@ -485,8 +485,10 @@ moe_gate_up_kernel(moe_args a, const float *__restrict__ x, const int32_t *ids,
     uint32_t e;
     router_sel r{nullptr, nullptr, true};
     if constexpr (ROUTE > 0) {
-        void *rl = reinterpret_cast<void *>(bsum + 2u * pairs);
-        rl = reinterpret_cast<void *>((reinterpret_cast<uintptr_t>(rl) + 7u) & ~(uintptr_t)7u);
+        // 8-byte aligned as it stands: xs is 16-byte aligned and 2*pairs floats
+        // follow 16*(pairs+1) vectors.  (Rounding the address up through an
+        // integer would hide from the compiler that this is LDS.)
+        void *rl = bsum + 2u * pairs;
         // only the workgroup that publishes the selection needs the probabilities
         r = router_select_block<ROUTE>(scores + (uint64_t)t * a.experts, rl, a.experts, a.top_k,
                                        blockIdx.x == 0 && slot == 0);
