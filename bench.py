@@ -272,7 +272,21 @@ def main():
                     c, ring6.data_ptr(), ring6.numel(), (i % 6) * nb6 * 210, xq.data_ptr(), xs.data_ptr(),
                     xq.numel(), yn.data_ptr(), yn.numel(), cols, r6, n)),
                     nb6 * 210 + n * (cols + cols // 4 + r6 * 4), 50, 10)
-            del ring6
+            # the head as a prefill product: 512 tokens on the matrix cores
+            tokens6 = 512
+            xh6 = torch.randn(tokens6, cols, device=dev, generator=gen).to(torch.float16)
+            yg6 = torch.empty(tokens6, r6, device=dev)
+            flop6 = 2.0 * tokens6 * r6 * cols
+
+            def gemm6_extra(ms):
+                tf = flop6 / (ms * 1e-3) / 1e12
+                return {"TFLOPs": tf, "mfma_frac_of_fp16_peak": tf / MFMA_F16_PEAK_TFLOPS,
+                        "bound": "mfma"}
+            run_other("q6_k_prefill_gemm_512x32000x4096", lambda i: must(lib.lev_hip_q6_k_gemm_prefill(
+                c, ring6.data_ptr(), ring6.numel(), (i % 6) * nb6 * 210, xh6.data_ptr(), xh6.numel(),
+                yg6.data_ptr(), yg6.numel(), cols, r6, tokens6)),
+                nb6 * 210 + tokens6 * cols * 2 + tokens6 * r6 * 4, 100, 200, gemm6_extra)
+            del ring6, xh6, yg6
 
         # ------------------------------------------- RMSNorm + Q4_K N columns
         if want("q4_k", "gemm"):

@@ -205,6 +205,13 @@ int lev_hip_q4_k_gemm_prefill(lev_ctx *ctx, const void *d_w, size_t w_bytes, uin
                               const uint16_t *d_x_f16, size_t x_count, float *d_y,
                               size_t y_capacity, uint32_t in_dim, uint32_t rows,
                               uint32_t tokens);
+/* The same for Q6_K weights (q6k gemm blocked, lev-forge/src/coopmat.rs:333-425):
+ * W is dequantised to fp16 as (d*sc)*(q-32) in f32, rounded to nearest even.
+ * Weights 2-byte aligned (GGUF), x 16-byte aligned. */
+int lev_hip_q6_k_gemm_prefill(lev_ctx *ctx, const void *d_w, size_t w_bytes, uint64_t w_off,
+                              const uint16_t *d_x_f16, size_t x_count, float *d_y,
+                              size_t y_capacity, uint32_t in_dim, uint32_t rows,
+                              uint32_t tokens);
 /* act_f16 (lev-forge/src/coopmat.rs:49): f32 -> f16, round to nearest even. */
 int lev_hip_f32_to_f16(lev_ctx *ctx, const float *d_x, uint16_t *d_out, size_t n);
 

@@ -92,6 +92,7 @@ SIGNATURES = {
     "lev_hip_swiglu_quant_q8": (_int, [_vp, _vp, _vp, _sz, _vp, _vp, _vp]),
     "lev_hip_embed_q4_k": (_int, [_vp, _vp, _sz, _u64, _vp, _u32, _vp, _sz, _u32, _u32]),
     "lev_hip_q4_k_gemm_prefill": (_int, [_vp, _vp, _sz, _u64, _vp, _sz, _vp, _sz, _u32, _u32, _u32]),
+    "lev_hip_q6_k_gemm_prefill": (_int, [_vp, _vp, _sz, _u64, _vp, _sz, _vp, _sz, _u32, _u32, _u32]),
     "lev_hip_f32_to_f16": (_int, [_vp, _vp, _vp, _sz]),
     "lev_hip_rmsnorm": (_int, [_vp, _vp, _vp, _u32, _u32, _vp, _f32]),
     "lev_hip_gelu_up": (_int, [_vp, _vp, _vp, _u32]),

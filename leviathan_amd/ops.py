@@ -219,6 +219,16 @@ class Context:
                                                        y.numel(), in_dim, rows, tokens))
         return y
 
+    def q6_k_gemm_prefill(self, w, x_f16, in_dim: int, rows: int, tokens: int, y=None, w_off: int = 0):
+        _dev(w, torch.uint8, "w")
+        _dev(x_f16, torch.float16, "x")
+        if y is None:
+            y = torch.empty((max(tokens, 1), max(rows, 1)), dtype=torch.float32, device=w.device)
+        self._check(self.lib.lev_hip_q6_k_gemm_prefill(self.ctx, _ptr(w), w.numel(), w_off,
+                                                       _ptr(x_f16), x_f16.numel(), _ptr(y),
+                                                       y.numel(), in_dim, rows, tokens))
+        return y
+
     def f32_to_f16(self, x):
         _dev(x, torch.float32, "x")
         out = torch.empty(x.shape, dtype=torch.float16, device=x.device)

@@ -922,6 +922,48 @@ int levo_q4_k_gemm_f16_oracle(const uint8_t *w, size_t w_bytes, int64_t rows, in
     return LEVO_OK;
 }
 
+/* The same gate for Q6_K weights (q6k gemm blocked, lev-forge coopmat.rs:333-425:
+ * float16_t(ds * float(q - 32)) with ds = d * float(scale)): the f32 value of
+ * decodeBlock, d * sc * level evaluated left to right, rounded to f16. */
+int levo_q6_k_gemm_f16_oracle(const uint8_t *w, size_t w_bytes, int64_t rows, int64_t cols,
+                              const uint16_t *x_f16, int64_t tokens, int64_t row0,
+                              int64_t row_step, double *y_out) {
+    if (rows <= 0 || cols <= 0 || cols % 256 != 0) return LEVO_BAD_DIMENSIONS;
+    const int64_t row_bytes = cols / 256 * 210;
+    if ((uint64_t)rows * (uint64_t)row_bytes > (uint64_t)w_bytes) return LEVO_BAD_DIMENSIONS;
+    if (tokens <= 0 || row_step <= 0 || row0 < 0) return LEVO_BAD_DIMENSIONS;
+    int64_t n_rows = row0 < rows ? (rows - row0 + row_step - 1) / row_step : 0;
+    double *wr = (double *)malloc(sizeof(double) * (size_t)cols);
+    double *xr = (double *)malloc(sizeof(double) * (size_t)cols * (size_t)tokens);
+    if (!wr || !xr) {
+        free(wr);
+        free(xr);
+        return LEVO_INVALID_ARGUMENT;
+    }
+    for (int64_t i = 0; i < cols * tokens; i++) xr[i] = levo_f16_to_f64(x_f16[i]);
+    float tmp[256];
+    int st = LEVO_OK;
+    int64_t k = 0;
+    for (int64_t r = row0; r < rows && st == LEVO_OK; r += row_step, k++) {
+        for (int64_t b = 0; b < cols / 256; b++) {
+            st = levo_q6_k_decode_block(w + r * row_bytes + b * 210, tmp);
+            if (st) break;
+            for (int i = 0; i < 256; i++)
+                wr[b * 256 + i] = levo_f16_to_f64(levo_f32_to_f16_bits(tmp[i]));
+        }
+        if (st) break;
+        for (int64_t t = 0; t < tokens; t++) {
+            double acc = 0.0;
+            const double *xt = xr + t * cols;
+            for (int64_t c = 0; c < cols; c++) acc += wr[c] * xt[c];
+            y_out[t * n_rows + k] = acc;
+        }
+    }
+    free(wr);
+    free(xr);
+    return st;
+}
+
 /* ------------------------------------------------------------------ */
 /* synthetic inputs (this build's own seeded generators)               */
 /* ------------------------------------------------------------------ */

@@ -190,6 +190,11 @@ int levo_q4_k_gemm_f16_oracle(const uint8_t *w, size_t w_bytes, int64_t rows, in
                               const uint16_t *x_f16, int64_t tokens,
                               int64_t row0, int64_t row_step, double *y_out);
 
+/* Q6_K weights through the same gate (lev-forge/src/coopmat.rs:333-425). */
+int levo_q6_k_gemm_f16_oracle(const uint8_t *w, size_t w_bytes, int64_t rows, int64_t cols,
+                              const uint16_t *x_f16, int64_t tokens,
+                              int64_t row0, int64_t row_step, double *y_out);
+
 /* ---- synthetic inputs for the benchmark configurations ----
  * These are this build's own seeded generators (the reference only fixes
  * the distributions).  Normal draws use Box-Muller over SplitMix64. */

@@ -49,8 +49,7 @@ def build(force: bool = False) -> str:
 
 
 def _load():
-    if not os.path.exists(_LIB_PATH):
-        build()
+    build()   # compiles only when the library is missing or older than its sources
     return C.CDLL(_LIB_PATH)
 
 
@@ -528,6 +527,21 @@ def q4_k_gemm_f16_oracle(w, rows, cols, x_f16_bits, tokens, row0=0, row_step=13)
     y = np.empty((tokens, n_rows), dtype=np.float64)
     _check(_gemm(wp, wb.size, rows, cols, xb.ctypes.data_as(_u16p), tokens, row0, row_step,
                  y.ctypes.data_as(_f64p)))
+    return y
+
+
+_gemm6 = _sig("levo_q6_k_gemm_f16_oracle", C.c_int, _u8p, C.c_size_t, C.c_int64, C.c_int64, _u16p,
+              C.c_int64, C.c_int64, C.c_int64, _f64p)
+
+
+def q6_k_gemm_f16_oracle(w, rows, cols, x_f16_bits, tokens, row0=0, row_step=13) -> np.ndarray:
+    """As q4_k_gemm_f16_oracle for Q6_K weights.  [tokens, n_rows]."""
+    wb, wp = _u8(w)
+    xb = np.ascontiguousarray(x_f16_bits, dtype=np.uint16)
+    n_rows = len(range(row0, rows, row_step))
+    y = np.empty((tokens, n_rows), dtype=np.float64)
+    _check(_gemm6(wp, wb.size, rows, cols, xb.ctypes.data_as(_u16p), tokens, row0, row_step,
+                  y.ctypes.data_as(_f64p)))
     return y
 
 

@@ -22,7 +22,7 @@ def test_header_declares_the_expected_surface():
     names = declared_functions()
     for must in ["lev_hip_ctx_create", "lev_hip_sync", "lev_hip_buf_alloc", "lev_hip_dequant",
                  "lev_hip_q4_0_gemv", "lev_hip_q6_k_gemv", "lev_hip_q4_k_gemv_ncol",
-                 "lev_hip_q4_k_gemm_prefill", "lev_hip_moe_route_topk", "lev_hip_moe_experts_q4_0",
+                 "lev_hip_q4_k_gemm_prefill", "lev_hip_q6_k_gemm_prefill", "lev_hip_moe_route_topk", "lev_hip_moe_experts_q4_0",
                  "lev_hip_moe_layer_q4_0", "lev_hip_rmsnorm", "lev_hip_gelu_up", "lev_hip_axpy",
                  "lev_hip_argmax", "lev_hip_q4_0_matvec_reporting", "lev_hip_q6_k_matvec_reporting"]:
         assert must in names

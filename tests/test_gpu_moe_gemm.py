@@ -364,3 +364,79 @@ def test_f32_to_f16_then_gemm_matches_direct(ctx):
     ctx.sync()
     ref = O.q4_k_gemm_f16_oracle(w, rows, cols, x32.astype(np.float16).view(np.uint16), tokens, 0, 1)
     assert O.max_rel_err(y.cpu().numpy(), ref) < GEMM_TOL
+
+
+# --------------------------------------------------- Q6_K prefill GEMM ----
+
+def gemm6(ctx, w, x16, rows, cols, tokens, w_off=0):
+    y = torch.full((tokens, rows), float("nan"), device="cuda")
+    ctx.q6_k_gemm_prefill(dev(w), dev(x16), cols, rows, tokens, y=y, w_off=w_off)
+    ctx.sync()
+    return y.cpu().numpy()
+
+
+def config4_q6(rows, cols, tokens, seed):
+    w = O.synth_q6_k(seed, rows * cols // 256, 0.01)
+    x = O.normal(tokens * cols, seed + 1000).astype(np.float16).reshape(tokens, cols)
+    return w, x
+
+
+@pytest.mark.parametrize("rows,cols,tokens", [(128, 256, 128), (64, 512, 32), (200, 1024, 37), (33, 256, 1),
+                                              # either side of the 128-row x 128-token workgroup tile
+                                              (129, 256, 129), (127, 512, 127), (256, 768, 256),
+                                              (300, 4096, 150)])
+def test_q6_gemm_small_shapes_every_row(ctx, rows, cols, tokens):
+    """coopmat.rs:333-425 against the gate of lev-cli main.rs:1201-1217 (W and X
+    rounded to fp16, f64 accumulation), every row and token."""
+    w, x = config4_q6(rows, cols, tokens, seed=rows + tokens)
+    got = gemm6(ctx, w, x, rows, cols, tokens)
+    ref = O.q6_k_gemm_f16_oracle(w, rows, cols, x.view(np.uint16), tokens, 0, 1)
+    assert O.max_rel_err(got, ref) < GEMM_TOL
+
+
+def test_q6_gemm_weights_at_a_2_byte_offset(ctx):
+    """GGUF aligns Q6_K tensors to 2 bytes only (210-byte blocks)."""
+    rows, cols, tokens = 96, 512, 48
+    w, x = config4_q6(rows, cols, tokens, seed=77)
+    shifted = np.concatenate([np.zeros(2, np.uint8), w])
+    got = gemm6(ctx, shifted, x, rows, cols, tokens, w_off=2)
+    ref = O.q6_k_gemm_f16_oracle(w, rows, cols, x.view(np.uint16), tokens, 0, 1)
+    assert O.max_rel_err(got, ref) < GEMM_TOL
+
+
+def test_q6_gemm_lm_head_size_sampled_rows(ctx):
+    """The 32000 x 4096 head at 256 tokens: every 13th row (lev-cli main.rs:1266-1278,
+    gate 1e-3), and exact linearity under a power-of-two scaling of X."""
+    rows, cols, tokens = 32000, 4096, 256
+    w, x = config4_q6(rows, cols, tokens, seed=6)
+    got = gemm6(ctx, w, x, rows, cols, tokens)
+    assert np.all(np.isfinite(got))
+    ref = O.q6_k_gemm_f16_oracle(w, rows, cols, x.view(np.uint16), tokens, 0, 13)
+    assert O.max_rel_err(got[:, 0::13], ref) < GEMM_TOL
+    got2 = gemm6(ctx, w, (x * np.float16(2)), rows, cols, tokens)
+    assert np.array_equal(got2.view(np.uint32), (got * 2).view(np.uint32))
+
+
+def test_q6_gemm_one_token_matches_the_gemv_within_rounding(ctx):
+    """One token through the GEMM against the f64 GEMV oracle on the same fp16
+    activations: the only difference is the fp16 rounding of W (2^-11 relative
+    per weight)."""
+    rows, cols = 160, 2048
+    w, x = config4_q6(rows, cols, 1, seed=12)
+    got = gemm6(ctx, w, x, rows, cols, 1)[0]
+    ref = O.q6_k_matvec_f64(w, rows, cols, x[0].astype(np.float32))
+    mag = np.abs(O.q6_k_dequant(w).reshape(rows, cols).astype(np.float64)) @ np.abs(x[0].astype(np.float64))
+    assert np.all(np.abs(got - ref) <= 2.0 ** -10 * mag)
+
+
+def test_q6_gemm_rejects_bad_arguments(ctx):
+    from leviathan_amd import ops
+    w, x = config4_q6(32, 256, 4, seed=3)
+    with pytest.raises(ops.LevError):
+        ctx.q6_k_gemm_prefill(dev(w), dev(x), 255, 32, 4)            # in_dim not a multiple of 256
+    with pytest.raises(ops.LevError):
+        ctx.q6_k_gemm_prefill(dev(w), dev(x), 256, 33, 4)            # weights too short for 33 rows
+    with pytest.raises(ops.LevError):
+        ctx.q6_k_gemm_prefill(dev(w), dev(x), 256, 32, 5)            # x too short for 5 tokens
+    with pytest.raises(ops.LevError):
+        ctx.q6_k_gemm_prefill(dev(w), dev(x), 256, 32, 0)

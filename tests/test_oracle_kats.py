@@ -674,3 +674,21 @@ def test_synthetic_generators():
     assert np.all(np.isfinite(c[:, :4].copy().view(np.float16).astype(np.float64)))
     n = O.normal(200000, 9)
     assert abs(n.mean()) < 0.01 and abs(n.std() - 1.0) < 0.01
+
+
+def test_q6_k_gemm_oracle_is_fp16_rounded_decode_times_x_in_f64():
+    """The Q6_K prefill gate (lev-forge coopmat.rs:333-425 with lev-cli main.rs:1201-1217):
+    W = fp16(decodeBlock value), X fp16, f64 accumulation -- against numpy on the
+    block decode that the reference's own known answers pin, and on the -315 block
+    (main.swift:1091-1120) whose weights are exact in fp16."""
+    rows, cols, tokens = 7, 512, 5
+    w = O.synth_q6_k(21, rows * cols // 256, 0.01)
+    x = O.normal(tokens * cols, 22).astype(np.float16).reshape(tokens, cols)
+    w16 = O.q6_k_dequant(w).astype(np.float16).astype(np.float64).reshape(rows, cols)
+    want = x.astype(np.float64) @ w16.T
+    got = O.q6_k_gemm_f16_oracle(w, rows, cols, x.view(np.uint16), tokens, 0, 1)
+    assert np.array_equal(got, want) or np.allclose(got, want, rtol=1e-13, atol=0)
+    sampled = O.q6_k_gemm_f16_oracle(w, rows, cols, x.view(np.uint16), tokens, 1, 3)
+    assert np.array_equal(sampled, got[:, 1::3])
+    with pytest.raises(O.OracleError):
+        O.q6_k_gemm_f16_oracle(w[:-1], rows, cols, x.view(np.uint16), tokens, 0, 1)
