@@ -59,13 +59,25 @@ __device__ __forceinline__ void q6g_load(const uint8_t *blk, uint32_t half, uint
     u.sc[1] = c.v[1];
 }
 
-// Four codes packed in `c` -> fp16 weights out[at..at+3] (ds * (q - 32), rounded once).
-__device__ __forceinline__ void q6g_put4(uint32_t c, float ds, f16x8 &out, int at) {
-#pragma unroll
-    for (int b = 0; b < 4; ++b) {
-        const float q = (float)((int)((c >> (8 * b)) & 0xFFu) - 32);
-        out[at + b] = (_Float16)(ds * q);
-    }
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+// Four codes packed in `c` -> fp16 weights out[at..at+3]: ds * (q - 32) in f32,
+// rounded once to fp16.  The f32 product is formed as fma(q, ds, -32*ds): the
+// fused operation rounds the exact q*ds - 32*ds = (q-32)*ds once, which is the
+// rounded product itself (-32*ds is exact), and it takes the code byte as it
+// stands (byte -> float conversion, no integer subtraction).
+__device__ __forceinline__ void q6g_put4(uint32_t c, float ds, float nb, f16x8 &out, int at) {
+    f32x2 lo, hi;
+    lo.x = fmaf((float)(c & 0xFFu), ds, nb);
+    lo.y = fmaf((float)((c >> 8) & 0xFFu), ds, nb);
+    hi.x = fmaf((float)((c >> 16) & 0xFFu), ds, nb);
+    hi.y = fmaf((float)(c >> 24), ds, nb);
+    const f16x2 l16 = __builtin_convertvector(lo, f16x2), h16 = __builtin_convertvector(hi, f16x2);
+    out[at + 0] = l16.x;
+    out[at + 1] = l16.y;
+    out[at + 2] = h16.x;
+    out[at + 3] = h16.y;
 }
 
 // Decodes the unit into its two 16-weight groups: lo = elements 16v.., hi = 64+16v..
@@ -76,13 +88,14 @@ __device__ __forceinline__ void q6g_decode(const q6g_unit &u, uint32_t v, f16x8 
     const float d = lev_f16_bits_to_f32(u.d);
     const float ds_lo = d * (float)(int)__builtin_amdgcn_sbfe((int)u.sc[0], 8u * bi, 8u);
     const float ds_hi = d * (float)(int)__builtin_amdgcn_sbfe((int)u.sc[1], 8u * bi, 8u);
+    const float nb_lo = -32.0f * ds_lo, nb_hi = -32.0f * ds_hi;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const uint32_t q = u.ql[i], h = u.qh[i];
         const uint32_t cl = (q & 0x0F0F0F0Fu) | ((h << shl) & 0x30303030u);
         const uint32_t ch = ((q >> 4) & 0x0F0F0F0Fu) | ((h >> shr) & 0x30303030u);
-        q6g_put4(cl, ds_lo, lo[i >> 1], 4 * (i & 1));
-        q6g_put4(ch, ds_hi, hi[i >> 1], 4 * (i & 1));
+        q6g_put4(cl, ds_lo, nb_lo, lo[i >> 1], 4 * (i & 1));
+        q6g_put4(ch, ds_hi, nb_hi, hi[i >> 1], 4 * (i & 1));
     }
 }
 

@@ -440,3 +440,23 @@ def test_q6_gemm_rejects_bad_arguments(ctx):
         ctx.q6_k_gemm_prefill(dev(w), dev(x), 256, 32, 5)            # x too short for 5 tokens
     with pytest.raises(ops.LevError):
         ctx.q6_k_gemm_prefill(dev(w), dev(x), 256, 32, 0)
+
+
+@pytest.mark.parametrize("kind", ["q4_k", "q6_k"])
+def test_gemm_weights_are_exactly_the_fp16_rounded_decode(ctx, kind):
+    """X = identity reads the fp16 weights the kernel multiplies with back out:
+    they must be the f32 decode rounded once to fp16 (coopmat.rs:236-323, 333-425),
+    exactly, wide scale range included."""
+    rows, cols = 70, 512
+    if kind == "q4_k":
+        w = O.synth_q4_k(31, rows * cols // 256, 0.3)
+        want = O.q4_k_dequant(w)
+        run = gemm
+    else:
+        w = O.synth_q6_k(32, rows * cols // 256, 0.3)
+        want = O.q6_k_dequant(w)
+        run = gemm6
+    want16 = want.reshape(rows, cols).astype(np.float16).astype(np.float32)
+    x = np.eye(cols, dtype=np.float16)
+    got = run(ctx, w, x, rows, cols, cols)            # [cols tokens][rows]
+    assert np.array_equal(got.T, want16)              # as values: the sign of a zero weight is immaterial
