@@ -5,16 +5,17 @@
 // there, W is dequantised to fp16 -- (d*sc) * (q-32) in f32, then
 // round-to-nearest-even -- and X arrives as fp16; products accumulate in f32.
 //
-// One workgroup = 128 rows x 128 tokens, four waves in a 2 x 2 arrangement;
+// One workgroup = 128 rows x 256 tokens, eight waves in a 2 x 4 arrangement;
 // a wave owns 64 rows x 64 tokens = four 32x32 accumulator tiles
 // (v_mfma_f32_32x32x16_f16, A = X, B = W^T: lane l holds output row l%32, so
-// the stores of Y run along rows).
+// the stores of Y run along rows).  The wide token tile is what keeps the
+// decode (done once per workgroup and K-step) below the matrix-core time.
 // K advances by 128 = one half of a superblock.  Per step
-//   - W: thread (row = tid/2, two of the half's four 32-weight units) decodes
-//     64 weights straight from global memory (2-byte aligned 16-byte runs, as
+//   - W: thread (row = tid/4, one of the half's four 32-weight units) decodes
+//     32 weights straight from global memory (2-byte aligned 16-byte runs, as
 //     the GGUF layout has them) into fp16 and writes them to LDS, row-major in
 //     k with 16 bytes of padding per row;
-//   - X: 128 tokens x 256 bytes, sixteen lanes per token row, to LDS in the
+//   - X: 256 tokens x 256 bytes, sixteen lanes per token row, to LDS in the
 //     same row-major layout;
 //   - the operands of step ks+1 are requested before the MFMAs of step ks and
 //     written to LDS after them (registers in between, two barriers a step).
@@ -28,10 +29,11 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 constexpr int kTR = 128;                 // rows per workgroup
-constexpr int kTT = 128;                 // tokens per workgroup
+constexpr int kTT = 256;                 // tokens per workgroup (128 measured 6 % slower at 512 tokens)
 constexpr int kTK = 128;                 // K-step
 constexpr int kRowHalfs = kTK + 8;       // LDS row: 128 fp16 + 16 bytes of padding
-constexpr int kGThreads = 256;
+constexpr int kGThreads = 2 * kTT;       // one wave per 64 rows x 64 tokens
+constexpr int kUnits = kTR * 4 / kGThreads;               // 32-weight units decoded per thread and step
 constexpr int kXLoads = kTT * kTK * 2 / 16 / kGThreads;   // 16-byte loads of X per thread and step
 
 struct __attribute__((packed, aligned(2))) u32x4_a2 { uint32_t v[4]; };
@@ -107,12 +109,12 @@ q6_k_gemm_kernel(const uint8_t *__restrict__ w, const uint16_t *__restrict__ x, 
     _Float16 *xsh = lds + kTR * kRowHalfs;        // [kTT][kRowHalfs]
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t lr = lane & 31u, lh = lane >> 5;
-    const uint32_t wr = wave & 1u, wt = wave >> 1;
+    const uint32_t wr = wave & 1u, wt = wave >> 1;   // 2 x kTT/64 waves
     const uint32_t row0 = blockIdx.x * kTR, tok0 = blockIdx.y * kTT;
     const uint32_t bpr = in_dim / 256u, steps = in_dim / kTK;
 
-    // decode role: row tid/2, units 2*(tid&1) and 2*(tid&1)+1 of the step's half
-    const uint32_t drow = tid >> 1, dv = 2u * (tid & 1u);
+    // decode role: kUnits consecutive units of the step's half of one row
+    const uint32_t drow = tid / (4u / kUnits), dv = kUnits * (tid % (4u / kUnits));
     const uint32_t wrow = min(row0 + drow, rows - 1u);   // rows past the end repeat the last one
     const uint8_t *wrow_p = w + (uint64_t)wrow * bpr * 210u;
     // X role: 16-byte piece i = tid + 256*j of the step: token i/16, piece i%16
@@ -124,19 +126,19 @@ q6_k_gemm_kernel(const uint8_t *__restrict__ w, const uint16_t *__restrict__ x, 
         xrow_p[j] = x + (uint64_t)t * in_dim + 8u * (i & 15u);
     }
 
-    q6g_unit U[2];
+    q6g_unit U[kUnits];
     lev_u32x4 XR[kXLoads];
     auto request = [&](uint32_t ks) {
         const uint8_t *blk = wrow_p + (uint64_t)(ks >> 1) * 210u;
-        q6g_load(blk, ks & 1u, dv, U[0]);
-        q6g_load(blk, ks & 1u, dv + 1u, U[1]);
+#pragma unroll
+        for (int k = 0; k < kUnits; ++k) q6g_load(blk, ks & 1u, dv + k, U[k]);
 #pragma unroll
         for (int j = 0; j < kXLoads; ++j)
             XR[j] = *reinterpret_cast<const lev_u32x4 *>(xrow_p[j] + (uint64_t)ks * kTK);
     };
     auto park = [&]() {
 #pragma unroll
-        for (int k = 0; k < 2; ++k) {
+        for (int k = 0; k < kUnits; ++k) {
             f16x8 lo[2], hi[2];
             q6g_decode(U[k], dv + k, lo, hi);
             _Float16 *dst = wsh + drow * kRowHalfs + 16u * (dv + k);
