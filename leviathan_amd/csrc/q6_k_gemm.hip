@@ -30,11 +30,12 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 constexpr int kTR = 128;                 // rows per workgroup
 constexpr int kTT = 256;                 // tokens per workgroup (128 measured 6 % slower at 512 tokens)
-constexpr int kTK = 128;                 // K-step
-constexpr int kRowHalfs = kTK + 8;       // LDS row: 128 fp16 + 16 bytes of padding
+constexpr int kTK = 64;                  // K-step: one nibble plane of a half superblock
+constexpr int kRowHalfs = kTK + 8;       // LDS row: 64 fp16 + 16 bytes of padding
+constexpr int kBufHalfs = (kTR + kTT) * kRowHalfs;        // one buffer: W rows, then X rows
 constexpr int kGThreads = 2 * kTT;       // one wave per 64 rows x 64 tokens
-constexpr int kUnits = kTR * 4 / kGThreads;               // 32-weight units decoded per thread and step
 constexpr int kXLoads = kTT * kTK * 2 / 16 / kGThreads;   // 16-byte loads of X per thread and step
+static_assert(kGThreads == kTR * 4, "one 32-weight unit per thread and half");
 
 struct __attribute__((packed, aligned(2))) u32x4_a2 { uint32_t v[4]; };
 struct __attribute__((packed, aligned(2))) u32x2_a2 { uint32_t v[2]; };
@@ -82,22 +83,21 @@ __device__ __forceinline__ void q6g_put4(uint32_t c, float ds, float nb, f16x8 &
     out[at + 3] = h16.y;
 }
 
-// Decodes the unit into its two 16-weight groups: lo = elements 16v.., hi = 64+16v..
-__device__ __forceinline__ void q6g_decode(const q6g_unit &u, uint32_t v, f16x8 lo[2], f16x8 hi[2]) {
+// Decodes one of the unit's two 16-weight groups: HIGH = false -> elements
+// 16v.. (low nibbles), true -> 64+16v.. (high nibbles) of the half.
+template <bool HIGH>
+__device__ __forceinline__ void q6g_decode(const q6g_unit &u, uint32_t v, f16x8 out[2]) {
     const uint32_t pair = v >> 1;
-    const uint32_t shl = 4u - 2u * pair, shr = 2u * pair;
     const uint32_t bi = (v & 1u) + 2u * pair;
     const float d = lev_f16_bits_to_f32(u.d);
-    const float ds_lo = d * (float)(int)__builtin_amdgcn_sbfe((int)u.sc[0], 8u * bi, 8u);
-    const float ds_hi = d * (float)(int)__builtin_amdgcn_sbfe((int)u.sc[1], 8u * bi, 8u);
-    const float nb_lo = -32.0f * ds_lo, nb_hi = -32.0f * ds_hi;
+    const float ds = d * (float)(int)__builtin_amdgcn_sbfe((int)u.sc[HIGH ? 1 : 0], 8u * bi, 8u);
+    const float nb = -32.0f * ds;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const uint32_t q = u.ql[i], h = u.qh[i];
-        const uint32_t cl = (q & 0x0F0F0F0Fu) | ((h << shl) & 0x30303030u);
-        const uint32_t ch = ((q >> 4) & 0x0F0F0F0Fu) | ((h >> shr) & 0x30303030u);
-        q6g_put4(cl, ds_lo, nb_lo, lo[i >> 1], 4 * (i & 1));
-        q6g_put4(ch, ds_hi, nb_hi, hi[i >> 1], 4 * (i & 1));
+        const uint32_t c = HIGH ? (((q >> 4) & 0x0F0F0F0Fu) | ((h >> (2u * pair)) & 0x30303030u))
+                                : ((q & 0x0F0F0F0Fu) | ((h << (4u - 2u * pair)) & 0x30303030u));
+        q6g_put4(c, ds, nb, out[i >> 1], 4 * (i & 1));
     }
 }
 
@@ -105,53 +105,48 @@ __global__ void __launch_bounds__(kGThreads)
 q6_k_gemm_kernel(const uint8_t *__restrict__ w, const uint16_t *__restrict__ x, float *__restrict__ y,
                  uint32_t in_dim, uint32_t rows, uint32_t tokens) {
     extern __shared__ _Float16 lds[];
-    _Float16 *wsh = lds;                          // [kTR][kRowHalfs]
-    _Float16 *xsh = lds + kTR * kRowHalfs;        // [kTT][kRowHalfs]
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t lr = lane & 31u, lh = lane >> 5;
-    const uint32_t wr = wave & 1u, wt = wave >> 1;   // 2 x kTT/64 waves
+    const uint32_t wr = wave & 1u, wt = wave >> 1;   // 2 x 4 waves
     const uint32_t row0 = blockIdx.x * kTR, tok0 = blockIdx.y * kTT;
-    const uint32_t bpr = in_dim / 256u, steps = in_dim / kTK;
+    const uint32_t bpr = in_dim / 256u, halves = in_dim / 128u;
 
-    // decode role: kUnits consecutive units of the step's half of one row
-    const uint32_t drow = tid / (4u / kUnits), dv = kUnits * (tid % (4u / kUnits));
+    // decode role: unit dv of the current half of row drow
+    const uint32_t drow = tid >> 2, dv = tid & 3u;
     const uint32_t wrow = min(row0 + drow, rows - 1u);   // rows past the end repeat the last one
     const uint8_t *wrow_p = w + (uint64_t)wrow * bpr * 210u;
-    // X role: 16-byte piece i = tid + 256*j of the step: token i/16, piece i%16
+    // X role: 16-byte piece i = tid + 512*j of the step: token i/8, piece i%8
     const uint16_t *xrow_p[kXLoads];
+    uint32_t xdst[kXLoads];
 #pragma unroll
     for (int j = 0; j < kXLoads; ++j) {
         const uint32_t i = tid + (uint32_t)j * kGThreads;
-        const uint32_t t = min(tok0 + (i >> 4), tokens - 1u);
-        xrow_p[j] = x + (uint64_t)t * in_dim + 8u * (i & 15u);
+        const uint32_t t = min(tok0 + (i >> 3), tokens - 1u);
+        xrow_p[j] = x + (uint64_t)t * in_dim + 8u * (i & 7u);
+        xdst[j] = kTR * kRowHalfs + (i >> 3) * kRowHalfs + 8u * (i & 7u);
     }
+    const uint32_t wdst = drow * kRowHalfs + 16u * dv;
 
-    q6g_unit U[kUnits];
-    lev_u32x4 XR[kXLoads];
-    auto request = [&](uint32_t ks) {
-        const uint8_t *blk = wrow_p + (uint64_t)(ks >> 1) * 210u;
-#pragma unroll
-        for (int k = 0; k < kUnits; ++k) q6g_load(blk, ks & 1u, dv + k, U[k]);
+    // Two register sets per operand: what is requested now is parked two steps
+    // later, so a request has two multiply phases to arrive.
+    q6g_unit Ucur, Unext;
+    lev_u32x4 XE[kXLoads], XO[kXLoads];   // activations of even / odd K-steps
+    const uint32_t steps = 2u * halves;
+    auto request_w = [&](uint32_t half, q6g_unit &U) {
+        half = half < halves ? half : halves - 1u;   // past the end: the last half again, never used
+        q6g_load(wrow_p + (uint64_t)(half >> 1) * 210u, half & 1u, dv, U);
+    };
+    auto request_x = [&](uint32_t ks, lev_u32x4 (&XR)[kXLoads]) {
+        ks = ks < steps ? ks : steps - 1u;
 #pragma unroll
         for (int j = 0; j < kXLoads; ++j)
             XR[j] = *reinterpret_cast<const lev_u32x4 *>(xrow_p[j] + (uint64_t)ks * kTK);
     };
-    auto park = [&]() {
+    auto park = [&](_Float16 *buf, const f16x8 wv[2], const lev_u32x4 (&XR)[kXLoads]) {
+        *reinterpret_cast<f16x8 *>(buf + wdst) = wv[0];
+        *reinterpret_cast<f16x8 *>(buf + wdst + 8) = wv[1];
 #pragma unroll
-        for (int k = 0; k < kUnits; ++k) {
-            f16x8 lo[2], hi[2];
-            q6g_decode(U[k], dv + k, lo, hi);
-            _Float16 *dst = wsh + drow * kRowHalfs + 16u * (dv + k);
-            *reinterpret_cast<f16x8 *>(dst) = lo[0];
-            *reinterpret_cast<f16x8 *>(dst + 8) = lo[1];
-            *reinterpret_cast<f16x8 *>(dst + 64) = hi[0];
-            *reinterpret_cast<f16x8 *>(dst + 72) = hi[1];
-        }
-#pragma unroll
-        for (int j = 0; j < kXLoads; ++j) {
-            const uint32_t i = tid + (uint32_t)j * kGThreads;
-            *reinterpret_cast<lev_u32x4 *>(xsh + (i >> 4) * kRowHalfs + 8u * (i & 15u)) = XR[j];
-        }
+        for (int j = 0; j < kXLoads; ++j) *reinterpret_cast<lev_u32x4 *>(buf + xdst[j]) = XR[j];
     };
 
     f32x16 acc[2][2];
@@ -162,33 +157,58 @@ q6_k_gemm_kernel(const uint8_t *__restrict__ w, const uint16_t *__restrict__ x, 
 #pragma unroll
             for (int i = 0; i < 16; ++i) acc[r][m][i] = 0.f;
 
-    request(0);
-    park();
-    __syncthreads();
-    const _Float16 *a_base = xsh + (64u * wt + lr) * kRowHalfs + 8u * lh;
-    const _Float16 *b_base = wsh + (64u * wr + lr) * kRowHalfs + 8u * lh;
-    for (uint32_t ks = 0; ks < steps; ++ks) {
-        // the next step's operands are requested unconditionally (the last step
-        // asks for its own again): a branch around the loads would make the
-        // compiler wait for them at its end
-        request(ks + 1u < steps ? ks + 1u : ks);
+    const uint32_t a_off = kTR * kRowHalfs + (64u * wt + lr) * kRowHalfs + 8u * lh;
+    const uint32_t b_off = (64u * wr + lr) * kRowHalfs + 8u * lh;
+    auto multiply = [&](const _Float16 *buf) {
 #pragma unroll
         for (int kk = 0; kk < kTK / 16; ++kk) {
             f16x8 a[2], b[2];
 #pragma unroll
             for (int m = 0; m < 2; ++m)
-                a[m] = *reinterpret_cast<const f16x8 *>(a_base + m * 32 * kRowHalfs + 16 * kk);
+                a[m] = *reinterpret_cast<const f16x8 *>(buf + a_off + m * 32 * kRowHalfs + 16 * kk);
 #pragma unroll
             for (int r = 0; r < 2; ++r)
-                b[r] = *reinterpret_cast<const f16x8 *>(b_base + r * 32 * kRowHalfs + 16 * kk);
+                b[r] = *reinterpret_cast<const f16x8 *>(buf + b_off + r * 32 * kRowHalfs + 16 * kk);
 #pragma unroll
             for (int r = 0; r < 2; ++r)
 #pragma unroll
                 for (int m = 0; m < 2; ++m)
                     acc[r][m] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[m], b[r], acc[r][m], 0, 0, 0);
         }
-        __syncthreads();   // every wave is done reading this step's tiles
-        if (ks + 1u < steps) park();
+    };
+
+    _Float16 *buf0 = lds, *buf1 = lds + kBufHalfs;
+    f16x8 wv[2];
+    request_w(0, Ucur);
+    request_x(0, XE);
+    request_x(1, XO);
+    request_w(1, Unext);
+    q6g_decode<false>(Ucur, dv, wv);
+    park(buf0, wv, XE);
+    request_x(2, XE);
+    __syncthreads();
+    // Two K-steps per half: the low-nibble groups (elements 0..63 of the half)
+    // from buffer 0, then the high-nibble groups (64..127) from buffer 1.  While
+    // a buffer is multiplied the other one is filled, so one barrier a step is
+    // enough.  Requests are unconditional (a branch around the loads would make
+    // the compiler wait for them at its end) and fenced against the scheduler,
+    // which would otherwise move them next to their first use.
+    for (uint32_t hf = 0; hf < halves; ++hf) {
+        multiply(buf0);                               // step 2hf
+        q6g_decode<true>(Ucur, dv, wv);
+        park(buf1, wv, XO);                           // -> step 2hf+1
+        __builtin_amdgcn_sched_barrier(0);
+        request_x(2u * hf + 3u, XO);
+        __builtin_amdgcn_sched_barrier(0);
+        __syncthreads();
+        multiply(buf1);                               // step 2hf+1
+        q6g_decode<false>(Unext, dv, wv);
+        park(buf0, wv, XE);                           // -> step 2hf+2
+        Ucur = Unext;
+        __builtin_amdgcn_sched_barrier(0);
+        request_x(2u * hf + 4u, XE);
+        request_w(hf + 2u, Unext);
+        __builtin_amdgcn_sched_barrier(0);
         __syncthreads();
     }
 
@@ -212,7 +232,7 @@ q6_k_gemm_kernel(const uint8_t *__restrict__ w, const uint16_t *__restrict__ x, 
 hipError_t lev_q6_k_gemm_launch(lev_ctx *ctx, const uint8_t *w, const uint16_t *x, float *y,
                                 uint32_t in_dim, uint32_t rows, uint32_t tokens) {
     static bool attr_set = false;
-    const size_t lds = (size_t)(kTR + kTT) * kRowHalfs * sizeof(_Float16);
+    const size_t lds = (size_t)2 * kBufHalfs * sizeof(_Float16);
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&q6_k_gemm_kernel),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
