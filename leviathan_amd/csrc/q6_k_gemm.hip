@@ -10,15 +10,19 @@
 // (v_mfma_f32_32x32x16_f16, A = X, B = W^T: lane l holds output row l%32, so
 // the stores of Y run along rows).  The wide token tile is what keeps the
 // decode (done once per workgroup and K-step) below the matrix-core time.
-// K advances by 128 = one half of a superblock.  Per step
-//   - W: thread (row = tid/4, one of the half's four 32-weight units) decodes
-//     32 weights straight from global memory (2-byte aligned 16-byte runs, as
-//     the GGUF layout has them) into fp16 and writes them to LDS, row-major in
+// K advances by 64 = one nibble plane of half a superblock: the low nibbles of
+// a half are its elements 0..63, the high nibbles 64..127, so a thread keeps
+// its 32-weight unit (16 ql bytes, 16 qh bytes, scales, d) for two steps.  Per
+// step
+//   - W: thread (row = tid/4, unit tid%4) decodes 16 weights straight from the
+//     2-byte aligned GGUF bytes into fp16 and writes them to LDS, row-major in
 //     k with 16 bytes of padding per row;
-//   - X: 256 tokens x 256 bytes, sixteen lanes per token row, to LDS in the
-//     same row-major layout;
-//   - the operands of step ks+1 are requested before the MFMAs of step ks and
-//     written to LDS after them (registers in between, two barriers a step).
+//   - X: 256 tokens x 128 bytes, eight lanes per token row, to LDS in the same
+//     row-major layout;
+//   - two LDS buffers: while one is multiplied the other is filled, one
+//     barrier per step; operands are requested two steps before they are
+//     written to LDS (two register sets), so that a request has two multiply
+//     phases to arrive.
 // Every lane's fragment is 8 consecutive k (16 bytes) of its row, for both
 // operands, so the natural k order is kept.
 #include "lev_common.hpp"
