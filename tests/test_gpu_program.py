@@ -113,7 +113,7 @@ def test_recorded_step_replays_bit_exact():
 
 
 def test_recorded_prefill_like_sequence_replays_bit_exact():
-    """f32 -> f16, prefill GEMM (first use of the kernel happens while recording),
+    """f32 -> f16, the two prefill GEMMs (first use of the kernels happens while recording),
     grouped MoE over 24 tokens, and a Q4_0 GEMV under a forge selection made before
     recording: three replays with changed inputs equal the eager results bit for bit."""
     from leviathan_amd import capi, ops
@@ -128,6 +128,7 @@ def test_recorded_prefill_like_sequence_replays_bit_exact():
     T, K, R = 24, 512, 200
     hidden, inter, experts, top_k = 512, 256, 12, 3
     wk = dev(O.synth_q4_k(11, R * K // 256))
+    w6 = dev(O.synth_q6_k(17, R * K // 256))
     w0 = dev(O.synth_q4_0(12, 300 * 2048 // 32))
     gu_bytes, dn_bytes = inter * (hidden // 32) * 18, hidden * (inter // 32) * 18
     pool = dev(np.concatenate([O.synth_q4_0(13, experts * gu_bytes // 18), O.synth_q4_0(14, experts * gu_bytes // 18),
@@ -138,6 +139,7 @@ def test_recorded_prefill_like_sequence_replays_bit_exact():
         x32 = torch.empty(T, K, device="cuda")
         x16 = torch.empty(T, K, dtype=torch.float16, device="cuda")
         yg = torch.empty(T, R, device="cuda")
+        yg6 = torch.empty(T, R, device="cuda")
         ymoe = torch.empty(T, hidden, device="cuda")
         ids = torch.empty(T, top_k, dtype=torch.int32, device="cuda")
         wts = torch.empty(T, top_k, device="cuda")
@@ -152,12 +154,13 @@ def test_recorded_prefill_like_sequence_replays_bit_exact():
     def step():
         must(lib.lev_hip_f32_to_f16(c, p(x32), p(x16), T * K))
         must(lib.lev_hip_q4_k_gemm_prefill(c, p(wk), wk.numel(), 0, p(x16), x16.numel(), p(yg), yg.numel(), K, R, T))
+        must(lib.lev_hip_q6_k_gemm_prefill(c, p(w6), w6.numel(), 0, p(x16), x16.numel(), p(yg6), yg6.numel(), K, R, T))
         must(lib.lev_hip_moe_layer_q4_0(c, C.byref(pools), p(router), None, p(x32), p(ymoe), p(ids), p(wts), top_k, T))
         must(lib.lev_hip_q4_0_gemv(c, p(w0), w0.numel(), 0, p(xv), 2048, p(yv), 300, 2048, 300))
 
     def snapshot():
         ctx.sync()
-        return [t.clone() for t in (x16, yg, ymoe, ids, wts, yv)]
+        return [t.clone() for t in (x16, yg, yg6, ymoe, ids, wts, yv)]
 
     # the MoE scratch is sized by an eager MoE call (it may not grow while recording);
     # the GEMM has NOT run yet: its first launch is the recorded one
@@ -180,6 +183,8 @@ def test_recorded_prefill_like_sequence_replays_bit_exact():
     # and the results are right, not merely repeatable
     ref = O.q4_k_gemm_f16_oracle(wk.cpu().numpy(), R, K, x16.cpu().numpy().view(np.uint16), T, 0, 1)
     assert O.max_rel_err(yg.cpu().numpy(), ref) < 1e-3
+    ref6 = O.q6_k_gemm_f16_oracle(w6.cpu().numpy(), R, K, x16.cpu().numpy().view(np.uint16), T, 0, 1)
+    assert O.max_rel_err(yg6.cpu().numpy(), ref6) < 1e-3
     assert O.max_rel_err(yv.cpu().numpy(), O.q4_0_matvec_f64(w0.cpu().numpy(), 300, 2048, xv.cpu().numpy())) < 1e-4
     ctx.forge_clear(capi.OP_Q4_0_GEMV, 2048, 300)
     prog.destroy()
