@@ -143,6 +143,58 @@ def test_router_selection_order_edge_cases(ctx, case, experts):
     assert np.allclose(wts2.cpu().numpy()[0], ref_w, rtol=1e-6, atol=0)
 
 
+@pytest.mark.parametrize("experts,top_k", [(8, 3), (64, 8), (128, 8), (200, 16), (256, 5), (1000, 32)])
+def test_router_selection_matches_the_oracle_on_adversarial_scores(ctx, experts, top_k):
+    """256 score vectors per expert count, built to sit on the edges of the
+    selection's two orderings: few distinct values (ties), neighbours one ulp
+    apart, magnitudes from 1e-30 to 1e3, gaps below 1e-6 and beyond 690.  One-hot
+    activations make the scores exactly the chosen values; ids must match the
+    reference's order bit for bit."""
+    cases = 256
+    rng = np.random.default_rng(1000 + experts)
+    scores = np.empty((cases, experts), np.float32)
+    for t in range(cases):
+        kind = t % 8
+        if kind == 0:      # few distinct values: many exact ties
+            scores[t] = rng.choice(np.array([-2.5, 0.0, 0.75, 3.0], np.float32), experts)
+        elif kind == 1:    # one-ulp neighbours of one value
+            base = np.float32(rng.uniform(-4, 4))
+            scores[t] = base
+            up = rng.random(experts) < 0.3
+            scores[t][up] = np.nextafter(base, np.float32(np.inf))
+            scores[t][rng.random(experts) < 0.2] = np.nextafter(base, np.float32(-np.inf))
+        elif kind == 2:    # tiny magnitudes: exp saturates at 1 for every score.  (Differences
+            # between 1e-19 and 1e-9 are left out on purpose: there the last bit of exp()
+            # decides which probabilities tie, and neither this build's nor the reference's
+            # libm promises that bit.)
+            scores[t] = (rng.standard_normal(experts) * 10.0 ** rng.integers(-30, -20)).astype(np.float32)
+        elif kind == 3:    # huge spread: exp underflows
+            scores[t] = (-rng.random(experts) * 1500.0).astype(np.float32)
+        elif kind == 4:    # ordinary router scores
+            scores[t] = (rng.standard_normal(experts) * 2.0).astype(np.float32)
+        elif kind == 5:    # ordinary, a handful within 1e-6 of the maximum
+            scores[t] = (rng.standard_normal(experts) * 2.0).astype(np.float32)
+            m = scores[t].max()
+            near = rng.choice(experts, min(4, experts), replace=False)
+            scores[t][near] = m - np.float32(1e-7) * rng.integers(0, 8, near.size).astype(np.float32)
+        elif kind == 6:    # gaps right at the edges of the fast ordering
+            scores[t] = rng.choice(np.array([0.0, -1e-6, -9.5e-7, -1.05e-6, -690.0, -689.9, -690.1, -5.0],
+                                            np.float32), experts)
+        else:              # all equal
+            scores[t] = np.float32(rng.uniform(-3, 3))
+    hidden = cases
+    wr = np.ascontiguousarray(scores.T)                 # [experts, hidden]: score[t][e] = wr[e][t]
+    x = np.eye(cases, dtype=np.float32)
+    ids, wts, got = ctx.moe_route_topk(dev(wr), dev(x), hidden, experts, top_k, cases, want_scores=True)
+    ctx.sync()
+    assert np.array_equal(got.cpu().numpy(), scores)
+    ids, wts = ids.cpu().numpy(), wts.cpu().numpy()
+    for t in range(cases):
+        ref_ids, ref_w = O.router_topk(scores[t], top_k)
+        assert ids[t].tolist() == ref_ids.tolist(), (t, t % 8)
+        assert np.allclose(wts[t], ref_w, rtol=2e-6, atol=0), (t, t % 8)
+
+
 # ------------------------------------------------------------- experts ----
 
 def run_experts(ctx, pool, offs, hidden, inter, experts, x, ids, wts):
