@@ -121,6 +121,18 @@ def test_prefill_gemm_random(ctx, rows, cols):
     assert O.max_rel_err(y.cpu().numpy(), ref) < GEMM_TOL, tokens
 
 
+@pytest.mark.parametrize("rows,cols", shapes(107, 10, 256, 330, 8))
+def test_q6_k_prefill_gemm_random(ctx, rows, cols):
+    tokens = int(np.random.default_rng(rows + cols + 1).integers(1, 600))
+    w = O.synth_q6_k(rows + tokens, rows * cols // 256, 0.01)
+    x = O.normal(tokens * cols, rows + 1000).astype(np.float16).reshape(tokens, cols)
+    y = torch.full((tokens, rows), float("nan"), device="cuda")
+    ctx.q6_k_gemm_prefill(dev(w), dev(x), cols, rows, tokens, y=y)
+    ctx.sync()
+    ref = O.q6_k_gemm_f16_oracle(w, rows, cols, x.view(np.uint16), tokens, 0, 1)
+    assert O.max_rel_err(y.cpu().numpy(), ref) < GEMM_TOL, tokens
+
+
 def moe_cases(seed, count):
     rng = np.random.default_rng(seed)
     out = []
