@@ -279,6 +279,26 @@ int lev_hip_moe_layer_q4_0(lev_ctx *ctx, const lev_moe_experts *pools, const flo
                            const float *d_expert_scale, const float *d_x, float *d_y,
                            int32_t *d_ids, float *d_weights, uint32_t top_k, uint32_t tokens);
 
+/* The same block for callers that cannot allocate device memory: code that is
+ * being captured into a HIP graph, tight serving loops, harnesses that forbid
+ * hipMalloc.  NO COUNTERPART IN THE REFERENCE (its MoE scratch is sized once by
+ * the engine, Gemma4.swift:2025-2059); it exists for those callers only.
+ * Arguments and results are those of lev_hip_moe_layer_q4_0, bit for bit; the
+ * router scores and the expert activations live in a static device array of
+ * LEV_NOALLOC_MOE_SCRATCH_BYTES that every GPU holds until the process ends,
+ * and the call itself allocates nothing.  Limits: tokens <=
+ * LEV_NOALLOC_MOE_MAX_TOKENS and 256-byte-rounded
+ * tokens*experts*4 + tokens*top_k*inter*4 <= LEV_NOALLOC_MOE_SCRATCH_BYTES,
+ * otherwise LEV_ERR_EXCEEDS_WORKING_SET and nothing is launched.  All calls on
+ * one GPU share the one array: calls that overlap in time on the same GPU
+ * (from two contexts or streams) race. */
+#define LEV_NOALLOC_MOE_SCRATCH_BYTES (1u << 20)
+#define LEV_NOALLOC_MOE_MAX_TOKENS 4u
+int lev_hip_moe_layer_q4_0_noalloc(lev_ctx *ctx, const lev_moe_experts *pools,
+                                   const float *d_router_w, const float *d_expert_scale,
+                                   const float *d_x, float *d_y, int32_t *d_ids, float *d_weights,
+                                   uint32_t top_k, uint32_t tokens);
+
 /* ---- host-array convenience twins of the standalone backends ----
  * Q4MetalBackend.matvecReporting (Q4.swift:165-269) and
  * Q6MetalBackend.matvecReporting (Q6.swift:199-285): validate, upload,

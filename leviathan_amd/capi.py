@@ -103,6 +103,8 @@ SIGNATURES = {
                                         _u32]),
     "lev_hip_moe_layer_q4_0": (_int, [_vp, C.POINTER(MoEExperts), _vp, _vp, _vp, _vp, _vp, _vp,
                                       _u32, _u32]),
+    "lev_hip_moe_layer_q4_0_noalloc": (_int, [_vp, C.POINTER(MoEExperts), _vp, _vp, _vp, _vp, _vp, _vp,
+                                              _u32, _u32]),
     "lev_hip_forge_candidates": (_int, [_vp, _u32, _u32, _u32, _u32, C.POINTER(Schedule), _u32,
                                         C.POINTER(_u32)]),
     "lev_hip_forge_select": (_int, [_vp, _u32, _u32, _u32, C.POINTER(Schedule)]),

@@ -127,6 +127,10 @@ extern "C" int lev_hip_ctx_create(int device, void *stream, lev_ctx **out) {
         return LEV_ERR_DEVICE_UNAVAILABLE;
     }
     *ctx->h_flag = 0;
+    if (lev_moe_static_scratch_init(ctx) != LEV_OK) {
+        lev_hip_ctx_destroy(ctx);
+        return LEV_ERR_KERNEL_LOAD_FAILED;
+    }
     *out = ctx;
     return LEV_OK;
 }

@@ -42,7 +42,13 @@ struct lev_ctx {
         lev_schedule schedule;
     };
     std::vector<selection> selections;
+    // Device address, on this context's GPU, of the static scratch array of
+    // lev_hip_moe_layer_q4_0_noalloc (looked up once at context creation).
+    void *moe_static_scratch = nullptr;
 };
+
+// Looks the static MoE scratch array up on the current device (moe.hip).
+int lev_moe_static_scratch_init(lev_ctx *ctx);
 
 // The schedule installed for this op and shape, or nullptr.
 const lev_schedule *lev_selected(const lev_ctx *ctx, uint32_t op, uint32_t in_dim, uint32_t rows, uint32_t ncol);

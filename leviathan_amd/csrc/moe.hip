@@ -1001,22 +1001,42 @@ extern "C" int lev_hip_moe_experts_q4_0(lev_ctx *ctx, const lev_moe_experts *poo
                          "moe experts launch");
 }
 
-extern "C" int lev_hip_moe_layer_q4_0(lev_ctx *ctx, const lev_moe_experts *pools,
-                                      const float *d_router_w, const float *d_expert_scale,
-                                      const float *d_x, float *d_y, int32_t *d_ids, float *d_weights,
-                                      uint32_t top_k, uint32_t tokens) {
-    LEV_REQUIRE_CTX(ctx);
+namespace {
+
+// Whole MoE block.  `fixed` == nullptr: the scratch comes from the context
+// (allocated or grown on demand).  Otherwise the caller supplies `fixed_bytes`
+// of device memory and nothing is allocated: shapes that need more, or the
+// many-token grouped path (which sizes a work area from the routing), are
+// refused.
+int moe_layer_impl(lev_ctx *ctx, const lev_moe_experts *pools, const float *d_router_w,
+                   const float *d_expert_scale, const float *d_x, float *d_y, int32_t *d_ids,
+                   float *d_weights, uint32_t top_k, uint32_t tokens, void *fixed, size_t fixed_bytes) {
     if (!d_router_w || !d_x || !d_y || !d_ids || !d_weights)
         return lev_fail(ctx, LEV_ERR_INVALID_ARGUMENT, "moe_layer: null pointer");
     moe_args a;
     int st = check_pools(ctx, pools, top_k, tokens, &a);
     if (st != LEV_OK) return st;
     if (a.experts > 4096u) return lev_fail(ctx, LEV_ERR_BAD_DIMENSIONS, "moe_layer: %u experts", a.experts);
-    const bool grouped = use_grouped(ctx, a, d_x, tokens);
+    const bool grouped = !fixed && use_grouped(ctx, a, d_x, tokens);
     moe_scratch s;
-    st = get_scratch(ctx, tokens, a.experts, top_k, a.inter, &s,
-                     grouped ? lev_moe_grouped_scratch_bytes(grouped_args(a, tokens)) : 0);
-    if (st != LEV_OK) return st;
+    if (fixed) {
+        if (tokens > LEV_NOALLOC_MOE_MAX_TOKENS)
+            return lev_fail(ctx, LEV_ERR_EXCEEDS_WORKING_SET,
+                            "moe_layer_noalloc: %u tokens, at most %u", tokens, LEV_NOALLOC_MOE_MAX_TOKENS);
+        const size_t s_bytes = ((size_t)tokens * a.experts * 4 + 255) & ~(size_t)255;
+        const size_t a_bytes = ((size_t)tokens * top_k * a.inter * 4 + 255) & ~(size_t)255;
+        if (s_bytes + a_bytes > fixed_bytes)
+            return lev_fail(ctx, LEV_ERR_EXCEEDS_WORKING_SET,
+                            "moe_layer_noalloc: needs %zu bytes of scratch, the static buffer holds %zu",
+                            s_bytes + a_bytes, fixed_bytes);
+        s.scores = static_cast<float *>(fixed);
+        s.act = reinterpret_cast<float *>(static_cast<char *>(fixed) + s_bytes);
+        s.grouped = nullptr;
+    } else {
+        st = get_scratch(ctx, tokens, a.experts, top_k, a.inter, &s,
+                         grouped ? lev_moe_grouped_scratch_bytes(grouped_args(a, tokens)) : 0);
+        if (st != LEV_OK) return st;
+    }
     st = lev_hip_check(ctx, run_scores(ctx, d_router_w, d_x, s.scores, a.hidden, a.experts, tokens),
                        "moe router scores launch");
     if (st != LEV_OK) return st;
@@ -1039,4 +1059,52 @@ extern "C" int lev_hip_moe_layer_q4_0(lev_ctx *ctx, const lev_moe_experts *pools
                              "moe grouped experts launch");
     return lev_hip_check(ctx, run_experts(ctx, a, d_x, rt, d_ids, d_weights, d_y, s.act, tokens, fast),
                          "moe experts launch");
+}
+
+}  // namespace
+
+extern "C" int lev_hip_moe_layer_q4_0(lev_ctx *ctx, const lev_moe_experts *pools,
+                                      const float *d_router_w, const float *d_expert_scale,
+                                      const float *d_x, float *d_y, int32_t *d_ids, float *d_weights,
+                                      uint32_t top_k, uint32_t tokens) {
+    LEV_REQUIRE_CTX(ctx);
+    return moe_layer_impl(ctx, pools, d_router_w, d_expert_scale, d_x, d_y, d_ids, d_weights, top_k,
+                          tokens, nullptr, 0);
+}
+
+// ---------------------------------------------------------------------------
+// The same block for callers that cannot allocate (code under HIP graph
+// capture, serving loops, harnesses that forbid hipMalloc): the router scores
+// and the expert activations live in a file-scope device array instead of the
+// context's grow-on-demand buffer.  Every GPU holds its own copy of the array
+// until the process ends; every call on a GPU uses that one copy, so calls
+// that overlap on one GPU (two contexts, two streams) race.  Both regions are
+// written in full before they are read, so nothing has to start at zero.
+// ---------------------------------------------------------------------------
+
+static __device__ __align__(256) unsigned char lev_moe_static_scratch_array[LEV_NOALLOC_MOE_SCRATCH_BYTES];
+
+// Set-up: called by lev_hip_ctx_create with the context's device current.  The
+// array's name is only a host-side handle; its device address differs per GPU
+// and comes from the runtime.
+int lev_moe_static_scratch_init(lev_ctx *ctx) {
+    void *p = nullptr;
+    hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(lev_moe_static_scratch_array));
+    if (e != hipSuccess || !p) {
+        ctx->moe_static_scratch = nullptr;
+        return lev_hip_check(ctx, e != hipSuccess ? e : hipErrorInvalidSymbol, "hipGetSymbolAddress(static MoE scratch)");
+    }
+    ctx->moe_static_scratch = p;
+    return LEV_OK;
+}
+
+extern "C" int lev_hip_moe_layer_q4_0_noalloc(lev_ctx *ctx, const lev_moe_experts *pools,
+                                              const float *d_router_w, const float *d_expert_scale,
+                                              const float *d_x, float *d_y, int32_t *d_ids,
+                                              float *d_weights, uint32_t top_k, uint32_t tokens) {
+    LEV_REQUIRE_CTX(ctx);
+    if (!ctx->moe_static_scratch)
+        return lev_fail(ctx, LEV_ERR_DEVICE_UNAVAILABLE, "moe_layer_noalloc: the static scratch has no device address");
+    return moe_layer_impl(ctx, pools, d_router_w, d_expert_scale, d_x, d_y, d_ids, d_weights, top_k,
+                          tokens, ctx->moe_static_scratch, LEV_NOALLOC_MOE_SCRATCH_BYTES);
 }

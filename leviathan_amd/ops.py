@@ -302,7 +302,10 @@ class Context:
         return (y, act) if want_act else y
 
     def moe_layer_q4_0(self, pools, router_w, x, top_k: int, tokens: int, expert_scale=None, y=None,
-                       ids=None, weights=None):
+                       ids=None, weights=None, noalloc: bool = False):
+        """``noalloc``: the entry point that allocates nothing inside the call (static
+        device scratch; pass ``y``, ``ids`` and ``weights`` so that this wrapper
+        allocates nothing either)."""
         _dev(x, torch.float32, "x")
         if y is None:
             y = torch.empty((max(tokens, 1), pools.hidden), dtype=torch.float32, device=x.device)
@@ -311,9 +314,9 @@ class Context:
         if weights is None:
             weights = torch.empty((max(tokens, 1), max(top_k, 1)), dtype=torch.float32,
                                   device=x.device)
-        self._check(self.lib.lev_hip_moe_layer_q4_0(self.ctx, C.byref(pools), _ptr(router_w),
-                                                    _ptr(expert_scale), _ptr(x), _ptr(y), _ptr(ids),
-                                                    _ptr(weights), top_k, tokens))
+        fn = self.lib.lev_hip_moe_layer_q4_0_noalloc if noalloc else self.lib.lev_hip_moe_layer_q4_0
+        self._check(fn(self.ctx, C.byref(pools), _ptr(router_w), _ptr(expert_scale), _ptr(x), _ptr(y),
+                       _ptr(ids), _ptr(weights), top_k, tokens))
         return y, ids, weights
 
 
