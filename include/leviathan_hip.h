@@ -103,9 +103,14 @@ int lev_hip_device_name(lev_ctx *ctx, char *out, size_t cap);
  * Gemma4.swift:2313-2376) ----
  * Between begin and end every operator call on the context is recorded
  * instead of executed; run() replays the whole sequence with one submission.
- * The context must own its stream or sit on a non-default stream.  Scratch
- * is never grown while recording: run each MoE shape once before recording
- * it.  Pointers and sizes are frozen into the program. */
+ * The context must own its stream or sit on a non-default stream.  Pointers
+ * and sizes are frozen into the program, the context's scratch address
+ * included.  Scratch is never grown while recording (run each MoE shape once
+ * before recording it; a call that would have to grow it fails with
+ * LEV_ERR_EXCEEDS_WORKING_SET and records nothing).  An eager call after
+ * recording may still grow the scratch: the buffer a live program was recorded
+ * with then stays allocated until the last program of the context is
+ * destroyed, so replaying stays valid. */
 typedef struct lev_program lev_program;
 int lev_hip_program_begin(lev_ctx *ctx);
 int lev_hip_program_end(lev_ctx *ctx, lev_program **out);

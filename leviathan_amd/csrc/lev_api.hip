@@ -32,8 +32,13 @@ void *lev_scratch(lev_ctx *ctx, size_t bytes) {
     // Growing replaces the buffer; earlier kernels on the stream may still be
     // using the old one, so drain the stream first.
     if (ctx->scratch) {
-        if (hipStreamSynchronize(ctx->stream) != hipSuccess) return nullptr;
-        (void)hipFree(ctx->scratch);
+        if (ctx->live_programs > 0) {
+            // a recorded program may hold this address: keep the memory alive
+            ctx->retired_scratch.push_back(ctx->scratch);
+        } else {
+            if (hipStreamSynchronize(ctx->stream) != hipSuccess) return nullptr;
+            (void)hipFree(ctx->scratch);
+        }
         ctx->scratch = nullptr;
         ctx->scratch_bytes = 0;
     }
@@ -119,7 +124,8 @@ extern "C" int lev_hip_ctx_create(int device, void *stream, lev_ctx **out) {
         }
         ctx->owns_stream = true;
     }
-    if (hipMalloc(reinterpret_cast<void **>(&ctx->d_flag), sizeof(int)) != hipSuccess ||
+    if (hipMalloc(&ctx->argmax_partials, (size_t)lev_ctx::kArgmaxPartials * 16u) != hipSuccess ||
+        hipMalloc(reinterpret_cast<void **>(&ctx->d_flag), sizeof(int)) != hipSuccess ||
         hipHostMalloc(reinterpret_cast<void **>(&ctx->h_flag), sizeof(int), hipHostMallocDefault) !=
             hipSuccess ||
         hipMemset(ctx->d_flag, 0, sizeof(int)) != hipSuccess) {
@@ -140,6 +146,8 @@ extern "C" int lev_hip_ctx_destroy(lev_ctx *ctx) {
     (void)hipSetDevice(ctx->device);
     if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
     if (ctx->scratch) (void)hipFree(ctx->scratch);
+    for (void *p : ctx->retired_scratch) (void)hipFree(p);
+    if (ctx->argmax_partials) (void)hipFree(ctx->argmax_partials);
     if (ctx->d_flag) (void)hipFree(ctx->d_flag);
     if (ctx->h_flag) (void)hipHostFree(ctx->h_flag);
     if (ctx->owns_stream && ctx->stream) (void)hipStreamDestroy(ctx->stream);
@@ -433,6 +441,7 @@ extern "C" int lev_hip_program_end(lev_ctx *ctx, lev_program **out) {
         delete p;
         return lev_hip_check(ctx, e, "hipGraphInstantiate");
     }
+    ++ctx->live_programs;
     *out = p;
     return LEV_OK;
 }
@@ -451,6 +460,11 @@ extern "C" int lev_hip_program_destroy(lev_ctx *ctx, lev_program *program) {
     if (program->exec) (void)hipGraphExecDestroy(program->exec);
     if (program->graph) (void)hipGraphDestroy(program->graph);
     delete program;
+    if (ctx->live_programs > 0 && --ctx->live_programs == 0) {
+        // no program is left that could hold a parked scratch address
+        for (void *p : ctx->retired_scratch) (void)hipFree(p);
+        ctx->retired_scratch.clear();
+    }
     return LEV_OK;
 }
 

@@ -28,8 +28,19 @@ struct lev_ctx {
     // it, Gemma4.swift:2025-2059).  Grown on demand, never shrunk.
     void *scratch = nullptr;
     size_t scratch_bytes = 0;
+    // Recorded programs keep the scratch address they were recorded with.  While
+    // any program is alive a buffer that has to make room for a larger one is
+    // parked here instead of freed, so replaying the program stays valid; the
+    // parked buffers go when the last program or the context is destroyed.
+    int live_programs = 0;
+    std::vector<void *> retired_scratch;
     // Device-side error flag written by kernels that validate device-resident
     // arguments (expert ids); read back by lev_hip_sync.
+    // Per-workgroup (best, second, index) partials of the greedy-token epilogue
+    // of the Q6_K GEMV: fixed size, allocated with the context and never moved,
+    // so a recorded GEMV needs no grow-on-demand scratch.
+    void *argmax_partials = nullptr;
+    static constexpr uint32_t kArgmaxPartials = 4096;   // entries of 16 bytes
     int *d_flag = nullptr;
     int *h_flag = nullptr;   // pinned
     // True between lev_hip_program_begin and lev_hip_program_end: the stream

@@ -419,8 +419,9 @@ hipError_t launch_units(lev_ctx *ctx, const uint8_t *w, const float *x, float *y
     if (blocks > cap) blocks = cap;
     lev_f32x4 *partials = nullptr;
     if (d_argmax || d_margin) {
-        partials = static_cast<lev_f32x4 *>(lev_scratch(ctx, (size_t)blocks * sizeof(lev_f32x4)));
-        if (!partials) return hipErrorOutOfMemory;
+        // one partial per workgroup, in the context's fixed buffer
+        if (blocks > lev_ctx::kArgmaxPartials) blocks = lev_ctx::kArgmaxPartials;
+        partials = static_cast<lev_f32x4 *>(ctx->argmax_partials);
     }
     hipLaunchKernelGGL((q6_k_gemv_units<L, P, S>), dim3(blocks), dim3(kThreads), lds, ctx->stream, w, x,
                        y, units, rows, partials);

@@ -189,3 +189,81 @@ def test_recorded_prefill_like_sequence_replays_bit_exact():
     ctx.forge_clear(capi.OP_Q4_0_GEMV, 2048, 300)
     prog.destroy()
     ctx.close()
+
+
+def test_scratch_growth_after_recording_keeps_the_program_valid():
+    """A recorded single-token MoE program holds the context's scratch address.  A
+    later eager call that needs more scratch (700 tokens, grouped path: several MiB against the first MiB) must not
+    free that buffer under the program: the replay still gives the eager bits.  And a
+    shape that would have to grow the scratch WHILE recording is refused, recording
+    nothing for it."""
+    from leviathan_amd import capi, ops
+    from tests import helpers as H
+    stream = torch.cuda.Stream()
+    ctx = ops.Context(0, stream=stream)
+    hidden, inter, experts, top_k = 512, 256, 16, 4
+    wr, pool, offs, x = H.config5(hidden, inter, experts, 700, seed=31)
+    pools = ops.Context.moe_pools(dev(pool), hidden, inter, experts, offs["gate_off"], offs["up_off"], offs["down_off"])
+    wr_d = dev(wr)
+    with torch.cuda.stream(stream):
+        x1, y1 = dev(x[:1]), torch.empty(1, hidden, device="cuda")
+        ids1 = torch.empty(1, top_k, dtype=torch.int32, device="cuda")
+        w1 = torch.empty(1, top_k, device="cuda")
+        xb = dev(x)
+        yB, idsB = torch.empty(700, hidden, device="cuda"), torch.empty(700, top_k, dtype=torch.int32, device="cuda")
+        wB = torch.empty(700, top_k, device="cuda")
+    ctx.moe_layer_q4_0(pools, wr_d, x1, top_k, 1, y=y1, ids=ids1, weights=w1)      # sizes the scratch for one token
+    ctx.sync()
+    want = y1.clone()
+    ctx.program_begin()
+    ctx.moe_layer_q4_0(pools, wr_d, x1, top_k, 1, y=y1, ids=ids1, weights=w1)
+    # 700 tokens need far more scratch than one: refused while recording
+    with pytest.raises(ops.LevError) as e:
+        ctx.moe_layer_q4_0(pools, wr_d, xb, top_k, 700, y=yB, ids=idsB, weights=wB)   # nothing allocated here
+    assert e.value.status == capi.EXCEEDS_WORKING_SET
+    prog = ctx.program_end()
+    # eager call that grows the scratch while the program is alive
+    yb, _, _ = ctx.moe_layer_q4_0(pools, wr_d, xb, top_k, 700)
+    ctx.sync()
+    for _ in range(3):
+        with torch.cuda.stream(stream):
+            y1.fill_(float("nan"))
+        prog.run()
+        ctx.sync()
+        assert torch.equal(y1, want)
+        yb2, _, _ = ctx.moe_layer_q4_0(pools, wr_d, xb, top_k, 700)               # eager work on the new scratch in between
+        ctx.sync()
+        assert torch.equal(yb2, yb)
+    prog.destroy()
+    ctx.close()
+
+
+def test_q6_k_argmax_records_on_a_fresh_context():
+    """The greedy-token epilogue needs no grow-on-demand scratch: a GEMV with argmax can be
+    recorded on a context that never ran anything eagerly."""
+    from leviathan_amd import ops
+    stream = torch.cuda.Stream()
+    ctx = ops.Context(0, stream=stream)
+    rows, cols = 640, 1024
+    w = O.synth_q6_k(21, rows * cols // 256)
+    xv = O.normal(cols, 22)
+    with torch.cuda.stream(stream):
+        w_d, x_d = dev(w), dev(xv)
+        y = torch.empty(rows, device="cuda")
+        idx = torch.zeros(1, dtype=torch.int32, device="cuda")
+        mg = torch.zeros(1, device="cuda")
+    lib, c = ctx.lib, ctx.ctx
+    ctx.program_begin()
+    st = lib.lev_hip_q6_k_gemv(c, p(w_d), w_d.numel(), 0, p(x_d), cols, p(y), rows, cols, rows, p(idx), p(mg))
+    prog = ctx.program_end()
+    assert st == 0, lib.lev_hip_last_error(c).decode()
+    for _ in range(2):
+        prog.run()
+        ctx.sync()
+        got = y.cpu().numpy()
+        assert O.max_rel_err(got, O.q6_k_matvec_f64(w, rows, cols, xv)) < 1e-4
+        assert int(idx.item()) == O.argmax(got)
+        top = np.sort(got)[::-1]
+        assert abs(float(mg.item()) - float(top[0] - top[1])) <= 1e-6 * max(1.0, abs(float(top[0])))
+    prog.destroy()
+    ctx.close()
