@@ -141,9 +141,39 @@ __device__ __forceinline__ float lev_group_sum(float v) {
     return v;
 }
 
+// The same in f64 (two DPP moves and one add per step).  For L <= 16 every lane
+// of a group ends with the group's sum; for L = 32 / 64 read the highest lane.
+template <int CTRL, int ROW_MASK = 0xF, bool BOUND = true>
+__device__ __forceinline__ double lev_dpp_add_f64(double v) {
+    const int lo = __builtin_amdgcn_update_dpp(0, __double2loint(v), CTRL, ROW_MASK, 0xF, BOUND);
+    const int hi = __builtin_amdgcn_update_dpp(0, __double2hiint(v), CTRL, ROW_MASK, 0xF, BOUND);
+    return v + __hiloint2double(hi, lo);
+}
+
+template <int L>
+__device__ __forceinline__ double lev_group_sum_f64(double v) {
+    if (L >= 2) v = lev_dpp_add_f64<0xB1>(v);
+    if (L >= 4) v = lev_dpp_add_f64<0x4E>(v);
+    if (L >= 8) v = lev_dpp_add_f64<0x141>(v);
+    if (L >= 16) v = lev_dpp_add_f64<0x140>(v);
+    if (L >= 32) v = lev_dpp_add_f64<0x142, 0xA, false>(v);
+    if (L >= 64) v = lev_dpp_add_f64<0x143, 0xC, false>(v);
+    return v;
+}
+
 __device__ __forceinline__ float lev_wave_sum_broadcast(float v) {
     v = lev_group_sum<64>(v);
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+
+// Workgroup barrier that orders LDS traffic only: it waits for this wave's LDS
+// operations and leaves its global loads in flight.  __syncthreads() carries a
+// workgroup fence for which the compiler drains every outstanding load first,
+// i.e. the prefetch of the next tile: inside a streaming loop that turns every
+// iteration into a full memory round trip.
+__device__ __forceinline__ void lev_barrier_lds() {
+    __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0); vmcnt and expcnt left open
+    asm volatile("s_barrier" ::: "memory");
 }
 
 // Overflow-safe tanh and gelu_tanh(g)*u exactly as the reference kernels

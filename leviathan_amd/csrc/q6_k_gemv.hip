@@ -14,17 +14,31 @@
 //                                  high nibbles -> elements E+64..E+79
 //   qh[32*half + 16*(v&1) .. +16)  bit pairs (v>>1)*2 and (v>>1)*2+4
 // with E = 128*half + 16*v inside the superblock, so both of its 16-element
-// groups have ONE sub-scale each (scales[8*half + (v&1) + 2*(v>>1)] and +4).
-// A lane keeps the 32 activations of its unit(s) in registers for every row
-// it visits; the -32 offset is folded out:  sc*(sum q*x - 32*sum x).
-// The 6-bit codes are assembled four per dword with byte-wise logic, turned
-// into fp16 subnormals (q * 2^-24) by masking and fed to v_fma_mix_f32.
+// groups have ONE sub-scale each (scales[8*half + v] and [8*half + 4 + v]).
+//
+// Arithmetic.  Logits are sums of 4096 terms that cancel from magnitudes of
+// several thousand down to O(1), and the gate is 1e-4 of max(1, |logit|): f32
+// accumulation sits at that bound whatever the order.  So the products are
+// formed EXACTLY, on integers: while staging, every 16-element group of x is
+// written as 27-bit integers X_i = rint(x_i * 2^(26-e)), 2^e > max|x| of the
+// group (exact for every element within 2^-3 of the group's maximum, 2^-27 of the
+// maximum otherwise), split into four balanced 7-bit digits held as int8
+//   X = l0*2^21 + l1*2^14 + l2*2^7 + l3,
+// and the 6-bit codes, assembled four per dword with byte-wise logic, go
+// straight into v_dot4_i32_i8 against each digit plane: four exact int32 dot
+// products per group, recombined in f64.  The -32 offset comes out through the
+// group's exact integer sum.  Scales, the sum over a row and the reduction
+// across lanes are f64; the result is rounded to f32 once.  A lane keeps the
+// digit planes of its unit(s) in registers for every row it visits.
 #include "lev_common.hpp"
 
 namespace {
 
-constexpr int kThreads = 512;
+constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / LEV_WAVE;
+#ifndef LEV_Q6_DEPTH
+#define LEV_Q6_DEPTH 3   // tiles in flight per wave of the one-unit-per-lane kernels
+#endif
 
 struct __attribute__((packed, aligned(2))) u32x4_a2 { uint32_t v[4]; };
 struct __attribute__((packed, aligned(2))) u32x2_a2 { uint32_t v[2]; };
@@ -45,6 +59,14 @@ struct q6_unit_w {
 __device__ __forceinline__ void q6_load_unit(const uint8_t *row, uint32_t g, q6_unit_w &u) {
     const uint32_t sb = g >> 3, half = (g >> 2) & 1u, v = g & 3u;
     const uint8_t *blk = row + (uint64_t)sb * 210u;
+#ifdef LEV_EXP_NO_LOADS
+    {
+        const uint32_t z = (uint32_t)(uintptr_t)blk * 2654435761u;
+        for (int i = 0; i < 4; ++i) u.ql[i] = z + i, u.qh[i] = z ^ i;
+        u.sc[0] = z; u.sc[1] = ~z; u.d = 0x2000u + (z & 255u);
+        return;
+    }
+#endif
     u32x4_a2 a = *reinterpret_cast<const u32x4_a2 *>(blk + 64u * half + 16u * v);
     u32x4_a2 b = *reinterpret_cast<const u32x4_a2 *>(blk + 128u + 32u * half + 16u * (v & 1u));
     u32x2_a2 c = *reinterpret_cast<const u32x2_a2 *>(blk + 192u + 8u * half);
@@ -58,6 +80,8 @@ __device__ __forceinline__ void q6_load_unit(const uint8_t *row, uint32_t g, q6_
     u.sc[1] = c.v[1];
 }
 
+// ---- f32 path of the generic kernel (any geometry, activations from global memory) ----
+
 // sum_i code_i * x_i over four code bytes packed in `c`, scaled by 2^-24.
 __device__ __forceinline__ float q6_dot4(uint32_t c, lev_f32x4 x, float acc) {
     lev_f16x2 e02 = __builtin_bit_cast(lev_f16x2, c & 0x00FF00FFu);
@@ -69,60 +93,150 @@ __device__ __forceinline__ float q6_dot4(uint32_t c, lev_f32x4 x, float acc) {
     return acc;
 }
 
-// Contribution of one unit to its row's dot product.  `v` = g & 3.
-__device__ __forceinline__ float q6_unit_dot(const q6_unit_w &u, const q6_unit_x &x, uint32_t v) {
+// Contribution of one unit to its row's dot product.  `v` = g & 3.  The two
+// 16-element sums are f32 (two chains each), everything behind them f64.
+__device__ __forceinline__ double q6_unit_dot(const q6_unit_w &u, const q6_unit_x &x, uint32_t v) {
     const uint32_t pair = v >> 1;              // 0: qh bit pairs 0 and 4, 1: pairs 2 and 6
     const uint32_t shl = 4u - 2u * pair;       // (qh << shl) & 0x30 -> top bits of the low set
     const uint32_t shr = 2u * pair;            // (qh >> shr) & 0x30 -> top bits of the high set
-    float lo = 0.f, hi = 0.f;
+    float lo0 = 0.f, lo1 = 0.f, hi0 = 0.f, hi1 = 0.f;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < 4; i += 2) {
         uint32_t q = u.ql[i], h = u.qh[i];
-        uint32_t cl = (q & 0x0F0F0F0Fu) | ((h << shl) & 0x30303030u);
-        uint32_t ch = ((q >> 4) & 0x0F0F0F0Fu) | ((h >> shr) & 0x30303030u);
-        lo = q6_dot4(cl, x.lo[i], lo);
-        hi = q6_dot4(ch, x.hi[i], hi);
+        lo0 = q6_dot4((q & 0x0F0F0F0Fu) | ((h << shl) & 0x30303030u), x.lo[i], lo0);
+        hi0 = q6_dot4(((q >> 4) & 0x0F0F0F0Fu) | ((h >> shr) & 0x30303030u), x.hi[i], hi0);
+        q = u.ql[i + 1], h = u.qh[i + 1];
+        lo1 = q6_dot4((q & 0x0F0F0F0Fu) | ((h << shl) & 0x30303030u), x.lo[i + 1], lo1);
+        hi1 = q6_dot4(((q >> 4) & 0x0F0F0F0Fu) | ((h >> shr) & 0x30303030u), x.hi[i + 1], hi1);
     }
-    // sub-scales: byte (v&1) + 2*pair for the low set, +4 for the high set
-    const uint32_t bi = (v & 1u) + 2u * pair;
-    float s_lo = (float)(int)__builtin_amdgcn_sbfe((int)u.sc[0], 8u * bi, 8u);
-    float s_hi = (float)(int)__builtin_amdgcn_sbfe((int)u.sc[1], 8u * bi, 8u);
-    float d = lev_f16_bits_to_f32(u.d);
-    float t = fmaf(s_lo, fmaf(lo, 16777216.0f, -32.0f * x.sum_lo),
-                   s_hi * fmaf(hi, 16777216.0f, -32.0f * x.sum_hi));
-    return d * t;
+    // sub-scales: byte v of the half's low four for the low set, of its high four for the high set
+    const double s_lo = (double)(int)__builtin_amdgcn_sbfe((int)u.sc[0], 8u * v, 8u);
+    const double s_hi = (double)(int)__builtin_amdgcn_sbfe((int)u.sc[1], 8u * v, 8u);
+    const double t_lo = fma(((double)lo0 + (double)lo1), 16777216.0, -32.0 * (double)x.sum_lo);
+    const double t_hi = fma(((double)hi0 + (double)hi1), 16777216.0, -32.0 * (double)x.sum_hi);
+    return (double)lev_f16_bits_to_f32(u.d) * fma(s_lo, t_lo, s_hi * t_hi);
 }
 
-// LDS layout of the activations: float4 slot q*(U+1)+g, q = 0..3 low set,
-// 4..7 high set of unit g; U = units per row.
-__device__ __forceinline__ void q6_stage_x(const float *__restrict__ x, lev_f32x4 *xs,
-                                           uint32_t units, uint32_t tid) {
+// ---- exact path ------------------------------------------------------------
+
+// Digit planes of one unit: lo[i] / hi[i] hold, for elements 4i..4i+3 of the
+// low / high set, the four dwords {l0, l1, l2, l3} of packed int8 digits.
+struct q6_unit_xi {
+    lev_u32x4 lo[4];
+    lev_u32x4 hi[4];
+};
+
+// Per 16-element group of x: p = 2^(e-26) and sx = sum of the group's integers X_i.
+struct q6_group_meta {
+    double p, sx;
+};
+
+// LDS: uint4 slot q*(U+1)+g holds the digit dwords of quad q (0..3 low set,
+// 4..7 high set) of unit g; then 2*U group records, group j = element / 16.
+__host__ __device__ constexpr size_t q6_lds_bytes(uint32_t units) {
+    return (size_t)8 * (units + 1u) * sizeof(lev_u32x4) + (size_t)2 * units * sizeof(q6_group_meta);
+}
+
+// Returns false (workgroup-uniform) when x holds a NaN or an infinity.
+__device__ __forceinline__ bool q6_stage_digits(const float *__restrict__ x, lev_u32x4 *xs,
+                                                q6_group_meta *meta, uint32_t units, uint32_t tid) {
     const lev_f32x4 *x4 = reinterpret_cast<const lev_f32x4 *>(x);
     const uint32_t n4 = units * 8u;
-    for (uint32_t i = tid; i < n4; i += kThreads) {
-        uint32_t e = i * 4u;
-        uint32_t c = e >> 7, r = e & 127u;
-        uint32_t g = 4u * c + ((r & 63u) >> 4);
-        uint32_t q = 4u * (r >> 6) + ((r & 15u) >> 2);
-        xs[q * (units + 1u) + g] = x4[i];
+    bool finite = true;
+    // whole passes: the four lanes of a group exchange their maxima and sums by DPP
+    for (uint32_t base = 0; base < n4; base += kThreads) {
+        const uint32_t i = base + tid;
+        const bool live = i < n4;
+        const lev_f32x4 v = x4[live ? i : n4 - 1u];
+        float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+#define LEV_Q6_MAXSTEP(CTRL)                                                                     \
+        amax = fmaxf(amax, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(                 \
+                               __builtin_bit_cast(int, amax), __builtin_bit_cast(int, amax), CTRL, 0xF, 0xF, false)))
+        LEV_Q6_MAXSTEP(0xB1);   // quad_perm [1,0,3,2]
+        LEV_Q6_MAXSTEP(0x4E);   // quad_perm [2,3,0,1]
+#undef LEV_Q6_MAXSTEP
+        uint32_t ex = __float_as_uint(amax) >> 23;          // biased exponent: amax < 2^(ex-126)
+        finite = finite && ex != 255u && !(v.x != v.x || v.y != v.y || v.z != v.z || v.w != v.w);
+        ex = ex < 25u ? 25u : (ex > 254u ? 254u : ex);      // keeps the scale 2^(152-ex) a normal number
+        const float scale = __uint_as_float((279u - ex) << 23);
+        int X[4] = {(int)rintf(v.x * scale), (int)rintf(v.y * scale), (int)rintf(v.z * scale),
+                    (int)rintf(v.w * scale)};
+        int sum = (X[0] + X[1]) + (X[2] + X[3]);            // |X| <= 2^26: sixteen of them fit
+        sum += __builtin_amdgcn_update_dpp(0, sum, 0xB1, 0xF, 0xF, false);
+        sum += __builtin_amdgcn_update_dpp(0, sum, 0x4E, 0xF, 0xF, false);
+        uint32_t dw[4] = {0u, 0u, 0u, 0u};                  // dw[3] = lowest digit l3 ... dw[0] = l0
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            int r = X[k];
+#pragma unroll
+            for (int dgt = 3; dgt >= 1; --dgt) {
+                const int l = __builtin_amdgcn_sbfe(r, 0u, 7u);   // signed low 7 bits: r - l is a multiple of 128
+                r = (r - l) >> 7;
+                dw[dgt] |= ((uint32_t)l & 0xFFu) << (8 * k);
+            }
+            dw[0] |= ((uint32_t)r & 0xFFu) << (8 * k);            // |r| <= 33
+        }
+        if (live) {
+            const uint32_t e = i * 4u;
+            const uint32_t c = e >> 7, rr = e & 127u;
+            const uint32_t g = 4u * c + ((rr & 63u) >> 4);
+            const uint32_t q = 4u * (rr >> 6) + ((rr & 15u) >> 2);
+            xs[q * (units + 1u) + g] = lev_u32x4{dw[0], dw[1], dw[2], dw[3]};
+            if ((i & 3u) == 3u) {
+                q6_group_meta m;
+                m.p = __hiloint2double((int)((ex + 871u) << 20), 0);   // 2^(ex-152)
+                m.sx = (double)sum;
+                meta[i >> 2] = m;
+            }
+        }
     }
+    return __syncthreads_and(finite ? 1 : 0) != 0;
 }
 
-__device__ __forceinline__ void q6_fetch_x(const lev_f32x4 *xs, uint32_t units, uint32_t g,
-                                           q6_unit_x &x) {
+__device__ __forceinline__ void q6_fetch_digits(const lev_u32x4 *xs, const q6_group_meta *meta,
+                                                uint32_t units, uint32_t g, q6_unit_xi &x,
+                                                q6_group_meta &mlo, q6_group_meta &mhi) {
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
         x.lo[q] = xs[q * (units + 1u) + g];
         x.hi[q] = xs[(4 + q) * (units + 1u) + g];
     }
-    float a = 0.f, b = 0.f;
+    const uint32_t j = 8u * (g >> 2) + (g & 3u);
+    mlo = meta[j];
+    mhi = meta[j + 4u];
+}
+
+// sum over a 16-element group of code * X, exact.
+__device__ __forceinline__ double q6_group_dot(const uint32_t c[4], const lev_u32x4 x[4]) {
+    int d0 = 0, d1 = 0, d2 = 0, d3 = 0;
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-        a += (x.lo[q].x + x.lo[q].y) + (x.lo[q].z + x.lo[q].w);
-        b += (x.hi[q].x + x.hi[q].y) + (x.hi[q].z + x.hi[q].w);
+    for (int i = 0; i < 4; ++i) {
+        d0 = __builtin_amdgcn_sdot4((int)c[i], (int)x[i].x, d0, false);
+        d1 = __builtin_amdgcn_sdot4((int)c[i], (int)x[i].y, d1, false);
+        d2 = __builtin_amdgcn_sdot4((int)c[i], (int)x[i].z, d2, false);
+        d3 = __builtin_amdgcn_sdot4((int)c[i], (int)x[i].w, d3, false);
     }
-    x.sum_lo = a;
-    x.sum_hi = b;
+    // |d_k| <= 16*63*64: the pairs fit 32 bits, the whole sum fits f64
+    return fma((double)((d0 << 7) + d1), 16384.0, (double)((d2 << 7) + d3));
+}
+
+__device__ __forceinline__ double q6_unit_dot_exact(const q6_unit_w &u, const q6_unit_xi &x,
+                                                    const q6_group_meta &mlo, const q6_group_meta &mhi,
+                                                    uint32_t v) {
+    const uint32_t pair = v >> 1;
+    const uint32_t shl = 4u - 2u * pair, shr = 2u * pair;
+    uint32_t cl[4], ch[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t q = u.ql[i], h = u.qh[i];
+        cl[i] = (q & 0x0F0F0F0Fu) | ((h << shl) & 0x30303030u);
+        ch[i] = ((q >> 4) & 0x0F0F0F0Fu) | ((h >> shr) & 0x30303030u);
+    }
+    const double t_lo = fma(-32.0, mlo.sx, q6_group_dot(cl, x.lo));   // sum (code - 32) * X
+    const double t_hi = fma(-32.0, mhi.sx, q6_group_dot(ch, x.hi));
+    const double s_lo = (double)(int)__builtin_amdgcn_sbfe((int)u.sc[0], 8u * v, 8u) * mlo.p;
+    const double s_hi = (double)(int)__builtin_amdgcn_sbfe((int)u.sc[1], 8u * v, 8u) * mhi.p;
+    return (double)lev_f16_bits_to_f32(u.d) * fma(s_lo, t_lo, s_hi * t_hi);
 }
 
 // ---- argmax + margin (lev-forge/src/ops.rs:479-516) ------------------------
@@ -164,7 +278,9 @@ __device__ __forceinline__ void q6_load_row(const uint8_t *__restrict__ w, uint6
                                             uint32_t units, q6_unit_w (&W)[P]) {
     // Lanes past the end of the matrix read a valid unit (clamped) and have
     // their block scale forced to zero: no divergent control flow around loads.
-    const uint32_t row_c = row < rows ? row : rows - 1u;
+    uint32_t row_c = row < rows ? row : rows - 1u;
+    // a whole wave per row: the row's address is wave-uniform (scalar base, one lane offset)
+    if (L == LEV_WAVE) row_c = (uint32_t)__builtin_amdgcn_readfirstlane((int)row_c);
 #pragma unroll
     for (int p = 0; p < P; ++p) {
         uint32_t g = lu + p * L;
@@ -174,45 +290,30 @@ __device__ __forceinline__ void q6_load_row(const uint8_t *__restrict__ w, uint6
     }
 }
 
-template <int L, int P>
-__device__ __forceinline__ void q6_finish_row(float *__restrict__ y, uint32_t row, uint32_t rows,
-                                              uint32_t lu, const q6_unit_w (&W)[P],
-                                              const q6_unit_x (&X)[P], top2 &m) {
-    float acc = 0.f;
-#pragma unroll
-    for (int p = 0; p < P; ++p) acc += q6_unit_dot(W[p], X[p], (lu + p * L) & 3u);
-    acc = lev_group_sum<L>(acc);
-    if (lu % L == L - 1 && row < rows) {
-        y[row] = acc;
-        // running top two of the rows this lane finishes (rows ascend, so a
-        // tie keeps the earlier, lower index)
-        if (acc > m.best) {
-            m.second = m.best;
-            m.best = acc;
-            m.idx = row;
-        } else if (acc > m.second) {
-            m.second = acc;
-        }
-    }
-}
-
 // L lanes per row-part, P passes of L units, S waves share a row (units <=
-// S*L*P; S > 1 only with L = 64): with S = 2 a 4096-wide row costs each lane
-// one unit instead of two, which brings the kernel under 128 VGPRs and five
-// waves per SIMD instead of three.  Persistent workgroups, weights
-// double-buffered.
+// S*L*P; S > 1 only with L = 64 and P = 1).  RESIDENT: the lane keeps the digit
+// planes of its P units in registers for every row; otherwise (rows wider than
+// 128 units) it reads them from LDS per row.
+// S = 2 is the shape of a 4096-wide row: one unit per lane keeps the kernel
+// under 100 registers, five waves per SIMD, which is what both the vector ALU
+// (a single wave issues one instruction every 8 cycles, the SIMD takes one
+// every 2) and the memory latency need; the two waves of a row meet in LDS, one
+// barrier per tile (two buffers).
+// Persistent workgroups of four waves, the next tile's weights in flight while
+// the current one is multiplied.
 // partials (optional): the workgroup's top two logits and the index of the
 // best, one float4 {best, second, idx bits, 0} per workgroup, for the greedy
 // token epilogue.
-template <int L, int P, int S>
+template <int L, int P, bool RESIDENT, int S>
 __global__ void __launch_bounds__(kThreads)
-q6_k_gemv_units(const uint8_t *__restrict__ w, const float *__restrict__ x, float *__restrict__ y,
+q6_k_gemv_exact(const uint8_t *__restrict__ w, const float *__restrict__ x, float *__restrict__ y,
                 uint32_t units, uint32_t rows, lev_f32x4 *__restrict__ partials) {
-    extern __shared__ lev_f32x4 xs[];
+    extern __shared__ lev_u32x4 xs[];
+    static_assert(S == 1 || (L == LEV_WAVE && P == 1), "rows are shared by whole waves only");
     constexpr int G = LEV_WAVE / L;
     constexpr uint32_t kRowsPerTile = kWaves * G / S;
-    static_assert(S == 1 || L == LEV_WAVE, "rows are shared by whole waves only");
-    __shared__ float part[2][S > 1 ? kWaves : 1];
+    __shared__ double part[2][S > 1 ? kWaves : 1];
+    q6_group_meta *meta = reinterpret_cast<q6_group_meta *>(xs + 8u * (units + 1u));
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & (LEV_WAVE - 1);
     const uint32_t wave = tid / LEV_WAVE;
@@ -226,66 +327,90 @@ q6_k_gemv_units(const uint8_t *__restrict__ w, const float *__restrict__ x, floa
     if (base >= rows) return;   // never: the grid has at most one workgroup per tile
 
     top2 m{kTop2Floor, kTop2Floor, 0xFFFFFFFFu};
-    q6_unit_w Wa[P], Wb[P];
-    q6_load_row<L, P>(w, row_bytes, base + in_tile, rows, lu, units, Wa);
-    q6_stage_x(x, xs, units, tid);
-    __syncthreads();
+    constexpr int kDepth = (P == 1) ? LEV_Q6_DEPTH : 2;
+    q6_unit_w W[kDepth][P];
+    q6_load_row<L, P>(w, row_bytes, base + in_tile, rows, lu, units, W[0]);
+    const bool finite = q6_stage_digits(x, xs, meta, units, tid);   // ends with a barrier
 
-    q6_unit_x X[P];
+    constexpr int PR = RESIDENT ? P : 1;
+    q6_unit_xi X[PR];
+    q6_group_meta Mlo[PR], Mhi[PR];
+    if (RESIDENT) {
 #pragma unroll
-    for (int p = 0; p < P; ++p) {
-        uint32_t g = lu + p * L;
-        if (g < units) {
-            q6_fetch_x(xs, units, g, X[p]);
-        } else {
-#pragma unroll
-            for (int q = 0; q < 4; ++q) X[p].lo[q] = X[p].hi[q] = lev_f32x4{0.f, 0.f, 0.f, 0.f};
-            X[p].sum_lo = X[p].sum_hi = 0.f;
+        for (int p = 0; p < P; ++p) {
+            const uint32_t g = lu + p * L;
+            q6_fetch_digits(xs, meta, units, g < units ? g : units - 1u, X[p], Mlo[p], Mhi[p]);
         }
     }
+    const float poison = finite ? 0.f : __builtin_nanf("");   // a NaN or infinity in x reaches every output
+    auto note = [&](float out, uint32_t row) {
+        // running top two of the rows this lane finishes (rows ascend, so a
+        // tie keeps the earlier, lower index)
+        if (out > m.best) {
+            m.second = m.best;
+            m.best = out;
+            m.idx = row;
+        } else if (out > m.second) {
+            m.second = out;
+        }
+    };
 
-    // The prefetch is unconditional (clamped past the end): a branch around the
-    // loads would make the compiler wait for them before the current row is used.
     uint32_t buf = 0;
-    auto finish = [&](uint32_t row0, const q6_unit_w (&W)[P]) {
+    auto finish = [&](uint32_t row, const q6_unit_w (&W)[P]) {
+        double acc = 0.0;
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+            const uint32_t g = lu + p * L;
+#ifdef LEV_EXP_NO_COMPUTE
+            acc += (double)(W[p].ql[0] ^ W[p].ql[1] ^ W[p].ql[2] ^ W[p].ql[3] ^ W[p].qh[0] ^ W[p].qh[1] ^ W[p].qh[2] ^ W[p].qh[3] ^ W[p].sc[0] ^ W[p].sc[1] ^ W[p].d);
+            continue;
+#endif
+            if (RESIDENT) {
+                acc += q6_unit_dot_exact(W[p], X[p], Mlo[p], Mhi[p], g & 3u);
+            } else {
+                q6_fetch_digits(xs, meta, units, g < units ? g : units - 1u, X[0], Mlo[0], Mhi[0]);
+                acc += q6_unit_dot_exact(W[p], X[0], Mlo[0], Mhi[0], g & 3u);
+            }
+        }
+        acc = lev_group_sum_f64<L>(acc);
         if constexpr (S == 1) {
-            q6_finish_row<L, P>(y, row0 + in_tile, rows, lu, W, X, m);
+            if (lane % L == L - 1 && row < rows) {
+                const float out = (float)acc + poison;
+                y[row] = out;
+                note(out, row);
+            }
         } else {
-            // the S waves of a row leave their parts in LDS; one thread per row
-            // adds them in wave order.  Two part buffers: one barrier per tile.
-            float acc = 0.f;
-#pragma unroll
-            for (int p = 0; p < P; ++p) acc += q6_unit_dot(W[p], X[p], (lu + p * L) & 3u);
-            acc = lev_group_sum<L>(acc);
-            if (lane == LEV_WAVE - 1) part[buf][wave] = acc;
-            __syncthreads();
-            if (tid < kRowsPerTile && row0 + tid < rows) {
-                float sum = part[buf][tid * S];
-#pragma unroll
-                for (int k = 1; k < S; ++k) sum += part[buf][tid * S + k];
-                y[row0 + tid] = sum;
-                if (sum > m.best) {
-                    m.second = m.best;
-                    m.best = sum;
-                    m.idx = row0 + tid;
-                } else if (sum > m.second) {
-                    m.second = sum;
-                }
+            // the odd wave of a row leaves its half in LDS, the even one adds and stores
+            if ((wave & 1u) && lane == LEV_WAVE - 1) part[buf][wave >> 1] = acc;
+            lev_barrier_lds();   // not __syncthreads(): the next tiles' loads stay in flight
+            if (!(wave & 1u) && lane == LEV_WAVE - 1 && row < rows) {
+                const float out = (float)(acc + part[buf][wave >> 1]) + poison;
+                y[row] = out;
+                note(out, row);
             }
             buf ^= 1u;
         }
     };
-    while (true) {
-        uint32_t next = base + step;
-        q6_load_row<L, P>(w, row_bytes, next + in_tile, rows, lu, units, Wb);
-        finish(base, Wa);
-        if (next >= rows) break;
-        base = next;
-        next = base + step;
-        q6_load_row<L, P>(w, row_bytes, next + in_tile, rows, lu, units, Wa);
-        finish(base, Wb);
-        if (next >= rows) break;
-        base = next;
+    // kDepth tiles in flight per wave (the one being multiplied and kDepth-1
+    // behind it): what the streaming rate of this kernel is made of is bytes in
+    // flight over memory latency.  The prefetch is unconditional (clamped past
+    // the end): a branch around the loads would make the compiler wait for them
+    // before the current row is used.
+#pragma unroll
+    for (int k = 1; k < kDepth - 1; ++k)
+        q6_load_row<L, P>(w, row_bytes, base + k * step + in_tile, rows, lu, units, W[k]);
+    for (bool more = true; more;) {
+#pragma unroll
+        for (int k = 0; k < kDepth; ++k) {
+            q6_load_row<L, P>(w, row_bytes, base + (kDepth - 1) * step + in_tile, rows, lu, units,
+                              W[(k + kDepth - 1) % kDepth]);
+            finish(base + in_tile, W[k]);
+            base += step;
+            if (base >= rows) {   // uniform over the workgroup
+                more = false;
+                break;
+            }
+        }
     }
     if (partials) {
         __shared__ float s_best[kWaves], s_second[kWaves];
@@ -305,18 +430,26 @@ q6_k_gemv_units(const uint8_t *__restrict__ w, const float *__restrict__ x, floa
     }
 }
 
-// One workgroup: merges the per-workgroup partials of the GEMV.
-__global__ void __launch_bounds__(256)
+// One workgroup: merges the per-workgroup partials of the GEMV (n <= 4096).
+// All of a thread's partials are requested before the first is used: one
+// memory round trip, not one per partial.
+__global__ void __launch_bounds__(1024)
 argmax_partials_kernel(const lev_f32x4 *__restrict__ partials, uint32_t n,
                        uint32_t *__restrict__ out_idx, float *__restrict__ out_margin) {
-    __shared__ float s_best[4], s_second[4];
-    __shared__ uint32_t s_idx[4];
+    __shared__ float s_best[16], s_second[16];
+    __shared__ uint32_t s_idx[16];
     const uint32_t t = threadIdx.x;
+    lev_f32x4 p[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const uint32_t i = t + 1024u * (uint32_t)k;
+        p[k] = partials[i < n ? i : n - 1u];
+    }
     top2 m{kTop2Floor, kTop2Floor, 0xFFFFFFFFu};
-    for (uint32_t i = t; i < n; i += 256u) {
-        lev_f32x4 p = partials[i];
-        const float idx_bits = p.z;   // a copy: bit_cast straight from a vector element reads element 0
-        m = top2_merge(m, top2{p.x, p.y, __float_as_uint(idx_bits)});
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const float idx_bits = p[k].z;   // a copy: bit_cast straight from a vector element reads element 0
+        if (t + 1024u * (uint32_t)k < n) m = top2_merge(m, top2{p[k].x, p[k].y, __float_as_uint(idx_bits)});
     }
     m = top2_wave(m);
     if ((t & 63u) == 0) {
@@ -327,13 +460,14 @@ argmax_partials_kernel(const lev_f32x4 *__restrict__ partials, uint32_t n,
     __syncthreads();
     if (t == 0) {
         top2 r{s_best[0], s_second[0], s_idx[0]};
-        for (int k = 1; k < 4; ++k) r = top2_merge(r, top2{s_best[k], s_second[k], s_idx[k]});
+        for (int k = 1; k < 16; ++k) r = top2_merge(r, top2{s_best[k], s_second[k], s_idx[k]});
         if (out_idx) out_idx[0] = r.idx == 0xFFFFFFFFu ? 0u : r.idx;   // nothing above -inf: first
         if (out_margin) out_margin[0] = r.best - r.second;
     }
 }
 
-// Any in_dim: one wave per row, activations read through the cache.
+// Any in_dim and alignment: one wave per row, activations read through the
+// cache, 16-element sums in f32 (two chains), everything behind them in f64.
 __global__ void __launch_bounds__(kThreads)
 q6_k_gemv_generic(const uint8_t *__restrict__ w, const float *__restrict__ x,
                   float *__restrict__ y, uint32_t units, uint32_t rows) {
@@ -341,7 +475,7 @@ q6_k_gemv_generic(const uint8_t *__restrict__ w, const float *__restrict__ x,
     const uint32_t row = blockIdx.x * kWaves + threadIdx.x / LEV_WAVE;
     if (row >= rows) return;
     const uint8_t *rp = w + (uint64_t)row * (units >> 3) * 210u;
-    float acc = 0.f;
+    double acc = 0.0;
     for (uint32_t g = lane; g < units; g += LEV_WAVE) {
         q6_unit_w u;
         q6_load_unit(rp, g, u);
@@ -359,8 +493,8 @@ q6_k_gemv_generic(const uint8_t *__restrict__ w, const float *__restrict__ x,
         ux.sum_hi = b;
         acc += q6_unit_dot(u, ux, g & 3u);
     }
-    acc = lev_group_sum<64>(acc);
-    if (lane == LEV_WAVE - 1) y[row] = acc;
+    acc = lev_group_sum_f64<64>(acc);
+    if (lane == LEV_WAVE - 1) y[row] = (float)acc;
 }
 
 __global__ void __launch_bounds__(1024)
@@ -403,16 +537,16 @@ argmax_kernel(const float *__restrict__ logits, uint32_t vocab, uint32_t *__rest
     }
 }
 
-template <int L, int P, int S = 1>
+template <int L, int P, bool RESIDENT = true, int S = 1>
 hipError_t launch_units(lev_ctx *ctx, const uint8_t *w, const float *x, float *y, uint32_t units,
                         uint32_t rows, uint32_t *d_argmax, float *d_margin) {
     constexpr uint32_t rows_per_tile = kWaves * (LEV_WAVE / L) / S;
     uint32_t blocks = (rows + rows_per_tile - 1) / rows_per_tile;
-    size_t lds = (size_t)8 * (units + 1) * sizeof(lev_f32x4);
+    const size_t lds = q6_lds_bytes(units);
     // persistent grid: exactly the workgroups that are resident at once, so
     // that no workgroup waits for a slot behind another one's whole loop
     int per_cu = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, q6_k_gemv_units<L, P, S>, kThreads, lds) !=
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, q6_k_gemv_exact<L, P, RESIDENT, S>, kThreads, lds) !=
             hipSuccess || per_cu < 1)
         per_cu = 2;
     uint32_t cap = (uint32_t)ctx->num_cus * (uint32_t)per_cu;
@@ -423,11 +557,11 @@ hipError_t launch_units(lev_ctx *ctx, const uint8_t *w, const float *x, float *y
         if (blocks > lev_ctx::kArgmaxPartials) blocks = lev_ctx::kArgmaxPartials;
         partials = static_cast<lev_f32x4 *>(ctx->argmax_partials);
     }
-    hipLaunchKernelGGL((q6_k_gemv_units<L, P, S>), dim3(blocks), dim3(kThreads), lds, ctx->stream, w, x,
-                       y, units, rows, partials);
+    hipLaunchKernelGGL((q6_k_gemv_exact<L, P, RESIDENT, S>), dim3(blocks), dim3(kThreads), lds, ctx->stream, w,
+                       x, y, units, rows, partials);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || !partials) return e;
-    hipLaunchKernelGGL(argmax_partials_kernel, dim3(1), dim3(256), 0, ctx->stream, partials, blocks,
+    hipLaunchKernelGGL(argmax_partials_kernel, dim3(1), dim3(1024), 0, ctx->stream, partials, blocks,
                        d_argmax, d_margin);
     return hipGetLastError();
 }
@@ -451,9 +585,8 @@ hipError_t lev_q6_k_gemv_argmax_launch(lev_ctx *ctx, const uint8_t *w, const flo
                            d_margin);
         return hipGetLastError();
     }
-    if (units > 192) return launch_units<64, 4>(ctx, w, x, y, units, rows, d_argmax, d_margin);
-    if (units > 128) return launch_units<64, 3>(ctx, w, x, y, units, rows, d_argmax, d_margin);
-    if (units > 64) return launch_units<64, 1, 2>(ctx, w, x, y, units, rows, d_argmax, d_margin);
+    if (units > 128) return launch_units<64, 4, false>(ctx, w, x, y, units, rows, d_argmax, d_margin);
+    if (units > 64) return launch_units<64, 1, true, 2>(ctx, w, x, y, units, rows, d_argmax, d_margin);
     if (units > 32) return launch_units<64, 1>(ctx, w, x, y, units, rows, d_argmax, d_margin);
     if (units > 16) return launch_units<32, 1>(ctx, w, x, y, units, rows, d_argmax, d_margin);
     if (units > 8) return launch_units<16, 1>(ctx, w, x, y, units, rows, d_argmax, d_margin);

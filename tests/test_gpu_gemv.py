@@ -249,28 +249,25 @@ def test_q6_k_one_hot_bit_exact(ctx):
 
 
 def test_q6_k_random_64x512_vs_fp64(ctx):
-    """main.swift:1028-1085: seeds 555 / 202, wide-range blocks (|d| up to 3,
+    """main.swift:1028-1085: seeds 555 / 202, wide-range blocks (|d| up to 1,
     sub-scales over the whole int8 range): single rows cancel from ~2e5 of
-    summed magnitudes down to ~16, which is beyond what ANY f32 accumulation
-    holds to 1e-4.  Restated on these bytes, the reference's own f32 paths give
-    1.96e-4 (matvec_q6k_f32, lev-cpu/src/lib.rs:261) and 1.69e-4 (the serial
-    order of g4_q6_matvec with fused multiply-add); only its f64-accumulating
-    Swift CPU path meets 1e-4.  Tolerance for the f32 HIP kernel on THIS
-    fixture: 4e-4 normalised and no worse than 2x the reference's f32 CPU path;
-    every other Q6_K case in this file is held to 1e-4."""
+    summed magnitudes down to ~16.  The reference gates its GPU kernel at 1e-4
+    on exactly these bytes (main.swift:1047-1081), and so does this test.  The
+    kernel's per-group dot products are exact integers and everything behind
+    them is f64, so it sits orders below the gate; the reference's own f32 CPU
+    order (matvec_q6k_f32, lev-cpu/src/lib.rs:261) measures 1.96e-4 here, its
+    f64-accumulating Swift CPU path < 1e-4."""
     w = H.swift_q6_k_blocks(555, 64 * 2)
     x = O.seeded_input(512, 1, 202)
     got = q6_gemv(ctx, w, x, 64, 512)
     ref = O.q6_k_matvec_f64(w, 64, 512, x)
     assert O.max_rel_err(O.q6_k_matvec_ref(w, 64, 512, x), ref) < TOL      # Swift CPU path (f64 acc)
-    cpu_f32 = O.max_rel_err(O.q6_k_matvec_f32(w, 64, 512, x), ref)          # Rust CPU path (f32)
-    err = O.max_rel_err(got, ref)
-    assert err < 4e-4 and err < 2 * cpu_f32
+    assert O.max_rel_err(got, ref) < TOL
     # scaled by the summed magnitudes (the reference's F32 matvec gate,
-    # main.swift:2615-2647) the kernel is four orders inside the bound
+    # main.swift:2615-2647) the kernel is at the rounding of its f32 output
     dq = O.q6_k_dequant(w).reshape(64, 512).astype(np.float64)
     mag = np.abs(dq) @ np.abs(x.astype(np.float64))
-    assert np.all(np.abs(got - ref) <= 1e-6 * mag + 1e-6)
+    assert np.all(np.abs(got - ref) <= 1e-7 * mag + 1e-6)
 
 
 @pytest.mark.parametrize("rows,cols", [(1, 256), (5, 768), (33, 2048), (17, 2816), (21, 4096),
@@ -279,6 +276,24 @@ def test_q6_k_shapes_vs_fp64(ctx, rows, cols):
     w = O.synth_q6_k(rows * 3 + cols, rows * cols // 256)
     x = O.seeded_input(cols, 1, 11)
     assert O.max_rel_err(q6_gemv(ctx, w, x, rows, cols), O.q6_k_matvec_f64(w, rows, cols, x)) < TOL
+
+
+def test_q6_k_non_finite_activation_reaches_the_output(ctx):
+    """The integer digit planes cannot carry a NaN or an infinity: the kernel
+    detects them while staging and poisons its outputs, as an f32 product would
+    (the runner re-checks outputs for finiteness, Q6.swift:260-268)."""
+    rows, cols = 9, 4096
+    w = O.synth_q6_k(77, rows * cols // 256)
+    for bad in (np.nan, np.inf, -np.inf):
+        x = O.seeded_input(cols, 1, 5)
+        x[1234] = bad
+        got = q6_gemv(ctx, w, x, rows, cols)
+        assert not np.any(np.isfinite(got)), bad
+    x = O.seeded_input(cols, 1, 5)
+    x[7] = 1e-40          # denormal: finite, must not poison
+    x[8] = 3e30
+    got = q6_gemv(ctx, w, x, rows, cols)
+    assert O.max_rel_err(got, O.q6_k_matvec_f64(w, rows, cols, x)) < TOL
 
 
 def test_q6_k_saturated_bytes_every_fourth_block(ctx):
@@ -295,10 +310,10 @@ def test_q6_k_config2_full_size_with_argmax(ctx):
     w, x = H.config2()
     got, idx, margin = q6_gemv(ctx, w, x, 32000, 4096, argmax=True)
     ref64 = O.q6_k_matvec_f64(w, 32000, 4096, x)
-    # logits of this configuration are O(200) with summed magnitudes O(7000):
-    # over 32000 rows an f32 accumulation lands within a factor ~2 of 1e-4
-    # (the reference's f32 CPU order, matvec_q6k_f32, measures 3e-4 here)
-    assert O.max_rel_err(got, ref64) < 2e-4
+    # logits of this configuration are O(200) with summed magnitudes O(7000): the
+    # reference's f32 CPU order (matvec_q6k_f32) measures 3e-4 here; the kernel
+    # (exact integer dot products per 16 weights, f64 behind them) holds 1e-4
+    assert O.max_rel_err(got, ref64) < TOL
     ref32 = O.q6_k_matvec_ref(w, 32000, 4096, x, threads=8)      # reference CPU path
     # the comparison is only meaningful if the CPU reference's own top-2 gap
     # is far above the summation-order noise; assert it, then demand equality
