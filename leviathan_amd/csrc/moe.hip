@@ -185,7 +185,7 @@ __device__ router_sel router_select_block(const float *__restrict__ srow, void *
             rank[lane + 64u * j] = 0u;
         }
     }
-    __syncthreads();
+    lev_barrier_lds();
     auto count_before = [&](uint32_t i, uint32_t j0, uint32_t j1) {
         uint32_t before = 0;
         if (by_key) {
@@ -210,7 +210,7 @@ __device__ router_sel router_select_block(const float *__restrict__ srow, void *
     } else {
         for (uint32_t i = tid; i < padded; i += blockDim.x) rank[i] = count_before(i, 0u, padded);
     }
-    __syncthreads();
+    lev_barrier_lds();
     if (wave == 0) {
 #pragma unroll
         for (int j = 0; j < J; ++j) {
@@ -222,7 +222,7 @@ __device__ router_sel router_select_block(const float *__restrict__ srow, void *
             }
         }
     }
-    __syncthreads();
+    lev_barrier_lds();
     return out;
 }
 
@@ -279,7 +279,7 @@ moe_scores_kernel(const float *__restrict__ wr, const float *__restrict__ x,
             acc = wave_sum_f64(acc);
             if (lane == 0) partial[t][wave] = acc;
         }
-        __syncthreads();
+        lev_barrier_lds();
         if (threadIdx.x < tokens) {
             double acc = partial[threadIdx.x][0];
             for (uint32_t w = 1; w < waves; ++w) acc += partial[threadIdx.x][w];
@@ -361,7 +361,7 @@ moe_scores_mfma_kernel(const float *__restrict__ wr, const float *__restrict__ x
     // D of the f64 16x16x4 product: register r of lane (i, kq) is row (token) 4*r + kq of column (expert) i
 #pragma unroll
     for (int r = 0; r < 4; ++r) part[wave][(4u * (uint32_t)r + kq) * 16u + i] = acc[r];
-    __syncthreads();
+    lev_barrier_lds();
     const uint32_t tt = (threadIdx.x >> 4) & 15u, ee = threadIdx.x & 15u;
     if (threadIdx.x < 256u && t0 + tt < tokens && e0 + ee < experts) {
         double total = part[0][threadIdx.x];
@@ -510,7 +510,7 @@ moe_gate_up_kernel(moe_args a, const float *__restrict__ x, const int32_t *ids,
     uint32_t i0 = i_begin + wave * R;
     gu_load_rows<P, R>(wbase, row_bytes, i0, a.inter, pairs, lp, Da);
     lev_q4_stage_x_store_sums<NS>(xt, xs, bsum, pairs, tid, kGuThreads, xv);
-    __syncthreads();
+    lev_barrier_lds();
     if constexpr (ROUTE > 0) {
         // the first workgroup of a token publishes the selection while its
         // weights are on their way
@@ -641,7 +641,7 @@ moe_down_kernel(moe_args a, const float *__restrict__ act, const int32_t *__rest
     }
     if (bad && lane == 0) atomicOr(flag, kFlagBadExpertId);
     if (wave == 0 && lane < a.top_k) w_slot[lane] = w_mine;
-    __syncthreads();
+    lev_barrier_lds();
     // ordered merge: y = sum over slots, in slot order, of w_slot * dn[slot]
     for (uint32_t r = tid; r < tile; r += kDnThreads) {
         uint32_t row = row_begin + r;

@@ -81,10 +81,10 @@ __device__ __forceinline__ void finish_tile(const uint8_t *__restrict__ w, uint6
         float s = lev_group_sum<L>(acc[r]);
         if (lp == L - 1) ysh[in_tile + r * G] = s;
     }
-    __syncthreads();
+    lev_barrier_lds();
     if (threadIdx.x < kRowsPerTile && tile_base + threadIdx.x < rows)
         y[tile_base + threadIdx.x] = ysh[threadIdx.x];
-    __syncthreads();   // ysh is reused by the next tile
+    lev_barrier_lds();   // ysh is reused by the next tile
 }
 
 // One tile per workgroup, straight-line code: used whenever the whole matrix
@@ -115,7 +115,7 @@ q4_0_gemv_tile(const uint8_t *__restrict__ w, const float *__restrict__ x, float
     uint32_t D[R][9];
     load_tile<L, R>(w, row_bytes, base + in_tile, rows, pairs, lp, D);
     lev_q4_stage_x_store_sums<NS, EXACT>(x, xs, bsum, pairs, tid, kThreads, xv);
-    __syncthreads();
+    lev_barrier_lds();
 
     lev_q4_pair_x px;
     const bool p_ok = EXACT || lp < pairs;
@@ -131,7 +131,7 @@ q4_0_gemv_tile(const uint8_t *__restrict__ w, const float *__restrict__ x, float
         float s = lev_group_sum<L>(lev_q4_pair_dot(D[r], px));
         if (lp == L - 1) ysh[in_tile + r * G] = s;
     }
-    __syncthreads();
+    lev_barrier_lds();
     if (tid < kRowsPerTile && base + tid < rows) y[base + tid] = ysh[tid];
 }
 
@@ -168,7 +168,7 @@ q4_0_gemv_pairs(const uint8_t *__restrict__ w, const float *__restrict__ x, floa
     uint32_t Da[R][9], Db[R][9];
     load_tile<L, R>(w, row_bytes, base + in_tile, rows, pairs, lp, Da);
     lev_q4_stage_x_store_sums<NS>(x, xs, bsum, pairs, tid, kThreads, xv);
-    __syncthreads();
+    lev_barrier_lds();
 
     // Activations of the lane's first pair stay in registers for every tile;
     // lanes past the end of the row hold zeros.

@@ -195,7 +195,7 @@ q4_k_gemv_ncol(const uint8_t *__restrict__ w, const float *__restrict__ x,
             if (lane == LEV_WAVE - 1) s_part[c][wave] = ss;
         }
     }
-    __syncthreads();
+    lev_barrier_lds();
     if (tid < NC) {
         float inv = 1.0f;
         if (gain) {
@@ -206,7 +206,7 @@ q4_k_gemv_ncol(const uint8_t *__restrict__ w, const float *__restrict__ x,
         }
         s_inv[tid] = inv;
     }
-    __syncthreads();
+    lev_barrier_lds();
 
     q4k_unit_x X[RESIDENT ? NC : 1];
     if (RESIDENT) {

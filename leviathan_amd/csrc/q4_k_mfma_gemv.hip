@@ -227,7 +227,7 @@ q4_k_mfma_gemv(const uint8_t *__restrict__ w, const float *__restrict__ x,
             }
         }
     }
-    __syncthreads();
+    lev_barrier_lds();
     issue(ci, W0);
     issue(ci, W1);
     issue(ci, W2);
@@ -251,7 +251,7 @@ q4_k_mfma_gemv(const uint8_t *__restrict__ w, const float *__restrict__ x,
             s_fac[NC + wave] = __uint_as_float((254u - ex) << 23);     // 2^(127-ex)
         }
     }
-    __syncthreads();   // s_run (aliasing xh) is dead from here
+    lev_barrier_lds();   // s_run (aliasing xh) is dead from here
 #pragma unroll
     for (int i = 0; i < CH; ++i) {
         if ((uint32_t)i * kMThreads >= total_slots) break;
@@ -299,7 +299,7 @@ q4_k_mfma_gemv(const uint8_t *__restrict__ w, const float *__restrict__ x,
     }
     // columns of the layout beyond ncol hold no data: the A rows that read them
     // (clamped to the last column) only feed outputs that are never stored
-    __syncthreads();
+    lev_barrier_lds();
 
     // ---- stream the weights ----
     const uint32_t colc = r < (uint32_t)NC ? r : (uint32_t)NC - 1u;   // A rows past NC: any valid address
@@ -357,7 +357,7 @@ q4_k_mfma_gemv(const uint8_t *__restrict__ w, const float *__restrict__ x,
             for (int i = 0; i < 4; ++i)
                 if (4u * g + (uint32_t)i < (uint32_t)NC) pp[(wave * 16u + r) * NC + 4u * g + i] = yacc[i];
             yacc = lev_f32x4{0.f, 0.f, 0.f, 0.f};
-            __syncthreads();
+            lev_barrier_lds();
             if (tid < 16u * NC) {
                 const uint32_t col = tid >> 4, rr = tid & 15u, row = rg * 16u + rr;
                 float sum = 0.f;

@@ -190,7 +190,16 @@ __device__ __forceinline__ bool q6_stage_digits(const float *__restrict__ x, lev
             }
         }
     }
-    return __syncthreads_and(finite ? 1 : 0) != 0;
+    // every wave leaves its verdict in LDS; the barrier waits for LDS traffic only, so the
+    // first tile's weight loads (already requested) stay in flight across it
+    __shared__ uint32_t s_finite[kWaves];
+    const bool wave_ok = __ballot(!finite) == 0ull;
+    if ((tid & (LEV_WAVE - 1)) == 0) s_finite[tid / LEV_WAVE] = wave_ok ? 1u : 0u;
+    lev_barrier_lds();
+    bool all_ok = true;
+#pragma unroll
+    for (int k = 0; k < kWaves; ++k) all_ok = all_ok && s_finite[k] != 0u;
+    return all_ok;
 }
 
 __device__ __forceinline__ void q6_fetch_digits(const lev_u32x4 *xs, const q6_group_meta *meta,

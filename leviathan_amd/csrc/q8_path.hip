@@ -83,7 +83,7 @@ norm_quant_kernel(float *__restrict__ x, const float *__restrict__ add,
 #pragma unroll
             for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off);
             if (lane == 0) s_part[t >> 6] = ss;
-            __syncthreads();
+            lev_barrier_lds();
             double tot = 0.0;
 #pragma unroll
             for (int k = 0; k < kNQThreads / 64; ++k) tot += s_part[k];
@@ -182,7 +182,7 @@ q4_k_gemv_q8_kernel(const uint8_t *__restrict__ w, const uint32_t *__restrict__ 
         if (c < ncol) v = *reinterpret_cast<const lev_f32x4 *>(xs + ((uint64_t)c * (in_dim >> 5) + sb * 8u) * 2u + k * 4u);
         *reinterpret_cast<lev_f32x4 *>(s_pairs + ((size_t)c * SB + sb) * kPairStride + k * 16u) = v;
     }
-    __syncthreads();
+    lev_barrier_lds();
 
     const uint32_t grp = lane >> 4, lp = lane & 15u;
     const uint64_t row_bytes = (uint64_t)SB * 144u;
@@ -317,7 +317,7 @@ q6_k_gemv_q8_kernel(const uint8_t *__restrict__ w, const uint32_t *__restrict__ 
         if (c < ncol) d = xs[((uint64_t)c * (in_dim >> 5) + sb * 8u + k) * 2u];
         reinterpret_cast<float *>(smem + ((size_t)c * SB + sb) * kQ6Stride + 272u)[k] = d;
     }
-    __syncthreads();
+    lev_barrier_lds();
 
     const uint32_t grp = lane >> 5, lp = lane & 31u;
     const uint32_t halves = SB * 2u;
@@ -585,7 +585,7 @@ q4_k_q8_mfma(const uint8_t *__restrict__ w, const uint8_t *__restrict__ xq, cons
             ssum[(size_t)k * NCL + ac] = __uint_as_float(v.y);
         }
     }
-    __syncthreads();
+    lev_barrier_lds();
 
     // ---- stream the weights ----
     const uint32_t colc = r < (uint32_t)NCL ? r : (uint32_t)NCL - 1u;    // A rows past NCL: any valid address
@@ -638,7 +638,7 @@ q4_k_q8_mfma(const uint8_t *__restrict__ w, const uint8_t *__restrict__ xq, cons
             for (int i = 0; i < 4; ++i)
                 if (4u * g + (uint32_t)i < (uint32_t)NCL) pp[(wave * 16u + r) * NCL + 4u * g + i] = yacc[i];
             yacc = lev_f32x4{0.f, 0.f, 0.f, 0.f};
-            __syncthreads();
+            lev_barrier_lds();
             if (tid < 16u * NCL) {
                 const uint32_t col = tid >> 4, rr = tid & 15u, row = rg * 16u + rr;
                 float sum = 0.f;

@@ -183,3 +183,27 @@ def write_gguf(kvs, tensors, version=3, alignment=None, pad_data_to=None) -> byt
     if pad_data_to is not None:
         out += b"\0" * max(0, pad_data_to - len(out))
     return out
+
+
+def check_moe_layer_token(y, ids, wts, ref_ids, ref_w, gate, up, down, hidden, inter, x, tol=1e-4):
+    """Parity of one token of the whole MoE block, stated as the reference states it:
+    the router and the expert composite have separate contracts.
+      * expert ids: bit-exact with the CPU route (F32 matvec + f64 softmax / top-k);
+      * routing weights: within 2e-5 relative of the CPU route (the device accumulates
+        the router scores in f64, the CPU reference in f32, so they are not bit-equal);
+      * expert composite: the output against the FP64 oracle evaluated on the routing
+        weights the device produced, at the reference's 1e-4 (MoESIMDOracle.contract);
+      * and against the FP64 oracle on the CPU route's weights the output may differ by
+        that 1e-4 plus what the weight difference itself moves it:
+        sum_slot |w_dev - w_cpu| * |down_slot|.
+    Returns the composite's error."""
+    assert ids.tolist() == list(ref_ids), (ids, ref_ids)
+    assert np.allclose(wts, ref_w, rtol=2e-5)
+    ref = O.moe_experts_f64(gate, up, down, hidden, inter, ids, wts, x)
+    err = O.max_rel_err(y, ref["y"])
+    assert err < tol, err
+    ref_cpu = O.moe_experts_f64(gate, up, down, hidden, inter, ref_ids, ref_w, x)
+    moved = np.abs(wts.astype(np.float64) - np.asarray(ref_w, np.float64)) @ np.abs(ref_cpu["dn"])
+    slack = tol * np.maximum(1.0, np.abs(ref_cpu["y"])) + moved
+    assert np.all(np.abs(y - ref_cpu["y"]) <= slack)
+    return err

@@ -16,11 +16,6 @@ pytestmark = pytest.mark.gpu
 
 TOL = 1e-4
 GEMM_TOL = 1e-3
-# Cases whose outputs are O(100) with summed magnitudes O(1000): there an f32
-# accumulation sits within a factor ~2 of 1e-4 whatever the order, and the
-# reference's own f32 CPU order measures 1.7e-4 on the same inputs.  These
-# carry the wider stated bound; everything else is held to 1e-4.
-TOL_WIDE = 2e-4
 
 
 @pytest.fixture(scope="module")
@@ -266,11 +261,20 @@ def test_moe_tail_region_fused_gate_up_layout(ctx):
     # merged output: three terms of up to 1e15 cancel, so the bound is relative
     # to the largest term
     assert np.max(np.abs(y[0] - y_ref)) <= 1e-5 * np.max(np.abs(y_ref))
-    # end to end against the full FP64 oracle (MoESIMDOracle.reference), where
-    # the stages' errors compound: relative accuracy at the wide bound
+    # end to end against the full FP64 oracle (MoESIMDOracle.reference): the activation
+    # may differ by the 1e-4 of its own stage plus what the (gated) error of the gate|up
+    # stage moves it: d(gelu(g)*u) <= |gelu'|*|u|*dg + |gelu(g)|*du with |gelu'| < 1.13
+    # and |gelu(g)| <= |g|.  With values up to 1e15 no fixed constant says that.
     ref = O.moe_experts_f64(gu, gu[up_rel:], dn, hidden, inter, [0, 1, 2], [1, 1, 1], x[0],
                             (gu_stride, gu_stride, dn_stride))
-    assert O.max_rel_err(act[0], ref["act"]) < TOL_WIDE
+    for slot in range(top_k):
+        gu_gpu = ctx.q4_0_gemv(gu_d, dev(x[0]), hidden, 2 * inter, w_off=slot * gu_stride)
+        ctx.sync()
+        gu_gpu = gu_gpu.cpu().numpy().astype(np.float64)
+        g_ref, u_ref = ref["gate"][slot], ref["up"][slot]
+        dg, du = np.abs(gu_gpu[:inter] - g_ref), np.abs(gu_gpu[inter:] - u_ref)
+        slack = TOL * np.maximum(1.0, np.abs(ref["act"][slot])) + 1.2 * (np.abs(u_ref) * dg + np.abs(g_ref) * du)
+        assert np.all(np.abs(act[0, slot] - ref["act"][slot]) <= slack)
     assert np.max(np.abs(y[0] - ref["y"])) <= 1e-3 * np.max(np.abs(ref["y"]))
 
 
@@ -322,16 +326,11 @@ def test_moe_layer_config5(ctx, tokens):
     ctx.sync()
     y, ids, wts = y.cpu().numpy(), ids.cpu().numpy(), wts.cpu().numpy()
     g, u, d = (pool[offs["gate_off"]:], pool[offs["up_off"]:], pool[offs["down_off"]:])
-    worst = 0.0
     for t in range(tokens):
         ref_scores, ref_ids, ref_w = cpu_route(wr, x[t], top_k)
         order = np.sort(ref_scores)[::-1]
         assert float(np.min(np.diff(-order[:top_k + 1]))) > 1e-5, "degenerate seed"
-        assert ids[t].tolist() == ref_ids.tolist()                  # expert ids bit-exact
-        assert np.allclose(wts[t], ref_w, rtol=2e-5)
-        ref = O.moe_experts_f64(g, u, d, hidden, inter, ref_ids, ref_w, x[t])
-        worst = max(worst, O.max_rel_err(y[t], ref["y"]))
-    assert worst < (TOL if tokens == 1 else TOL_WIDE)
+        H.check_moe_layer_token(y[t], ids[t], wts[t], ref_ids, ref_w, g, u, d, hidden, inter, x[t], TOL)
     # batch invariance (main.swift:9053-9056: a schedule gives the same bits whatever
     # else is in the batch).  Two schedules exist here: up to four tokens every
     # (token, slot) streams its expert alone on the vector ALU; from five tokens
@@ -365,10 +364,7 @@ def test_moe_layer_small_and_odd_expert_counts(ctx, hidden, inter, experts, top_
     g, u, d = (pool[offs["gate_off"]:], pool[offs["up_off"]:], pool[offs["down_off"]:])
     for t in range(tokens):
         _, ref_ids, ref_w = cpu_route(wr, x[t], top_k)
-        assert ids[t].tolist() == ref_ids.tolist()
-        assert np.allclose(wts[t], ref_w, rtol=2e-5)
-        ref = O.moe_experts_f64(g, u, d, hidden, inter, ref_ids, ref_w, x[t])
-        assert O.max_rel_err(y[t], ref["y"]) < TOL_WIDE
+        H.check_moe_layer_token(y[t], ids[t], wts[t], ref_ids, ref_w, g, u, d, hidden, inter, x[t], TOL)
 
 
 # ---------------------------------------------------------- prefill GEMM ----
