@@ -92,11 +92,17 @@ __device__ __forceinline__ void wave_lds_fence() {
 __host__ __device__ constexpr size_t router_lds_bytes(uint32_t j) {
     return (size_t)(64u * j) * 12u + 64u * 8u + 64u * 4u;
 }
+// ... plus the eight waves' partial rank counts of the register-based selection
+__host__ __device__ constexpr size_t router_lds_bytes_fast(uint32_t j) {
+    return router_lds_bytes(j) + (size_t)8u * (64u * j) * 4u;
+}
 
 struct router_sel {
     const double *sel_p;     // LDS: probabilities of the selected experts, selection order
     const uint32_t *sel_id;  // LDS: their indices
     bool ok;                 // false: a score was not finite, nothing selected
+    uint32_t e_slot = 0xFFFFFFFFu;   // register-based selection: the expert of the slot asked for;
+                                     // sel_p / sel_id are then only filled when need_p was set
 };
 
 // softmax (f64) + top-k (ties -> lower index) for one token
@@ -116,25 +122,51 @@ struct router_sel {
 // same result), so the only exchanges are the table, the ranks and the winners.
 // need_p = false (uniform over the workgroup): the caller only wants the ids;
 // sel_p is then not meaningful.
+// The token's scores as every wave holds them: lane l keeps experts j*64 + l.
+template <int J>
+__device__ __forceinline__ void router_load_scores(const float *__restrict__ srow, uint32_t experts,
+                                                   float (&sc)[J]) {
+    const uint32_t lane = threadIdx.x & 63u;
+#pragma unroll
+    for (int j = 0; j < J; ++j) {
+        const uint32_t i = lane + 64u * j;
+        sc[j] = srow[i < experts ? i : experts - 1u];
+    }
+}
+
+template <int J>
+__device__ router_sel router_select_regs(const float (&sc)[J], void *lds, uint32_t experts,
+                                         uint32_t top_k, bool need_p, bool fast, uint32_t slot = 0);
+
 template <int J>
 __device__ router_sel router_select_block(const float *__restrict__ srow, void *lds,
                                           uint32_t experts, uint32_t top_k, bool need_p = true) {
+    float sc[J];
+    router_load_scores<J>(srow, experts, sc);
+    return router_select_regs<J>(sc, lds, experts, top_k, need_p, false);
+}
+
+// fast (workgroup-uniform, J <= 8, blockDim = 512): ranks are counted from
+// registers, the waves splitting the table between them: a wave broadcasts its
+// share of the keys lane by lane (v_readlane) and every lane compares its own
+// J keys against them; the waves' partial counts meet in LDS.  One barrier
+// less than the table walk and no LDS atomics.  Only when the integer keys
+// order the probabilities (the common case); the result is the same.
+template <int J>
+__device__ router_sel router_select_regs(const float (&sc)[J], void *lds, uint32_t experts,
+                                         uint32_t top_k, bool need_p, bool fast, uint32_t slot) {
     constexpr uint32_t padded = 64u * J;
     uint64_t *table = static_cast<uint64_t *>(lds);   // probabilities (f64) or order keys
     double *sel_p = reinterpret_cast<double *>(table + padded);
     uint32_t *rank = reinterpret_cast<uint32_t *>(sel_p + 64);
     uint32_t *sel_id = rank + padded;
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-    router_sel out{sel_p, sel_id, true};
+    router_sel out{sel_p, sel_id, true, 0xFFFFFFFFu};
 
-    float sc[J];
     float mx = -INFINITY;
     bool finite = true;
 #pragma unroll
     for (int j = 0; j < J; ++j) {
-        const uint32_t i = lane + 64u * j;
-        const bool valid = i < experts;
-        sc[j] = srow[valid ? i : experts - 1u];
         finite = finite && isfinite(sc[j]);
         mx = fmaxf(mx, sc[j]);
     }
@@ -175,6 +207,62 @@ __device__ router_sel router_select_block(const float *__restrict__ srow, void *
         sum = wave_sum_f64(sum);
 #pragma unroll
         for (int j = 0; j < J; ++j) p[j] = lane + 64u * j < experts ? p[j] / sum : 0.0;
+    }
+    if constexpr (J <= 8) {
+        if (fast && by_key && blockDim.x == 512u) {
+            // wave w broadcasts table entries w*share .. +share (one register set: share divides 64)
+            constexpr uint32_t share = padded / 8u;
+            // the wave index as a scalar: the lane selects below must be uniform registers
+            const uint32_t first = (uint32_t)__builtin_amdgcn_readfirstlane((int)wave) * share;
+            uint64_t src = key[0];
+#pragma unroll
+            for (int j = 1; j < J; ++j) src = (first >> 6) == (uint32_t)j ? key[j] : src;
+            const uint32_t lo = (uint32_t)src, hi = (uint32_t)(src >> 32);
+            uint32_t cnt[J];
+#pragma unroll
+            for (int j = 0; j < J; ++j) cnt[j] = 0u;
+#pragma unroll
+            for (uint32_t k = 0; k < share; ++k) {
+                const uint32_t l = (first & 63u) + k;
+                const uint64_t other = ((uint64_t)(uint32_t)__builtin_amdgcn_readlane((int)hi, l) << 32) |
+                                       (uint32_t)__builtin_amdgcn_readlane((int)lo, l);
+#pragma unroll
+                for (int j = 0; j < J; ++j) cnt[j] += other < key[j] ? 1u : 0u;
+            }
+            uint32_t *part = sel_id + 64;   // partial counts [wave][padded], behind the regular areas
+#pragma unroll
+            for (int j = 0; j < J; ++j) part[wave * padded + lane + 64u * j] = cnt[j];
+            lev_barrier_lds();
+            // every wave adds up the ranks of its own copies of the keys: no second exchange
+            uint32_t total[J];
+#pragma unroll
+            for (int j = 0; j < J; ++j) {
+                uint32_t r = 0;
+#pragma unroll
+                for (uint32_t w = 0; w < 8u; ++w) r += part[w * padded + lane + 64u * j];
+                total[j] = lane + 64u * j < experts ? r : 0xFFFFFFFFu;
+            }
+            // the expert of `slot`: the one element whose rank is slot (ranks are a permutation)
+            uint32_t found = 0xFFFFFFFFu;
+#pragma unroll
+            for (int j = 0; j < J; ++j) {
+                const unsigned long long hit = __ballot(total[j] == slot);
+                if (hit != 0ull) found = (uint32_t)__builtin_ctzll(hit) + 64u * (uint32_t)j;
+            }
+            out.e_slot = found;
+            if (need_p) {   // the publishing workgroup also lists all winners with their probabilities
+                if (wave == 0) {
+#pragma unroll
+                    for (int j = 0; j < J; ++j)
+                        if (total[j] < top_k) {
+                            sel_id[total[j]] = lane + 64u * j;
+                            sel_p[total[j]] = p[j];
+                        }
+                }
+                lev_barrier_lds();
+            }
+            return out;
+        }
     }
     if (wave == 0) {
 #pragma unroll
@@ -396,6 +484,20 @@ moe_topk_kernel(const float *__restrict__ scores, const float *__restrict__ expe
 // other slot names the same one.  Run by a whole wave (top_k <= 64): lane k
 // reads ids[k], so the check costs one memory round trip however many slots
 // there are.
+__device__ __forceinline__ int32_t expert_ids_request(const int32_t *ids, uint32_t top_k) {
+    const uint32_t lane = threadIdx.x & 63u;
+    return ids[lane < top_k ? lane : top_k - 1u];
+}
+
+__device__ __forceinline__ bool expert_ids_verdict(int32_t mine, uint32_t top_k, uint32_t slot,
+                                                   uint32_t experts, uint32_t *expert) {
+    const uint32_t lane = threadIdx.x & 63u;
+    const int32_t me = __builtin_amdgcn_readlane(mine, slot);
+    const unsigned long long same = __ballot(lane < top_k && mine == me);
+    *expert = (uint32_t)me;
+    return me >= 0 && (uint32_t)me < experts && __popcll(same) == 1;
+}
+
 __device__ __forceinline__ bool expert_ids_ok(const int32_t *ids, uint32_t top_k, uint32_t slot,
                                               uint32_t experts, uint32_t *expert) {
     const uint32_t lane = threadIdx.x & 63u;
@@ -479,20 +581,24 @@ moe_gate_up_kernel(moe_args a, const float *__restrict__ x, const int32_t *ids,
     float *bsum = reinterpret_cast<float *>(xs + 16u * (pairs + 1u));
     const float *xt = x + (uint64_t)t * a.hidden;
 
+    // Request order = return order on a CU (its memory pipeline hands data back in
+    // the order it was asked for): the scores, which the expert id and with it
+    // every weight address hang on, go out first, the activations second.
+    float sc[ROUTE > 0 ? ROUTE : 1];
+    if constexpr (ROUTE > 0) router_load_scores<ROUTE>(scores + (uint64_t)t * a.experts, a.experts, sc);
     lev_f32x4 xv[NS];
     lev_q4_stage_x_load<NS>(xt, pairs, tid, kGuThreads, xv);
 
     uint32_t e;
-    router_sel r{nullptr, nullptr, true};
+    router_sel r{nullptr, nullptr, true, 0xFFFFFFFFu};
     if constexpr (ROUTE > 0) {
         // 8-byte aligned as it stands: xs is 16-byte aligned and 2*pairs floats
         // follow 16*(pairs+1) vectors.  (Rounding the address up through an
         // integer would hide from the compiler that this is LDS.)
         void *rl = bsum + 2u * pairs;
         // only the workgroup that publishes the selection needs the probabilities
-        r = router_select_block<ROUTE>(scores + (uint64_t)t * a.experts, rl, a.experts, a.top_k,
-                                       blockIdx.x == 0 && slot == 0);
-        e = r.ok ? r.sel_id[slot] : slot;
+        r = router_select_regs<ROUTE>(sc, rl, a.experts, a.top_k, blockIdx.x == 0 && slot == 0, true, slot);
+        e = !r.ok ? slot : r.e_slot != 0xFFFFFFFFu ? r.e_slot : r.sel_id[slot];
     } else {
         const int32_t *tids = ids + (uint64_t)t * a.top_k;
         if (!expert_ids_ok(tids, a.top_k, slot, a.experts, &e)) {
@@ -508,8 +614,11 @@ moe_gate_up_kernel(moe_args a, const float *__restrict__ x, const int32_t *ids,
 
     uint32_t Da[P][R][9], Db[P][R][9];
     uint32_t i0 = i_begin + wave * R;
-    gu_load_rows<P, R>(wbase, row_bytes, i0, a.inter, pairs, lp, Da);
+    // The activations were requested before anything else and have landed by
+    // now: they go to LDS before the weight requests leave, so that the wait for
+    // them cannot end up behind the weights.
     lev_q4_stage_x_store_sums<NS>(xt, xs, bsum, pairs, tid, kGuThreads, xv);
+    gu_load_rows<P, R>(wbase, row_bytes, i0, a.inter, pairs, lp, Da);
     lev_barrier_lds();
     if constexpr (ROUTE > 0) {
         // the first workgroup of a token publishes the selection while its
@@ -593,8 +702,15 @@ moe_down_kernel(moe_args a, const float *__restrict__ act, const int32_t *__rest
 
     bool bad = false;
     for (uint32_t slot = wave; slot < a.top_k; slot += kDnWaves) {
+        // request order = return order: the ids (the weight addresses hang on them)
+        // first, then this slot's activations, so that both are on their way while
+        // the id is checked and neither waits behind the weights
+        const int32_t ids_mine = expert_ids_request(tids, a.top_k);
+        const float *av = act + ((uint64_t)t * a.top_k + slot) * a.inter;
+        lev_f32x4 av4[kLevStageSlots];
+        lev_q4_stage_x_load<kLevStageSlots>(av, pairs, lane, 64u, av4);
         uint32_t e;
-        if (!expert_ids_ok(tids, a.top_k, slot, a.experts, &e)) {
+        if (!expert_ids_verdict(ids_mine, a.top_k, slot, a.experts, &e)) {
             bad = true;
             for (uint32_t r = lane; r < tile; r += 64u) partial[slot * tile + r] = 0.f;
             continue;
@@ -609,8 +725,7 @@ moe_down_kernel(moe_args a, const float *__restrict__ act, const int32_t *__rest
         };
         load_row(0, Da);
         // this wave's slot activations -> its private LDS region (wave-local)
-        const float *av = act + ((uint64_t)t * a.top_k + slot) * a.inter;
-        lev_q4_stage_x(av, xs, pairs, lane, 64u);
+        lev_q4_stage_x_store<kLevStageSlots>(av, xs, pairs, lane, 64u, av4);
         // wave-private region: LDS executes one wave's accesses in order, the
         // fences only stop the compiler from moving the reads above the writes
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -748,8 +863,10 @@ hipError_t launch_gate_up(lev_ctx *ctx, const moe_args &a, const float *x, const
     uint64_t slots = (uint64_t)a.top_k * tokens;
     uint32_t want_blocks_per_slot = (uint32_t)(((uint64_t)ctx->num_cus * 2u + slots - 1) / slots);
     if (want_blocks_per_slot < 1) want_blocks_per_slot = 1;
+    // (not rounded to whole steps: with 12 rows per workgroup half of its waves take
+    // a second row, which beats 16 rows on three quarters of the workgroups)
     uint32_t rows_per_block = (a.inter + want_blocks_per_slot - 1) / want_blocks_per_slot;
-    rows_per_block = (rows_per_block + step - 1) / step * step;
+    (void)step;
     uint32_t chunks = (a.inter + rows_per_block - 1) / rows_per_block;
     const uint32_t pairs = a.hidden / 64u;
     size_t lds = (size_t)16 * (pairs + 1u) * sizeof(lev_f32x4) + (size_t)2 * pairs * sizeof(float);
@@ -759,7 +876,7 @@ hipError_t launch_gate_up(lev_ctx *ctx, const moe_args &a, const float *x, const
                            a, x, rt.ids, nullptr, nullptr, nullptr, nullptr, act, ctx->d_flag,
                            rows_per_block);
     } else {
-        lds += 8 + router_lds_bytes(a.experts <= 128u ? 2u : 4u);
+        lds += 8 + router_lds_bytes_fast(a.experts <= 128u ? 2u : 4u);
         if (a.experts <= 128u)
             hipLaunchKernelGGL((moe_gate_up_kernel<P, R, NS, 2>), grid, dim3(kGuThreads), lds, ctx->stream,
                                a, x, nullptr, rt.scores, rt.expert_scale, rt.ids_out, rt.weights_out,
@@ -781,7 +898,7 @@ hipError_t launch_down(lev_ctx *ctx, const moe_args &a, const float *act, const 
     if (want_tiles < 1) want_tiles = 1;
     uint32_t tile = (a.hidden + want_tiles - 1) / want_tiles;
     uint32_t steps = (tile + G - 1) / G;
-    if (steps < 2) steps = 2;
+    if (steps < 1) steps = 1;
     if (steps > 64) steps = 64;
     tile = steps * G;
     uint32_t tiles = (a.hidden + tile - 1) / tile;
@@ -859,7 +976,10 @@ hipError_t run_experts(lev_ctx *ctx, const moe_args &a, const float *x, const gu
                            ctx->stream, a, act, ids, weights, y, ctx->d_flag);
         return hipGetLastError();
     }
-    if (a.hidden <= 2048u) e = launch_gate_up<1, 3, 1>(ctx, a, x, rt, act, tokens);
+    // One row pair per wave and step: what a wave does after its last byte has
+    // landed is issued at one instruction per eight cycles whatever else runs
+    // on the SIMD, so many short waves finish sooner than few long ones.
+    if (a.hidden <= 2048u) e = launch_gate_up<1, 1, 1>(ctx, a, x, rt, act, tokens);
     else e = launch_gate_up<2, 1, 2>(ctx, a, x, rt, act, tokens);
     if (e != hipSuccess) return e;
     const uint32_t dp = a.inter / 64u;

@@ -59,14 +59,6 @@ struct q6_unit_w {
 __device__ __forceinline__ void q6_load_unit(const uint8_t *row, uint32_t g, q6_unit_w &u) {
     const uint32_t sb = g >> 3, half = (g >> 2) & 1u, v = g & 3u;
     const uint8_t *blk = row + (uint64_t)sb * 210u;
-#ifdef LEV_EXP_NO_LOADS
-    {
-        const uint32_t z = (uint32_t)(uintptr_t)blk * 2654435761u;
-        for (int i = 0; i < 4; ++i) u.ql[i] = z + i, u.qh[i] = z ^ i;
-        u.sc[0] = z; u.sc[1] = ~z; u.d = 0x2000u + (z & 255u);
-        return;
-    }
-#endif
     u32x4_a2 a = *reinterpret_cast<const u32x4_a2 *>(blk + 64u * half + 16u * v);
     u32x4_a2 b = *reinterpret_cast<const u32x4_a2 *>(blk + 128u + 32u * half + 16u * (v & 1u));
     u32x2_a2 c = *reinterpret_cast<const u32x2_a2 *>(blk + 192u + 8u * half);
@@ -370,10 +362,6 @@ q6_k_gemv_exact(const uint8_t *__restrict__ w, const float *__restrict__ x, floa
 #pragma unroll
         for (int p = 0; p < P; ++p) {
             const uint32_t g = lu + p * L;
-#ifdef LEV_EXP_NO_COMPUTE
-            acc += (double)(W[p].ql[0] ^ W[p].ql[1] ^ W[p].ql[2] ^ W[p].ql[3] ^ W[p].qh[0] ^ W[p].qh[1] ^ W[p].qh[2] ^ W[p].qh[3] ^ W[p].sc[0] ^ W[p].sc[1] ^ W[p].d);
-            continue;
-#endif
             if (RESIDENT) {
                 acc += q6_unit_dot_exact(W[p], X[p], Mlo[p], Mhi[p], g & 3u);
             } else {
