@@ -335,17 +335,14 @@ hipError_t lev_q4_k_mfma_gemv_launch(lev_ctx *ctx, const uint8_t *w, const float
                                      float eps, float *y, uint32_t in_dim, uint32_t rows,
                                      uint32_t ncol);
 
-// Built-in kernel family (1 = matrix cores, 0 = vector ALU), from measurements on
-// MI355X: a single column of rows up to 8192 wide runs fastest on the vector-ALU
-// kernel (12288x4096: 8.1 against 10.6 us; it also starts faster: 2.5 against 4.6 us
-// for a small matrix), two columns only for rows up to 2048 wide or small matrices;
-// everything else on the matrix cores, where their activation staging fits.
+// Built-in kernel family (1 = integer matrix cores, 0 = vector ALU).  The
+// matrix-core kernel forms every dot product without rounding and is the choice
+// wherever its activation staging fits; the vector-ALU kernel (f32 FMA chains)
+// takes the other shapes and stays a candidate for lev_hip_forge_select.
 static uint32_t q4k_builtin_family(const lev_ctx *ctx, uint32_t in_dim, uint32_t rows, uint32_t ncol) {
-    if (lev_q4_k_mfma_cols(ctx, in_dim) == 0u) return 0u;
-    const uint32_t units = in_dim / 64u;
-    if (ncol == 1u && units <= 128u) return 0u;
-    if (ncol == 2u && (units <= 32u || (uint64_t)rows * in_dim <= (8u << 20))) return 0u;
-    return 1u;
+    (void)rows;
+    (void)ncol;
+    return lev_q4_k_mfma_cols(ctx, in_dim) == 0u ? 0u : 1u;
 }
 
 hipError_t lev_q4_k_gemv_launch(lev_ctx *ctx, const uint8_t *w, const float *x, const float *gain,

@@ -66,8 +66,8 @@ def test_q4_k_candidates_pass_the_gate(ctx, rows, cols, ncol):
     ref = np.stack([O.q4_k_matvec_f64(w, rows, cols, x[c]) for c in range(ncol)])
     dw, dx = dev(w), dev(x)
     cands = ctx.forge_candidates(capi.OP_Q4_K_GEMV, cols, rows, ncol)
-    # one column of rows up to 4096 wide: the vector-ALU kernel is the built-in choice; else the matrix cores
-    assert [c.family for c in cands] == ([0, 1] if ncol == 1 else [1, 0])
+    # the integer matrix-core kernel (exact sums) is the built-in choice wherever its staging fits
+    assert [c.family for c in cands] == [1, 0]
     outs = []
     try:
         for s in cands:

@@ -378,15 +378,12 @@ def test_q4_k_rust_fixture_16x1024(ctx):
     assert O.max_rel_err(got, O.q4_k_matvec_f64(w, 16, 1024, x)) < TOL
 
 
-# Tolerance of the Q4_K cases drawn from the benchmark distribution (uniform
-# codes, 6-bit scales, d and dmin ~ |N(0, 0.01)|): every output is the small
-# difference of a d*sc*q sum and a dmin*m sum, so ANY 24-bit accumulation sits
-# near 1e-4 of max(1, |y|) -- the reference's own f32 CPU order
-# (matvec_q4k_f32, lev-cpu/src/lib.rs:158-176) measures 1.2e-4 to 4.4e-4 against
-# FP64 on these very inputs.  The matrix-core kernel carries x as two fp16
-# halves (22 bits) and lands at <= 1.1e-4.  The reference's own fixtures
-# (test_q4_k_rust_fixture_16x1024 above) stay at 1e-4.
-TOL_Q4K_BENCH = 2e-4
+# The Q4_K cases drawn from the benchmark distribution (uniform codes, 6-bit
+# scales, d and dmin ~ |N(0, 0.01)|) are hard for 24-bit accumulation: every
+# output is the small difference of a d*sc*q sum and a dmin*m sum, and the
+# reference's own f32 CPU order (matvec_q4k_f32, lev-cpu/src/lib.rs:158-176)
+# measures 1.2e-4 to 4.4e-4 against FP64 on these very inputs.  The kernel forms
+# the sums without rounding and is held to the reference's 1e-4 like every other case.
 
 
 @pytest.mark.parametrize("ncol", [1, 2, 3, 4, 5, 8, 16])
@@ -396,10 +393,10 @@ def test_q4_k_ncol_shapes_with_rmsnorm(ctx, rows, cols, ncol):
     got = q4k_gemv(ctx, w, x, rows, cols, ncol, gain)
     xn = H.rmsnorm_rows(x, gain)
     for c in range(ncol):
-        assert O.max_rel_err(got[c], O.q4_k_matvec_f64(w, rows, cols, xn[c])) < TOL_Q4K_BENCH, c
+        assert O.max_rel_err(got[c], O.q4_k_matvec_f64(w, rows, cols, xn[c])) < TOL, c
     plain = q4k_gemv(ctx, w, x, rows, cols, ncol)                # no norm
     for c in range(ncol):
-        assert O.max_rel_err(plain[c], O.q4_k_matvec_f64(w, rows, cols, x[c])) < TOL_Q4K_BENCH, c
+        assert O.max_rel_err(plain[c], O.q4_k_matvec_f64(w, rows, cols, x[c])) < TOL, c
 
 
 @pytest.mark.parametrize("ncol", [1, 2, 3, 4, 8])
@@ -408,15 +405,62 @@ def test_q4_k_config3_full_size(ctx, ncol):
     got = q4k_gemv(ctx, w, x, 12288, 4096, ncol, gain)
     xn = H.rmsnorm_rows(x, gain)
     for c in range(ncol):
-        assert O.max_rel_err(got[c], O.q4_k_matvec_f64(w, 12288, 4096, xn[c])) < TOL_Q4K_BENCH, c
-    # columns are independent: column 0 alone gives the same bits when the same kernel
-    # serves it (one column runs on the vector-ALU kernel, two and more on the matrix
-    # cores at this shape), and the same value to 1e-5 otherwise
+        assert O.max_rel_err(got[c], O.q4_k_matvec_f64(w, 12288, 4096, xn[c])) < TOL, c
+    # columns are independent: column 0 alone gives the same bits
     alone = q4k_gemv(ctx, w, x[:1], 12288, 4096, 1, gain)
-    if ncol == 1:
-        assert np.array_equal(bits(alone[0]), bits(got[0]))
-    else:   # two f32 accumulation orders, each within TOL_Q4K_BENCH of the FP64 oracle
-        assert O.max_rel_err(alone[0], got[0].astype(np.float64)) < TOL_Q4K_BENCH
+    assert np.array_equal(bits(alone[0]), bits(got[0]))
+
+
+@pytest.mark.parametrize("ncol", [1, 4, 8])
+@pytest.mark.parametrize("rows,cols", [(16389, 1024), (5000, 8192)])
+def test_q4_k_many_row_groups_per_workgroup(ctx, rows, cols, ncol):
+    """More than three tasks per wave (tall matrices, rows of 32 superblocks): the kernel's
+    loop with three loads in flight instead of its straight-line form."""
+    w, x, gain = H.config3(rows, cols, ncol, seed=rows % 97 + ncol)
+    got = q4k_gemv(ctx, w, x, rows, cols, ncol, gain)
+    xn = H.rmsnorm_rows(x, gain)
+    for c in range(ncol):
+        assert O.max_rel_err(got[c], O.q4_k_matvec_f64(w, rows, cols, xn[c])) < TOL, c
+
+
+def test_q4_k_exact_sums_do_not_depend_on_the_scale_of_x(ctx):
+    """The dot products are formed in integers per superblock: scaling x by a power of two
+    scales every output by exactly that power, and tiny or huge activations lose nothing."""
+    rows, cols = 64, 4096
+    w, x, _ = H.config3(rows, cols, 2, seed=21)
+    base = q4k_gemv(ctx, w, x, rows, cols, 2)
+    for e in (-60, -20, 20, 60):
+        got = q4k_gemv(ctx, w, np.ldexp(x, e).astype(np.float32), rows, cols, 2)
+        assert np.array_equal(bits(got), bits(np.ldexp(base, e).astype(np.float32))), e
+
+
+def test_q4_k_mixed_magnitudes_within_a_row(ctx):
+    """Superblocks of very different magnitude in one row: each carries its own power of two."""
+    rows, cols = 48, 4096
+    w, x, gain = H.config3(rows, cols, 3, seed=8)
+    x = x.copy()
+    x[:, 256:512] *= 1e-6
+    x[:, 1024:1280] *= 3e4
+    x[1, 2048:2304] = 0.0
+    got = q4k_gemv(ctx, w, x, rows, cols, 3)
+    for c in range(3):
+        assert O.max_rel_err(got[c], O.q4_k_matvec_f64(w, rows, cols, x[c])) < TOL, c
+
+
+def test_q4_k_non_finite_activation_reaches_the_output(ctx):
+    """A NaN or an infinity in a column of x makes that column's outputs NaN (the
+    reference's sums would hold NaN or infinities there); the other columns are untouched."""
+    rows, cols = 40, 4096
+    w, x, gain = H.config3(rows, cols, 3, seed=13)
+    clean = q4k_gemv(ctx, w, x, rows, cols, 3, gain)
+    for bad in (np.nan, np.inf, -np.inf):
+        xb = x.copy()
+        xb[1, 777] = bad
+        got = q4k_gemv(ctx, w, xb, rows, cols, 3)
+        assert np.isnan(got[1]).all(), bad
+        plain = q4k_gemv(ctx, w, x, rows, cols, 3)
+        assert np.array_equal(bits(got[0]), bits(plain[0])) and np.array_equal(bits(got[2]), bits(plain[2]))
+    assert np.isfinite(clean).all()
 
 
 def test_q4_k_embedding_gather_bit_exact(ctx):
