@@ -501,6 +501,22 @@ public:
         check(lev_hip_axpy(ctx_, xp, y.floats(), c, (uint32_t)n), "axpy");
     }
 
+    // ---- Gemma4.swift:3742-3773: the shared expert beside the routed ones ----
+    // bufH = rmsnorm(bufX, ffn_norm); gate|up fused into bufGU ([0..I) gate, [I..2I) up through a
+    // 256-aligned byte offset); bufAct = geluUp(bufGU); bufShared = rmsnorm(down bufAct,
+    // post_ffw_norm_1).  bufH is left holding the normed input for the routed experts.
+    void sharedExpert(const std::string &prefix, const DeviceBuffer &bufX, DeviceBuffer &bufH,
+                      DeviceBuffer &bufGU, DeviceBuffer &bufAct, DeviceBuffer &bufShared, int64_t hidden,
+                      int64_t sharedIntermediate) {
+        rmsnorm(bufX, bufH, hidden, 1, prefix + "ffn_norm.weight");
+        matvec(prefix + "ffn_gate.weight", bufH, hidden, bufGU, 2 * sharedIntermediate);
+        matvec(prefix + "ffn_up.weight", bufH, hidden, bufGU, 2 * sharedIntermediate, 0, std::nullopt,
+               sharedIntermediate * 4);
+        geluUp(bufGU, bufAct, sharedIntermediate);
+        matvec(prefix + "ffn_down.weight", bufAct, sharedIntermediate, bufShared, hidden);
+        rmsnorm(bufShared, bufShared, hidden, 1, prefix + "post_ffw_norm_1.weight");
+    }
+
     // ---- Gemma4.swift:3795-3810: router scores, softmax, top-k, renormalise ----
     // routerTensor is F32 [experts][hidden].  Returns (topIdx, weights) for one token.
     std::pair<std::vector<int>, std::vector<float>>

@@ -257,6 +257,31 @@ class Context:
         self._check(self.lib.lev_hip_axpy(self.ctx, _ptr(x), _ptr(y), c, n))
         return y
 
+    def shared_expert_ffn(self, x, ffn_norm, gate_w, up_w, down_w, post_norm, hidden: int, inter: int,
+                          eps: float = 1e-6, bufs=None):
+        """The shared expert that runs beside the routed ones (Gemma4.swift:3742-3773):
+        h = rmsnorm(x, ffn_norm); gu = [gate h | up h] (Q4_0 matvecs, up at float offset
+        `inter` of the one buffer); act = gelu_up(gu); shared = rmsnorm(down act, post_norm).
+        `bufs` = (h, gu, act, shared) to reuse buffers (a recorded program needs fixed ones).
+        Returns (h, shared): h also feeds the routed experts."""
+        if inter % 32 or hidden % 32 or (inter * 4) % 256:
+            raise LevError(capi.BAD_DIMENSIONS,
+                           f"shared expert: hidden {hidden} / intermediate {inter} (blocks of 32, up half 256-byte aligned)")
+        if bufs is None:
+            dev = x.device
+            bufs = (torch.empty(hidden, dtype=torch.float32, device=dev),
+                    torch.empty(2 * inter, dtype=torch.float32, device=dev),
+                    torch.empty(inter, dtype=torch.float32, device=dev),
+                    torch.empty(hidden, dtype=torch.float32, device=dev))
+        h, gu, act, shared = bufs
+        self.rmsnorm(x, hidden, 1, weight=ffn_norm, eps=eps, y=h)
+        self.q4_0_gemv(gate_w, h, hidden, inter, y=gu)
+        self.q4_0_gemv(up_w, h, hidden, inter, y=gu[inter:])
+        self.gelu_up(gu, inter, y=act)
+        self.q4_0_gemv(down_w, act, inter, hidden, y=shared)
+        self.rmsnorm(shared, hidden, 1, weight=post_norm, eps=eps, y=shared)
+        return h, shared
+
     def argmax(self, logits, vocab: int, ncol: int = 1):
         _dev(logits, torch.float32, "logits")
         idx = torch.empty(max(ncol, 1), dtype=torch.int32, device=logits.device)

@@ -146,6 +146,7 @@ struct Model {
     // one weight buffer: a Q4_0 matrix, a Q6_K matrix, an F32 norm weight, an
     // F32 router and the expert tensors of layer 0, at 256-byte aligned offsets
     static constexpr int hidden = 256, inter = 128, experts = 8, topK = 2, vocab = 96;
+    static constexpr int sharedInter = 192;   // a multiple of 64: the up half of gate|up starts 256-byte aligned
     std::vector<uint8_t> bytes;
     std::map<std::string, TensorRef> table;
     MoEBinding binding;
@@ -175,6 +176,17 @@ struct Model {
             [](uint8_t *p, size_t n) { levo_fill_normal(34, 0.f, 0.02f, reinterpret_cast<float *>(p), n / 4); });
         add("blk.0.ffn_up.weight", GGMLTensorType::q4_K, hidden, 64, 1,
             [](uint8_t *p, size_t n) { levo_synth_q4_k(37, 0.01f, p, n / 144); });
+        // the shared expert of layer 1 (Gemma4.swift:3742-3773)
+        add("blk.1.ffn_norm.weight", GGMLTensorType::float32, hidden, 1, 1,
+            [](uint8_t *p, size_t n) { levo_fill_normal(61, 1.f, 0.1f, reinterpret_cast<float *>(p), n / 4); });
+        add("blk.1.post_ffw_norm_1.weight", GGMLTensorType::float32, hidden, 1, 1,
+            [](uint8_t *p, size_t n) { levo_fill_normal(62, 1.f, 0.1f, reinterpret_cast<float *>(p), n / 4); });
+        add("blk.1.ffn_gate.weight", GGMLTensorType::q4_0, hidden, sharedInter, 1,
+            [](uint8_t *p, size_t n) { levo_synth_q4_0(63, 0.02f, p, n / 18); });
+        add("blk.1.ffn_up.weight", GGMLTensorType::q4_0, hidden, sharedInter, 1,
+            [](uint8_t *p, size_t n) { levo_synth_q4_0(64, 0.02f, p, n / 18); });
+        add("blk.1.ffn_down.weight", GGMLTensorType::q4_0, sharedInter, hidden, 1,
+            [](uint8_t *p, size_t n) { levo_synth_q4_0(65, 0.02f, p, n / 18); });
         // fused gate|up [2I, H] per expert, as the reference stores it
         int64_t gu = add("blk.0.ffn_gate_up_exps.weight", GGMLTensorType::q4_0, hidden, 2 * inter, experts,
                          [](uint8_t *p, size_t n) { levo_synth_q4_0(35, 0.02f, p, n / 18); });
@@ -669,6 +681,43 @@ void forge_matvec(Runner &r) {
     EXPECT(lev_hip_forge_candidates(ctx, LEV_OP_Q4_0_GEMV, 4096, 512, 1, nullptr, 0, &n) == LEV_OK && n == 6);
 }
 
+// Gemma4.swift:3742-3773: rmsnorm -> gate, up (one buffer) -> geluUp -> down -> rmsnorm,
+// against the same chain on the CPU (FP64 matvecs and norms, f32 between the steps)
+void runner_shared_expert(Runner &r, const Model &m) {
+    const int H = Model::hidden, I = Model::sharedInter;
+    std::vector<float> x(H);
+    levo_fill_normal(71, 0.f, 1.f, x.data(), H);
+    DeviceBuffer dx = r.makeBuffer(x), dh = r.makeBuffer((int64_t)H * 4), dgu = r.makeBuffer((int64_t)2 * I * 4),
+                 dact = r.makeBuffer((int64_t)I * 4), dsh = r.makeBuffer((int64_t)H * 4);
+    r.sharedExpert("blk.1.", dx, dh, dgu, dact, dsh, H, I);
+    std::vector<float> got = r.read<float>(dsh, H), got_h = r.read<float>(dh, H);
+
+    auto f32 = [](const std::vector<double> &v) { return std::vector<float>(v.begin(), v.end()); };
+    auto tensor_bytes = [&](const char *name) { const TensorRef &t = m.table.at(name); return (size_t)(t.end - t.offset); };
+    std::vector<double> hd(H), gd(I), ud(I), dd(H), sd(H);
+    levo_rmsnorm_f64(x.data(), reinterpret_cast<const float *>(m.at("blk.1.ffn_norm.weight")), 1e-6, H, hd.data());
+    EXPECT(rel_err(got_h, hd) < 1e-5);
+    std::vector<float> h = f32(hd);
+    EXPECT(levo_q4_0_matvec_f64(m.at("blk.1.ffn_gate.weight"), tensor_bytes("blk.1.ffn_gate.weight"), I, H, h.data(), H, gd.data()) == 0);
+    EXPECT(levo_q4_0_matvec_f64(m.at("blk.1.ffn_up.weight"), tensor_bytes("blk.1.ffn_up.weight"), I, H, h.data(), H, ud.data()) == 0);
+    std::vector<float> g = f32(gd), u = f32(ud), act(I);
+    for (int i = 0; i < I; ++i) act[i] = levo_gelu_up_f32(g[i], u[i]);
+    EXPECT(levo_q4_0_matvec_f64(m.at("blk.1.ffn_down.weight"), tensor_bytes("blk.1.ffn_down.weight"), H, I, act.data(), I, dd.data()) == 0);
+    std::vector<float> d = f32(dd);
+    levo_rmsnorm_f64(d.data(), reinterpret_cast<const float *>(m.at("blk.1.post_ffw_norm_1.weight")), 1e-6, H, sd.data());
+    EXPECT(rel_err(got, sd) < 1e-4);
+    // the two halves of gate|up are where the reference binds them
+    std::vector<float> gu = r.read<float>(dgu, (size_t)2 * I);
+    EXPECT(rel_err(std::vector<float>(gu.begin(), gu.begin() + I), gd) < 1e-4);
+    EXPECT(rel_err(std::vector<float>(gu.begin() + I, gu.end()), ud) < 1e-4);
+    // guards: an intermediate size whose up half would not start 256-byte aligned, short buffers
+    DeviceBuffer small = r.makeBuffer((int64_t)I * 4);
+    EXPECT(throws_geometry([&] { r.sharedExpert("blk.1.", dx, dh, small, dact, dsh, H, I); }));
+    EXPECT(throws_geometry([&] { r.sharedExpert("blk.1.", dx, dh, dgu, dact, dsh, H, I - 32); }));
+    EXPECT(throws_geometry([&] { r.sharedExpert("blk.7.", dx, dh, dgu, dact, dsh, H, I); }));
+    r.flushOpenSegment();
+}
+
 int main(int argc, char **argv) {
     Model model;
     std::unique_ptr<Runner> runner;
@@ -688,6 +737,7 @@ int main(int argc, char **argv) {
         {"runner_matvec", [&] { runner_matvec(R(), model); }},
         {"runner_elementwise", [&] { runner_elementwise(R(), model); }},
         {"runner_int8_path", [&] { runner_int8_path(R(), model); }},
+        {"runner_shared_expert", [&] { runner_shared_expert(R(), model); }},
         {"runner_moe", [&] { runner_moe(R(), model); }},
         {"runner_moe_hand_computed", [&] { runner_moe_hand_computed(R()); }},
         {"runner_gguf_file", [&] { runner_gguf_file(R(), model); }},

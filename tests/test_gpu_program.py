@@ -267,3 +267,77 @@ def test_q6_k_argmax_records_on_a_fresh_context():
         assert abs(float(mg.item()) - float(top[0] - top[1])) <= 1e-6 * max(1.0, abs(float(top[0])))
     prog.destroy()
     ctx.close()
+
+
+def test_shared_expert_ffn_recorded_program_matches_the_cpu_chain():
+    """The shared expert beside the routed ones (Gemma4.swift:3742-3773) at the model's
+    sizes (hidden 2048, shared intermediate 2112): rmsnorm -> gate, up into one buffer ->
+    geluUp -> down -> rmsnorm, then x += shared.  Eager against the same chain on the CPU
+    (FP64 matvecs and norms, f32 between the steps) at 1e-4; recorded once and replayed
+    with changed inputs, with the program's own eager work in between, bit for bit."""
+    from leviathan_amd import ops
+    hidden, inter = 2048, 2112
+    stream = torch.cuda.Stream()
+    ctx = ops.Context(0, stream=stream)
+    gate = O.synth_q4_0(81, inter * hidden // 32, 0.02)
+    up = O.synth_q4_0(82, inter * hidden // 32, 0.02)
+    down = O.synth_q4_0(83, hidden * inter // 32, 0.02)
+    ffn_norm = O.normal(hidden, 84, 1.0, 0.1)
+    post_norm = O.normal(hidden, 85, 1.0, 0.1)
+    xs = [O.normal(hidden, 90 + i) for i in range(4)]
+    dgate, dup, ddown, dfn, dpn = dev(gate), dev(up), dev(down), dev(ffn_norm), dev(post_norm)
+    x = torch.zeros(hidden, device="cuda")
+    resid = torch.zeros(hidden, device="cuda")
+    bufs = (torch.empty(hidden, device="cuda"), torch.empty(2 * inter, device="cuda"),
+            torch.empty(inter, device="cuda"), torch.empty(hidden, device="cuda"))
+
+    def step():
+        h, shared = ctx.shared_expert_ffn(x, dfn, dgate, dup, ddown, dpn, hidden, inter, bufs=bufs)
+        ctx.axpy(shared, resid, 1.0, hidden)                    # x += shared (Gemma4.swift:3115)
+        return h, shared
+
+    def load(v):
+        with torch.cuda.stream(stream):
+            x.copy_(torch.from_numpy(v))
+            resid.copy_(torch.from_numpy(v))
+
+    def cpu_chain(v):
+        h = O.rmsnorm_f64(v, ffn_norm, 1e-6).astype(np.float32)
+        g = O.q4_0_matvec_f64(gate, inter, hidden, h).astype(np.float32)
+        u = O.q4_0_matvec_f64(up, inter, hidden, h).astype(np.float32)
+        act = np.array([O.gelu_up_f32(float(a), float(b)) for a, b in zip(g, u)], np.float32)
+        d = O.q4_0_matvec_f64(down, hidden, inter, act).astype(np.float32)
+        return h, g, u, act, O.rmsnorm_f64(d, post_norm, 1e-6)
+
+    eager = []
+    for v in xs:
+        load(v)
+        h, shared = step()
+        ctx.sync()
+        ref_h, ref_g, ref_u, ref_act, ref_shared = cpu_chain(v)
+        assert O.max_rel_err(h.cpu().numpy(), ref_h.astype(np.float64)) < 1e-5
+        gu = bufs[1].cpu().numpy()
+        assert O.max_rel_err(gu[:inter], ref_g.astype(np.float64)) < 1e-4     # gate half
+        assert O.max_rel_err(gu[inter:], ref_u.astype(np.float64)) < 1e-4     # up half, at its byte offset
+        assert O.max_rel_err(shared.cpu().numpy(), ref_shared) < 1e-4
+        assert O.max_rel_err(resid.cpu().numpy(), v.astype(np.float64) + ref_shared) < 1e-4
+        eager.append([t.clone() for t in (*bufs, resid)])
+
+    load(xs[0])
+    ctx.program_begin()
+    step()
+    prog = ctx.program_end()
+    assert prog.node_count() >= 7                               # 2 norms, 3 matvecs, geluUp, axpy
+    for i in (2, 0, 3, 1, 2):
+        load(xs[i])
+        prog.run()
+        ctx.sync()
+        for a, b in zip([*bufs, resid], eager[i]):
+            assert torch.equal(a, b), i
+        load(xs[(i + 1) % 4])                                   # eager work between the replays
+        step()
+        ctx.sync()
+    prog.destroy()
+    with pytest.raises(ops.LevError):
+        ctx.shared_expert_ffn(x, dfn, dgate, dup, ddown, dpn, hidden, 2112 - 32, bufs=bufs)   # up half unaligned
+    ctx.close()
