@@ -323,16 +323,28 @@ int lev_hip_q6_k_matvec_reporting(const uint8_t *blocks, size_t blocks_count, in
  * schedule names one of the precompiled kernel variants.  Candidate 0 is
  * always the built-in choice (the reference's BASELINE).  A selection applies
  * to exactly one (op, in_dim, rows, ncol) on this context and is consulted by
- * lev_hip_q4_0_gemv / lev_hip_q4_k_gemv_ncol / lev_hip_q4_k_gemv_q8 before their
- * built-in choice. */
+ * the operator's entry point before its built-in choice.  The Q6_K head and the
+ * MoE layer have candidates as the reference's own forges do (vk_q6k,
+ * lev-cli/src/main.rs:467 and lev-forge/src/q6k.rs:175; MoELoweringForge.forge,
+ * MoELowering.swift:1896-1985).  For LEV_OP_MOE_LAYER_Q4_0 the shape is
+ * (in_dim = hidden, rows = expert intermediate size, ncol = tokens, 1..4). */
 #define LEV_OP_Q4_0_GEMV 1u
 #define LEV_OP_Q4_K_GEMV 2u
 #define LEV_OP_Q4_K_GEMV_Q8 3u
+#define LEV_OP_Q6_K_GEMV 4u
+#define LEV_OP_Q6_K_GEMV_Q8 5u
+#define LEV_OP_MOE_LAYER_Q4_0 6u
 typedef struct lev_schedule {
     uint32_t op;             /* LEV_OP_* */
-    uint32_t family;         /* Q4_K: 1 = matrix-core kernel, 0 = vector-ALU (int8: dot4) kernel; Q4_0: 0 */
-    uint32_t rows_in_flight; /* Q4_0: rows a wave keeps in flight (1, 2, 4; 0 = no variants for the shape) */
-    uint32_t persistent;     /* Q4_0: 0 = one workgroup per row tile, 1 = resident grid walking the tiles */
+    uint32_t family;         /* Q4_K: 1 = matrix-core kernel, 0 = vector-ALU (int8: dot4) kernel; Q4_0: 0;
+                                Q6_K: 0 = exact digit-plane kernel, 1 = one wave per row with f64 sums;
+                                Q6_K x int8: 0; MoE layer: 1 = the gate/up workgroups select the experts
+                                themselves, 0 = a top-k kernel of its own ahead of them */
+    uint32_t rows_in_flight; /* Q4_0: rows a wave keeps in flight (1, 2, 4; 0 = no variants for the shape);
+                                Q6_K: waves that share a row (1, 2); Q6_K x int8: columns per pass over the
+                                weights; MoE layer: gate/up workgroups aimed at per CU (1, 2, 4) */
+    uint32_t persistent;     /* Q4_0, Q6_K x int8: 0 = one workgroup per row tile, 1 = resident grid walking
+                                the tiles */
 } lev_schedule;
 /* Writes min(*count, capacity) candidates; *count is the full number. */
 int lev_hip_forge_candidates(lev_ctx *ctx, uint32_t op, uint32_t in_dim, uint32_t rows,

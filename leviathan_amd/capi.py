@@ -57,6 +57,7 @@ class Schedule(C.Structure):
 
 
 OP_Q4_0_GEMV, OP_Q4_K_GEMV, OP_Q4_K_GEMV_Q8 = 1, 2, 3
+OP_Q6_K_GEMV, OP_Q6_K_GEMV_Q8, OP_MOE_LAYER_Q4_0 = 4, 5, 6
 
 _vp, _sz, _u64, _u32, _f32, _i64, _int = (C.c_void_p, C.c_size_t, C.c_uint64, C.c_uint32, C.c_float,
                                           C.c_int64, C.c_int)

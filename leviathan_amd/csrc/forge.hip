@@ -16,6 +16,12 @@ uint32_t lev_q4_k_gemv_candidates(const lev_ctx *ctx, uint32_t in_dim, uint32_t 
                                   lev_schedule *out, uint32_t capacity);
 uint32_t lev_q4_k_gemv_q8_candidates(const lev_ctx *ctx, uint32_t in_dim, uint32_t rows, uint32_t ncol,
                                      lev_schedule *out, uint32_t capacity);
+uint32_t lev_q6_k_gemv_candidates(const lev_ctx *ctx, uint32_t in_dim, uint32_t rows, lev_schedule *out,
+                                  uint32_t capacity);
+uint32_t lev_q6_k_gemv_q8_candidates(const lev_ctx *ctx, uint32_t in_dim, uint32_t rows, uint32_t ncol,
+                                     lev_schedule *out, uint32_t capacity);
+uint32_t lev_moe_layer_candidates(const lev_ctx *ctx, uint32_t hidden, uint32_t inter, uint32_t tokens,
+                                  lev_schedule *out, uint32_t capacity);
 
 const lev_schedule *lev_selected(const lev_ctx *ctx, uint32_t op, uint32_t in_dim, uint32_t rows, uint32_t ncol) {
     for (const lev_ctx::selection &s : ctx->selections)
@@ -28,13 +34,15 @@ namespace {
 constexpr uint32_t kMaxCandidates = 16;
 
 int shape_ok(lev_ctx *ctx, uint32_t op, uint32_t in_dim, uint32_t rows, uint32_t ncol) {
-    const uint32_t block = op == LEV_OP_Q4_0_GEMV ? 32u : 256u;
-    if (op != LEV_OP_Q4_0_GEMV && op != LEV_OP_Q4_K_GEMV && op != LEV_OP_Q4_K_GEMV_Q8)
+    if (op < LEV_OP_Q4_0_GEMV || op > LEV_OP_MOE_LAYER_Q4_0)
         return lev_fail(ctx, LEV_ERR_INVALID_ARGUMENT, "forge: unknown op %u", op);
-    if (in_dim == 0 || rows == 0 || in_dim % block != 0 || in_dim > LEV_MAX_Q4_INPUT_DIM ||
-        rows > LEV_MAX_Q4_OUTPUT_DIM)
+    const bool moe = op == LEV_OP_MOE_LAYER_Q4_0;
+    const uint32_t block = op == LEV_OP_Q4_0_GEMV || moe ? 32u : 256u;
+    if (in_dim == 0 || rows == 0 || in_dim % block != 0 || (moe && rows % block != 0) ||
+        in_dim > LEV_MAX_Q4_INPUT_DIM || rows > LEV_MAX_Q4_OUTPUT_DIM)
         return lev_fail(ctx, LEV_ERR_BAD_DIMENSIONS, "forge: %u x %u is not a shape of this op", rows, in_dim);
-    if (ncol == 0 || ncol > LEV_MAX_GEMV_COLUMNS || (op == LEV_OP_Q4_0_GEMV && ncol != 1))
+    const bool one_column = op == LEV_OP_Q4_0_GEMV || op == LEV_OP_Q6_K_GEMV;
+    if (ncol == 0 || ncol > (moe ? 4u : (uint32_t)LEV_MAX_GEMV_COLUMNS) || (one_column && ncol != 1))
         return lev_fail(ctx, LEV_ERR_BAD_DIMENSIONS, "forge: %u columns", ncol);
     return LEV_OK;
 }
@@ -43,6 +51,9 @@ uint32_t candidates(const lev_ctx *ctx, uint32_t op, uint32_t in_dim, uint32_t r
                     lev_schedule *out, uint32_t capacity) {
     if (op == LEV_OP_Q4_0_GEMV) return lev_q4_0_gemv_candidates(ctx, in_dim, rows, out, capacity);
     if (op == LEV_OP_Q4_K_GEMV) return lev_q4_k_gemv_candidates(ctx, in_dim, rows, ncol, out, capacity);
+    if (op == LEV_OP_Q6_K_GEMV) return lev_q6_k_gemv_candidates(ctx, in_dim, rows, out, capacity);
+    if (op == LEV_OP_Q6_K_GEMV_Q8) return lev_q6_k_gemv_q8_candidates(ctx, in_dim, rows, ncol, out, capacity);
+    if (op == LEV_OP_MOE_LAYER_Q4_0) return lev_moe_layer_candidates(ctx, in_dim, rows, ncol, out, capacity);
     return lev_q4_k_gemv_q8_candidates(ctx, in_dim, rows, ncol, out, capacity);
 }
 

@@ -856,12 +856,12 @@ struct gu_route {
 
 template <int P, int R, int NS>
 hipError_t launch_gate_up(lev_ctx *ctx, const moe_args &a, const float *x, const gu_route &rt,
-                          float *act, uint32_t tokens) {
-    // rows per workgroup: about two workgroups per CU at one token, more rows
-    // per workgroup (less re-staging of x) at many
+                          float *act, uint32_t tokens, uint32_t per_cu) {
+    // rows per workgroup: about per_cu (two, unless a schedule says otherwise)
+    // workgroups per CU at one token, more rows per workgroup (less re-staging of x) at many
     constexpr uint32_t step = kGuWaves * R;
     uint64_t slots = (uint64_t)a.top_k * tokens;
-    uint32_t want_blocks_per_slot = (uint32_t)(((uint64_t)ctx->num_cus * 2u + slots - 1) / slots);
+    uint32_t want_blocks_per_slot = (uint32_t)(((uint64_t)ctx->num_cus * per_cu + slots - 1) / slots);
     if (want_blocks_per_slot < 1) want_blocks_per_slot = 1;
     // (not rounded to whole steps: with 12 rows per workgroup half of its waves take
     // a second row, which beats 16 rows on three quarters of the workgroups)
@@ -966,7 +966,7 @@ bool experts_fast(const moe_args &a, const float *x) {
 // fast path: callers test experts_fast() first.
 hipError_t run_experts(lev_ctx *ctx, const moe_args &a, const float *x, const gu_route &rt,
                        const int32_t *ids, const float *weights, float *y, float *act,
-                       uint32_t tokens, bool fast) {
+                       uint32_t tokens, bool fast, uint32_t gu_per_cu = 2u) {
     hipError_t e;
     if (!fast) {
         hipLaunchKernelGGL(moe_gate_up_generic, dim3((a.inter + 3) / 4, a.top_k, tokens), dim3(256), 0,
@@ -979,8 +979,8 @@ hipError_t run_experts(lev_ctx *ctx, const moe_args &a, const float *x, const gu
     // One row pair per wave and step: what a wave does after its last byte has
     // landed is issued at one instruction per eight cycles whatever else runs
     // on the SIMD, so many short waves finish sooner than few long ones.
-    if (a.hidden <= 2048u) e = launch_gate_up<1, 1, 1>(ctx, a, x, rt, act, tokens);
-    else e = launch_gate_up<2, 1, 2>(ctx, a, x, rt, act, tokens);
+    if (a.hidden <= 2048u) e = launch_gate_up<1, 1, 1>(ctx, a, x, rt, act, tokens, gu_per_cu);
+    else e = launch_gate_up<2, 1, 2>(ctx, a, x, rt, act, tokens, gu_per_cu);
     if (e != hipSuccess) return e;
     const uint32_t dp = a.inter / 64u;
     if (dp > 32) return launch_down<64>(ctx, a, act, ids, weights, y, tokens);
@@ -1162,7 +1162,12 @@ int moe_layer_impl(lev_ctx *ctx, const lev_moe_experts *pools, const float *d_ro
     if (st != LEV_OK) return st;
     const bool fast = experts_fast(a, d_x);
     gu_route rt{d_ids, nullptr, nullptr, nullptr, nullptr};
-    if (fast && tokens <= 4u && a.experts <= kRouteInKernelMax) {
+    // a schedule installed for this shape (lev_hip_forge_select) overrides the built-in choice
+    const lev_schedule *sel = tokens <= 4u ? lev_selected(ctx, LEV_OP_MOE_LAYER_Q4_0, a.hidden, a.inter, tokens)
+                                           : nullptr;
+    const bool select_in_kernel = !(sel && sel->family == 0u);
+    const uint32_t gu_per_cu = sel && sel->rows_in_flight ? sel->rows_in_flight : 2u;
+    if (fast && tokens <= 4u && a.experts <= kRouteInKernelMax && select_in_kernel) {
         // few tokens: the gate/up workgroups select the experts themselves
         rt = gu_route{nullptr, s.scores, d_expert_scale, d_ids, d_weights};
     } else {
@@ -1177,11 +1182,38 @@ int moe_layer_impl(lev_ctx *ctx, const lev_moe_experts *pools, const float *d_ro
                              lev_moe_grouped_launch(ctx, grouped_args(a, tokens), d_x, d_ids, d_weights,
                                                     d_y, s.act, s.grouped),
                              "moe grouped experts launch");
-    return lev_hip_check(ctx, run_experts(ctx, a, d_x, rt, d_ids, d_weights, d_y, s.act, tokens, fast),
+    return lev_hip_check(ctx,
+                         run_experts(ctx, a, d_x, rt, d_ids, d_weights, d_y, s.act, tokens, fast, gu_per_cu),
                          "moe experts launch");
 }
 
 }  // namespace
+
+// Candidate schedules of the MoE layer at one to four tokens, the built-in choice
+// first (MoELoweringForge.forge, MoELowering.swift:1896-1985, derives and gates the
+// lowered layer the same way): who selects the experts (the gate/up workgroups
+// themselves, or a top-k kernel of its own ahead of them: one launch more, no
+// redundant selection) and how many gate/up workgroups per CU the rows are cut
+// into.  Every candidate computes each row with the same lanes in the same order:
+// their outputs agree bit for bit.  (Shapes the streaming kernels cannot take run
+// the generic kernels whatever is selected.)
+uint32_t lev_moe_layer_candidates(const lev_ctx *ctx, uint32_t hidden, uint32_t inter, uint32_t tokens,
+                                  lev_schedule *out, uint32_t capacity) {
+    (void)ctx;
+    (void)hidden;
+    (void)inter;
+    (void)tokens;
+    uint32_t n = 0;
+    auto add = [&](uint32_t family, uint32_t per_cu) {
+        if (n < capacity) out[n] = lev_schedule{LEV_OP_MOE_LAYER_Q4_0, family, per_cu, 0u};
+        ++n;
+    };
+    add(1u, 2u);
+    add(1u, 1u);
+    add(1u, 4u);
+    add(0u, 2u);
+    return n;
+}
 
 extern "C" int lev_hip_moe_layer_q4_0(lev_ctx *ctx, const lev_moe_experts *pools,
                                       const float *d_router_w, const float *d_expert_scale,

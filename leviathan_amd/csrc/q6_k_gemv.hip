@@ -565,13 +565,46 @@ hipError_t launch_units(lev_ctx *ctx, const uint8_t *w, const float *x, float *y
 
 }  // namespace
 
+namespace {
+bool q6_exact_usable(const uint8_t *w, const float *x, uint32_t units) {
+    return ((reinterpret_cast<uintptr_t>(w) & 1u) == 0u) && ((reinterpret_cast<uintptr_t>(x) & 15u) == 0u) &&
+           units <= 256u;
+}
+}  // namespace
+
+// Candidate schedules of a Q6_K GEMV shape, the built-in choice first (vk_q6k,
+// lev-cli/src/main.rs:467; the q6k.matvec variants of lev-forge/src/q6k.rs:175):
+// the exact digit-plane kernel, for rows of 65..128 units with two waves or one
+// wave per row, and the one-wave-per-row kernel with f64 sums.  (Pointer alignment
+// is not part of a shape: a selection of the exact kernel is ignored for operands
+// it cannot take.)
+uint32_t lev_q6_k_gemv_candidates(const lev_ctx *ctx, uint32_t in_dim, uint32_t rows, lev_schedule *out,
+                                  uint32_t capacity) {
+    (void)ctx;
+    (void)rows;
+    const uint32_t units = in_dim / 32u;
+    uint32_t n = 0;
+    auto add = [&](uint32_t family, uint32_t waves) {
+        if (n < capacity) out[n] = lev_schedule{LEV_OP_Q6_K_GEMV, family, waves, 0u};
+        ++n;
+    };
+    if (units <= 256u) {
+        const bool pair = units > 64u && units <= 128u;
+        add(0u, pair ? 2u : 1u);
+        if (pair) add(0u, 1u);
+    }
+    add(1u, 1u);
+    return n;
+}
+
 // GEMV with the greedy-token epilogue: d_argmax / d_margin may be NULL.
 hipError_t lev_q6_k_gemv_argmax_launch(lev_ctx *ctx, const uint8_t *w, const float *x, float *y,
                                        uint32_t in_dim, uint32_t rows, uint32_t *d_argmax,
                                        float *d_margin) {
     const uint32_t units = in_dim / 32u;   // 8 per superblock
-    const bool fast = ((reinterpret_cast<uintptr_t>(w) & 1u) == 0u) &&
-                      ((reinterpret_cast<uintptr_t>(x) & 15u) == 0u) && units <= 256u;
+    // a schedule installed for this shape (lev_hip_forge_select) overrides the built-in choice
+    const lev_schedule *sel = lev_selected(ctx, LEV_OP_Q6_K_GEMV, in_dim, rows, 1);
+    const bool fast = q6_exact_usable(w, x, units) && !(sel && sel->family == 1u);
     if (!fast) {
         uint32_t blocks = (rows + kWaves - 1) / kWaves;
         hipLaunchKernelGGL(q6_k_gemv_generic, dim3(blocks), dim3(kThreads), 0, ctx->stream, w, x, y,
@@ -583,7 +616,11 @@ hipError_t lev_q6_k_gemv_argmax_launch(lev_ctx *ctx, const uint8_t *w, const flo
         return hipGetLastError();
     }
     if (units > 128) return launch_units<64, 4, false>(ctx, w, x, y, units, rows, d_argmax, d_margin);
-    if (units > 64) return launch_units<64, 1, true, 2>(ctx, w, x, y, units, rows, d_argmax, d_margin);
+    if (units > 64) {
+        if (sel && sel->rows_in_flight == 1u)
+            return launch_units<64, 2, true, 1>(ctx, w, x, y, units, rows, d_argmax, d_margin);
+        return launch_units<64, 1, true, 2>(ctx, w, x, y, units, rows, d_argmax, d_margin);
+    }
     if (units > 32) return launch_units<64, 1>(ctx, w, x, y, units, rows, d_argmax, d_margin);
     if (units > 16) return launch_units<32, 1>(ctx, w, x, y, units, rows, d_argmax, d_margin);
     if (units > 8) return launch_units<16, 1>(ctx, w, x, y, units, rows, d_argmax, d_margin);

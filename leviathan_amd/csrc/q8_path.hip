@@ -393,7 +393,7 @@ q6_k_gemv_q8_kernel(const uint8_t *__restrict__ w, const uint32_t *__restrict__ 
 
 template <int NC>
 hipError_t launch_q6_q8(lev_ctx *ctx, const uint8_t *w, const uint32_t *xq, const float *xs, float *y,
-                        uint32_t in_dim, uint32_t rows, uint32_t ncol) {
+                        uint32_t in_dim, uint32_t rows, uint32_t ncol, bool persistent) {
     const size_t lds = (size_t)NC * (in_dim >> 8) * kQ6Stride;
     static size_t configured = 0;
     if (lds > 48 * 1024 && lds > configured) {
@@ -408,7 +408,7 @@ hipError_t launch_q6_q8(lev_ctx *ctx, const uint8_t *w, const uint32_t *xq, cons
         per_cu = 1;
     const uint32_t tiles = (rows + kQ6Rows - 1u) / kQ6Rows;
     uint32_t blocks = (uint32_t)ctx->num_cus * (uint32_t)per_cu;
-    if (blocks > tiles) blocks = tiles;
+    if (blocks > tiles || !persistent) blocks = tiles;
     hipLaunchKernelGGL((q6_k_gemv_q8_kernel<NC>), dim3(blocks), dim3(kQ6Threads), lds, ctx->stream, w, xq,
                        xs, y, in_dim, rows, ncol);
     return hipGetLastError();
@@ -822,6 +822,41 @@ extern "C" int lev_hip_q4_k_gemv_q8(lev_ctx *ctx, const void *d_w, size_t w_byte
     return LEV_OK;
 }
 
+// Columns one pass of the Q6_K x int8 kernel takes: the staged activations of up to
+// eight columns must fit the LDS (0: not even one does).
+static uint32_t q6_q8_cols_per_pass(const lev_ctx *ctx, uint32_t in_dim, uint32_t ncol) {
+    const size_t limit = ctx->props.sharedMemPerBlockOptin > ctx->props.sharedMemPerBlock
+                             ? ctx->props.sharedMemPerBlockOptin
+                             : ctx->props.sharedMemPerBlock;
+    const size_t per_col = (size_t)(in_dim >> 8) * kQ6Stride;
+    if (per_col > limit) return 0;
+    uint32_t fit = 8;
+    while (fit > 1u && fit * per_col > limit) fit >>= 1;
+    uint32_t nc = 1;
+    while (nc < ncol && nc < fit) nc <<= 1;   // the kernel is built for 1, 2, 4 and 8 columns
+    return nc;
+}
+
+// Candidate schedules of a Q6_K x int8 GEMV shape, the built-in choice first
+// (q6k.matvec over int8 activations, lev-forge/src/q8.rs:328-447): a resident grid
+// or a workgroup per row tile, all columns in one pass over the weights or half
+// of them in each of two.
+uint32_t lev_q6_k_gemv_q8_candidates(const lev_ctx *ctx, uint32_t in_dim, uint32_t rows, uint32_t ncol,
+                                     lev_schedule *out, uint32_t capacity) {
+    (void)rows;
+    const uint32_t all = q6_q8_cols_per_pass(ctx, in_dim, ncol);
+    uint32_t n = 0;
+    auto add = [&](uint32_t cols, uint32_t persistent) {
+        if (n < capacity) out[n] = lev_schedule{LEV_OP_Q6_K_GEMV_Q8, 0u, cols, persistent};
+        ++n;
+    };
+    if (all == 0) return 0;
+    add(all, 1u);
+    add(all, 0u);
+    if (all >= 2u) add(all / 2u, 1u);
+    return n;
+}
+
 extern "C" int lev_hip_q6_k_gemv_q8(lev_ctx *ctx, const void *d_w, size_t w_bytes, uint64_t w_off,
                                     const int8_t *d_xq, const float *d_xs, size_t x_count, float *d_y,
                                     size_t y_capacity, uint32_t in_dim, uint32_t rows, uint32_t ncol) {
@@ -846,8 +881,13 @@ extern "C" int lev_hip_q6_k_gemv_q8(lev_ctx *ctx, const void *d_w, size_t w_byte
     const size_t per_col = (size_t)(in_dim >> 8) * kQ6Stride;
     if (per_col > limit)
         return lev_fail(ctx, LEV_ERR_EXCEEDS_MODEL_WORKLOAD, "q6_k_gemv_q8: inDim %u does not fit the staging", in_dim);
-    uint32_t fit = 8;
-    while (fit > 1u && fit * per_col > limit) fit >>= 1;
+    uint32_t fit = q6_q8_cols_per_pass(ctx, in_dim, ncol);
+    bool persistent = true;
+    // a schedule installed for this shape (lev_hip_forge_select) overrides the built-in choice
+    if (const lev_schedule *sel = lev_selected(ctx, LEV_OP_Q6_K_GEMV_Q8, in_dim, rows, ncol)) {
+        if (sel->rows_in_flight >= 1u && sel->rows_in_flight < fit) fit = sel->rows_in_flight;
+        persistent = sel->persistent != 0u;
+    }
     const uint32_t *xq = reinterpret_cast<const uint32_t *>(d_xq);
     uint32_t done = 0;
     while (done < ncol) {
@@ -857,10 +897,10 @@ extern "C" int lev_hip_q6_k_gemv_q8(lev_ctx *ctx, const void *d_w, size_t w_byte
         const float *xsc = d_xs + (uint64_t)done * (in_dim >> 5) * 2u;
         float *yc = d_y + (uint64_t)done * rows;
         hipError_t e;
-        if (nc > 4) e = launch_q6_q8<8>(ctx, w, xqc, xsc, yc, in_dim, rows, nc);
-        else if (nc > 2) e = launch_q6_q8<4>(ctx, w, xqc, xsc, yc, in_dim, rows, nc);
-        else if (nc > 1) e = launch_q6_q8<2>(ctx, w, xqc, xsc, yc, in_dim, rows, nc);
-        else e = launch_q6_q8<1>(ctx, w, xqc, xsc, yc, in_dim, rows, nc);
+        if (nc > 4) e = launch_q6_q8<8>(ctx, w, xqc, xsc, yc, in_dim, rows, nc, persistent);
+        else if (nc > 2) e = launch_q6_q8<4>(ctx, w, xqc, xsc, yc, in_dim, rows, nc, persistent);
+        else if (nc > 1) e = launch_q6_q8<2>(ctx, w, xqc, xsc, yc, in_dim, rows, nc, persistent);
+        else e = launch_q6_q8<1>(ctx, w, xqc, xsc, yc, in_dim, rows, nc, persistent);
         if (e != hipSuccess) return lev_hip_check(ctx, e, "q6_k_gemv_q8 launch");
         done += nc;
     }

@@ -9,8 +9,11 @@
 // beats the baseline's by more than 2 %.  The reference compiles an emitted
 // shader per candidate and caches the binary by source hash; here a candidate is
 // a precompiled kernel variant of the library (lev_hip_forge_candidates) and the
-// cache holds the selection, keyed by operator, shape, device name and ABI
-// version.  The FP64 products below follow matvec_q4k_f64 / dequant_block_f64
+// cache holds the selection, keyed by operator, shape, device name, ABI version and
+// a hash of this build's candidate table for the shape; a cached selection is gated
+// again (one launch) before it is installed.  Candidates are timed over rotating
+// copies of the weights, so that a matrix that fits the last-level cache is timed as
+// decode meets it: from HBM.  The FP64 products below follow matvec_q4k_f64 / dequant_block_f64
 // (lev-cpu/src/lib.rs:134-195) and Q4Oracle.matvecFP64 (Q4Lowering.swift:1215);
 // they only accept or reject a candidate and never supply an output.
 #pragma once
@@ -59,8 +62,9 @@ struct ForgeOptions {
     double margin = 0.02;         // a non-baseline candidate must be more than this much faster
     uint64_t seed = 0x4C455649ull;
     std::string cachePath;        // empty: no cache
-    // Q4_K only: forge the int8-activation GEMV (lev_hip_q4_k_gemv_q8) instead of the
-    // f32 one.  The activations are quantised on the device and the oracle is the FP64
+    size_t rotateBytes = (size_t)512 << 20;   // weight copies cycled through while timing (at most 64)
+    // Q4_K and Q6_K: forge the int8-activation GEMV (lev_hip_q4_k_gemv_q8,
+    // lev_hip_q6_k_gemv_q8) instead of the f32 one.  The activations are quantised on the device and the oracle is the FP64
     // product over those same codes (q * d), as `lev vk-q8` gates it
     // (lev-cli/src/main.rs:1788-1868).
     bool int8Activations = false;
@@ -127,6 +131,28 @@ inline void q4_kRowF64(const uint8_t *row, int64_t inDim, const float *x, double
     }
 }
 
+// q6k_unpack + matvec_q6k_f64, lev-cpu/src/lib.rs:203-300
+inline void q6_kRowF64(const uint8_t *row, int64_t inDim, const float *x, double &sum) {
+    for (int64_t b = 0; b < inDim / 256; ++b) {
+        const uint8_t *blk = row + b * 210, *ql = blk, *qh = blk + 128;
+        const int8_t *sc = reinterpret_cast<const int8_t *>(blk + 192);
+        const double d = halfToDouble((uint16_t)(blk[208] | blk[209] << 8));
+        for (int half = 0; half < 2; ++half)
+            for (int l = 0; l < 32; ++l) {
+                const int is = l / 16, h = qh[32 * half + l];
+                const int q1 = ((ql[64 * half + l] & 0xF) | ((h & 3) << 4)) - 32;
+                const int q2 = ((ql[64 * half + 32 + l] & 0xF) | (((h >> 2) & 3) << 4)) - 32;
+                const int q3 = ((ql[64 * half + l] >> 4) | (((h >> 4) & 3) << 4)) - 32;
+                const int q4 = ((ql[64 * half + 32 + l] >> 4) | (((h >> 6) & 3) << 4)) - 32;
+                const float *xb = x + b * 256 + 128 * half;
+                const int8_t *s8 = sc + 8 * half;
+                sum += d * s8[is] * q1 * (double)xb[l];
+                sum += d * s8[is + 2] * q2 * (double)xb[32 + l];
+                sum += d * s8[is + 4] * q3 * (double)xb[64 + l];
+                sum += d * s8[is + 6] * q4 * (double)xb[96 + l];
+            }
+    }
+}
 inline double maxRelErr(const std::vector<float> &got, const std::vector<double> &ref) {
     if (got.size() != ref.size() || got.empty()) return -1.0;
     double worst = 0;
@@ -137,31 +163,64 @@ inline double maxRelErr(const std::vector<float> &got, const std::vector<double>
     return worst;
 }
 
-inline std::string cacheKey(uint32_t op, int64_t inDim, int64_t rows, int64_t ncol, std::string device) {
+// FNV-1a over the candidate table: a build whose variants differ has different keys
+inline uint64_t tableHash(const lev_schedule *list, uint32_t n) {
+    uint64_t h = 0xcbf29ce484222325ull;
+    auto mix = [&](uint32_t v) {
+        for (int i = 0; i < 4; ++i) {
+            h ^= (v >> (8 * i)) & 0xFFu;
+            h *= 0x100000001b3ull;
+        }
+    };
+    mix(n);
+    for (uint32_t i = 0; i < n; ++i) {
+        mix(list[i].op);
+        mix(list[i].family);
+        mix(list[i].rows_in_flight);
+        mix(list[i].persistent);
+    }
+    return h;
+}
+inline std::string cacheKey(uint32_t op, int64_t inDim, int64_t rows, int64_t ncol, std::string device,
+                            uint64_t table) {
     std::replace(device.begin(), device.end(), ' ', '_');
     std::ostringstream k;
-    k << "leviathan-forge-1 " << lev_hip_abi_version() << " " << device << " " << op << " " << inDim << " "
-      << rows << " " << ncol;
+    k << "leviathan-forge-2 " << lev_hip_abi_version() << " " << device << " " << table << " " << op << " "
+      << inDim << " " << rows << " " << ncol;
     return k.str();
+}
+inline double median(std::vector<double> v) {
+    if (v.empty()) return 0;
+    std::sort(v.begin(), v.end());
+    return v[v.size() / 2];
+}
+// candidate 0 must pass; the fastest passing candidate wins if it beats it by more than the margin
+inline int choose(const std::vector<ForgeCandidate> &c, double margin) {
+    if (c.empty() || !c[0].pass) return -1;
+    size_t best = 0;
+    for (size_t i = 1; i < c.size(); ++i)
+        if (c[i].pass && c[i].medianUs < c[best].medianUs) best = i;
+    return best != 0 && c[best].medianUs < c[0].medianUs * (1.0 - margin) ? (int)best : 0;
 }
 
 }  // namespace forge_detail
 
 class MatvecForge {
 public:
-    // `weights`: rows x inDim in the tensor's GGUF block layout (Q4_0 or Q4_K),
+    // `weights`: rows x inDim in the tensor's GGUF block layout (Q4_0, Q4_K or Q6_K),
     // as read from the file.  Leaves the selection installed on the runner's
     // context (or the built-in choice, when that won) and returns the report.
     static ForgeReport forge(Runner &r, GGMLTensorType type, const std::vector<uint8_t> &weights, int64_t rows,
                              int64_t inDim, int64_t ncol = 1, const ForgeOptions &opt = ForgeOptions()) {
         using namespace forge_detail;
-        if (type != GGMLTensorType::q4_0 && type != GGMLTensorType::q4_K)
-            throw Gemma4Error(Gemma4Error::badTensorGeometry, "forge: only Q4_0 and Q4_K matvecs have schedules");
-        if (opt.int8Activations && type != GGMLTensorType::q4_K)
-            throw Gemma4Error(Gemma4Error::badTensorGeometry, "forge: the int8-activation GEMV is Q4_K");
+        if (type != GGMLTensorType::q4_0 && type != GGMLTensorType::q4_K && type != GGMLTensorType::q6_K)
+            throw Gemma4Error(Gemma4Error::badTensorGeometry, "forge: Q4_0, Q4_K and Q6_K matvecs have schedules");
+        if (opt.int8Activations && type == GGMLTensorType::q4_0)
+            throw Gemma4Error(Gemma4Error::badTensorGeometry, "forge: the int8-activation GEMVs are Q4_K and Q6_K");
+        const bool q6 = type == GGMLTensorType::q6_K;
         const uint32_t op = type == GGMLTensorType::q4_0 ? LEV_OP_Q4_0_GEMV
-                            : opt.int8Activations       ? LEV_OP_Q4_K_GEMV_Q8
-                                                        : LEV_OP_Q4_K_GEMV;
+                            : q6 ? (opt.int8Activations ? LEV_OP_Q6_K_GEMV_Q8 : LEV_OP_Q6_K_GEMV)
+                                 : (opt.int8Activations ? LEV_OP_Q4_K_GEMV_Q8 : LEV_OP_Q4_K_GEMV);
         const int64_t per = elementsPerBlock(type), bpb = bytesPerBlock(type);
         if (rows <= 0 || inDim <= 0 || ncol <= 0 || inDim % per != 0 ||
             (int64_t)weights.size() != rows * (inDim / per) * bpb)
@@ -175,47 +234,23 @@ public:
         char name[256] = {0};
         check(ctx, lev_hip_device_name(ctx, name, sizeof name));
         rep.device = name;
-
         lev_schedule list[16];
         uint32_t n = 0;
         check(ctx, lev_hip_forge_candidates(ctx, op, (uint32_t)inDim, (uint32_t)rows, (uint32_t)ncol, list, 16, &n));
         n = std::min<uint32_t>(n, 16);
+        const std::string key = cacheKey(op, inDim, rows, ncol, rep.device, tableHash(list, n));
 
-        const std::string key = cacheKey(op, inDim, rows, ncol, rep.device);
-        if (!opt.cachePath.empty()) {
-            std::ifstream in(opt.cachePath);
-            std::string line;
-            while (std::getline(in, line)) {
-                if (line.compare(0, key.size() + 1, key + " ") != 0) continue;
-                std::istringstream f(line.substr(key.size() + 1));
-                ForgeCandidate c;
-                c.schedule.op = op;
-                int baseline = 0;
-                if (!(f >> c.schedule.family >> c.schedule.rows_in_flight >> c.schedule.persistent >> c.medianUs >>
-                      c.maxRelErr >> baseline))
-                    continue;
-                // a cached schedule that is no longer a candidate (another build) is ignored
-                bool legal = false;
-                for (uint32_t i = 0; i < n; ++i)
-                    legal = legal || (list[i].family == c.schedule.family &&
-                                      list[i].rows_in_flight == c.schedule.rows_in_flight &&
-                                      list[i].persistent == c.schedule.persistent);
-                if (!legal) continue;
-                c.pass = true;
-                rep.candidates.push_back(c);
-                rep.selected = 0;
-                rep.fromCache = true;
-                install(ctx, rep, baseline != 0);
-                return rep;
-            }
-        }
-
+        // inputs, oracle and the launch closure (also needed to gate a cached selection)
         SplitMix64 rng{opt.seed};
         std::vector<float> x((size_t)(inDim * ncol));
         for (float &v : x) v = rng.nextSignedUnit();
         std::vector<double> ref((size_t)(rows * ncol), 0.0);
         const int64_t rowBytes = inDim / per * bpb;
-        DeviceBuffer dw = r.makeBuffer(weights), dx = r.makeBuffer(x), dy = r.makeBuffer(rows * ncol * 4);
+        size_t copies = weights.empty() ? 1 : opt.rotateBytes / weights.size();
+        copies = std::max<size_t>(1, std::min<size_t>(copies, 64));
+        std::vector<DeviceBuffer> dws;
+        for (size_t k = 0; k < copies; ++k) dws.push_back(r.makeBuffer(weights));
+        DeviceBuffer dx = r.makeBuffer(x), dy = r.makeBuffer(rows * ncol * 4);
         DeviceBuffer dxq, dxs;
         if (opt.int8Activations) {
             // quantise on the device, then continue with the values the codes stand for
@@ -232,34 +267,80 @@ public:
         for (int64_t c = 0; c < ncol; ++c)
             for (int64_t i = 0; i < rows; ++i) {
                 double s = 0;
-                if (op == LEV_OP_Q4_0_GEMV) q4_0RowF64(weights.data() + i * rowBytes, inDim, x.data() + c * inDim, s);
-                else q4_kRowF64(weights.data() + i * rowBytes, inDim, x.data() + c * inDim, s);
+                const uint8_t *row = weights.data() + i * rowBytes;
+                if (op == LEV_OP_Q4_0_GEMV) q4_0RowF64(row, inDim, x.data() + c * inDim, s);
+                else if (q6) q6_kRowF64(row, inDim, x.data() + c * inDim, s);
+                else q4_kRowF64(row, inDim, x.data() + c * inDim, s);
                 ref[(size_t)(c * rows + i)] = s;
             }
-
+        size_t turn = 0;
         auto launch = [&]() {
-            if (op == LEV_OP_Q4_K_GEMV_Q8)
+            const DeviceBuffer &dw = dws[turn++ % copies];
+            const size_t yn = (size_t)(rows * ncol);
+            switch (op) {
+            case LEV_OP_Q4_K_GEMV_Q8:
                 return lev_hip_q4_k_gemv_q8(ctx, dw.contents(), weights.size(), 0,
                                             static_cast<const int8_t *>(dxq.contents()), dxs.floats(), x.size(),
-                                            dy.floats(), (size_t)(rows * ncol), (uint32_t)inDim, (uint32_t)rows,
-                                            (uint32_t)ncol);
-            if (op == LEV_OP_Q4_0_GEMV)
+                                            dy.floats(), yn, (uint32_t)inDim, (uint32_t)rows, (uint32_t)ncol);
+            case LEV_OP_Q6_K_GEMV_Q8:
+                return lev_hip_q6_k_gemv_q8(ctx, dw.contents(), weights.size(), 0,
+                                            static_cast<const int8_t *>(dxq.contents()), dxs.floats(), x.size(),
+                                            dy.floats(), yn, (uint32_t)inDim, (uint32_t)rows, (uint32_t)ncol);
+            case LEV_OP_Q4_0_GEMV:
                 return lev_hip_q4_0_gemv(ctx, dw.contents(), weights.size(), 0, dx.floats(), (size_t)inDim,
                                          dy.floats(), (size_t)rows, (uint32_t)inDim, (uint32_t)rows);
-            return lev_hip_q4_k_gemv_ncol(ctx, dw.contents(), weights.size(), 0, dx.floats(), x.size(), nullptr,
-                                          0.f, dy.floats(), (size_t)(rows * ncol), (uint32_t)inDim, (uint32_t)rows,
-                                          (uint32_t)ncol);
+            case LEV_OP_Q6_K_GEMV:
+                return lev_hip_q6_k_gemv(ctx, dw.contents(), weights.size(), 0, dx.floats(), (size_t)inDim,
+                                         dy.floats(), (size_t)rows, (uint32_t)inDim, (uint32_t)rows, nullptr, nullptr);
+            default:
+                return lev_hip_q4_k_gemv_ncol(ctx, dw.contents(), weights.size(), 0, dx.floats(), x.size(), nullptr,
+                                              0.f, dy.floats(), yn, (uint32_t)inDim, (uint32_t)rows, (uint32_t)ncol);
+            }
         };
-        for (uint32_t i = 0; i < n; ++i) {
-            ForgeCandidate c;
-            c.schedule = list[i];
-            check(ctx, lev_hip_forge_select(ctx, (uint32_t)inDim, (uint32_t)rows, (uint32_t)ncol, &list[i]));
-            // poison the output so that a candidate that writes nothing cannot pass on the previous one's result
+        // one launch into a poisoned output (a candidate that writes nothing cannot pass on
+        // the previous one's result), compared with the oracle
+        auto gate = [&](const lev_schedule &sch) {
+            check(ctx, lev_hip_forge_select(ctx, (uint32_t)inDim, (uint32_t)rows, (uint32_t)ncol, &sch));
             std::vector<float> poison((size_t)(rows * ncol), NAN);
             check(ctx, lev_hip_buf_upload(ctx, dy.contents(), poison.data(), poison.size() * 4));
             check(ctx, launch());
             check(ctx, lev_hip_sync(ctx));
-            c.maxRelErr = maxRelErr(r.read<float>(dy, (size_t)(rows * ncol)), ref);
+            return maxRelErr(r.read<float>(dy, (size_t)(rows * ncol)), ref);
+        };
+
+        if (!opt.cachePath.empty()) {
+            std::ifstream in(opt.cachePath);
+            std::string line;
+            while (std::getline(in, line)) {
+                if (line.compare(0, key.size() + 1, key + " ") != 0) continue;
+                std::istringstream f(line.substr(key.size() + 1));
+                ForgeCandidate c;
+                c.schedule.op = op;
+                int baseline = 0;
+                if (!(f >> c.schedule.family >> c.schedule.rows_in_flight >> c.schedule.persistent >> c.medianUs >>
+                      c.maxRelErr >> baseline))
+                    continue;
+                bool legal = false;
+                for (uint32_t i = 0; i < n; ++i)
+                    legal = legal || (list[i].family == c.schedule.family &&
+                                      list[i].rows_in_flight == c.schedule.rows_in_flight &&
+                                      list[i].persistent == c.schedule.persistent);
+                if (!legal) continue;
+                // the cached choice is gated again by this build before it is installed
+                c.maxRelErr = gate(c.schedule);
+                c.pass = c.maxRelErr >= 0 && c.maxRelErr < opt.gate;
+                if (!c.pass) continue;
+                rep.candidates.push_back(c);
+                rep.selected = 0;
+                rep.fromCache = true;
+                install(ctx, rep, baseline != 0);
+                return rep;
+            }
+        }
+        for (uint32_t i = 0; i < n; ++i) {
+            ForgeCandidate c;
+            c.schedule = list[i];
+            c.maxRelErr = gate(list[i]);
             c.pass = c.maxRelErr >= 0 && c.maxRelErr < opt.gate;
             std::vector<double> samples;
             for (int s = 0; s < opt.warm + opt.timed; ++s) {
@@ -271,21 +352,10 @@ public:
                     samples.push_back(std::chrono::duration<double, std::micro>(t1 - t0).count() /
                                       opt.launchesPerSample);
             }
-            std::sort(samples.begin(), samples.end());
-            c.medianUs = samples.empty() ? 0 : samples[samples.size() / 2];
+            c.medianUs = median(samples);
             rep.candidates.push_back(c);
         }
-
-        // baseline must pass; the fastest passing candidate wins if it beats the baseline by more than the margin
-        rep.selected = -1;
-        if (!rep.candidates.empty() && rep.candidates[0].pass) {
-            rep.selected = 0;
-            size_t best = 0;
-            for (size_t i = 1; i < rep.candidates.size(); ++i)
-                if (rep.candidates[i].pass && rep.candidates[i].medianUs < rep.candidates[best].medianUs) best = i;
-            if (best != 0 && rep.candidates[best].medianUs < rep.candidates[0].medianUs * (1.0 - opt.margin))
-                rep.selected = (int)best;
-        }
+        rep.selected = choose(rep.candidates, opt.margin);
         install(ctx, rep, rep.selected <= 0);
         if (!opt.cachePath.empty() && rep.selected >= 0) {
             const ForgeCandidate &c = rep.candidates[(size_t)rep.selected];
@@ -297,6 +367,7 @@ public:
     }
 
 private:
+    friend class MoELayerForge;
     static void check(lev_ctx *ctx, int st) {
         if (st != LEV_OK)
             throw Gemma4Error(Gemma4Error::commandFailed, std::string("forge: ") + lev_hip_last_error(ctx));
@@ -308,6 +379,156 @@ private:
         else
             check(ctx, lev_hip_forge_select(ctx, (uint32_t)rep.inDim, (uint32_t)rep.rows, (uint32_t)rep.ncol,
                                             &rep.candidates[(size_t)rep.selected].schedule));
+    }
+};
+
+// The MoE layer at one to four tokens (MoELoweringForge.forge, MoELowering.swift:1896-1985:
+// derive the lowered layer's candidates, gate each against the FP64 oracle, time, select).
+// The gate has two parts, as the layer has two contracts: the routing must be a top-k of
+// the FP64 router probabilities (ties within 1e-6 may fall either way), and the output must
+// agree with the FP64 expert chain evaluated on the routing the device chose.
+class MoELayerForge {
+public:
+    // `pool`: the bytes `binding`'s offsets refer to; `router`: F32 [experts][hidden].
+    static ForgeReport forge(Runner &r, const std::vector<uint8_t> &pool, const MoEBinding &binding,
+                             const std::vector<float> &router, int tokens, const ForgeOptions &opt = ForgeOptions()) {
+        using namespace forge_detail;
+        const int H = binding.hidden, I = binding.expertIntermediate, E = binding.experts, K = binding.topK;
+        if (H <= 0 || I <= 0 || E <= 0 || K <= 0 || K > E || H % 32 || I % 32 || tokens < 1 || tokens > 4 ||
+            (int64_t)router.size() != (int64_t)E * H)
+            throw Gemma4Error(Gemma4Error::badTensorGeometry, "forge: MoE layer dims");
+        lev_ctx *ctx = r.context();
+        ForgeReport rep;
+        rep.op = LEV_OP_MOE_LAYER_Q4_0;
+        rep.inDim = H;
+        rep.rows = I;
+        rep.ncol = tokens;
+        char name[256] = {0};
+        MatvecForge::check(ctx, lev_hip_device_name(ctx, name, sizeof name));
+        rep.device = name;
+        lev_schedule list[16];
+        uint32_t n = 0;
+        MatvecForge::check(ctx, lev_hip_forge_candidates(ctx, rep.op, (uint32_t)H, (uint32_t)I, (uint32_t)tokens, list,
+                                                         16, &n));
+        n = std::min<uint32_t>(n, 16);
+
+        SplitMix64 rng{opt.seed};
+        std::vector<float> x((size_t)tokens * H);
+        for (float &v : x) v = rng.nextSignedUnit();
+        // FP64 router probabilities per token
+        std::vector<std::vector<double>> prob((size_t)tokens, std::vector<double>((size_t)E));
+        for (int t = 0; t < tokens; ++t) {
+            double top = -INFINITY, den = 0;
+            for (int e = 0; e < E; ++e) {
+                double s = 0;
+                for (int i = 0; i < H; ++i) s += (double)router[(size_t)e * H + i] * (double)x[(size_t)t * H + i];
+                prob[(size_t)t][(size_t)e] = s;
+                top = std::max(top, s);
+            }
+            for (double &p : prob[(size_t)t]) den += (p = std::exp(p - top));
+            for (double &p : prob[(size_t)t]) p /= den;
+        }
+        size_t copies = pool.empty() ? 1 : opt.rotateBytes / pool.size();
+        copies = std::max<size_t>(1, std::min<size_t>(copies, 8));
+        std::vector<DeviceBuffer> pools;
+        for (size_t k = 0; k < copies; ++k) pools.push_back(r.makeBuffer(pool));
+        DeviceBuffer dr = r.makeBuffer(router), dx = r.makeBuffer(x), dy = r.makeBuffer((int64_t)tokens * H * 4),
+                     dids = r.makeBuffer((int64_t)tokens * K * 4), dwts = r.makeBuffer((int64_t)tokens * K * 4);
+        size_t turn = 0;
+        auto launch = [&]() {
+            lev_moe_experts p;
+            p.d_base = pools[turn++ % copies].contents();
+            p.base_bytes = pool.size();
+            p.gate_off = (uint64_t)binding.gateOffset;
+            p.up_off = (uint64_t)binding.upOffset;
+            p.down_off = (uint64_t)binding.downOffset;
+            p.gate_stride = (uint64_t)binding.gateStride;
+            p.up_stride = (uint64_t)binding.upStride;
+            p.down_stride = (uint64_t)binding.downStride;
+            p.hidden = (uint32_t)H;
+            p.inter = (uint32_t)I;
+            p.experts = (uint32_t)E;
+            return lev_hip_moe_layer_q4_0(ctx, &p, dr.floats(), nullptr, dx.floats(), dy.floats(),
+                                          static_cast<int32_t *>(dids.contents()), dwts.floats(), (uint32_t)K,
+                                          (uint32_t)tokens);
+        };
+        // FP64 expert chain on a given routing (runMoeBatchedRouted, Gemma4.swift:2073; g4_gelu_up :4364-4388)
+        auto chain = [&](int t, const int32_t *ids, const float *wts, std::vector<double> &y) {
+            y.assign((size_t)H, 0.0);
+            const int64_t guRow = H / 32 * 18, dnRow = I / 32 * 18;
+            std::vector<float> act((size_t)I);
+            for (int k = 0; k < K; ++k) {
+                const uint8_t *g = pool.data() + binding.gateOffset + (int64_t)ids[k] * binding.gateStride;
+                const uint8_t *u = pool.data() + binding.upOffset + (int64_t)ids[k] * binding.upStride;
+                const uint8_t *d = pool.data() + binding.downOffset + (int64_t)ids[k] * binding.downStride;
+                for (int i = 0; i < I; ++i) {
+                    double gs = 0, us = 0;
+                    q4_0RowF64(g + i * guRow, H, x.data() + (size_t)t * H, gs);
+                    q4_0RowF64(u + i * guRow, H, x.data() + (size_t)t * H, us);
+                    const double inner = 0.7978845608028654 * (gs + 0.044715 * gs * gs * gs);
+                    act[(size_t)i] = (float)(0.5 * gs * (1.0 + std::tanh(inner)) * us);
+                }
+                for (int i = 0; i < H; ++i) {
+                    double s = 0;
+                    q4_0RowF64(d + i * dnRow, I, act.data(), s);
+                    y[(size_t)i] += (double)wts[k] * s;
+                }
+            }
+        };
+        auto gate = [&](const lev_schedule &sch) {
+            MatvecForge::check(ctx, lev_hip_forge_select(ctx, (uint32_t)H, (uint32_t)I, (uint32_t)tokens, &sch));
+            std::vector<float> poison((size_t)tokens * H, NAN);
+            MatvecForge::check(ctx, lev_hip_buf_upload(ctx, dy.contents(), poison.data(), poison.size() * 4));
+            MatvecForge::check(ctx, launch());
+            MatvecForge::check(ctx, lev_hip_sync(ctx));
+            const std::vector<float> y = r.read<float>(dy, (size_t)tokens * H), wts = r.read<float>(dwts, (size_t)tokens * K);
+            const std::vector<int32_t> ids = r.read<int32_t>(dids, (size_t)tokens * K);
+            double worst = 0;
+            for (int t = 0; t < tokens; ++t) {
+                // routing: K distinct experts in range, none of them clearly below an expert left out
+                std::vector<char> chosen((size_t)E, 0);
+                double least = INFINITY, psum = 0;
+                for (int k = 0; k < K; ++k) {
+                    const int32_t e = ids[(size_t)t * K + k];
+                    if (e < 0 || e >= E || chosen[(size_t)e]) return -1.0;
+                    chosen[(size_t)e] = 1;
+                    least = std::min(least, prob[(size_t)t][(size_t)e]);
+                    psum += prob[(size_t)t][(size_t)e];
+                }
+                for (int e = 0; e < E; ++e)
+                    if (!chosen[(size_t)e] && prob[(size_t)t][(size_t)e] > least + 1e-6) return -1.0;
+                for (int k = 0; k < K; ++k)   // renormalised probabilities (Gemma4.swift:3795-3810)
+                    worst = std::max(worst, std::fabs((double)wts[(size_t)t * K + k] -
+                                                      prob[(size_t)t][(size_t)ids[(size_t)t * K + k]] / psum));
+                std::vector<double> ref;
+                chain(t, ids.data() + (size_t)t * K, wts.data() + (size_t)t * K, ref);
+                const double e = maxRelErr(std::vector<float>(y.begin() + (size_t)t * H, y.begin() + (size_t)(t + 1) * H), ref);
+                if (e < 0) return -1.0;
+                worst = std::max(worst, e);
+            }
+            return worst;
+        };
+        for (uint32_t i = 0; i < n; ++i) {
+            ForgeCandidate c;
+            c.schedule = list[i];
+            c.maxRelErr = gate(list[i]);
+            c.pass = c.maxRelErr >= 0 && c.maxRelErr < opt.gate;
+            std::vector<double> samples;
+            for (int s = 0; s < opt.warm + opt.timed; ++s) {
+                auto t0 = std::chrono::steady_clock::now();
+                for (int k = 0; k < opt.launchesPerSample; ++k) MatvecForge::check(ctx, launch());
+                MatvecForge::check(ctx, lev_hip_sync(ctx));
+                auto t1 = std::chrono::steady_clock::now();
+                if (s >= opt.warm)
+                    samples.push_back(std::chrono::duration<double, std::micro>(t1 - t0).count() /
+                                      opt.launchesPerSample);
+            }
+            c.medianUs = median(samples);
+            rep.candidates.push_back(c);
+        }
+        rep.selected = choose(rep.candidates, opt.margin);
+        MatvecForge::install(ctx, rep, rep.selected <= 0);
+        return rep;
     }
 };
 

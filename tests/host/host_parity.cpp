@@ -601,21 +601,25 @@ void forge_matvec(Runner &r) {
     struct Shape { GGMLTensorType type; int rows, cols, ncol; };
     const Shape shapes[] = {{GGMLTensorType::q4_0, 512, 4096, 1}, {GGMLTensorType::q4_0, 300, 2048, 1},
                             {GGMLTensorType::q4_0, 64, 256, 1}, {GGMLTensorType::q4_K, 256, 1024, 1},
-                            {GGMLTensorType::q4_K, 128, 512, 3}};
+                            {GGMLTensorType::q4_K, 128, 512, 3}, {GGMLTensorType::q6_K, 200, 4096, 1},
+                            {GGMLTensorType::q6_K, 96, 1024, 1}};
     const std::string cache = "/tmp/leviathan_forge_test_cache.txt";
     std::remove(cache.c_str());
     for (const Shape &sh : shapes) {
-        const bool q40 = sh.type == GGMLTensorType::q4_0;
-        std::vector<uint8_t> w((size_t)sh.rows * sh.cols / (q40 ? 32 : 256) * (q40 ? 18 : 144));
+        const bool q40 = sh.type == GGMLTensorType::q4_0, q6 = sh.type == GGMLTensorType::q6_K;
+        std::vector<uint8_t> w((size_t)sh.rows * sh.cols / (q40 ? 32 : 256) * (q40 ? 18 : q6 ? 210 : 144));
         if (q40) levo_synth_q4_0(51, 0.02f, w.data(), w.size() / 18);
+        else if (q6) levo_synth_q6_k(54, 0.01f, w.data(), w.size() / 210);
         else levo_synth_q4_k(52, 0.01f, w.data(), w.size() / 144);
         ForgeOptions opt;
         opt.launchesPerSample = 5;
         opt.cachePath = cache;
+        opt.rotateBytes = 8 << 20;
         ForgeReport rep = MatvecForge::forge(r, sh.type, w, sh.rows, sh.cols, sh.ncol, opt);
         EXPECT(!rep.fromCache);
         EXPECT(!rep.candidates.empty());
-        EXPECT(q40 || rep.candidates.size() == 2);                       // matrix-core and vector-ALU kernel
+        EXPECT(q40 || q6 || rep.candidates.size() == 2);                 // matrix-core and vector-ALU kernel
+        EXPECT(!q6 || rep.candidates.size() == (sh.cols == 4096 ? 3u : 2u));   // exact kernel (two waves, one wave a row), f64-sum kernel
         EXPECT(!q40 || sh.cols < 1024 || rep.candidates.size() == 6);      // 3 depths x 2 grids, baseline first
         EXPECT(!q40 || sh.cols >= 1024 || rep.candidates.size() == 1);     // narrow rows: the built-in choice only
         for (const ForgeCandidate &c : rep.candidates) {
@@ -631,11 +635,13 @@ void forge_matvec(Runner &r) {
         levo_fill_signed_unit(0x4C455649ull, x.data(), x.size());
         std::vector<double> ref((size_t)sh.rows), mine((size_t)sh.rows, 0.0);
         if (q40) levo_q4_0_matvec_f64(w.data(), w.size(), sh.rows, sh.cols, x.data(), sh.cols, ref.data());
+        else if (q6) levo_q6_k_matvec_f64(w.data(), w.size(), sh.rows, sh.cols, x.data(), sh.cols, ref.data());
         else levo_q4_k_matvec_f64(w.data(), w.size(), sh.rows, sh.cols, x.data(), sh.cols, ref.data());
         const size_t row_bytes = w.size() / (size_t)sh.rows;
         double worst = 0;
         for (int i = 0; i < sh.rows; ++i) {
             if (q40) forge_detail::q4_0RowF64(w.data() + i * row_bytes, sh.cols, x.data(), mine[(size_t)i]);
+            else if (q6) forge_detail::q6_kRowF64(w.data() + i * row_bytes, sh.cols, x.data(), mine[(size_t)i]);
             else forge_detail::q4_kRowF64(w.data() + i * row_bytes, sh.cols, x.data(), mine[(size_t)i]);
             worst = std::max(worst, std::fabs(mine[(size_t)i] - ref[(size_t)i]) / std::max(1.0, std::fabs(ref[(size_t)i])));
         }
@@ -654,6 +660,20 @@ void forge_matvec(Runner &r) {
         ForgeReport none = MatvecForge::forge(r, sh.type, w, sh.rows, sh.cols, sh.ncol, strict);
         EXPECT(none.selected == -1);
     }
+    // a cached selection is gated again before it is installed: with a gate nobody passes the
+    // cache line is skipped and the candidates are run (and rejected) afresh
+    {
+        std::vector<uint8_t> w((size_t)300 * 2048 / 32 * 18);
+        levo_synth_q4_0(51, 0.02f, w.data(), w.size() / 18);
+        ForgeOptions strict;
+        strict.launchesPerSample = 1;
+        strict.timed = 1;
+        strict.warm = 0;
+        strict.gate = 0.0;
+        strict.cachePath = cache;
+        ForgeReport none = MatvecForge::forge(r, GGMLTensorType::q4_0, w, 300, 2048, 1, strict);
+        EXPECT(!none.fromCache && none.selected == -1);
+    }
     std::remove(cache.c_str());
     // the int8-activation GEMV: dot4 kernel and integer matrix-core kernel, gated on the device's own codes
     for (int ncol : {1, 12}) {
@@ -669,6 +689,20 @@ void forge_matvec(Runner &r) {
         for (const ForgeCandidate &c : rep.candidates) EXPECT(c.pass && c.maxRelErr < 1e-4);
         EXPECT(rep.selected >= 0);
     }
+    // the Q6_K head over int8 activations: grids and column passes, all the same bits
+    for (int ncol : {1, 4}) {
+        const int rows = 160, cols = 1024;
+        std::vector<uint8_t> w((size_t)rows * cols / 256 * 210);
+        levo_synth_q6_k(55, 0.01f, w.data(), w.size() / 210);
+        ForgeOptions opt;
+        opt.launchesPerSample = 5;
+        opt.int8Activations = true;
+        opt.rotateBytes = 8 << 20;
+        ForgeReport rep = MatvecForge::forge(r, GGMLTensorType::q6_K, w, rows, cols, ncol, opt);
+        EXPECT(rep.op == LEV_OP_Q6_K_GEMV_Q8 && rep.candidates.size() == (ncol == 1 ? 2u : 3u));
+        for (const ForgeCandidate &c : rep.candidates) EXPECT(c.pass && c.maxRelErr < 1e-4 && c.medianUs > 0);
+        EXPECT(rep.selected >= 0);
+    }
     // misuse of the selection ABI
     lev_ctx *ctx = r.context();
     lev_schedule bogus{LEV_OP_Q4_0_GEMV, 0u, 3u, 0u};
@@ -679,6 +713,38 @@ void forge_matvec(Runner &r) {
     EXPECT(lev_hip_forge_candidates(ctx, LEV_OP_Q4_K_GEMV, 100, 8, 1, nullptr, 0, &n) == LEV_ERR_BAD_DIMENSIONS);
     EXPECT(lev_hip_forge_candidates(ctx, LEV_OP_Q4_0_GEMV, 4096, 8, 2, nullptr, 0, &n) == LEV_ERR_BAD_DIMENSIONS);
     EXPECT(lev_hip_forge_candidates(ctx, LEV_OP_Q4_0_GEMV, 4096, 512, 1, nullptr, 0, &n) == LEV_OK && n == 6);
+}
+
+// MoELoweringForge.forge (MoELowering.swift:1896-1985) on the test model's layer 0
+void forge_moe_layer(Runner &r, const Model &m) {
+    const TensorRef &rt = m.table.at("blk.0.ffn_gate_inp.weight");
+    std::vector<float> router((size_t)Model::experts * Model::hidden);
+    std::memcpy(router.data(), m.bytes.data() + rt.offset, router.size() * 4);
+    for (int tokens : {1, 3}) {
+        ForgeOptions opt;
+        opt.launchesPerSample = 3;
+        opt.timed = 5;
+        opt.rotateBytes = 4 << 20;
+        ForgeReport rep = MoELayerForge::forge(r, m.bytes, m.binding, router, tokens, opt);
+        EXPECT(rep.op == LEV_OP_MOE_LAYER_Q4_0 && rep.candidates.size() == 4);
+        EXPECT(rep.candidates[0].schedule.family == 1u && rep.candidates[0].schedule.rows_in_flight == 2u);
+        for (const ForgeCandidate &c : rep.candidates) EXPECT(c.pass && c.maxRelErr >= 0 && c.maxRelErr < 1e-4 && c.medianUs > 0);
+        EXPECT(rep.selected >= 0 && rep.selected < 4);
+        if (rep.selected > 0)
+            EXPECT(rep.candidates[(size_t)rep.selected].medianUs < 0.98 * rep.candidates[0].medianUs);
+        ForgeOptions strict = opt;
+        strict.gate = 0.0;
+        EXPECT(MoELayerForge::forge(r, m.bytes, m.binding, router, tokens, strict).selected == -1);
+        // leave the built-in choice installed for the cases that follow
+        EXPECT(lev_hip_forge_clear(r.context(), LEV_OP_MOE_LAYER_Q4_0, Model::hidden, Model::inter, (uint32_t)tokens) == LEV_OK);
+    }
+    bool threw = false;
+    try {
+        MoELayerForge::forge(r, m.bytes, m.binding, router, 5);
+    } catch (const Gemma4Error &) {
+        threw = true;
+    }
+    EXPECT(threw);
 }
 
 // Gemma4.swift:3742-3773: rmsnorm -> gate, up (one buffer) -> geluUp -> down -> rmsnorm,
@@ -742,6 +808,7 @@ int main(int argc, char **argv) {
         {"runner_moe_hand_computed", [&] { runner_moe_hand_computed(R()); }},
         {"runner_gguf_file", [&] { runner_gguf_file(R(), model); }},
         {"forge_matvec", [&] { forge_matvec(R()); }},
+        {"forge_moe_layer", [&] { forge_moe_layer(R(), model); }},
     };
     if (argc > 1 && std::strcmp(argv[1], "--list") == 0) {
         for (auto &c : cases) std::printf("%s\n", c.name);

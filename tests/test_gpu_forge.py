@@ -11,6 +11,7 @@ import pytest
 import torch
 
 import oracle as O
+from tests import helpers as H
 
 pytestmark = pytest.mark.gpu
 
@@ -83,6 +84,98 @@ def test_q4_k_candidates_pass_the_gate(ctx, rows, cols, ncol):
     assert not np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
     again = ctx.q4_k_gemv_ncol(dw, dx, cols, rows, ncol).cpu().numpy()
     assert np.array_equal(again.view(np.uint32), outs[0].view(np.uint32))   # cleared: built-in again
+
+
+@pytest.mark.parametrize("rows,cols,expected", [(500, 4096, [(0, 2), (0, 1), (1, 1)]), (300, 2048, [(0, 1), (1, 1)]),
+                                                (64, 8192, [(0, 1), (1, 1)]), (40, 12288, [(1, 1)])])
+def test_q6_k_candidates_pass_the_gate(ctx, rows, cols, expected):
+    """vk_q6k (lev-cli/src/main.rs:467): the head's candidates, the forge's own input and gate.
+    With the argmax epilogue on: every candidate names the same token."""
+    from leviathan_amd import capi
+    w = O.synth_q6_k(rows + cols, rows * cols // 256)
+    x = O.signed_units(cols, FORGE_SEED)
+    ref = O.q6_k_matvec_f64(w, rows, cols, x)
+    dw, dx = dev(w), dev(x)
+    cands = ctx.forge_candidates(capi.OP_Q6_K_GEMV, cols, rows)
+    assert [(c.family, c.rows_in_flight) for c in cands] == expected
+    outs = []
+    try:
+        for s in cands:
+            ctx.forge_select(cols, rows, s)
+            y, idx, margin = ctx.q6_k_gemv(dw, dx, cols, rows, argmax=True)
+            ctx.sync()
+            outs.append(y.cpu().numpy())
+            assert O.max_rel_err(outs[-1], ref) < GATE, s.key()
+            assert int(idx.item()) == O.argmax(outs[-1]), s.key()
+    finally:
+        ctx.forge_clear(capi.OP_Q6_K_GEMV, cols, rows)
+    again = ctx.q6_k_gemv(dw, dx, cols, rows).cpu().numpy()
+    assert np.array_equal(again.view(np.uint32), outs[0].view(np.uint32))   # cleared: built-in again
+    if len(outs) > 1:   # the f64-sum kernel is a different kernel: a selection really switches
+        assert not np.array_equal(outs[0].view(np.uint32), outs[-1].view(np.uint32))
+
+
+@pytest.mark.parametrize("rows,cols,ncol,expected", [(200, 4096, 1, [(1, 1), (1, 0)]),
+                                                      (96, 1024, 4, [(4, 1), (4, 0), (2, 1)]),
+                                                      (130, 4352, 5, [(8, 1), (8, 0), (4, 1)])])
+def test_q6_k_q8_candidates_pass_the_gate_and_agree_bitwise(ctx, rows, cols, ncol, expected):
+    from leviathan_amd import capi
+    w = O.synth_q6_k(rows + ncol, rows * cols // 256)
+    x = O.signed_units(cols * ncol, FORGE_SEED).reshape(ncol, cols)
+    dw = dev(w)
+    xq, xs = ctx.norm_quant_q8(dev(x), cols, ncol)
+    ctx.sync()
+    hq, hs = xq.cpu().numpy(), xs.cpu().numpy()
+    ref = np.stack([O.q6_k_matvec_q8_f64(w, rows, cols, hq[c], hs[c, :, 0]) for c in range(ncol)])
+    cands = ctx.forge_candidates(capi.OP_Q6_K_GEMV_Q8, cols, rows, ncol)
+    assert [(c.rows_in_flight, c.persistent) for c in cands] == expected
+    outs = []
+    try:
+        for s in cands:
+            ctx.forge_select(cols, rows, s, ncol)
+            y = torch.full((ncol, rows), float("nan"), device="cuda")
+            ctx.q6_k_gemv_q8(dw, xq, xs, cols, rows, ncol, y=y)
+            ctx.sync()
+            outs.append(y.cpu().numpy())
+            assert O.max_rel_err(outs[-1], ref) < GATE, s.key()
+            # a row is summed by the same lanes in the same order whatever the grid or the pass
+            assert np.array_equal(outs[-1].view(np.uint32), outs[0].view(np.uint32)), s.key()
+    finally:
+        ctx.forge_clear(capi.OP_Q6_K_GEMV_Q8, cols, rows, ncol)
+
+
+@pytest.mark.parametrize("hidden,inter,experts,top_k,tokens", [(2048, 768, 128, 8, 1), (512, 256, 20, 4, 3)])
+def test_moe_layer_candidates_pass_the_gate_and_agree_bitwise(ctx, hidden, inter, experts, top_k, tokens):
+    """MoELoweringForge.forge (MoELowering.swift:1896-1985): every candidate of the layer
+    routes to the same experts and gives the same bits; the composite is gated at 1e-4."""
+    from leviathan_amd import capi, ops
+    wr, pool, offs, x = H.config5(hidden, inter, experts, tokens, seed=experts + tokens)
+    pools = ops.Context.moe_pools(dev(pool), hidden, inter, experts, offs["gate_off"], offs["up_off"],
+                                  offs["down_off"])
+    dwr, dx = dev(wr), dev(x)
+    g, u, d = (pool[offs["gate_off"]:], pool[offs["up_off"]:], pool[offs["down_off"]:])
+    cands = ctx.forge_candidates(capi.OP_MOE_LAYER_Q4_0, hidden, inter, tokens)
+    assert [(c.family, c.rows_in_flight) for c in cands] == [(1, 2), (1, 1), (1, 4), (0, 2)]
+    outs = []
+    try:
+        for s in cands:
+            ctx.forge_select(hidden, inter, s, tokens)
+            y, ids, wts = ctx.moe_layer_q4_0(pools, dwr, dx, top_k, tokens)
+            ctx.sync()
+            outs.append((y.cpu().numpy(), ids.cpu().numpy(), wts.cpu().numpy()))
+            for t in range(tokens):
+                scores = O.f32_matvec(wr, experts, hidden, x[t])
+                ref_ids, ref_w = O.router_topk(scores, top_k, None)
+                H.check_moe_layer_token(outs[-1][0][t], outs[-1][1][t], outs[-1][2][t], ref_ids, ref_w, g, u, d,
+                                        hidden, inter, x[t], GATE)
+            for a, b in zip(outs[-1], outs[0]):
+                assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), s.key()
+    finally:
+        ctx.forge_clear(capi.OP_MOE_LAYER_Q4_0, hidden, inter, tokens)
+    with pytest.raises(ops.LevError):
+        ctx.forge_candidates(capi.OP_MOE_LAYER_Q4_0, hidden, inter, 5)     # the grouped path has one schedule
+    with pytest.raises(ops.LevError):
+        ctx.forge_select(hidden, inter, capi.Schedule(capi.OP_MOE_LAYER_Q4_0, 1, 3, 0), tokens)
 
 
 def test_selection_applies_to_one_shape_only(ctx):
