@@ -60,7 +60,11 @@ def parse_args():
     p.add_argument("--skip-others", action="store_true", help="headline only")
     p.add_argument("--skip-cpu", action="store_true", help="no cpu_baseline leg")
     p.add_argument("--only", default="", help="comma-separated kernel families to run (for "
-                   "profiling): q4_0, q6_k, q4_k, gemm, moe1, moe64, copy")
+                   "profiling): q4_0, q6_k, q4_k, gemm, moe1, moe64, copy, floor (= sweep of the cold "
+                   "9 MiB streaming read over workgroup counts; only when named)")
+    p.add_argument("--select", action="append", default=[], metavar="OP:IN_DIM:ROWS:NCOL:FAMILY:ROWS_IN_FLIGHT:PERSISTENT",
+                   help="install a forge schedule (lev_hip_forge_select) on the bench context before running, "
+                        "to time a candidate other than the built-in choice; may be repeated")
     return p.parse_args()
 
 
@@ -87,6 +91,9 @@ def main():
     stream = torch.cuda.Stream(device=dev)
     torch.cuda.set_stream(stream)
     ctx = ops.Context(0, stream=stream)
+    for spec in args.select:
+        op, in_dim, nrows, ncol, fam, rif, pers = (int(v) for v in spec.split(":"))
+        ctx.forge_select(in_dim, nrows, capi.Schedule(op, fam, rif, pers), ncol)
     gen = torch.Generator(device=dev)
     gen.manual_seed(1)
 
@@ -281,6 +288,22 @@ def main():
             dst = torch.empty_like(src)
             run_other("copy_256MiB", lambda i: dst.copy_(src), 2 << 28, 20, 5)
             del buf, src, dst
+
+        # ------------------------------------- floor of a cold read of the headline's bytes
+        if "floor" in only_set:
+            # One pass over 9 MiB that no cache holds (a different part of 1 GiB every launch),
+            # by plain 128-bit loads and nothing else, for a range of grids: 256 threads a
+            # workgroup, so 589,824 loads / (256 * workgroups) loads per thread, four in flight.
+            buf = rand_bytes(1 << 30)
+            sink = torch.zeros(4, dtype=torch.int32, device=dev)
+            nrot = (1 << 30) // q4_bytes_w
+            for wg in (128, 256, 512, 1024, 2048, 4096, 8192):
+                run_other(f"stream_read_9MiB_rotating_wg{wg}", lambda i, wg=wg: must(lib.lev_hip_stream_read_probe(
+                    c, buf.data_ptr() + (i % nrot) * q4_bytes_w, q4_bytes_w, sink.data_ptr(), wg)), q4_bytes_w,
+                    600, 20, extra=lambda ms, wg=wg: {"workgroups": wg,
+                                                      "loads_per_thread": q4_bytes_w / 16 / (256 * wg)})
+            run_other("empty_kernel_launch", lambda i: must(lib.lev_hip_empty_launch(c)), 0, 1000, 100)
+            del buf
 
         # ---------------------------------------------- Q4_0 large streaming
         if want("q4_0"):
