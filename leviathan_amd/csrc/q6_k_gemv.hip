@@ -34,7 +34,7 @@
 
 namespace {
 
-constexpr int kThreads = 256;
+constexpr int kThreads = 512;
 constexpr int kWaves = kThreads / LEV_WAVE;
 #ifndef LEV_Q6_DEPTH
 #define LEV_Q6_DEPTH 3   // tiles in flight per wave of the one-unit-per-lane kernels
