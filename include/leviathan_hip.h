@@ -338,8 +338,9 @@ typedef struct lev_schedule {
     uint32_t op;             /* LEV_OP_* */
     uint32_t family;         /* Q4_K: 1 = matrix-core kernel, 0 = vector-ALU (int8: dot4) kernel; Q4_0: 0;
                                 Q6_K: 0 = exact digit-plane kernel, 1 = one wave per row with f64 sums;
-                                Q6_K x int8: 0; MoE layer: 1 = the gate/up workgroups select the experts
-                                themselves, 0 = a top-k kernel of its own ahead of them */
+                                Q6_K x int8: 0; MoE layer: who selects the experts: 1 = the gate/up workgroups
+                                themselves, 2 = the last workgroup of the router kernel to finish, 0 = a top-k
+                                kernel of its own ahead of them */
     uint32_t rows_in_flight; /* Q4_0: rows a wave keeps in flight (1, 2, 4; 0 = no variants for the shape);
                                 Q6_K: waves that share a row (1, 2); Q6_K x int8: columns per pass over the
                                 weights; MoE layer: gate/up workgroups aimed at per CU (1, 2, 4) */

@@ -125,10 +125,10 @@ extern "C" int lev_hip_ctx_create(int device, void *stream, lev_ctx **out) {
         ctx->owns_stream = true;
     }
     if (hipMalloc(&ctx->argmax_partials, (size_t)lev_ctx::kArgmaxPartials * 16u) != hipSuccess ||
-        hipMalloc(reinterpret_cast<void **>(&ctx->d_flag), sizeof(int)) != hipSuccess ||
+        hipMalloc(reinterpret_cast<void **>(&ctx->d_flag), lev_ctx::kFlagWords * sizeof(int)) != hipSuccess ||
         hipHostMalloc(reinterpret_cast<void **>(&ctx->h_flag), sizeof(int), hipHostMallocDefault) !=
             hipSuccess ||
-        hipMemset(ctx->d_flag, 0, sizeof(int)) != hipSuccess) {
+        hipMemset(ctx->d_flag, 0, lev_ctx::kFlagWords * sizeof(int)) != hipSuccess) {
         lev_hip_ctx_destroy(ctx);
         return LEV_ERR_DEVICE_UNAVAILABLE;
     }

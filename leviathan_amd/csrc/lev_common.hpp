@@ -41,7 +41,11 @@ struct lev_ctx {
     // so a recorded GEMV needs no grow-on-demand scratch.
     void *argmax_partials = nullptr;
     static constexpr uint32_t kArgmaxPartials = 4096;   // entries of 16 bytes
+    // word 0: error flags raised by kernels (read and cleared by lev_hip_sync);
+    // words kTicketWord..+3: arrival counters of the router kernel, one per token,
+    // zero between launches (the last workgroup to arrive resets its counter)
     int *d_flag = nullptr;
+    static constexpr uint32_t kFlagWords = 64, kTicketWord = 16;
     int *h_flag = nullptr;   // pinned
     // True between lev_hip_program_begin and lev_hip_program_end: the stream
     // is being captured, so nothing may allocate or synchronise.

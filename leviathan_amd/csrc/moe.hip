@@ -476,6 +476,80 @@ moe_topk_kernel(const float *__restrict__ scores, const float *__restrict__ expe
     }
 }
 
+// Up to four tokens: scores AND selection in one launch.  Workgroup (g, t) scores
+// experts 8g..8g+7 of token t, one router row per wave (f64 sums, rounded to f32
+// once); the last workgroup of a token to finish (an arrival counter per token)
+// reads all of the token's scores and runs the selection, so that the gate/up
+// kernel starts from finished ids instead of every one of its workgroups ranking
+// the scores for itself.  Sixteen workgroups per token keep the counter short (a
+// counter over one workgroup per expert would serialise 128 arrivals).  The
+// counter is zero again when the kernel ends.  A forge candidate, not the built-in
+// choice: see lev_moe_layer_candidates.
+template <int J>
+__global__ void __launch_bounds__(512)
+moe_scores_select_kernel(const float *__restrict__ wr, const float *__restrict__ x, float *scores,
+                         const float *__restrict__ expert_scale, int32_t *__restrict__ ids,
+                         float *__restrict__ weights, int *__restrict__ flag, uint32_t *tickets,
+                         uint32_t hidden, uint32_t experts, uint32_t top_k) {
+    extern __shared__ double s_router[];
+    __shared__ uint32_t s_ticket;
+    __shared__ float s_score[8];
+    const uint32_t t = blockIdx.y, tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t e = blockIdx.x * 8u + wave;
+    if (e < experts) {   // wave-uniform
+        const float *row = wr + (uint64_t)e * hidden;
+        const float *xv = x + (uint64_t)t * hidden;
+        double acc;
+        if ((hidden & 3u) == 0u &&
+            ((reinterpret_cast<uintptr_t>(wr) | reinterpret_cast<uintptr_t>(x)) & 15u) == 0u) {
+            const lev_f32x4 *r4 = reinterpret_cast<const lev_f32x4 *>(row);
+            const lev_f32x4 *x4 = reinterpret_cast<const lev_f32x4 *>(xv);
+            double a0 = 0.0, a1 = 0.0;
+#pragma unroll 8
+            for (uint32_t i = lane; i < hidden / 4u; i += 64u) {
+                const lev_f32x4 a = r4[i], b = x4[i];
+                a0 = fma((double)a.x, (double)b.x, a0);
+                a1 = fma((double)a.y, (double)b.y, a1);
+                a0 = fma((double)a.z, (double)b.z, a0);
+                a1 = fma((double)a.w, (double)b.w, a1);
+            }
+            acc = a0 + a1;
+        } else {
+            acc = 0.0;
+            for (uint32_t i = lane; i < hidden; i += 64u) acc = fma((double)row[i], (double)xv[i], acc);
+        }
+        acc = wave_sum_f64(acc);
+        if (lane == 0) s_score[wave] = (float)acc;
+    }
+    lev_barrier_lds();
+    // One wave stores the workgroup's eight scores, makes them visible beyond this
+    // XCD (a fence writes the L2's dirty lines back: once per workgroup, not per
+    // wave) and takes the workgroup's arrival number.
+    if (wave == 0) {
+        const uint32_t eo = blockIdx.x * 8u + lane;
+        if (lane < 8u && eo < experts) scores[(uint64_t)t * experts + eo] = s_score[lane];
+        __threadfence();
+        if (lane == 0) s_ticket = atomicAdd(&tickets[t], 1u);
+    }
+    __syncthreads();
+    if (s_ticket != gridDim.x - 1u) return;
+    if (tid == 0) tickets[t] = 0u;
+    // the other workgroups' scores are read with device-scope loads below
+    float sc[J];
+#pragma unroll
+    for (int j = 0; j < J; ++j) {
+        const uint32_t i = lane + 64u * j;
+        sc[j] = __hip_atomic_load(&scores[(uint64_t)t * experts + (i < experts ? i : experts - 1u)],
+                                  __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    const router_sel r = router_select_regs<J>(sc, s_router, experts, top_k, true, true, 0u);
+    if (!r.ok && tid == 0) atomicOr(flag, kFlagNonFiniteScore);
+    if (tid < top_k) {
+        ids[(uint64_t)t * top_k + tid] = r.ok ? (int32_t)r.sel_id[tid] : (int32_t)tid;
+        weights[(uint64_t)t * top_k + tid] = r.ok ? router_weight(r, expert_scale, top_k, tid) : 0.f;
+    }
+}
+
 // ---------------------------------------------------------------------------
 // expert ids: bounds + distinctness (MoEModelBinding.offsets requires both)
 // ---------------------------------------------------------------------------
@@ -1044,6 +1118,21 @@ hipError_t run_scores(lev_ctx *ctx, const float *wr, const float *x, float *scor
     return hipGetLastError();
 }
 
+// scores and selection in one launch (tokens <= 4, experts <= kRouteInKernelMax)
+hipError_t run_scores_select(lev_ctx *ctx, const float *wr, const float *x, float *scores, const float *scale,
+                             int32_t *ids, float *weights, uint32_t hidden, uint32_t experts, uint32_t top_k,
+                             uint32_t tokens) {
+    uint32_t *tickets = reinterpret_cast<uint32_t *>(ctx->d_flag) + lev_ctx::kTicketWord;
+    const dim3 grid((experts + 7u) / 8u, tokens);
+    if (experts <= 128u)
+        hipLaunchKernelGGL((moe_scores_select_kernel<2>), grid, dim3(512), router_lds_bytes_fast(2), ctx->stream, wr,
+                           x, scores, scale, ids, weights, ctx->d_flag, tickets, hidden, experts, top_k);
+    else
+        hipLaunchKernelGGL((moe_scores_select_kernel<4>), grid, dim3(512), router_lds_bytes_fast(4), ctx->stream, wr,
+                           x, scores, scale, ids, weights, ctx->d_flag, tickets, hidden, experts, top_k);
+    return hipGetLastError();
+}
+
 hipError_t run_topk(lev_ctx *ctx, const float *scores, const float *scale, int32_t *ids,
                     float *weights, uint32_t experts, uint32_t top_k, uint32_t tokens) {
 #define LEV_TOPK(J)                                                                               \
@@ -1157,25 +1246,35 @@ int moe_layer_impl(lev_ctx *ctx, const lev_moe_experts *pools, const float *d_ro
                          grouped ? lev_moe_grouped_scratch_bytes(grouped_args(a, tokens)) : 0);
         if (st != LEV_OK) return st;
     }
-    st = lev_hip_check(ctx, run_scores(ctx, d_router_w, d_x, s.scores, a.hidden, a.experts, tokens),
-                       "moe router scores launch");
-    if (st != LEV_OK) return st;
     const bool fast = experts_fast(a, d_x);
     gu_route rt{d_ids, nullptr, nullptr, nullptr, nullptr};
     // a schedule installed for this shape (lev_hip_forge_select) overrides the built-in choice
     const lev_schedule *sel = tokens <= 4u ? lev_selected(ctx, LEV_OP_MOE_LAYER_Q4_0, a.hidden, a.inter, tokens)
                                            : nullptr;
-    const bool select_in_kernel = !(sel && sel->family == 0u);
+    const uint32_t family = sel ? sel->family : 1u;
     const uint32_t gu_per_cu = sel && sel->rows_in_flight ? sel->rows_in_flight : 2u;
-    if (fast && tokens <= 4u && a.experts <= kRouteInKernelMax && select_in_kernel) {
-        // few tokens: the gate/up workgroups select the experts themselves
-        rt = gu_route{nullptr, s.scores, d_expert_scale, d_ids, d_weights};
-    } else {
+    const bool few = fast && tokens <= 4u && a.experts <= kRouteInKernelMax;
+    if (few && family == 2u) {
+        // few tokens: the router kernel's last workgroup selects the experts
         st = lev_hip_check(ctx,
-                           run_topk(ctx, s.scores, d_expert_scale, d_ids, d_weights, a.experts, top_k,
-                                    tokens),
-                           "moe router top-k launch");
+                           run_scores_select(ctx, d_router_w, d_x, s.scores, d_expert_scale, d_ids, d_weights,
+                                             a.hidden, a.experts, top_k, tokens),
+                           "moe router launch");
         if (st != LEV_OK) return st;
+    } else {
+        st = lev_hip_check(ctx, run_scores(ctx, d_router_w, d_x, s.scores, a.hidden, a.experts, tokens),
+                           "moe router scores launch");
+        if (st != LEV_OK) return st;
+        if (few && family == 1u) {
+            // the gate/up workgroups select the experts themselves
+            rt = gu_route{nullptr, s.scores, d_expert_scale, d_ids, d_weights};
+        } else {
+            st = lev_hip_check(ctx,
+                               run_topk(ctx, s.scores, d_expert_scale, d_ids, d_weights, a.experts, top_k,
+                                        tokens),
+                               "moe router top-k launch");
+            if (st != LEV_OK) return st;
+        }
     }
     if (grouped)
         return lev_hip_check(ctx,
@@ -1191,10 +1290,12 @@ int moe_layer_impl(lev_ctx *ctx, const lev_moe_experts *pools, const float *d_ro
 
 // Candidate schedules of the MoE layer at one to four tokens, the built-in choice
 // first (MoELoweringForge.forge, MoELowering.swift:1896-1985, derives and gates the
-// lowered layer the same way): who selects the experts (the gate/up workgroups
-// themselves, or a top-k kernel of its own ahead of them: one launch more, no
-// redundant selection) and how many gate/up workgroups per CU the rows are cut
-// into.  Every candidate computes each row with the same lanes in the same order:
+// lowered layer the same way): who selects the experts (family 1: the gate/up
+// workgroups themselves, the built-in choice; 2: the last workgroup of the router
+// kernel to finish; 0: a top-k kernel of its own, one launch more) and how many
+// gate/up workgroups per CU the rows are cut into.  On MI355X the hand-over inside
+// the router kernel (a fence and an arrival counter over 16 workgroups) costs as
+// much as the launch it saves: 18.8 us a layer against 15.9 and 18.9.  Every candidate computes each row with the same lanes in the same order:
 // their outputs agree bit for bit.  (Shapes the streaming kernels cannot take run
 // the generic kernels whatever is selected.)
 uint32_t lev_moe_layer_candidates(const lev_ctx *ctx, uint32_t hidden, uint32_t inter, uint32_t tokens,
@@ -1211,6 +1312,7 @@ uint32_t lev_moe_layer_candidates(const lev_ctx *ctx, uint32_t hidden, uint32_t 
     add(1u, 2u);
     add(1u, 1u);
     add(1u, 4u);
+    add(2u, 2u);
     add(0u, 2u);
     return n;
 }

@@ -79,6 +79,16 @@ __device__ __forceinline__ void q4k_exchange(lev_u4 &v) {
     v.w = s1[1];
 }
 
+// Byte offset of 16-byte unit u (= 8*kg + A row / 2) inside a sub-block's 512 bytes
+// of digit planes.  The staging threads of one wave write units 8*kg + 2*(column % 4)
+// of many sub-blocks at once; unswizzled, k-groups 0 and 2 and all sub-blocks would
+// meet in the same banks.  Flipping bit 0 for the upper two k-groups and bit 1 for
+// odd sub-blocks spreads eight consecutive lanes over eight bank groups, and is a
+// permutation of the units inside a sub-block, so the MFMA's reads stay conflict-free.
+__device__ __forceinline__ uint32_t q4k_unit(uint32_t u, uint32_t kg, uint32_t j) {
+    return (u ^ (kg >> 1) ^ ((j & 1u) << 1)) * 16u;
+}
+
 // LDS, for SB superblocks and NL = 4*NX layout columns:
 //   dig  [8*SB][NX][4 k-groups][16 A rows][8 bytes]   digit planes, A row = 4*(column % 4) + plane
 //   sxd  [SB][NL][8] f64                               sum of X per sub-block
@@ -298,9 +308,11 @@ q4_k_mfma_gemv(const uint8_t *__restrict__ w, const float *__restrict__ x,
         sum += __builtin_amdgcn_update_dpp(0, sum, 0x4E, 0xF, 0xF, true);
         if (real) {
             const uint32_t j = k8 >> 2, kg = k8 & 3u;       // sub-block, k-group
-            uint8_t *at = dig + ((((size_t)j * NX + (c >> 2)) * 4u + kg) * 16u + 4u * (c & 3u)) * 8u;
-            *reinterpret_cast<lev_u4 *>(at) = lev_u4{dw[3][0], dw[3][1], dw[2][0], dw[2][1]};
-            *reinterpret_cast<lev_u4 *>(at + 16u) = lev_u4{dw[1][0], dw[1][1], dw[0][0], dw[0][1]};
+            // 16-byte unit u = 8*kg + (A row)/2 of the sub-block's 512 bytes, stored at q4k_unit(u, kg, j)
+            uint8_t *blk = dig + ((size_t)j * NX + (c >> 2)) * 512u;
+            const uint32_t u = 8u * kg + 2u * (c & 3u);
+            *reinterpret_cast<lev_u4 *>(blk + q4k_unit(u, kg, j)) = lev_u4{dw[3][0], dw[3][1], dw[2][0], dw[2][1]};
+            *reinterpret_cast<lev_u4 *>(blk + q4k_unit(u + 1u, kg, j)) = lev_u4{dw[1][0], dw[1][1], dw[0][0], dw[0][1]};
             if (kg == 3u) sxd[((j >> 3) * NL + c) * 8u + (j & 7u)] = (double)sum;
             if ((k8 & 31u) == 31u) psb[(j >> 3) * NL + c] = __hiloint2double((int)((ex + 872u) << 20), 0);   // 2^(ex-151)
         }
@@ -339,7 +351,9 @@ q4_k_mfma_gemv(const uint8_t *__restrict__ w, const float *__restrict__ x,
 #pragma unroll
             for (int h = 0; h < 4; ++h) SX[q][h] = *reinterpret_cast<const lev_d2 *>(sxd + m * 8u + 2u * h);
         }
-        const uint8_t *arow = dig + (size_t)sb * 8u * NX * 512u + lane * 8u;
+        // lane (r, g) reads A row r, k-group g: unit 8g + r/2, its low or high 8 bytes
+        const uint8_t *ablk = dig + (size_t)sb * 8u * NX * 512u;
+        const uint32_t aoff = q4k_unit(8u * g + (r >> 1), g, 0u) + 8u * (r & 1u);
         lev_u4 ca = W.a, cb = W.b;
         q4k_exchange(ca);
         q4k_exchange(cb);
@@ -354,7 +368,7 @@ q4_k_mfma_gemv(const uint8_t *__restrict__ w, const float *__restrict__ x,
             const long B = __builtin_bit_cast(long, wv);
 #pragma unroll
             for (int q = 0; q < NX; ++q) {
-                const long A = *reinterpret_cast<const long *>(arow + ((size_t)j * NX + q) * 512u);
+                const long A = *reinterpret_cast<const long *>(ablk + ((size_t)j * NX + q) * 512u + (aoff ^ (32u * (j & 1))));
                 const lev_i4 D = __builtin_amdgcn_mfma_i32_16x16x32_i8(A, B, lev_i4{0, 0, 0, 0}, 0, 0, 0);
                 // |D| <= 32*15*128 < 2^16, sc < 2^6: eight of the products fit 32 bits with room
 #pragma unroll

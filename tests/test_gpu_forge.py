@@ -155,7 +155,7 @@ def test_moe_layer_candidates_pass_the_gate_and_agree_bitwise(ctx, hidden, inter
     dwr, dx = dev(wr), dev(x)
     g, u, d = (pool[offs["gate_off"]:], pool[offs["up_off"]:], pool[offs["down_off"]:])
     cands = ctx.forge_candidates(capi.OP_MOE_LAYER_Q4_0, hidden, inter, tokens)
-    assert [(c.family, c.rows_in_flight) for c in cands] == [(1, 2), (1, 1), (1, 4), (0, 2)]
+    assert [(c.family, c.rows_in_flight) for c in cands] == [(1, 2), (1, 1), (1, 4), (2, 2), (0, 2)]
     outs = []
     try:
         for s in cands:
@@ -176,6 +176,8 @@ def test_moe_layer_candidates_pass_the_gate_and_agree_bitwise(ctx, hidden, inter
         ctx.forge_candidates(capi.OP_MOE_LAYER_Q4_0, hidden, inter, 5)     # the grouped path has one schedule
     with pytest.raises(ops.LevError):
         ctx.forge_select(hidden, inter, capi.Schedule(capi.OP_MOE_LAYER_Q4_0, 1, 3, 0), tokens)
+    with pytest.raises(ops.LevError):
+        ctx.forge_select(hidden, inter, capi.Schedule(capi.OP_MOE_LAYER_Q4_0, 3, 2, 0), tokens)
 
 
 def test_selection_applies_to_one_shape_only(ctx):
