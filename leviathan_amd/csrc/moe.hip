@@ -146,12 +146,10 @@ __device__ router_sel router_select_block(const float *__restrict__ srow, void *
     return router_select_regs<J>(sc, lds, experts, top_k, need_p, false);
 }
 
-// fast (workgroup-uniform, J <= 8, blockDim = 512): ranks are counted from
-// registers, the waves splitting the table between them: a wave broadcasts its
-// share of the keys lane by lane (v_readlane) and every lane compares its own
-// J keys against them; the waves' partial counts meet in LDS.  One barrier
-// less than the table walk and no LDS atomics.  Only when the integer keys
-// order the probabilities (the common case); the result is the same.
+// fast (workgroup-uniform, J <= 8): every wave extracts the minima of the integer
+// keys from its own registers, round by round, with no exchange at all (see
+// below).  Only when the integer keys order the probabilities (the common case);
+// the result is the same.
 template <int J>
 __device__ router_sel router_select_regs(const float (&sc)[J], void *lds, uint32_t experts,
                                          uint32_t top_k, bool need_p, bool fast, uint32_t slot) {
@@ -209,56 +207,61 @@ __device__ router_sel router_select_regs(const float (&sc)[J], void *lds, uint32
         for (int j = 0; j < J; ++j) p[j] = lane + 64u * j < experts ? p[j] / sum : 0.0;
     }
     if constexpr (J <= 8) {
-        if (fast && by_key && blockDim.x == 512u) {
-            // wave w broadcasts table entries w*share .. +share (one register set: share divides 64)
-            constexpr uint32_t share = padded / 8u;
-            // the wave index as a scalar: the lane selects below must be uniform registers
-            const uint32_t first = (uint32_t)__builtin_amdgcn_readfirstlane((int)wave) * share;
-            uint64_t src = key[0];
+        if (fast && by_key) {
+            // Repeated extraction of the minimum key, as the reference extracts the
+            // maximum probability: every wave holds all keys (two per lane for 128
+            // experts) and needs no one else.  A round is a wave-wide minimum of the
+            // |d| bits (DPP), a ballot for the lowest index that holds it, and its
+            // removal: about twenty instructions.  The workgroup of `slot` stops after
+            // slot + 1 rounds; only the publishing workgroup runs all top_k and lists
+            // the winners with their probabilities.
+            uint32_t dk[J];
 #pragma unroll
-            for (int j = 1; j < J; ++j) src = (first >> 6) == (uint32_t)j ? key[j] : src;
-            const uint32_t lo = (uint32_t)src, hi = (uint32_t)(src >> 32);
-            uint32_t cnt[J];
-#pragma unroll
-            for (int j = 0; j < J; ++j) cnt[j] = 0u;
-#pragma unroll
-            for (uint32_t k = 0; k < share; ++k) {
-                const uint32_t l = (first & 63u) + k;
-                const uint64_t other = ((uint64_t)(uint32_t)__builtin_amdgcn_readlane((int)hi, l) << 32) |
-                                       (uint32_t)__builtin_amdgcn_readlane((int)lo, l);
-#pragma unroll
-                for (int j = 0; j < J; ++j) cnt[j] += other < key[j] ? 1u : 0u;
-            }
-            uint32_t *part = sel_id + 64;   // partial counts [wave][padded], behind the regular areas
-#pragma unroll
-            for (int j = 0; j < J; ++j) part[wave * padded + lane + 64u * j] = cnt[j];
-            lev_barrier_lds();
-            // every wave adds up the ranks of its own copies of the keys: no second exchange
-            uint32_t total[J];
-#pragma unroll
-            for (int j = 0; j < J; ++j) {
-                uint32_t r = 0;
-#pragma unroll
-                for (uint32_t w = 0; w < 8u; ++w) r += part[w * padded + lane + 64u * j];
-                total[j] = lane + 64u * j < experts ? r : 0xFFFFFFFFu;
-            }
-            // the expert of `slot`: the one element whose rank is slot (ranks are a permutation)
+            for (int j = 0; j < J; ++j) dk[j] = lane + 64u * j < experts ? (uint32_t)(key[j] >> 32) : 0xFFFFFFFFu;
+            const uint32_t rounds = need_p ? top_k : slot + 1u;
             uint32_t found = 0xFFFFFFFFu;
+            for (uint32_t rnd = 0; rnd < rounds; ++rnd) {
+                uint32_t m = dk[0];
 #pragma unroll
-            for (int j = 0; j < J; ++j) {
-                const unsigned long long hit = __ballot(total[j] == slot);
-                if (hit != 0ull) found = (uint32_t)__builtin_ctzll(hit) + 64u * (uint32_t)j;
-            }
-            out.e_slot = found;
-            if (need_p) {   // the publishing workgroup also lists all winners with their probabilities
-                if (wave == 0) {
-#pragma unroll
-                    for (int j = 0; j < J; ++j)
-                        if (total[j] < top_k) {
-                            sel_id[total[j]] = lane + 64u * j;
-                            sel_p[total[j]] = p[j];
-                        }
+                for (int j = 1; j < J; ++j) m = dk[j] < m ? dk[j] : m;
+#define LEV_MOE_MINSTEP(CTRL, ROWS)                                                                \
+                {                                                                                  \
+                    const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp((int)m, (int)m, CTRL, ROWS, 0xF, false); \
+                    m = o < m ? o : m;                                                             \
                 }
+                LEV_MOE_MINSTEP(0xB1, 0xF)    // quad_perm [1,0,3,2]
+                LEV_MOE_MINSTEP(0x4E, 0xF)    // quad_perm [2,3,0,1]
+                LEV_MOE_MINSTEP(0x141, 0xF)   // row_half_mirror
+                LEV_MOE_MINSTEP(0x140, 0xF)   // row_mirror
+                LEV_MOE_MINSTEP(0x142, 0xA)   // row_bcast:15 into rows 1 and 3
+                LEV_MOE_MINSTEP(0x143, 0xC)   // row_bcast:31 into rows 2 and 3: lane 63 holds the minimum
+#undef LEV_MOE_MINSTEP
+                const uint32_t best = (uint32_t)__builtin_amdgcn_readlane((int)m, 63);
+                uint32_t wl = 0, wj = 0;
+                bool seen = false;
+#pragma unroll
+                for (int j = 0; j < J; ++j) {   // ascending j, lowest lane: the lowest index among equals
+                    const unsigned long long hit = __ballot(dk[j] == best);
+                    if (!seen && hit != 0ull) {
+                        wl = (uint32_t)__builtin_ctzll(hit);
+                        wj = (uint32_t)j;
+                        seen = true;
+                    }
+                }
+                found = wl + 64u * wj;
+#pragma unroll
+                for (int j = 0; j < J; ++j) {
+                    const bool mine = lane == wl && wj == (uint32_t)j;
+                    if (need_p && wave == 0 && mine) {
+                        sel_id[rnd] = found;
+                        sel_p[rnd] = p[j];
+                    }
+                    dk[j] = mine ? 0xFFFFFFFFu : dk[j];
+                }
+            }
+            out.e_slot = found;   // need_p: the last winner; the publisher reads sel_id instead
+            if (need_p) {
+                out.e_slot = 0xFFFFFFFFu;
                 lev_barrier_lds();
             }
             return out;
