@@ -387,7 +387,8 @@ def test_q4_k_rust_fixture_16x1024(ctx):
 
 
 @pytest.mark.parametrize("ncol", [1, 2, 3, 4, 5, 8, 16])
-@pytest.mark.parametrize("rows,cols", [(37, 1024), (64, 4096), (20, 12288), (9, 256)])
+@pytest.mark.parametrize("rows,cols", [(37, 1024), (64, 4096), (20, 12288), (9, 256), (130, 4352), (33, 7936),
+                                       (17, 8192)])
 def test_q4_k_ncol_shapes_with_rmsnorm(ctx, rows, cols, ncol):
     w, x, gain = H.config3(rows, cols, ncol, seed=rows + ncol)
     got = q4k_gemv(ctx, w, x, rows, cols, ncol, gain)
