@@ -472,23 +472,39 @@ swiglu_quant_kernel(const float *__restrict__ gate, const float *__restrict__ up
 // LDS: codes [sub-block][NCL columns][32 B] (a wave's A read is 512 contiguous
 // bytes), d and s as [sub-block][NCL] floats.
 // ---------------------------------------------------------------------------
-constexpr uint32_t kQ8MfmaMinCols = 9;   // measured on 12288x4096: the dot4 kernel wins up to 8 columns
+constexpr uint32_t kQ8MfmaMinCols = 4;   // measured on 12288x4096: the dot4 kernel wins up to 3 columns (12.2 against 14.9 us at 2, 16.6 against 15.1 at 4)
 constexpr int kMThreads = 1024;
 constexpr int kMWaves = kMThreads / LEV_WAVE;
 typedef int lev_i32x4 __attribute__((ext_vector_type(4)));
 constexpr int kQ8mPieces = 6;   // 16-byte pieces of a column's codes a thread stages without a loop
 
 struct q8m_regs {
-    lev_u32x4 hdr;
-    lev_u32x2 c[4];
+    lev_u32x4 hdr, a, b;
 };
 
+// Three 16-byte loads per lane: the header, and bytes [16*(g/2), +16) of chunk
+// 2i + g%2 for i = 0, 1: a wave's load covers 64 contiguous bytes per row (five
+// loads of 8 bytes cost more in the L1 than the bytes they save).
 __device__ __forceinline__ void q8m_issue(const uint8_t *__restrict__ w, uint64_t row_bytes, uint32_t row,
                                           uint32_t sb, uint32_t g, q8m_regs &R) {
     const uint8_t *p = w + (uint64_t)row * row_bytes + (uint64_t)sb * 144u;
     R.hdr = *reinterpret_cast<const lev_u32x4 *>(p);
-#pragma unroll
-    for (int c = 0; c < 4; ++c) R.c[c] = *reinterpret_cast<const lev_u32x2 *>(p + 16u + 32u * c + 8u * g);
+    const uint8_t *q = p + 16u + 32u * (g & 1u) + 16u * (g >> 1);
+    R.a = *reinterpret_cast<const lev_u32x4 *>(q);
+    R.b = *reinterpret_cast<const lev_u32x4 *>(q + 64u);
+}
+
+// The MFMA wants bytes [8g, 8g+8) of every chunk in lane group g.  Lane groups g
+// and g^1 (16 lanes apart) hold each other's second piece; one row swap per dword
+// puts both in place: afterwards (x, y) is the lane's piece of chunk 2i and (z, w)
+// of chunk 2i+1.
+__device__ __forceinline__ void q8m_exchange(lev_u32x4 &v) {
+    const auto s0 = __builtin_amdgcn_permlane16_swap(v.x, v.z, false, false);
+    const auto s1 = __builtin_amdgcn_permlane16_swap(v.y, v.w, false, false);
+    v.x = s0[0];
+    v.z = s0[1];
+    v.y = s1[0];
+    v.w = s1[1];
 }
 
 // NCL: columns the LDS layout holds (>= ncol).  SHORT: no wave has more than
@@ -559,8 +575,10 @@ q4_k_q8_mfma(const uint8_t *__restrict__ w, const uint8_t *__restrict__ xq, cons
     cursor ci{0u, blockIdx.x, 0u}, cc{0u, blockIdx.x, 0u};
     q8m_regs W0, W1, W2;
     issue(ci, W0);
-    issue(ci, W1);
-    issue(ci, W2);
+    if constexpr (!SHORT) {
+        issue(ci, W1);
+        issue(ci, W2);
+    }
 
     // the activation loads were issued first and return first
 #pragma unroll
@@ -601,6 +619,11 @@ q4_k_q8_mfma(const uint8_t *__restrict__ w, const uint8_t *__restrict__ xq, cons
         const uint32_t S0 = W.hdr.y, S1 = W.hdr.z, S2 = W.hdr.w;
         const float d = live ? lev_f16_bits_to_f32(W.hdr.x & 0xFFFFu) : 0.f;
         const float dmin = live ? lev_f16_bits_to_f32(W.hdr.x >> 16) : 0.f;
+        lev_u32x4 ca = W.a, cb = W.b;
+        q8m_exchange(ca);
+        q8m_exchange(cb);
+        const lev_u32x2 chunk[4] = {lev_u32x2{ca.x, ca.y}, lev_u32x2{ca.z, ca.w}, lev_u32x2{cb.x, cb.y},
+                                    lev_u32x2{cb.z, cb.w}};
         const uint8_t *xrow = xa + ((size_t)sb * 8u * NCL + colc) * 32u + gm8;
         const float *drow = sd + (size_t)sb * 8u * NCL + gq;
         lev_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
@@ -610,7 +633,7 @@ q4_k_q8_mfma(const uint8_t *__restrict__ w, const uint8_t *__restrict__ xq, cons
             const uint32_t sc = j < 4 ? (S0 >> (8 * j)) & 63u
                                       : ((S2 >> (8 * (j - 4))) & 0xFu) | (((S0 >> (8 * (j - 4) + 6)) & 3u) << 4);
             const float scl = d * (float)sc;
-            lev_u32x2 wv = W.c[j >> 1];
+            lev_u32x2 wv = chunk[j >> 1];
             if (j & 1) wv >>= 4;
             wv &= 0x0F0F0F0Fu;
             const long B = __builtin_bit_cast(long, wv);
@@ -651,7 +674,15 @@ q4_k_q8_mfma(const uint8_t *__restrict__ w, const uint8_t *__restrict__ xq, cons
     };
 
     if constexpr (SHORT) {
+        // A wave that issues a load while the CU's memory queue is full waits in the
+        // issue: the second and third task are requested just ahead of the multiply
+        // that precedes their use, not up front.
+        issue(ci, W1);
+        __builtin_amdgcn_sched_barrier(0);
         compute(cc, W0);
+        __builtin_amdgcn_sched_barrier(0);
+        issue(ci, W2);
+        __builtin_amdgcn_sched_barrier(0);
         if (ntasks > 1u) compute(cc, W1);
         if (ntasks > 2u) compute(cc, W2);
         return;

@@ -184,14 +184,14 @@ def test_q4_k_q8_shapes(ctx, rows, cols, ncol):
                                             (5000, 4096, 12), (16, 16384, 5), (40, 28672, 4)])
 def test_q4_k_q8_both_kernels_every_column_count(ctx, rows, cols, ncol, family):
     """A forge selection pins the kernel: family 1 the integer matrix-core kernel
-    (built-in choice from 9 columns), 0 the dot4 kernel (built-in below); both meet
+    (built-in choice from 4 columns), 0 the dot4 kernel (built-in below); both meet
     the gate everywhere.  5000 rows give a wave more than three tasks (the looping
     variant); 28672 columns exceed the unrolled staging of the matrix-core kernel
     (its tail loops)."""
     from leviathan_amd import capi
     cands = ctx.forge_candidates(capi.OP_Q4_K_GEMV_Q8, cols, rows, ncol)
     assert sorted(c.family for c in cands) == [0, 1]
-    assert cands[0].family == (1 if ncol >= 9 else 0)          # candidate 0 is the built-in choice
+    assert cands[0].family == (1 if ncol >= 4 else 0)          # candidate 0 is the built-in choice
     ctx.forge_select(cols, rows, [c for c in cands if c.family == family][0], ncol)
     try:
         w, x, gain = H.config3(rows, cols, ncol, seed=rows + ncol)
