@@ -218,9 +218,12 @@ moe_grouped_kernel(lev_moe_grouped_args a, const _Float16 *__restrict__ xh,
             s_us[tid] = unscale[PAIRED ? p / (int32_t)a.top_k : p];
         }
         __syncthreads();
-        // stage the columns: 16-byte runs, global rows are contiguous
+        // stage the columns in 16-byte runs.  Consecutive threads take the kNC columns of one
+        // run, then the next run: their LDS writes are contiguous (column-major threads wrote
+        // 16 bytes at a stride of kNC*16 bytes, every lane of a wave into the same four
+        // banks), and a wave still reads whole 128-byte segments of each activation row.
         for (uint32_t i = tid; i < runs * kNC; i += kGrpThreads) {
-            const uint32_t c = i / runs, q = i - c * runs;
+            const uint32_t c = i % kNC, q = i / kNC;
             const int32_t p = s_pair[c];
             const uint64_t src = (uint64_t)(PAIRED ? p / (int32_t)a.top_k : p) * in_len + 8u * q;
             *reinterpret_cast<g_h8 *>(sxh + (q * kNC + c) * 8u) = *reinterpret_cast<const g_h8 *>(xh + src);
