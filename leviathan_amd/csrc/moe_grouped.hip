@@ -30,12 +30,15 @@
 // through a small wave-private LDS area so that each MFMA sees one block.
 #include "moe_grouped.hpp"
 
+#include <cstdlib>
+
 namespace {
 
 constexpr int kGrpThreads = 1024;
 constexpr int kGrpWaves = kGrpThreads / LEV_WAVE;
 constexpr int kNC = 8;                 // token columns per pass
 constexpr int kFlagBadExpertId = 1;    // same bit as the per-token kernels
+constexpr uint32_t kGrpScaleDw = 10;   // dwords per row of block scales in a wave's exchange area
 
 typedef _Float16 g_h8 __attribute__((ext_vector_type(8)));
 typedef uint32_t g_u4 __attribute__((ext_vector_type(4)));
@@ -168,7 +171,7 @@ __device__ __forceinline__ g_h8 q4_0_operand(g_u2 codes, uint32_t sh, uint32_t m
 
 template <bool PAIRED>
 __global__ void __launch_bounds__(kGrpThreads)
-moe_grouped_kernel(lev_moe_grouped_args a, const _Float16 *__restrict__ xh,
+moe_grouped_kernel(lev_moe_grouped_args a, uint32_t tiles_per_wg, const _Float16 *__restrict__ xh,
                    const _Float16 *__restrict__ xl, const float *__restrict__ unscale,
                    const int32_t *__restrict__ goff, const int32_t *__restrict__ glist,
                    float *__restrict__ out) {
@@ -181,35 +184,62 @@ moe_grouped_kernel(lev_moe_grouped_args a, const _Float16 *__restrict__ xh,
     const uint32_t n = (uint32_t)(goff[e + 1] - first);
     if (n == 0u) return;
 
-    constexpr int NM = 1;   // matrices per wave
     const uint32_t plane = runs * kNC * 8u;                      // halfs
     _Float16 *sxh = reinterpret_cast<_Float16 *>(smem);           // [run][col][8]
     _Float16 *sxl = sxh + plane;
-    // wave-private exchange area: per matrix 16 rows x (8 blocks x 4 dwords + 4 pad), then 16 x 8 scales
+    // wave-private exchange area: 16 rows x (8 blocks x 4 dwords + 4 pad), then 16 rows of
+    // 8 scales + 2 pad (a stride of 8 dwords put rows r and r+8 into the same bank for every read)
     uint32_t *xch = reinterpret_cast<uint32_t *>(sxl + plane);
-    constexpr uint32_t kRowDw = 36, kXchDw = 16 * kRowDw + 16 * 8;
+    constexpr uint32_t kRowDw = 36, kXchDw = 16 * kRowDw + 16 * kGrpScaleDw;
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-    uint32_t *my = xch + wave * (NM * kXchDw);
+    uint32_t *area = xch + wave * kXchDw;
     __shared__ int32_t s_pair[kNC];
     __shared__ float s_us[kNC];
-    __shared__ float s_gate[PAIRED ? (kGrpWaves / 2) * 16 * kNC : 1];   // [tile row][col]
+    __shared__ float s_gate[PAIRED ? 2 * (kGrpWaves / 2) * 16 * kNC : 1];   // [tile parity][tile row][col]
 
     const uint32_t r = lane & 15u, g = lane >> 4;
     const uint32_t is_up = PAIRED ? wave / (kGrpWaves / 2) : 0u;
-    const uint32_t wv = PAIRED ? wave % (kGrpWaves / 2) : wave;          // 16-row slice of the tile
+    const uint32_t wv = PAIRED ? wave % (kGrpWaves / 2) : wave;          // 16-row slice of a tile
     const uint32_t tile_rows = PAIRED ? (kGrpWaves / 2) * 16 : kGrpWaves * 16;
-    const uint32_t row = blockIdx.x * tile_rows + wv * 16u + r;
-    const uint32_t rowc = row < out_rows ? row : out_rows - 1u;
+    const uint32_t ntile = (out_rows + tile_rows - 1u) / tile_rows;
+    // this workgroup's row tiles: the activation planes are staged once for all of them and the
+    // weight requests run ahead across tile boundaries
+    const uint32_t t0 = blockIdx.x * tiles_per_wg;
+    const uint32_t t1 = t0 + tiles_per_wg < ntile ? t0 + tiles_per_wg : ntile;
     const uint64_t row_bytes = (uint64_t)nblk * 18u;
-    const uint8_t *wrow[NM];
+    const uint8_t *mat;
     if (PAIRED)
-        wrow[0] = a.base + (is_up ? a.up_off + e * a.up_stride : a.gate_off + e * a.gate_stride) +
-                  rowc * row_bytes;
+        mat = a.base + (is_up ? a.up_off + e * a.up_stride : a.gate_off + e * a.gate_stride);
     else
-        wrow[0] = a.base + a.down_off + e * a.down_stride + rowc * row_bytes;
+        mat = a.base + a.down_off + e * a.down_stride;
+
+    // groups of 8 blocks = 4 pairs; lane (r, g) fetches pair g of row r of a tile
+    const uint32_t ngrp = nblk >> 3;
+    auto fetch = [&](uint32_t tile, uint32_t grp, uint32_t (&D)[9]) {
+        const uint32_t tc = tile < t1 ? tile : t1 - 1u;          // past the end: any valid address
+        const uint32_t row = tc * tile_rows + wv * 16u + r;
+        const uint32_t rowc = row < out_rows ? row : out_rows - 1u;
+        const uint8_t *p = mat + rowc * row_bytes + (uint64_t)(grp * 4u + g) * 36u;
+        lev_u32x4_a4 v0 = *reinterpret_cast<const lev_u32x4_a4 *>(p);
+        lev_u32x4_a4 v1 = *reinterpret_cast<const lev_u32x4_a4 *>(p + 16);
+        lev_u32_a4 v2 = *reinterpret_cast<const lev_u32_a4 *>(p + 32);
+        D[0] = v0.v[0]; D[1] = v0.v[1]; D[2] = v0.v[2]; D[3] = v0.v[3];
+        D[4] = v1.v[0]; D[5] = v1.v[1]; D[6] = v1.v[2]; D[7] = v1.v[3];
+        D[8] = v2.v;
+    };
+    const uint32_t nib_shift = 4u * (g >> 1);
+    uint32_t k_mask = 0x000F000Fu, k_magic = 0x64006400u;
+    asm("" : "+v"(k_mask), "+v"(k_magic));   // keep both in registers (see q4_0_operand)
+    const uint32_t colc = r < (uint32_t)kNC ? r : (uint32_t)kNC - 1u;   // A rows past kNC: any valid address
 
     for (uint32_t pass = 0; pass * kNC < n; ++pass) {
         const uint32_t ncols = n - pass * kNC < (uint32_t)kNC ? n - pass * kNC : (uint32_t)kNC;
+        // the first weights are requested ahead of everything that only concerns the activations
+        uint32_t Dc[9], Dn[9];
+        uint32_t ft = t0, fg = 0;                                 // the next group to request
+        auto advance = [&] { if (++fg == ngrp) { fg = 0; ++ft; } };
+        fetch(ft, fg, Dc);
+        advance();
         __syncthreads();   // previous pass done with the planes and s_pair
         if (tid < (uint32_t)kNC) {
             // columns past the end repeat the last pair (never stored)
@@ -218,117 +248,93 @@ moe_grouped_kernel(lev_moe_grouped_args a, const _Float16 *__restrict__ xh,
             s_us[tid] = unscale[PAIRED ? p / (int32_t)a.top_k : p];
         }
         __syncthreads();
-        // stage the columns in 16-byte runs.  Consecutive threads take the kNC columns of one
+        // stage the pass's columns in 16-byte runs.  Consecutive threads take the kNC columns of one
         // run, then the next run: their LDS writes are contiguous (column-major threads wrote
         // 16 bytes at a stride of kNC*16 bytes, every lane of a wave into the same four
-        // banks), and a wave still reads whole 128-byte segments of each activation row.
+        // banks).  Columns past the end keep what the area held: an MFMA row of A only reaches its
+        // own row of outputs, which is never stored.
         for (uint32_t i = tid; i < runs * kNC; i += kGrpThreads) {
             const uint32_t c = i % kNC, q = i / kNC;
-            const int32_t p = s_pair[c];
-            const uint64_t src = (uint64_t)(PAIRED ? p / (int32_t)a.top_k : p) * in_len + 8u * q;
-            *reinterpret_cast<g_h8 *>(sxh + (q * kNC + c) * 8u) = *reinterpret_cast<const g_h8 *>(xh + src);
-            *reinterpret_cast<g_h8 *>(sxl + (q * kNC + c) * 8u) = *reinterpret_cast<const g_h8 *>(xl + src);
+            if (c < ncols) {
+                const int32_t p = s_pair[c];
+                const uint64_t src = (uint64_t)(PAIRED ? p / (int32_t)a.top_k : p) * in_len + 8u * q;
+                *reinterpret_cast<g_h8 *>(sxh + (q * kNC + c) * 8u) = *reinterpret_cast<const g_h8 *>(xh + src);
+                *reinterpret_cast<g_h8 *>(sxl + (q * kNC + c) * 8u) = *reinterpret_cast<const g_h8 *>(xl + src);
+            }
         }
         __syncthreads();
 
-        lev_f32x4 y[NM];
+        for (uint32_t tile = t0; tile < t1; ++tile) {
+            lev_f32x4 y = {0.f, 0.f, 0.f, 0.f};
+            for (uint32_t grp = 0; grp < ngrp; ++grp) {
+                // the next group (of this tile or the next) is requested before this one is multiplied;
+                // unconditional (clamped past the end): no branch around loads
+                fetch(ft, fg, Dn);
+                advance();
+                // hand the pair's two blocks to the lanes that need them
+                {
+                    const uint32_t *D = Dc;
+                    g_u4 qa, qb;
+                    qa.x = __builtin_amdgcn_alignbit(D[1], D[0], 16);
+                    qa.y = __builtin_amdgcn_alignbit(D[2], D[1], 16);
+                    qa.z = __builtin_amdgcn_alignbit(D[3], D[2], 16);
+                    qa.w = __builtin_amdgcn_alignbit(D[4], D[3], 16);
+                    qb.x = D[5]; qb.y = D[6]; qb.z = D[7]; qb.w = D[8];
+                    *reinterpret_cast<g_u4 *>(area + r * kRowDw + (2u * g) * 4u) = qa;
+                    *reinterpret_cast<g_u4 *>(area + r * kRowDw + (2u * g + 1u) * 4u) = qb;
+                    typedef float f32x2 __attribute__((ext_vector_type(2)));
+                    *reinterpret_cast<f32x2 *>(area + 16 * kRowDw + r * kGrpScaleDw + 2u * g) =
+                        f32x2{lev_f16_bits_to_f32(D[0] & 0xFFFFu), lev_f16_bits_to_f32(D[4] >> 16)};
+                }
+                // wave-private area: the hardware runs one wave's LDS accesses in order
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
-        for (int m = 0; m < NM; ++m) y[m] = lev_f32x4{0.f, 0.f, 0.f, 0.f};
-        const uint32_t colc = r < (uint32_t)kNC ? r : (uint32_t)kNC - 1u;   // A rows past kNC: any valid address
-
-        // groups of 8 blocks = 4 pairs; lane (r, g) fetches pair g of row r
-        const uint32_t ngrp = nblk >> 3;
-        auto fetch = [&](uint32_t grp, uint32_t (&D)[NM][9]) {
-            const uint32_t gc = grp < ngrp ? grp : ngrp - 1u;
-#pragma unroll
-            for (int m = 0; m < NM; ++m) {
-                const uint8_t *p = wrow[m] + (uint64_t)(gc * 4u + g) * 36u;
-                lev_u32x4_a4 v0 = *reinterpret_cast<const lev_u32x4_a4 *>(p);
-                lev_u32x4_a4 v1 = *reinterpret_cast<const lev_u32x4_a4 *>(p + 16);
-                lev_u32_a4 v2 = *reinterpret_cast<const lev_u32_a4 *>(p + 32);
-                D[m][0] = v0.v[0]; D[m][1] = v0.v[1]; D[m][2] = v0.v[2]; D[m][3] = v0.v[3];
-                D[m][4] = v1.v[0]; D[m][5] = v1.v[1]; D[m][6] = v1.v[2]; D[m][7] = v1.v[3];
-                D[m][8] = v2.v;
-            }
-        };
-        const uint32_t nib_shift = 4u * (g >> 1);
-        uint32_t k_mask = 0x000F000Fu, k_magic = 0x64006400u;
-        asm("" : "+v"(k_mask), "+v"(k_magic));   // keep both in registers (see q4_0_operand)
-        auto process = [&](uint32_t grp, const uint32_t (&Dcur)[NM][9]) {
-            // hand the pair's two blocks to the lanes that need them
-#pragma unroll
-            for (int m = 0; m < NM; ++m) {
-                const uint32_t *D = Dcur[m];
-                uint32_t *area = my + m * kXchDw;
-                g_u4 qa, qb;
-                qa.x = __builtin_amdgcn_alignbit(D[1], D[0], 16);
-                qa.y = __builtin_amdgcn_alignbit(D[2], D[1], 16);
-                qa.z = __builtin_amdgcn_alignbit(D[3], D[2], 16);
-                qa.w = __builtin_amdgcn_alignbit(D[4], D[3], 16);
-                qb.x = D[5]; qb.y = D[6]; qb.z = D[7]; qb.w = D[8];
-                *reinterpret_cast<g_u4 *>(area + r * kRowDw + (2u * g) * 4u) = qa;
-                *reinterpret_cast<g_u4 *>(area + r * kRowDw + (2u * g + 1u) * 4u) = qb;
-                float *sc = reinterpret_cast<float *>(area + 16 * kRowDw) + r * 8u + 2u * g;
-                sc[0] = lev_f16_bits_to_f32(D[0] & 0xFFFFu);
-                sc[1] = lev_f16_bits_to_f32(D[4] >> 16);
-            }
-            // wave-private area: the hardware runs one wave's LDS accesses in order
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-#pragma unroll
-            for (uint32_t b = 0; b < 8u; ++b) {
-                const uint32_t at = (((grp * 8u + b) * 4u + g) * kNC + colc) * 8u;
-                const g_h8 Ah = *reinterpret_cast<const g_h8 *>(sxh + at);
-                const g_h8 Al = *reinterpret_cast<const g_h8 *>(sxl + at);
-#pragma unroll
-                for (int m = 0; m < NM; ++m) {
-                    const uint32_t *area = my + m * kXchDw;
+                for (uint32_t b = 0; b < 8u; ++b) {
+                    const uint32_t at = (((grp * 8u + b) * 4u + g) * kNC + colc) * 8u;
+                    const g_h8 Ah = *reinterpret_cast<const g_h8 *>(sxh + at);
+                    const g_h8 Al = *reinterpret_cast<const g_h8 *>(sxl + at);
                     const g_u2 codes = *reinterpret_cast<const g_u2 *>(area + r * kRowDw + b * 4u + 2u * (g & 1u));
-                    const float d = reinterpret_cast<const float *>(area + 16 * kRowDw)[r * 8u + b];
+                    const float d = reinterpret_cast<const float *>(area + 16 * kRowDw)[r * kGrpScaleDw + b];
                     const g_h8 B = q4_0_operand(codes, nib_shift, k_mask, k_magic);
                     lev_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
                     acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ah, B, acc, 0, 0, 0);
                     acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(Al, B, acc, 0, 0, 0);
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) y[m][i] = fmaf(d, acc[i], y[m][i]);
+                    for (int i = 0; i < 4; ++i) y[i] = fmaf(d, acc[i], y[i]);
                 }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();   // reads done before the next group's writes
+#pragma unroll
+                for (int k = 0; k < 9; ++k) Dc[k] = Dn[k];
             }
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();   // reads done before the next group's writes
-        };
-        // the next group is requested before the current one is multiplied
-        // (a third group in flight costs more in registers than it gains)
-        uint32_t Dc[NM][9], Dn[NM][9];
-        fetch(0, Dc);
-        for (uint32_t grp = 0; grp < ngrp; ++grp) {
-            fetch(grp + 1u, Dn);   // unconditional (clamped): no branch around loads
-            process(grp, Dc);
-#pragma unroll
-            for (int m = 0; m < NM; ++m)
-#pragma unroll
-                for (int k = 0; k < 9; ++k) Dc[m][k] = Dn[m][k];
-        }
 
-        // output lane (r, g): weight row r, columns 4g..4g+3
-        if (PAIRED) {
-            if (!is_up) {
+            // output lane (r, g): weight row r of the tile, columns 4g..4g+3
+            const uint32_t row = tile * tile_rows + wv * 16u + r;
+            // gate values wait for the up waves in the buffer of the tile's parity: a gate wave
+            // cannot reach the same buffer again before the up waves have passed the barrier of
+            // the tile between, which lies behind their reads
+            float *sg = s_gate + (PAIRED ? ((tile - t0) & 1u) * ((kGrpWaves / 2) * 16 * kNC) : 0u);
+            if (PAIRED) {
+                if (!is_up) {
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    if (4u * g + i < (uint32_t)kNC) s_gate[(wv * 16u + r) * kNC + 4u * g + i] = y[0][i] * s_us[4u * g + i];
+                    for (int i = 0; i < 4; ++i)
+                        if (4u * g + i < (uint32_t)kNC) sg[(wv * 16u + r) * kNC + 4u * g + i] = y[i] * s_us[4u * g + i];
+                }
+                __syncthreads();
             }
-            __syncthreads();
-        }
-        if (row < out_rows && (!PAIRED || is_up)) {
+            if (row < out_rows && (!PAIRED || is_up)) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const uint32_t col = 4u * g + i;
-                if (col < ncols) {
-                    const int32_t p = s_pair[col];
-                    const float us = s_us[col];
-                    float v = y[0][i] * us;
-                    if (PAIRED) v = lev_gelu_up_value(s_gate[(wv * 16u + r) * kNC + col], v);
-                    out[(uint64_t)p * out_rows + row] = v;
+                for (int i = 0; i < 4; ++i) {
+                    const uint32_t col = 4u * g + i;
+                    if (col < ncols) {
+                        const int32_t p = s_pair[col];
+                        const float us = s_us[col];
+                        float v = y[i] * us;
+                        if (PAIRED) v = lev_gelu_up_value(sg[(wv * 16u + r) * kNC + col], v);
+                        out[(uint64_t)p * out_rows + row] = v;
+                    }
                 }
             }
         }
@@ -377,7 +383,23 @@ grouped_layout layout_of(const lev_moe_grouped_args &a) {
 
 size_t grouped_lds(uint32_t in_len, bool paired) {
     (void)paired;
-    return (size_t)2 * (in_len / 8) * kNC * 16 + (size_t)kGrpWaves * (16 * 36 + 16 * 8) * 4;
+    return (size_t)2 * (in_len / 8) * kNC * 16 + (size_t)kGrpWaves * (16 * 36 + 16 * kGrpScaleDw) * 4;
+}
+
+// Row tiles per workgroup.  A workgroup pays for its activation planes (a chain of dependent reads
+// and three barriers) whatever it multiplies afterwards, and its weight requests only run ahead
+// inside its own tiles: as many tiles as still leave one workgroup per CU.  The experts that
+// take part are not known on the host; at most min(experts, pairs) do.
+uint32_t tiles_per_wg(const lev_ctx *ctx, const lev_moe_grouped_args &a, uint32_t tiles, int down) {
+    static const char *env[2] = {getenv("LEV_MOE_GROUPED_TILES_GU"), getenv("LEV_MOE_GROUPED_TILES_DN")};
+    if (env[down] && atoi(env[down]) > 0) return (uint32_t)atoi(env[down]);
+    const uint64_t pairs = (uint64_t)a.tokens * a.top_k;
+    const uint64_t active = pairs < a.experts ? pairs : a.experts;
+    const uint64_t cus = (uint64_t)ctx->props.multiProcessorCount;
+    uint64_t t = (uint64_t)tiles * active / (cus ? cus : 1);
+    if (t < 1) t = 1;
+    if (t > tiles) t = tiles;
+    return (uint32_t)t;
 }
 
 }  // namespace
@@ -431,15 +453,18 @@ hipError_t lev_moe_grouped_launch(lev_ctx *ctx, const lev_moe_grouped_args &a, c
         lds_set[1] = lds_dn;
     }
     const uint32_t rows_per_wg = kGrpWaves * 16, rows_per_wg_gu = rows_per_wg / 2;
-    hipLaunchKernelGGL((moe_grouped_kernel<true>), dim3((a.inter + rows_per_wg_gu - 1) / rows_per_wg_gu, a.experts),
-                       dim3(kGrpThreads), lds_gu, ctx->stream, a, xh, xl, xus, goff, glist, act);
+    const uint32_t tiles_gu = (a.inter + rows_per_wg_gu - 1) / rows_per_wg_gu;
+    const uint32_t tiles_dn = (a.hidden + rows_per_wg - 1) / rows_per_wg;
+    const uint32_t tpw_gu = tiles_per_wg(ctx, a, tiles_gu, 0), tpw_dn = tiles_per_wg(ctx, a, tiles_dn, 1);
+    hipLaunchKernelGGL((moe_grouped_kernel<true>), dim3((tiles_gu + tpw_gu - 1) / tpw_gu, a.experts),
+                       dim3(kGrpThreads), lds_gu, ctx->stream, a, tpw_gu, xh, xl, xus, goff, glist, act);
     if ((e = hipGetLastError()) != hipSuccess) return e;
     // rows of act that belong to dropped pairs are never written; prep reads
     // them all the same (any finite or non-finite value: they are never used)
     hipLaunchKernelGGL(moe_prep_kernel, dim3(pairs), dim3(256), 0, ctx->stream, act, a.inter, ah, al, aus);
     if ((e = hipGetLastError()) != hipSuccess) return e;
-    hipLaunchKernelGGL((moe_grouped_kernel<false>), dim3((a.hidden + rows_per_wg - 1) / rows_per_wg, a.experts),
-                       dim3(kGrpThreads), lds_dn, ctx->stream, a, ah, al, aus, goff, glist, dn);
+    hipLaunchKernelGGL((moe_grouped_kernel<false>), dim3((tiles_dn + tpw_dn - 1) / tpw_dn, a.experts),
+                       dim3(kGrpThreads), lds_dn, ctx->stream, a, tpw_dn, ah, al, aus, goff, glist, dn);
     if ((e = hipGetLastError()) != hipSuccess) return e;
     hipLaunchKernelGGL(moe_merge_kernel, dim3((a.hidden + 255) / 256, a.tokens), dim3(256), 0, ctx->stream,
                        dn, weights, valid, y, a.hidden, a.top_k);
