@@ -10,12 +10,15 @@
 // again (64 tokens x top-8 = 512 x 2.65 MB against 126 distinct experts).
 //
 // Pipeline (all on the context's stream):
-//   1. group:  histogram of expert ids -> offsets; list of pairs per expert.
-//   2. prep:   rows of f32 activations -> two fp16 planes (high + low half,
-//              after a power-of-two row scale), in the k-slot order of step 3.
-//   3. gate/up on MFMA -> act = gelu_tanh(g)*u (f32, [pair][inter]).
-//   4. prep(act), down on MFMA -> dn (f32, [pair][hidden]).
-//   5. merge:  y[t] = sum over slots, IN SLOT ORDER, fmaf(w_slot, dn_slot, acc).
+//   1. group:  histogram of expert ids -> offsets; list of pairs per expert;
+//              beside it, one workgroup per token writes x as two fp16 planes
+//              (high + low half, after a power-of-two row scale), in the k-slot
+//              order of step 2.
+//   2. gate/up on MFMA -> act = gelu_tanh(g)*u (f32, [pair][inter]) and the
+//              largest |act| of every pair (atomic maximum on the bit patterns).
+//   3. down on MFMA -> dn (f32, [pair][hidden]); it splits act into planes
+//              while it copies the rows into LDS.
+//   4. merge:  y[t] = sum over slots, IN SLOT ORDER, fmaf(w_slot, dn_slot, acc).
 //
 // MFMA formulation (v_mfma_f32_16x16x32_f16), per Q4_0 block of 32 weights:
 //   B = 16 weight rows x the block's 32 codes as exact fp16 integers n-8
@@ -45,18 +48,78 @@ typedef uint32_t g_u4 __attribute__((ext_vector_type(4)));
 typedef uint32_t g_u2 __attribute__((ext_vector_type(2)));
 
 // ---------------------------------------------------------------------------
+// Activation planes.  A row is scaled by the power of two that brings its maximum into [1, 2)
+// (zero, denormal and non-finite maxima: no scaling) and split into fp16 high and low halves;
+// inside each run of 8 elements the planes hold elements 0,2,1,3,4,6,5,7: the order in which
+// the masks of the matrix-core kernel deliver the code bytes of a dword pair.
+// ---------------------------------------------------------------------------
+struct grp_scale { float scale, unscale; };
+__device__ __forceinline__ grp_scale grp_row_scale(uint32_t max_bits) {
+    uint32_t ex = (max_bits >> 23) & 0xFFu;
+    if (ex == 0u || ex >= 254u) ex = 127u;
+    return grp_scale{__uint_as_float((254u - ex) << 23), __uint_as_float(ex << 23)};
+}
+__device__ __forceinline__ void grp_split_run(lev_f32x4 a, lev_f32x4 b, float scale, g_h8 &h, g_h8 &l) {
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+    a = a * scale;
+    b = b * scale;
+    const float m[8] = {a.x, a.z, a.y, a.w, b.x, b.z, b.y, b.w};
+#pragma unroll
+    for (int k = 0; k < 8; k += 2) {
+        const f32x2 pair = {m[k], m[k + 1]};
+        const f16x2 hp = __builtin_convertvector(pair, f16x2);
+        const f32x2 rest = {pair.x - (float)hp.x, pair.y - (float)hp.y};
+        const f16x2 lp = __builtin_convertvector(rest, f16x2);
+        h[k] = hp.x; h[k + 1] = hp.y;
+        l[k] = lp.x; l[k + 1] = lp.y;
+    }
+}
+
+// ---------------------------------------------------------------------------
 // 1. group pairs by expert.  One workgroup.  A pair is dropped (and flagged)
 // when its id is out of range or repeats an earlier slot of the same token,
 // as MoEModelBinding.offsets requires (MoEModelBinding.swift:174-214).
 // goff[e] .. goff[e+1]: expert e's pairs in glist; valid[p]: pair p takes part.
 // ---------------------------------------------------------------------------
+// Workgroups 1..tokens: the fp16 planes of x[t][:] and its row maximum (bit pattern of the largest
+// |x|; NaNs are passed over, as fmaxf does).  Workgroup 0 also clears amax (the per-pair maxima
+// step 2 builds).
 __global__ void __launch_bounds__(1024)
 moe_group_kernel(const int32_t *__restrict__ ids, uint32_t pairs, uint32_t experts, uint32_t top_k,
                  int32_t *__restrict__ goff, int32_t *__restrict__ glist,
-                 uint8_t *__restrict__ valid, int *__restrict__ flag) {
+                 uint8_t *__restrict__ valid, int *__restrict__ flag, const float *__restrict__ x,
+                 uint32_t hidden, _Float16 *__restrict__ xh, _Float16 *__restrict__ xl,
+                 uint32_t *__restrict__ xmax, uint32_t *__restrict__ amax) {
     extern __shared__ int32_t s_cnt[];          // [experts] counts, then [experts] cursors
     int32_t *s_cur = s_cnt + experts;
     const uint32_t tid = threadIdx.x;
+    if (blockIdx.x != 0u) {
+        __shared__ float s_max[16];
+        const uint32_t t = blockIdx.x - 1u, runs = hidden >> 3;
+        const lev_f32x4 *s4 = reinterpret_cast<const lev_f32x4 *>(x + (uint64_t)t * hidden);
+        float mx = 0.f;
+        for (uint32_t q = tid; q < 2u * runs; q += 1024u) {
+            const lev_f32x4 v = s4[q];
+            mx = fmaxf(mx, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
+        if ((tid & 63u) == 0u) s_max[tid >> 6] = mx;
+        __syncthreads();
+        float m = s_max[0];
+        for (int w = 1; w < 16; ++w) m = fmaxf(m, s_max[w]);
+        if (tid == 0) xmax[t] = __float_as_uint(m);
+        const float scale = grp_row_scale(__float_as_uint(m)).scale;
+        for (uint32_t q = tid; q < runs; q += 1024u) {
+            g_h8 h, l;
+            grp_split_run(s4[2u * q], s4[2u * q + 1u], scale, h, l);
+            *reinterpret_cast<g_h8 *>(xh + (uint64_t)t * hidden + 8u * q) = h;
+            *reinterpret_cast<g_h8 *>(xl + (uint64_t)t * hidden + 8u * q) = l;
+        }
+        return;
+    }
+    for (uint32_t p = tid; p < pairs; p += 1024u) amax[p] = 0u;
     for (uint32_t e = tid; e < experts; e += 1024u) s_cnt[e] = 0;
     __syncthreads();
     bool bad_seen = false;
@@ -88,61 +151,7 @@ moe_group_kernel(const int32_t *__restrict__ ids, uint32_t pairs, uint32_t exper
 }
 
 // ---------------------------------------------------------------------------
-// 2. prep: one workgroup of 256 threads per row of `len` floats (len % 32 == 0).
-// hi/lo planes keep the row order except inside each run of 8 elements, which
-// is stored as elements 0,2,1,3,4,6,5,7: the order in which the masks of step 3
-// deliver the code bytes of a dword pair.  unscale[row] undoes the row scale.
-// ---------------------------------------------------------------------------
-__global__ void __launch_bounds__(256)
-moe_prep_kernel(const float *__restrict__ src, uint32_t len, _Float16 *__restrict__ hi,
-                _Float16 *__restrict__ lo, float *__restrict__ unscale) {
-    __shared__ float s_max[4];
-    __shared__ float s_scale;
-    const uint32_t row = blockIdx.x, tid = threadIdx.x;
-    const lev_f32x4 *s4 = reinterpret_cast<const lev_f32x4 *>(src + (uint64_t)row * len);
-    const uint32_t runs = len >> 3;
-    float mx = 0.f;
-    for (uint32_t q = tid; q < runs; q += 256u) {
-        const lev_f32x4 a = s4[2u * q], b = s4[2u * q + 1u];
-        mx = fmaxf(mx, fmaxf(fmaxf(fabsf(a.x), fabsf(a.y)), fmaxf(fabsf(a.z), fabsf(a.w))));
-        mx = fmaxf(mx, fmaxf(fmaxf(fabsf(b.x), fabsf(b.y)), fmaxf(fabsf(b.z), fabsf(b.w))));
-    }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
-    if ((tid & 63u) == 0u) s_max[tid >> 6] = mx;
-    __syncthreads();
-    if (tid == 0) {
-        const float m = fmaxf(fmaxf(s_max[0], s_max[1]), fmaxf(s_max[2], s_max[3]));
-        // power-of-two scale that brings the row maximum into [1, 2)
-        uint32_t ex = (__float_as_uint(m) >> 23) & 0xFFu;
-        if (ex == 0u || ex >= 254u) ex = 127u;      // zero / denormal / non-finite row: no scaling
-        s_scale = __uint_as_float((254u - ex) << 23);
-        unscale[row] = __uint_as_float(ex << 23);
-    }
-    __syncthreads();
-    const float scale = s_scale;
-    typedef float f32x2 __attribute__((ext_vector_type(2)));
-    typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
-    for (uint32_t q = tid; q < runs; q += 256u) {
-        const lev_f32x4 a = s4[2u * q] * scale, b = s4[2u * q + 1u] * scale;
-        const float m[8] = {a.x, a.z, a.y, a.w, b.x, b.z, b.y, b.w};
-        g_h8 h, l;
-#pragma unroll
-        for (int k = 0; k < 8; k += 2) {
-            const f32x2 pair = {m[k], m[k + 1]};
-            const f16x2 hp = __builtin_convertvector(pair, f16x2);
-            const f32x2 rest = {pair.x - (float)hp.x, pair.y - (float)hp.y};
-            const f16x2 lp = __builtin_convertvector(rest, f16x2);
-            h[k] = hp.x; h[k + 1] = hp.y;
-            l[k] = lp.x; l[k + 1] = lp.y;
-        }
-        *reinterpret_cast<g_h8 *>(hi + (uint64_t)row * len + 8u * q) = h;
-        *reinterpret_cast<g_h8 *>(lo + (uint64_t)row * len + 8u * q) = l;
-    }
-}
-
-// ---------------------------------------------------------------------------
-// 3./4. grouped matrix-core kernel, 16 waves.  Down: grid (row tiles of 256,
+// 2./3. grouped matrix-core kernel, 16 waves.  Down: grid (row tiles of 256,
 // experts), wave w owns rows 16w..16w+15 of the tile.  PAIRED (gate/up): grid
 // (row tiles of 128, experts), waves 0..7 own the tile's gate rows, waves 8..15
 // the same rows of the up matrix; gate values meet the up waves in LDS.
@@ -171,10 +180,11 @@ __device__ __forceinline__ g_h8 q4_0_operand(g_u2 codes, uint32_t sh, uint32_t m
 
 template <bool PAIRED>
 __global__ void __launch_bounds__(kGrpThreads)
-moe_grouped_kernel(lev_moe_grouped_args a, uint32_t tiles_per_wg, const _Float16 *__restrict__ xh,
-                   const _Float16 *__restrict__ xl, const float *__restrict__ unscale,
-                   const int32_t *__restrict__ goff, const int32_t *__restrict__ glist,
-                   float *__restrict__ out) {
+moe_grouped_kernel(lev_moe_grouped_args a, uint32_t tiles_per_wg, const float *__restrict__ src,
+                   const _Float16 *__restrict__ src_h, const _Float16 *__restrict__ src_l,
+                   const uint32_t *__restrict__ src_max, const int32_t *__restrict__ goff,
+                   const int32_t *__restrict__ glist, float *__restrict__ out,
+                   uint32_t *__restrict__ out_max) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const uint32_t in_len = PAIRED ? a.hidden : a.inter;
     const uint32_t out_rows = PAIRED ? a.inter : a.hidden;
@@ -194,7 +204,7 @@ moe_grouped_kernel(lev_moe_grouped_args a, uint32_t tiles_per_wg, const _Float16
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     uint32_t *area = xch + wave * kXchDw;
     __shared__ int32_t s_pair[kNC];
-    __shared__ float s_us[kNC];
+    __shared__ float s_us[kNC], s_scale[kNC];
     __shared__ float s_gate[PAIRED ? 2 * (kGrpWaves / 2) * 16 * kNC : 1];   // [tile parity][tile row][col]
 
     const uint32_t r = lane & 15u, g = lane >> 4;
@@ -245,10 +255,12 @@ moe_grouped_kernel(lev_moe_grouped_args a, uint32_t tiles_per_wg, const _Float16
             // columns past the end repeat the last pair (never stored)
             const int32_t p = glist[first + pass * kNC + (tid < ncols ? tid : ncols - 1u)];
             s_pair[tid] = p;
-            s_us[tid] = unscale[PAIRED ? p / (int32_t)a.top_k : p];
+            const grp_scale sc = grp_row_scale(src_max[PAIRED ? p / (int32_t)a.top_k : p]);
+            s_us[tid] = sc.unscale;
+            s_scale[tid] = sc.scale;
         }
         __syncthreads();
-        // stage the pass's columns in 16-byte runs.  Consecutive threads take the kNC columns of one
+        // stage the pass's columns in runs of 8 values -> 16 bytes per plane.  Consecutive threads take the kNC columns of one
         // run, then the next run: their LDS writes are contiguous (column-major threads wrote
         // 16 bytes at a stride of kNC*16 bytes, every lane of a wave into the same four
         // banks).  Columns past the end keep what the area held: an MFMA row of A only reaches its
@@ -257,9 +269,19 @@ moe_grouped_kernel(lev_moe_grouped_args a, uint32_t tiles_per_wg, const _Float16
             const uint32_t c = i % kNC, q = i / kNC;
             if (c < ncols) {
                 const int32_t p = s_pair[c];
-                const uint64_t src = (uint64_t)(PAIRED ? p / (int32_t)a.top_k : p) * in_len + 8u * q;
-                *reinterpret_cast<g_h8 *>(sxh + (q * kNC + c) * 8u) = *reinterpret_cast<const g_h8 *>(xh + src);
-                *reinterpret_cast<g_h8 *>(sxl + (q * kNC + c) * 8u) = *reinterpret_cast<const g_h8 *>(xl + src);
+                g_h8 h, l;
+                if (PAIRED) {
+                    // x: planes written beside the grouping
+                    const uint64_t at = (uint64_t)(p / (int32_t)a.top_k) * in_len + 8u * q;
+                    h = *reinterpret_cast<const g_h8 *>(src_h + at);
+                    l = *reinterpret_cast<const g_h8 *>(src_l + at);
+                } else {
+                    // act: split here, its row maximum was only complete when gate/up ended
+                    const lev_f32x4 *s4 = reinterpret_cast<const lev_f32x4 *>(src + (uint64_t)p * in_len + 8u * q);
+                    grp_split_run(s4[0], s4[1], s_scale[c], h, l);
+                }
+                *reinterpret_cast<g_h8 *>(sxh + (q * kNC + c) * 8u) = h;
+                *reinterpret_cast<g_h8 *>(sxl + (q * kNC + c) * 8u) = l;
             }
         }
         __syncthreads();
@@ -267,7 +289,8 @@ moe_grouped_kernel(lev_moe_grouped_args a, uint32_t tiles_per_wg, const _Float16
         for (uint32_t tile = t0; tile < t1; ++tile) {
             lev_f32x4 y = {0.f, 0.f, 0.f, 0.f};
             for (uint32_t grp = 0; grp < ngrp; ++grp) {
-                // the next group (of this tile or the next) is requested before this one is multiplied;
+                // the next group (of this tile or the next) is requested before this one is multiplied
+                // (two groups on their way measured 6 % slower);
                 // unconditional (clamped past the end): no branch around loads
                 fetch(ft, fg, Dn);
                 advance();
@@ -324,16 +347,29 @@ moe_grouped_kernel(lev_moe_grouped_args a, uint32_t tiles_per_wg, const _Float16
                 }
                 __syncthreads();
             }
-            if (row < out_rows && (!PAIRED || is_up)) {
+            if (!PAIRED || is_up) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const uint32_t col = 4u * g + i;
-                    if (col < ncols) {
-                        const int32_t p = s_pair[col];
-                        const float us = s_us[col];
-                        float v = y[i] * us;
+                    const bool live = col < ncols && row < out_rows;
+                    const int32_t p = s_pair[col < (uint32_t)kNC ? col : 0u];
+                    float v = 0.f;
+                    if (live) {
+                        v = y[i] * s_us[col];
                         if (PAIRED) v = lev_gelu_up_value(sg[(wv * 16u + r) * kNC + col], v);
                         out[(uint64_t)p * out_rows + row] = v;
+                    }
+                    if (PAIRED) {
+                        // largest |act| of the pair: over the wave's 16 rows first, then one atomic per
+                        // column; the bit patterns of non-negative floats order as the floats do, and a
+                        // NaN ranks above every number (the down stage then leaves the row unscaled)
+                        uint32_t m = __float_as_uint(fabsf(v));
+#pragma unroll
+                        for (int off = 1; off < 16; off <<= 1) {
+                            const uint32_t o = (uint32_t)__shfl_xor((int)m, off);
+                            m = m > o ? m : o;
+                        }
+                        if (r == 0u && col < ncols && m != 0u) atomicMax(out_max + p, m);
                     }
                 }
             }
@@ -341,7 +377,7 @@ moe_grouped_kernel(lev_moe_grouped_args a, uint32_t tiles_per_wg, const _Float16
     }
 }
 
-// 5. merge in slot order (g4_axpy chain, Gemma4.swift:2171-2175); dropped pairs add nothing.
+// 4. merge in slot order (g4_axpy chain, Gemma4.swift:2171-2175); dropped pairs add nothing.
 __global__ void __launch_bounds__(256)
 moe_merge_kernel(const float *__restrict__ dn, const float *__restrict__ weights,
                  const uint8_t *__restrict__ valid, float *__restrict__ y, uint32_t hidden,
@@ -360,7 +396,7 @@ moe_merge_kernel(const float *__restrict__ dn, const float *__restrict__ weights
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct grouped_layout {
-    size_t goff, glist, valid, xh, xl, xus, ah, al, aus, dn, total;
+    size_t goff, glist, valid, xh, xl, xmax, amax, dn, total;
 };
 
 grouped_layout layout_of(const lev_moe_grouped_args &a) {
@@ -372,10 +408,8 @@ grouped_layout layout_of(const lev_moe_grouped_args &a) {
     L.valid = o; o += align256(pairs);
     L.xh = o; o += align256((size_t)a.tokens * a.hidden * 2);
     L.xl = o; o += align256((size_t)a.tokens * a.hidden * 2);
-    L.xus = o; o += align256((size_t)a.tokens * 4);
-    L.ah = o; o += align256(pairs * a.inter * 2);
-    L.al = o; o += align256(pairs * a.inter * 2);
-    L.aus = o; o += align256(pairs * 4);
+    L.xmax = o; o += align256((size_t)a.tokens * 4);
+    L.amax = o; o += align256(pairs * 4);
     L.dn = o; o += align256(pairs * a.hidden * 4);
     L.total = o;
     return L;
@@ -426,16 +460,14 @@ hipError_t lev_moe_grouped_launch(lev_ctx *ctx, const lev_moe_grouped_args &a, c
     int32_t *glist = reinterpret_cast<int32_t *>(s + L.glist);
     uint8_t *valid = reinterpret_cast<uint8_t *>(s + L.valid);
     _Float16 *xh = reinterpret_cast<_Float16 *>(s + L.xh), *xl = reinterpret_cast<_Float16 *>(s + L.xl);
-    _Float16 *ah = reinterpret_cast<_Float16 *>(s + L.ah), *al = reinterpret_cast<_Float16 *>(s + L.al);
-    float *xus = reinterpret_cast<float *>(s + L.xus), *aus = reinterpret_cast<float *>(s + L.aus);
+    uint32_t *xmax = reinterpret_cast<uint32_t *>(s + L.xmax), *amax = reinterpret_cast<uint32_t *>(s + L.amax);
     float *dn = reinterpret_cast<float *>(s + L.dn);
     const uint32_t pairs = a.tokens * a.top_k;
     hipError_t e;
 
-    hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), (size_t)2 * a.experts * 4, ctx->stream, ids,
-                       pairs, a.experts, a.top_k, goff, glist, valid, ctx->d_flag);
-    if ((e = hipGetLastError()) != hipSuccess) return e;
-    hipLaunchKernelGGL(moe_prep_kernel, dim3(a.tokens), dim3(256), 0, ctx->stream, x, a.hidden, xh, xl, xus);
+    hipLaunchKernelGGL(moe_group_kernel, dim3(1 + a.tokens), dim3(1024), (size_t)2 * a.experts * 4,
+                       ctx->stream, ids, pairs, a.experts, a.top_k, goff, glist, valid, ctx->d_flag, x,
+                       a.hidden, xh, xl, xmax, amax);
     if ((e = hipGetLastError()) != hipSuccess) return e;
 
     static size_t lds_set[2] = {0, 0};
@@ -457,14 +489,11 @@ hipError_t lev_moe_grouped_launch(lev_ctx *ctx, const lev_moe_grouped_args &a, c
     const uint32_t tiles_dn = (a.hidden + rows_per_wg - 1) / rows_per_wg;
     const uint32_t tpw_gu = tiles_per_wg(ctx, a, tiles_gu, 0), tpw_dn = tiles_per_wg(ctx, a, tiles_dn, 1);
     hipLaunchKernelGGL((moe_grouped_kernel<true>), dim3((tiles_gu + tpw_gu - 1) / tpw_gu, a.experts),
-                       dim3(kGrpThreads), lds_gu, ctx->stream, a, tpw_gu, xh, xl, xus, goff, glist, act);
+                       dim3(kGrpThreads), lds_gu, ctx->stream, a, tpw_gu, nullptr, xh, xl, xmax, goff, glist, act, amax);
     if ((e = hipGetLastError()) != hipSuccess) return e;
-    // rows of act that belong to dropped pairs are never written; prep reads
-    // them all the same (any finite or non-finite value: they are never used)
-    hipLaunchKernelGGL(moe_prep_kernel, dim3(pairs), dim3(256), 0, ctx->stream, act, a.inter, ah, al, aus);
-    if ((e = hipGetLastError()) != hipSuccess) return e;
+    // rows of act that belong to dropped pairs are never written and never read
     hipLaunchKernelGGL((moe_grouped_kernel<false>), dim3((tiles_dn + tpw_dn - 1) / tpw_dn, a.experts),
-                       dim3(kGrpThreads), lds_dn, ctx->stream, a, tpw_dn, ah, al, aus, goff, glist, dn);
+                       dim3(kGrpThreads), lds_dn, ctx->stream, a, tpw_dn, act, nullptr, nullptr, amax, goff, glist, dn, nullptr);
     if ((e = hipGetLastError()) != hipSuccess) return e;
     hipLaunchKernelGGL(moe_merge_kernel, dim3((a.hidden + 255) / 256, a.tokens), dim3(256), 0, ctx->stream,
                        dn, weights, valid, y, a.hidden, a.top_k);
