@@ -164,6 +164,18 @@ int lev_hip_q4_k_gemv_ncol(lev_ctx *ctx, const void *d_w, size_t w_bytes, uint64
                            float *d_y, size_t y_capacity, uint32_t in_dim, uint32_t rows,
                            uint32_t ncol);
 
+/* Q6_K multi-column GEMV on f32 activations: the LM head (or any Q6_K tensor) applied to
+ * ncol columns per weight read, as Builder::matvec does for Q4_K
+ * (lev-model/src/gpu.rs:334-370; single-column q6k.matvec, lev-forge/src/q6k.rs:61-187),
+ * with the same optional RMSNorm in front (d_gain == NULL skips it).  Same layouts as
+ * lev_hip_q4_k_gemv_ncol: x is [ncol][in_dim], y[col*rows + row].  Sums are formed
+ * without rounding, so a column's result does not depend on ncol.  Weights 2-byte
+ * aligned (GGUF), x and gain 16-byte aligned, in_dim a multiple of 256. */
+int lev_hip_q6_k_gemv_ncol(lev_ctx *ctx, const void *d_w, size_t w_bytes, uint64_t w_off,
+                           const float *d_x, size_t x_count, const float *d_gain, float eps,
+                           float *d_y, size_t y_capacity, uint32_t in_dim, uint32_t rows,
+                           uint32_t ncol);
+
 /* ---- int8-activation decode path ----
  * Activation quantiser: groups of 32, d = amax/127, q = roundEven(v * 127/amax),
  * s = d * sum(q) (quantize_q8, lev-cpu/src/lib.rs:295-322; emit_quantize,
@@ -337,12 +349,14 @@ int lev_hip_q6_k_matvec_reporting(const uint8_t *blocks, size_t blocks_count, in
 typedef struct lev_schedule {
     uint32_t op;             /* LEV_OP_* */
     uint32_t family;         /* Q4_K: 1 = matrix-core kernel, 0 = vector-ALU (int8: dot4) kernel; Q4_0: 0;
-                                Q6_K: 0 = exact digit-plane kernel, 1 = one wave per row with f64 sums;
+                                Q6_K: 2 = integer matrix-core kernel, 0 = digit-plane dot4 kernel (both exact),
+                                1 = one wave per row with f64 sums;
                                 Q6_K x int8: 0; MoE layer: who selects the experts: 1 = the gate/up workgroups
                                 themselves, 2 = the last workgroup of the router kernel to finish, 0 = a top-k
                                 kernel of its own ahead of them */
     uint32_t rows_in_flight; /* Q4_0: rows a wave keeps in flight (1, 2, 4; 0 = no variants for the shape);
-                                Q6_K: waves that share a row (1, 2); Q6_K x int8: columns per pass over the
+                                Q6_K: waves that share a row (family 0: 1, 2) or a group of 16 rows (family 2:
+                                2, 4, 8, 16); Q6_K x int8: columns per pass over the
                                 weights; MoE layer: gate/up workgroups aimed at per CU (1, 2, 4) */
     uint32_t persistent;     /* Q4_0, Q6_K x int8: 0 = one workgroup per row tile, 1 = resident grid walking
                                 the tiles */

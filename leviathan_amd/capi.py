@@ -87,6 +87,8 @@ SIGNATURES = {
     "lev_hip_q6_k_gemv": (_int, [_vp, _vp, _sz, _u64, _vp, _sz, _vp, _sz, _u32, _u32, _vp, _vp]),
     "lev_hip_q4_k_gemv_ncol": (_int, [_vp, _vp, _sz, _u64, _vp, _sz, _vp, _f32, _vp, _sz, _u32,
                                       _u32, _u32]),
+    "lev_hip_q6_k_gemv_ncol": (_int, [_vp, _vp, _sz, _u64, _vp, _sz, _vp, _f32, _vp, _sz, _u32,
+                                      _u32, _u32]),
     "lev_hip_norm_quant_q8": (_int, [_vp, _vp, _sz, _vp, _vp, _f32, _vp, _vp, _vp, _u32, _u32]),
     "lev_hip_q4_k_gemv_q8": (_int, [_vp, _vp, _sz, _u64, _vp, _vp, _sz, _vp, _sz, _u32, _u32, _u32]),
     "lev_hip_q6_k_gemv_q8": (_int, [_vp, _vp, _sz, _u64, _vp, _vp, _sz, _vp, _sz, _u32, _u32, _u32]),

@@ -31,6 +31,9 @@
 // across lanes are f64; the result is rounded to f32 once.  A lane keeps the
 // digit planes of its unit(s) in registers for every row it visits.
 #include "lev_common.hpp"
+#include "top2.hpp"
+
+#include <cstdlib>
 
 namespace {
 
@@ -242,36 +245,6 @@ __device__ __forceinline__ double q6_unit_dot_exact(const q6_unit_w &u, const q6
 
 // ---- argmax + margin (lev-forge/src/ops.rs:479-516) ------------------------
 
-struct top2 {
-    float best, second;
-    uint32_t idx;
-};
-
-__device__ __forceinline__ top2 top2_merge(top2 a, top2 b) {
-    // take b when strictly larger, or equal with the lower index (ops.rs:508)
-    bool take = b.best > a.best || (b.best == a.best && b.idx < a.idx);
-    top2 r;
-    r.best = take ? b.best : a.best;
-    r.idx = take ? b.idx : a.idx;
-    float other = take ? fmaxf(a.best, b.second) : fmaxf(b.best, a.second);
-    r.second = fmaxf(other, take ? a.second : b.second);
-    return r;
-}
-
-
-__device__ __forceinline__ top2 top2_wave(top2 m) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-        top2 o;
-        o.best = __shfl_xor(m.best, off);
-        o.second = __shfl_xor(m.second, off);
-        o.idx = __shfl_xor(m.idx, off);
-        m = top2_merge(m, o);
-    }
-    return m;
-}
-
-constexpr float kTop2Floor = -INFINITY;
 
 template <int L, int P>
 __device__ __forceinline__ void q6_load_row(const uint8_t *__restrict__ w, uint64_t row_bytes,
@@ -565,7 +538,18 @@ hipError_t launch_units(lev_ctx *ctx, const uint8_t *w, const float *x, float *y
 
 }  // namespace
 
+uint32_t lev_q6_k_mfma_cols(const lev_ctx *ctx, uint32_t in_dim);
+uint32_t lev_q6_k_mfma_waves(const lev_ctx *ctx, uint32_t in_dim, uint32_t rows);
+hipError_t lev_q6_k_mfma_gemv_launch(lev_ctx *ctx, const uint8_t *w, const float *x, const float *gain,
+                                     float eps, float *y, uint32_t in_dim, uint32_t rows, uint32_t ncol,
+                                     uint32_t waves, lev_f32x4 *partials, uint32_t *blocks_out);
+
 namespace {
+bool q6_mfma_usable(const lev_ctx *ctx, const uint8_t *w, const float *x, uint32_t in_dim) {
+    return ((reinterpret_cast<uintptr_t>(w) & 1u) == 0u) && ((reinterpret_cast<uintptr_t>(x) & 15u) == 0u) &&
+           lev_q6_k_mfma_cols(ctx, in_dim) >= 1u;
+}
+
 bool q6_exact_usable(const uint8_t *w, const float *x, uint32_t units) {
     return ((reinterpret_cast<uintptr_t>(w) & 1u) == 0u) && ((reinterpret_cast<uintptr_t>(x) & 15u) == 0u) &&
            units <= 256u;
@@ -574,20 +558,26 @@ bool q6_exact_usable(const uint8_t *w, const float *x, uint32_t units) {
 
 // Candidate schedules of a Q6_K GEMV shape, the built-in choice first (vk_q6k,
 // lev-cli/src/main.rs:467; the q6k.matvec variants of lev-forge/src/q6k.rs:175):
-// the exact digit-plane kernel, for rows of 65..128 units with two waves or one
-// wave per row, and the one-wave-per-row kernel with f64 sums.  (Pointer alignment
+// the integer matrix-core kernel (family 2; rows_in_flight = waves per row group: the
+// built-in count, then 2 and 4 where they differ), the digit-plane dot4 kernel (family
+// 0), for rows of 65..128 units with two waves or one wave per row, and the
+// one-wave-per-row kernel with f64 sums (family 1).  (Pointer alignment
 // is not part of a shape: a selection of the exact kernel is ignored for operands
 // it cannot take.)
 uint32_t lev_q6_k_gemv_candidates(const lev_ctx *ctx, uint32_t in_dim, uint32_t rows, lev_schedule *out,
                                   uint32_t capacity) {
-    (void)ctx;
-    (void)rows;
     const uint32_t units = in_dim / 32u;
     uint32_t n = 0;
     auto add = [&](uint32_t family, uint32_t waves) {
         if (n < capacity) out[n] = lev_schedule{LEV_OP_Q6_K_GEMV, family, waves, 0u};
         ++n;
     };
+    if (lev_q6_k_mfma_cols(ctx, in_dim) >= 1u) {
+        const uint32_t builtin = lev_q6_k_mfma_waves(ctx, in_dim, rows);
+        add(2u, builtin);
+        if (builtin != 2u) add(2u, 2u);
+        if (builtin != 4u) add(2u, 4u);
+    }
     if (units <= 256u) {
         const bool pair = units > 64u && units <= 128u;
         add(0u, pair ? 2u : 1u);
@@ -604,7 +594,19 @@ hipError_t lev_q6_k_gemv_argmax_launch(lev_ctx *ctx, const uint8_t *w, const flo
     const uint32_t units = in_dim / 32u;   // 8 per superblock
     // a schedule installed for this shape (lev_hip_forge_select) overrides the built-in choice
     const lev_schedule *sel = lev_selected(ctx, LEV_OP_Q6_K_GEMV, in_dim, rows, 1);
-    const bool fast = q6_exact_usable(w, x, units) && !(sel && sel->family == 1u);
+    const uint32_t family = sel ? sel->family : 2u;
+    if (family == 2u && q6_mfma_usable(ctx, w, x, in_dim)) {
+        const bool top = d_argmax || d_margin;
+        uint32_t blocks = 0;
+        lev_f32x4 *partials = top ? static_cast<lev_f32x4 *>(ctx->argmax_partials) : nullptr;
+        hipError_t e = lev_q6_k_mfma_gemv_launch(ctx, w, x, nullptr, 0.f, y, in_dim, rows, 1,
+                                                 sel ? sel->rows_in_flight : 0u, partials, &blocks);
+        if (e != hipSuccess || !top) return e;
+        hipLaunchKernelGGL(argmax_partials_kernel, dim3(1), dim3(1024), 0, ctx->stream, partials, blocks,
+                           d_argmax, d_margin);
+        return hipGetLastError();
+    }
+    const bool fast = q6_exact_usable(w, x, units) && family != 1u;
     if (!fast) {
         uint32_t blocks = (rows + kWaves - 1) / kWaves;
         hipLaunchKernelGGL(q6_k_gemv_generic, dim3(blocks), dim3(kThreads), 0, ctx->stream, w, x, y,
@@ -653,6 +655,42 @@ extern "C" int lev_hip_q6_k_gemv(lev_ctx *ctx, const void *d_w, size_t w_bytes, 
                          lev_q6_k_gemv_argmax_launch(ctx, w, d_x, d_y, in_dim, out_rows, d_argmax,
                                                      d_margin),
                          "q6_k_gemv launch");
+}
+
+extern "C" int lev_hip_q6_k_gemv_ncol(lev_ctx *ctx, const void *d_w, size_t w_bytes, uint64_t w_off,
+                                      const float *d_x, size_t x_count, const float *d_gain,
+                                      float eps, float *d_y, size_t y_capacity, uint32_t in_dim,
+                                      uint32_t rows, uint32_t ncol) {
+    LEV_REQUIRE_CTX(ctx);
+    if (ncol == 0 || ncol > LEV_MAX_GEMV_COLUMNS)
+        return lev_fail(ctx, LEV_ERR_BAD_DIMENSIONS, "q6_k_gemv_ncol: %u columns (1..%d)", ncol,
+                        LEV_MAX_GEMV_COLUMNS);
+    if (d_gain && !(eps >= 0.f))
+        return lev_fail(ctx, LEV_ERR_BAD_DIMENSIONS, "q6_k_gemv_ncol: eps %g", (double)eps);
+    lev_geom g;
+    int st = lev_check_matvec(ctx, "q6_k_gemv_ncol", 256, 210, d_w, w_bytes, w_off, d_x, x_count,
+                              (uint64_t)in_dim * ncol, d_y, y_capacity, (uint64_t)rows * ncol,
+                              in_dim, rows, &g);
+    if (st != LEV_OK) return st;
+    const uint8_t *w = static_cast<const uint8_t *>(d_w) + w_off;
+    if ((reinterpret_cast<uintptr_t>(w) & 1u) || (reinterpret_cast<uintptr_t>(d_x) & 15u) ||
+        (d_gain && (reinterpret_cast<uintptr_t>(d_gain) & 15u)))
+        return lev_fail(ctx, LEV_ERR_BAD_DIMENSIONS,
+                        "q6_k_gemv_ncol: weights must be 2-byte, x and gain 16-byte aligned");
+    const uint32_t per_launch = lev_q6_k_mfma_cols(ctx, in_dim);
+    if (per_launch == 0)
+        return lev_fail(ctx, LEV_ERR_EXCEEDS_MODEL_WORKLOAD,
+                        "q6_k_gemv_ncol: inDim %u does not fit the activation staging", in_dim);
+    for (uint32_t c0 = 0; c0 < ncol; c0 += per_launch) {
+        const uint32_t nc = ncol - c0 < per_launch ? ncol - c0 : per_launch;
+        st = lev_hip_check(ctx,
+                           lev_q6_k_mfma_gemv_launch(ctx, w, d_x + (uint64_t)c0 * in_dim, d_gain, eps,
+                                                     d_y + (uint64_t)c0 * rows, in_dim, rows, nc, 0u, nullptr,
+                                                     nullptr),
+                           "q6_k_gemv_ncol launch");
+        if (st != LEV_OK) return st;
+    }
+    return LEV_OK;
 }
 
 extern "C" int lev_hip_argmax(lev_ctx *ctx, const float *d_logits, uint32_t vocab, uint32_t ncol,

@@ -1,0 +1,572 @@
+// (RMSNorm +) Q6_K GEMV for one to eight columns of f32 activations on the
+// integer matrix cores of gfx950, every sum formed without rounding.
+//
+// Stands in for g4_q6_matvec / q6k.matvec (Gemma4.swift:4065;
+// lev-forge/src/q6k.rs:61-187) applied to nb columns at once as Builder::matvec
+// does for Q4_K (rust/crates/lev-model/src/gpu.rs:334-370), with the RMSNorm of
+// Builder::norm_quant (gpu.rs:295; rmsnorm, lev-model/src/lib.rs:110-114)
+// optionally fused in front, and for the argmax step behind a single column
+// (lev-forge/src/ops.rs:479-516).
+//
+// A Q6_K superblock (Q6.swift:4-62; dequantize_row_q6_K order) is 16 groups of 16
+// weights w = d * sc_group * (q - 32), q = ql nibble | qh bit pair << 4.  Element
+// 128*half + 32*j + l (j = 0..3, l = 0..31) has its nibble in ql[64*half + 32*(j&1) + l]
+// (low for j < 2, high otherwise), its bit pair j in qh[32*half + l], and the scale
+// sc[8*half + 2*j + l/16].
+//
+// Arithmetic, per superblock of a row and column of x:
+//   * the activations become integers X = rint(x * 2^(30-e)), 2^e the power of two
+//     above the superblock's largest magnitude (|X| <= 2^30: every value within 2^-6
+//     of that maximum is represented exactly), written in four balanced base-256
+//     digits, the bytes of (X + 0x808080) ^ 0x808080 read as int8: four digit planes;
+//   * v_mfma_i32_16x16x64_i8: B = 16 weight rows x 64 codes, each lane group (16
+//     lanes) supplying ONE 16-element scale group as bytes 4*(q - 32); A row
+//     4*gs + p holds digit plane p of the elements lane group gs supplies and zeros
+//     elsewhere, so output row 4*gs + p is the exact sum of 4*(q-32)*digit_p over
+//     that one group — and lands in the lane group that loaded the group's codes;
+//   * the lane multiplies its four plane sums by the group's int8 scale and adds
+//     them up over the superblock in 32-bit integers (|sum| < 2^29), then recombines
+//     the planes in f64 (below 2^53: exact) and applies d and the power of two;
+//   * partial sums of a row (lane groups, waves) are added in f64 and rounded to
+//     f32 once.
+// Nothing depends on the order of the additions.
+//
+// lane (r, g) = (l % 16, l / 16) multiplies weight row r of the task's 16 rows, chunk g
+// of the superblock = ql bytes [32g, 32g+32) (half g/2, j in {g%2, g%2 + 2}) with the 32
+// qh bytes of that half, 8 scale bytes and d.  The bytes do not come from memory in that
+// shape: the L1 takes one tag lookup per 64 bytes a group of four lanes touches, and
+// with one row per lane (16 bytes here, 16 bytes 3360 bytes further on) every lane is a
+// lookup of its own (measured: 27 M lookups per launch, one per CU and clock, 39 us).
+// So a load instruction reads 4 rows x 256 contiguous bytes (16 lanes x 16 bytes per
+// row: the superblock's 210 bytes), four of them a task, and the wave turns the
+// pieces round through a private LDS area (written as loaded, read per (row, chunk);
+// pieces rotated by 4 per row and a 16-byte skew per instruction keep both sides
+// free of bank conflicts).
+//
+// Workgroup = 16 waves.  S waves share a group of 16 rows (each takes 1/S of the
+// row's superblocks), 16/S row groups per workgroup and round; the partial sums of
+// a round meet in LDS.  A NaN or infinity in a column of x makes every output of
+// that column NaN.
+#include "lev_common.hpp"
+#include "top2.hpp"
+
+#include <cstdlib>
+
+namespace {
+
+constexpr int kQThreads = 1024;
+constexpr int kQWaves = kQThreads / LEV_WAVE;
+constexpr uint32_t kQZeroBytes = 512;   // what masked lanes read as their A operand
+
+typedef int q6m_i4 __attribute__((ext_vector_type(4)));
+struct __attribute__((packed, aligned(2))) q6m_u4 { uint32_t v[4]; };
+struct __attribute__((packed, aligned(2))) q6m_u2 { uint32_t v[2]; };
+
+constexpr uint32_t kQAreaStride = 1024 + 16;              // one load instruction's pieces + skew
+constexpr uint32_t kQAreaBytes = 4 * kQAreaStride;        // per wave
+
+struct q6m_regs {
+    q6m_i4 p[4];   // instruction i: row 4i + l/16, piece (l%16 - 4*(l/16)) % 16 of its superblock
+};
+
+// Byte offset, from the start of a superblock, of the piece a lane loads.  Superblocks are
+// 210 bytes: even ones start on a dword boundary, odd ones two bytes past one, and a 16-byte
+// load from such an address costs the L1 several lookups (4 us of 29 at 32000 x 4096).  So
+// the 14 pieces of an odd superblock start 14 bytes early, at [-14 + 16p, +16): dword
+// aligned, ending exactly at the block's end, the logical piece P = bytes [16P, 16P+16) being
+// the last two bytes of piece P and the first 14 of piece P+1.  An even superblock's pieces
+// are [16p, +16) for p < 13.  Piece 13 is bytes [194, 210) for both, so that d is its last
+// two bytes and nothing behind the block is read (for an even superblock that one piece is
+// off the dword boundary).  Lanes 14 and 15 of a row repeat piece 1: never used.
+__device__ __forceinline__ int32_t q6m_piece_offset(uint32_t lane, uint32_t odd) {
+    const uint32_t p = ((lane & 15u) - 4u * (lane >> 4)) & 15u;
+    if (p == 13u) return 194;
+    return (int32_t)(16u * (p < 13u ? p : 1u)) - (odd ? 14 : 0);
+}
+
+__device__ __forceinline__ void q6m_issue(const uint8_t *__restrict__ w, uint64_t row_bytes, uint32_t row0,
+                                          uint32_t rows, uint32_t sb, uint32_t lane, int32_t poff,
+                                          q6m_regs &R) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        uint32_t row = row0 + 4u * (uint32_t)i + (lane >> 4);
+        row = row < rows ? row : rows - 1u;
+        const q6m_u4 v = *reinterpret_cast<const q6m_u4 *>(
+            w + (uint64_t)row * row_bytes + (uint64_t)(int64_t)((int32_t)(sb * 210u) + poff));
+        R.p[i] = q6m_i4{(int)v.v[0], (int)v.v[1], (int)v.v[2], (int)v.v[3]};
+    }
+}
+
+// LDS, for SB superblocks and NC columns:
+//   dig  [NC][16*SB groups][4 planes][16 bytes]
+//   zero [512 bytes]
+//   psb  [NC][SB] f64     2^(e-32) per superblock (the 4 of the codes included)
+//   ssq  [NC][SB] f64     sums of squares (RMSNorm)
+//   part [pb][16 waves][16 rows][NC] f64
+//   inv  [NC] f64, bad [NC] u32
+//   area [16 waves][4 x (1024 + 16) bytes]           the weights of a task on their way round
+template <int NC>
+struct q6m_lds {
+    static __host__ __device__ size_t dig_bytes(uint32_t cols) { return (size_t)NC * cols * 4u; }
+    static __host__ __device__ size_t total(uint32_t cols, uint32_t pb) {
+        return dig_bytes(cols) + kQZeroBytes + (size_t)2 * NC * (cols >> 8) * 8u +
+               (size_t)pb * kQWaves * 16u * NC * 8u + (size_t)NC * 16u + (size_t)kQWaves * kQAreaBytes;
+    }
+};
+
+// NC: columns staged (1, 2, 4 or 8; >= ncol).  S: waves per row group (2..16, a
+// power of two).  partials (optional, ncol == 1): the workgroup's top two outputs.
+template <int NC>
+__global__ void __launch_bounds__(kQThreads)
+q6_k_mfma_gemv(const uint8_t *__restrict__ w, const float *__restrict__ x, const float *__restrict__ gain,
+               float eps, float *__restrict__ y, uint32_t cols, uint32_t rows, uint32_t ncol, uint32_t S,
+               uint32_t pb, double rcols, lev_f32x4 *__restrict__ partials) {
+    using L = q6m_lds<NC>;
+    constexpr uint32_t kLogNC = NC == 8 ? 3u : NC == 4 ? 2u : NC == 2 ? 1u : 0u;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const uint32_t SB = cols >> 8;
+    uint8_t *dig = smem;
+    uint8_t *zero = smem + L::dig_bytes(cols);
+    double *psb = reinterpret_cast<double *>(zero + kQZeroBytes);
+    double *ssq = psb + (size_t)NC * SB;
+    double *part = ssq + (size_t)NC * SB;
+    double *s_inv = part + (size_t)pb * kQWaves * 16u * NC;
+    uint32_t *s_bad = reinterpret_cast<uint32_t *>(s_inv + NC);
+    uint8_t *area_all = reinterpret_cast<uint8_t *>(s_inv) + (size_t)NC * 16u;
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+
+    // ---- geometry of the weight stream ----
+    const uint32_t r = lane & 15u, g = lane >> 4;
+    const uint64_t row_bytes = (uint64_t)SB * 210u;
+    const uint32_t ngroups = (rows + 15u) >> 4;
+    const uint32_t slots = kQWaves / S;                    // row groups per workgroup and round
+    const uint32_t slot = wave / S, kpart = wave % S;
+    const uint32_t tpr = (SB + S - 1u) / S;                // tasks per round and wave
+    const uint32_t wgrounds = (ngroups + slots - 1u) / slots;
+    const uint32_t nrounds = (wgrounds - blockIdx.x + gridDim.x - 1u) / gridDim.x;
+    const uint32_t ntasks = nrounds * tpr;
+    // A cursor walks the wave's tasks in order: round rd, within it superblock
+    // kpart + S*t for t < tpr (S is even: all of a wave's superblocks are even or all odd).
+    // A task past the end reads the first bytes of the matrix.
+    struct cursor {
+        uint32_t k, rd, t;
+    };
+    auto advance = [&](cursor &c) {
+        ++c.k;
+        if (++c.t == tpr) {
+            c.t = 0;
+            ++c.rd;
+        }
+    };
+    const uint32_t odd = kpart & 1u;
+    const int32_t poff = q6m_piece_offset(lane, odd), poff_even = q6m_piece_offset(lane, 0u);
+    auto group_of = [&](uint32_t rd, uint32_t sl) { return (rd * gridDim.x + blockIdx.x) * slots + sl; };
+    auto issue = [&](cursor &c, q6m_regs &W) {
+        const uint32_t sbw = kpart + S * c.t;
+        const bool real = c.k < ntasks && sbw < SB;
+        // (past the end: the first superblock of the matrix, pieces as for an even one)
+        q6m_issue(w, row_bytes, real ? group_of(c.rd, slot) * 16u : 0u, rows, real ? sbw : 0u, lane,
+                  real ? poff : poff_even, W);
+        advance(c);
+    };
+    cursor ci{0u, 0u, 0u}, cc{0u, 0u, 0u};
+    q6m_regs W0, W1, W2;
+
+    // ---- stage the activations ----
+    // A wave takes one superblock of one column per pass (unit u = wave + 16*i: column
+    // u / SB, superblock u % SB), a lane four consecutive elements of it.  All loads
+    // are requested before the first is used; passes beyond the data are skipped.
+    constexpr int CH = 8;                                   // passes: NC*cols <= 32768
+    const uint32_t units = ncol * SB;
+    lev_f32x4 v[CH];
+    if (tid < (uint32_t)NC) s_bad[tid] = 0u;
+    if (tid < kQZeroBytes / 4u) reinterpret_cast<uint32_t *>(zero)[tid] = 0u;
+    {
+        lev_f32x4 gv[CH];
+#pragma unroll
+        for (int i = 0; i < CH; ++i) {
+            if ((uint32_t)i * kQWaves >= units) break;      // workgroup-uniform
+            const uint32_t u = wave + (uint32_t)i * kQWaves;
+            const uint32_t uc = u < units ? u : 0u;
+            const uint32_t c = uc / SB, sb = uc % SB;
+            v[i] = reinterpret_cast<const lev_f32x4 *>(x + (uint64_t)c * cols)[sb * 64u + lane];
+            if (gain) gv[i] = reinterpret_cast<const lev_f32x4 *>(gain)[sb * 64u + lane];
+        }
+        if (gain) {
+            // RMSNorm as the reference computes it: mean square and 1/sqrt in f64, then
+            // (f32)(x * inv) * gain
+#pragma unroll
+            for (int i = 0; i < CH; ++i) {
+                if ((uint32_t)i * kQWaves >= units) break;
+                const uint32_t u = wave + (uint32_t)i * kQWaves;
+                const lev_f32x4 a = v[i];
+                double ss = (double)a.x * (double)a.x;
+                ss = fma((double)a.y, (double)a.y, ss);
+                ss = fma((double)a.z, (double)a.z, ss);
+                ss = fma((double)a.w, (double)a.w, ss);
+                ss = lev_group_sum_f64<64>(ss);
+                if (lane == 63u && u < units) ssq[u] = ss;   // u = c*SB + sb
+            }
+        }
+        // every wave of the workgroup has its activations before the first weights are
+        // requested: a CU's memory pipeline is one queue
+        lev_barrier_lds();
+        issue(ci, W0);
+        if (gain) {
+            if (wave < ncol) {
+                double ss = 0.0;
+                for (uint32_t k = lane; k < SB; k += 64u) ss += ssq[wave * SB + k];
+                ss = lev_group_sum_f64<64>(ss);
+                // 1/sqrt(mean + eps): the hardware estimate and two Newton steps (full f64 accuracy)
+                const double a = fma(ss, rcols, (double)eps);
+                double rs = __builtin_amdgcn_rsq(a);
+                rs = rs * fma(-0.5 * a * rs, rs, 1.5);
+                rs = rs * fma(-0.5 * a * rs, rs, 1.5);
+                if (lane == 63u) s_inv[wave] = rs;
+            }
+            lev_barrier_lds();
+#pragma unroll
+            for (int i = 0; i < CH; ++i) {
+                if ((uint32_t)i * kQWaves >= units) break;
+                const uint32_t u = wave + (uint32_t)i * kQWaves;
+                const double inv = s_inv[u < units ? u / SB : 0u];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) v[i][k] = (float)((double)v[i][k] * inv) * gv[i][k];
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+        if ((uint32_t)i * kQWaves >= units) break;
+        const uint32_t u = wave + (uint32_t)i * kQWaves;
+        const bool real = u < units;
+        const uint32_t c = real ? u / SB : 0u, sb = real ? u % SB : 0u;
+        const lev_f32x4 a = v[i];
+        const float e4[4] = {a.x, a.y, a.z, a.w};
+        // largest magnitude of the superblock as an integer: NaN and infinity sort above every number
+        uint32_t mb = 0u;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const uint32_t bits = __float_as_uint(e4[k]) & 0x7FFFFFFFu;
+            mb = bits > mb ? bits : mb;
+        }
+#define LEV_Q6M_MAXSTEP(CTRL)                                                                       \
+        {                                                                                          \
+            const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp((int)mb, (int)mb, CTRL, 0xF, 0xF, false); \
+            mb = o > mb ? o : mb;                                                                  \
+        }
+        LEV_Q6M_MAXSTEP(0xB1);    // quad_perm [1,0,3,2]
+        LEV_Q6M_MAXSTEP(0x4E);    // quad_perm [2,3,0,1]
+        LEV_Q6M_MAXSTEP(0x141);   // row_half_mirror
+        LEV_Q6M_MAXSTEP(0x140);   // row_mirror: all 16 lanes of a row hold the row's maximum
+#undef LEV_Q6M_MAXSTEP
+        {
+            const uint32_t m0 = (uint32_t)__builtin_amdgcn_readlane((int)mb, 0);
+            const uint32_t m1 = (uint32_t)__builtin_amdgcn_readlane((int)mb, 16);
+            const uint32_t m2 = (uint32_t)__builtin_amdgcn_readlane((int)mb, 32);
+            const uint32_t m3 = (uint32_t)__builtin_amdgcn_readlane((int)mb, 48);
+            const uint32_t ma = m0 > m1 ? m0 : m1, mc = m2 > m3 ? m2 : m3;
+            mb = ma > mc ? ma : mc;
+        }
+        uint32_t ex = mb >> 23;                             // biased exponent: |x| < 2^(ex-126)
+        if (real && ex == 255u && lane == 0u) atomicOr(&s_bad[c], 1u);
+        ex = ex < 30u ? 30u : (ex > 254u ? 254u : ex);      // keeps both powers of two normal numbers
+        const float scale = __uint_as_float((283u - ex) << 23);   // 2^(156-ex): |x*scale| < 2^30
+        uint32_t Y[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int X = (int)rintf(e4[k] * scale);
+            // balanced base-256 digits: adding 0x80 to each of the low three bytes carries into
+            // the next digit where a byte exceeds 127, and flipping bit 7 subtracts it again
+            Y[k] = ((uint32_t)X + 0x00808080u) ^ 0x00808080u;
+        }
+        // 4x4 byte transpose: digit k of the four elements in one dword, element 0 lowest
+        const uint32_t t0 = __builtin_amdgcn_perm(Y[1], Y[0], 0x05010400u);   // a0 b0 a1 b1
+        const uint32_t t1 = __builtin_amdgcn_perm(Y[1], Y[0], 0x07030602u);   // a2 b2 a3 b3
+        const uint32_t t2 = __builtin_amdgcn_perm(Y[3], Y[2], 0x05010400u);
+        const uint32_t t3 = __builtin_amdgcn_perm(Y[3], Y[2], 0x07030602u);
+        const uint32_t dw[4] = {__builtin_amdgcn_perm(t2, t0, 0x05040100u), __builtin_amdgcn_perm(t2, t0, 0x07060302u),
+                                __builtin_amdgcn_perm(t3, t1, 0x05040100u), __builtin_amdgcn_perm(t3, t1, 0x07060302u)};
+        if (real) {
+            // group 16*sb + lane/4, plane p at +16p, the lane's four elements at +4*(lane%4)
+            uint8_t *at = dig + (size_t)c * cols * 4u + (size_t)(16u * sb + (lane >> 2)) * 64u + 4u * (lane & 3u);
+#pragma unroll
+            for (int p = 0; p < 4; ++p) *reinterpret_cast<uint32_t *>(at + 16 * p) = dw[p];
+            if (lane == 0u) psb[c * SB + sb] = __hiloint2double((int)((ex + 865u) << 20), 0);   // 2^(ex-158)
+        }
+    }
+    // columns of the layout beyond ncol hold no data: they only feed outputs that are never stored
+    lev_barrier_lds();
+
+    // ---- stream the weights ----
+    const uint32_t hf = g >> 1, jb = g & 1u;
+    const bool feeds = (r >> 2) == g;                      // this lane's A row belongs to its own lane group
+    const uint32_t maskq = jb ? 0xCCCCCCCCu : 0x33333333u;  // the bit pairs jb and jb+2 of a qh byte
+    const uint32_t rot[2] = {26u + 2u * jb, (30u + 2u * jb) & 31u};   // rotate right: pair jb + 2*nb to bits 6..7
+    const uint32_t scoff[2] = {16u * jb, 16u * jb + 8u};   // bit offset of scale 2*jb + lh in its dword
+    // where (row r, piece P) of a task sits in the wave's area: instruction r/4 wrote row r%4's
+    // pieces to lanes 16*(r%4) + (P + 4*(r%4)) % 16
+    uint8_t *area = area_all + wave * kQAreaBytes;
+    auto piece_at = [&](uint32_t P) {
+        return (r >> 2) * kQAreaStride + (16u * (r & 3u) + ((P + 4u * (r & 3u)) & 15u)) * 16u;
+    };
+    // logical piece P: an even wave reads piece P; an odd one piece P+1 and, for its first
+    // two bytes, the last dword of piece P.  `sel` picks per byte from {next, previous} dword.
+    const uint32_t sel = odd ? 0x05040302u : 0x07060504u;
+    const uint32_t at_ql[2] = {piece_at(2u * g + odd), piece_at(2u * g + 1u + odd)};
+    const uint32_t at_qh[2] = {piece_at(8u + 2u * hf + odd), piece_at(9u + 2u * hf + odd)};
+    const uint32_t c3_ql[2] = {piece_at(2u * g) + 12u, piece_at(2u * g + 1u) + 12u};
+    const uint32_t c3_qh[2] = {piece_at(8u + 2u * hf) + 12u, piece_at(9u + 2u * hf) + 12u};
+    // the eight scale bytes 192 + 8*hf ..: three dwords A0..A2, the wanted two being
+    // {A1, A2} (even) or the bytes 2.. of {A0, A1, A2} (odd: stream position 206 + 8*hf)
+    const uint32_t at_sc[3] = {odd ? (hf ? piece_at(13u) + 4u : piece_at(12u) + 12u) : piece_at(12u),
+                               odd ? (hf ? piece_at(13u) + 8u : piece_at(13u)) : piece_at(12u) + 8u * hf,
+                               odd ? (hf ? piece_at(13u) + 12u : piece_at(13u) + 4u) : piece_at(12u) + 8u * hf + 4u};
+    const uint32_t at_d = piece_at(13u) + 14u;
+    double yacc[NC];
+#pragma unroll
+    for (int q = 0; q < NC; ++q) yacc[q] = 0.0;
+    top2 best{kTop2Floor, kTop2Floor, 0xFFFFFFFFu};
+
+    uint32_t parity = 0;
+    auto compute = [&](cursor &c, const q6m_regs &W) {
+        const uint32_t rd = c.rd, t = c.t;
+        const uint32_t sbw = kpart + S * t;
+        const bool live = sbw < SB;
+        const uint32_t sb = live ? sbw : SB - 1u;
+        // B operands of the four MFMAs (nb = nibble, lh = which 16 of the chunk's 32 bytes): byte =
+        // nibble << 2 | bit pair << 6 with bit 7 flipped = 4*(q - 32) as int8.  The qh dwords are
+        // cleaned once (both pairs this lane uses survive, their top bits flipped); rotated so that
+        // the wanted pair sits in bits 6..7 the other one falls into bits 2..3, which the merge
+        // takes from the nibbles.
+        // the task's pieces go round through the wave's area: written as loaded, read as
+        // (row r, chunk g) wants them.  One wave's LDS operations run in order.
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            *reinterpret_cast<q6m_i4 *>(area + (uint32_t)i * kQAreaStride + lane * 16u) = W.p[i];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        auto piece = [&](uint32_t at, uint32_t c3) {
+            const q6m_i4 n = *reinterpret_cast<const q6m_i4 *>(area + at);
+            const uint32_t prev = *reinterpret_cast<const uint32_t *>(area + c3);
+            return q6m_i4{(int)__builtin_amdgcn_perm((uint32_t)n.x, prev, sel),
+                          (int)__builtin_amdgcn_perm((uint32_t)n.y, (uint32_t)n.x, sel),
+                          (int)__builtin_amdgcn_perm((uint32_t)n.z, (uint32_t)n.y, sel),
+                          (int)__builtin_amdgcn_perm((uint32_t)n.w, (uint32_t)n.z, sel)};
+        };
+        const q6m_i4 ql[2] = {piece(at_ql[0], c3_ql[0]), piece(at_ql[1], c3_ql[1])};
+        const q6m_i4 qh[2] = {piece(at_qh[0], c3_qh[0]), piece(at_qh[1], c3_qh[1])};
+        const uint32_t sa0 = *reinterpret_cast<const uint32_t *>(area + at_sc[0]);
+        const uint32_t sa1 = *reinterpret_cast<const uint32_t *>(area + at_sc[1]);
+        const uint32_t sa2 = *reinterpret_cast<const uint32_t *>(area + at_sc[2]);
+        const uint32_t scw[2] = {__builtin_amdgcn_perm(sa1, sa0, sel), __builtin_amdgcn_perm(sa2, sa1, sel)};
+        const uint32_t dbits = *reinterpret_cast<const uint16_t *>(area + at_d);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();   // the reads are issued before the next task's writes
+        q6m_i4 B[2][2];
+        int sc[2][2];
+#pragma unroll
+        for (int lh = 0; lh < 2; ++lh) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t qc = ((uint32_t)qh[lh][i] ^ 0xAAAAAAAAu) & maskq;
+#pragma unroll
+                for (int nb = 0; nb < 2; ++nb) {
+                    const uint32_t nib = nb ? (uint32_t)ql[lh][i] >> 2 : (uint32_t)ql[lh][i] << 2;
+                    const uint32_t top = __builtin_amdgcn_alignbit(qc, qc, rot[nb]);
+                    B[nb][lh][i] = (int)((nib & 0x3C3C3C3Cu) | (top & ~0x3C3C3C3Cu));
+                }
+            }
+#pragma unroll
+            for (int nb = 0; nb < 2; ++nb) sc[nb][lh] = __builtin_amdgcn_sbfe((int)scw[nb], scoff[lh], 8u);
+        }
+        // a task past the wave's last superblock contributes nothing
+        const double d = live ? (double)lev_f16_bits_to_f32(dbits) : 0.0;
+        // lane (r, g) feeds A row r = 4*gs + p: plane p of group 16*sb + 8*hf + 2*jb (+ 4*nb + lh)
+        // when gs == g, zeros otherwise
+        const uint32_t aoff = (uint32_t)((16u * sb + 8u * hf + 2u * jb) * 64u + 16u * (r & 3u));
+#pragma unroll
+        for (int q = 0; q < NC; ++q) {
+            const uint8_t *ab = feeds ? dig + (size_t)q * cols * 4u + aoff : zero;
+            int E[4] = {0, 0, 0, 0};
+#pragma unroll
+            for (int nb = 0; nb < 2; ++nb) {
+#pragma unroll
+                for (int lh = 0; lh < 2; ++lh) {
+                    const q6m_i4 A = *reinterpret_cast<const q6m_i4 *>(ab + (4 * nb + lh) * 64);
+                    const q6m_i4 D =
+                        __builtin_amdgcn_mfma_i32_16x16x64_i8(A, B[nb][lh], q6m_i4{0, 0, 0, 0}, 0, 0, 0);
+                    // |D| <= 16*128*128 = 2^18, |sc| <= 2^7: four products per plane stay below 2^27
+#pragma unroll
+                    for (int p = 0; p < 4; ++p) {
+                        E[p] += __mul24(D[p], sc[nb][lh]);
+                        asm("" : "+v"(E[p]));   // one multiply-add per plane: keeps the sums from being regrouped
+                    }
+                }
+            }
+            const double hi = fma((double)E[3], 256.0, (double)E[2]);
+            const double lo = fma((double)E[1], 256.0, (double)E[0]);
+            const double dot = fma(hi, 65536.0, lo);
+            yacc[q] = fma(psb[q * SB + sb] * d, dot, yacc[q]);
+        }
+
+        if (t + 1u == tpr) {   // workgroup-uniform: the round ends
+            double *pp = part + parity * (kQWaves * 16u * NC);
+            parity ^= pb - 1u;
+#pragma unroll
+            for (int q = 0; q < NC; ++q) {
+                double s = yacc[q];
+                s += __shfl_xor(s, 16);
+                s += __shfl_xor(s, 32);
+                if (g == 0u) pp[(wave * 16u + r) * NC + q] = s;
+                yacc[q] = 0.0;
+            }
+            lev_barrier_lds();
+            for (uint32_t i = tid; i < slots * 16u * NC; i += kQThreads) {
+                const uint32_t rr = i & 15u, col = (i >> 4) & (NC - 1u), sl = i >> (4u + kLogNC);
+                const uint32_t row = group_of(rd, sl) * 16u + rr;
+                double sum = 0.0;
+                for (uint32_t k = 0; k < S; ++k) sum += pp[((sl * S + k) * 16u + rr) * NC + col];
+                if (col < ncol && row < rows) {
+                    const float out = s_bad[col] ? __builtin_nanf("") : (float)sum;
+                    y[(uint64_t)col * rows + row] = out;
+                    // running top two of the rows this thread finishes (rows ascend, so a tie
+                    // keeps the earlier, lower index)
+                    if (out > best.best) {
+                        best.second = best.best;
+                        best.best = out;
+                        best.idx = row;
+                    } else if (out > best.second) {
+                        best.second = out;
+                    }
+                }
+            }
+            if (pb == 1u) lev_barrier_lds();   // the one buffer is written again by the next round
+        }
+        advance(c);
+    };
+
+    // Three tasks in flight per wave.  The scheduling barriers keep a refill's loads
+    // behind the compute that frees its registers: hoisted above it they would be
+    // younger than the data the compute waits for, and the wait would cover them too.
+    issue(ci, W1);
+    issue(ci, W2);
+    while (true) {
+        compute(cc, W0);
+        __builtin_amdgcn_sched_barrier(0);
+        issue(ci, W0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (cc.k >= ntasks) break;
+        compute(cc, W1);
+        __builtin_amdgcn_sched_barrier(0);
+        issue(ci, W1);
+        __builtin_amdgcn_sched_barrier(0);
+        if (cc.k >= ntasks) break;
+        compute(cc, W2);
+        __builtin_amdgcn_sched_barrier(0);
+        issue(ci, W2);
+        __builtin_amdgcn_sched_barrier(0);
+        if (cc.k >= ntasks) break;
+    }
+
+    if (partials) {
+        __shared__ float s_best[kQWaves], s_second[kQWaves];
+        __shared__ uint32_t s_idx[kQWaves];
+        best = top2_wave(best);
+        if (lane == 0u) {
+            s_best[wave] = best.best;
+            s_second[wave] = best.second;
+            s_idx[wave] = best.idx;
+        }
+        __syncthreads();
+        if (tid == 0u) {
+            top2 m{s_best[0], s_second[0], s_idx[0]};
+            for (int k = 1; k < kQWaves; ++k) m = top2_merge(m, top2{s_best[k], s_second[k], s_idx[k]});
+            partials[blockIdx.x] = lev_f32x4{m.best, m.second, __builtin_bit_cast(float, m.idx), 0.f};
+        }
+    }
+}
+
+size_t q6m_lds_limit(const lev_ctx *ctx) {
+    return ctx->props.sharedMemPerBlockOptin > ctx->props.sharedMemPerBlock ? ctx->props.sharedMemPerBlockOptin
+                                                                            : ctx->props.sharedMemPerBlock;
+}
+
+size_t q6m_lds_bytes(uint32_t cols, uint32_t nc, uint32_t pb) {
+    switch (nc) {
+    case 8: return q6m_lds<8>::total(cols, pb);
+    case 4: return q6m_lds<4>::total(cols, pb);
+    case 2: return q6m_lds<2>::total(cols, pb);
+    default: return q6m_lds<1>::total(cols, pb);
+    }
+}
+
+// Waves per row group.  The busiest workgroup runs ceil(rounds / grid) rounds of SB/S tasks:
+// the smallest S that makes that product smallest (fewer partial sums to add up).
+uint32_t q6m_waves_per_group(const lev_ctx *ctx, uint32_t cols, uint32_t rows) {
+    static const char *env = getenv("LEV_Q6_MFMA_WAVES");
+    if (env && atoi(env) > 1) return (uint32_t)atoi(env);
+    const uint32_t SB = cols >> 8, ngroups = (rows + 15u) / 16u, cus = (uint32_t)ctx->num_cus;
+    uint32_t best = 2, best_cost = 0xFFFFFFFFu;
+    for (uint32_t s = 2; s <= (uint32_t)kQWaves; s <<= 1) {   // even: a wave's superblocks share their parity
+        const uint32_t slots = kQWaves / s, wgrounds = (ngroups + slots - 1u) / slots;
+        const uint32_t cost = ((wgrounds + cus - 1u) / cus) * ((SB + s - 1u) / s);
+        if (cost < best_cost) best_cost = cost, best = s;
+    }
+    return best;
+}
+
+template <int NC>
+hipError_t q6m_launch(lev_ctx *ctx, const uint8_t *w, const float *x, const float *gain, float eps, float *y,
+                      uint32_t cols, uint32_t rows, uint32_t ncol, uint32_t waves, lev_f32x4 *partials,
+                      uint32_t *blocks_out) {
+    const uint32_t pb = q6m_lds_bytes(cols, NC, 2u) <= q6m_lds_limit(ctx) ? 2u : 1u;
+    const size_t lds = q6m_lds_bytes(cols, NC, pb);
+    static size_t configured = 0;   // per instantiation: raise the dynamic LDS limit once per size
+    if (lds > 48 * 1024 && lds > configured) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&q6_k_mfma_gemv<NC>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        configured = lds;
+    }
+    const uint32_t S = waves ? waves : q6m_waves_per_group(ctx, cols, rows);
+    const uint32_t slots = kQWaves / S, ngroups = (rows + 15u) / 16u;
+    const uint32_t wgrounds = (ngroups + slots - 1u) / slots;
+    uint32_t blocks = wgrounds < (uint32_t)ctx->num_cus ? wgrounds : (uint32_t)ctx->num_cus;
+    if (partials && blocks > lev_ctx::kArgmaxPartials) blocks = lev_ctx::kArgmaxPartials;
+    if (blocks_out) *blocks_out = blocks;
+    hipLaunchKernelGGL((q6_k_mfma_gemv<NC>), dim3(blocks), dim3(kQThreads), lds, ctx->stream, w, x, gain, eps,
+                       y, cols, rows, ncol, S, pb, 1.0 / (double)cols, partials);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+// Columns one launch of the matrix-core kernel can take for this in_dim (0: not usable).
+uint32_t lev_q6_k_mfma_cols(const lev_ctx *ctx, uint32_t in_dim) {
+    if (in_dim % 256u != 0u || in_dim == 0u) return 0;
+    uint32_t nc = 8;
+    const size_t limit = q6m_lds_limit(ctx);
+    while (nc >= 1u && ((uint64_t)nc * in_dim > 32768u || q6m_lds_bytes(in_dim, nc, 1u) > limit)) nc >>= 1;
+    return nc;
+}
+
+// The built-in number of waves per row group for a shape.
+uint32_t lev_q6_k_mfma_waves(const lev_ctx *ctx, uint32_t in_dim, uint32_t rows) {
+    return q6m_waves_per_group(ctx, in_dim, rows);
+}
+
+// ncol <= lev_q6_k_mfma_cols(ctx, in_dim); w 2-byte, x and gain 16-byte aligned.  waves: 2, 4,
+// 8 or 16 waves per row group, 0 for the built-in choice.  partials (ncol == 1 only): one
+// top-two record per workgroup, *blocks_out of them.
+hipError_t lev_q6_k_mfma_gemv_launch(lev_ctx *ctx, const uint8_t *w, const float *x, const float *gain,
+                                     float eps, float *y, uint32_t in_dim, uint32_t rows, uint32_t ncol,
+                                     uint32_t waves, lev_f32x4 *partials, uint32_t *blocks_out) {
+    if (waves != 2u && waves != 4u && waves != 8u && waves != 16u) waves = 0u;
+    if (ncol > 4) return q6m_launch<8>(ctx, w, x, gain, eps, y, in_dim, rows, ncol, waves, partials, blocks_out);
+    if (ncol > 2) return q6m_launch<4>(ctx, w, x, gain, eps, y, in_dim, rows, ncol, waves, partials, blocks_out);
+    if (ncol > 1) return q6m_launch<2>(ctx, w, x, gain, eps, y, in_dim, rows, ncol, waves, partials, blocks_out);
+    return q6m_launch<1>(ctx, w, x, gain, eps, y, in_dim, rows, ncol, waves, partials, blocks_out);
+}

@@ -137,6 +137,20 @@ class Context:
                                                     in_dim, rows, ncol))
         return y
 
+    def q6_k_gemv_ncol(self, w, x, in_dim: int, rows: int, ncol: int, gain=None, eps: float = 1e-6,
+                       y=None, w_off: int = 0):
+        """Q6_K GEMV of ``ncol`` f32 columns per weight read (optional RMSNorm in front)."""
+        _dev(w, torch.uint8, "w")
+        _dev(x, torch.float32, "x")
+        if gain is not None:
+            _dev(gain, torch.float32, "gain")
+        if y is None:
+            y = torch.empty((max(ncol, 1), max(rows, 1)), dtype=torch.float32, device=w.device)
+        self._check(self.lib.lev_hip_q6_k_gemv_ncol(self.ctx, _ptr(w), w.numel(), w_off, _ptr(x),
+                                                    x.numel(), _ptr(gain), eps, _ptr(y), y.numel(),
+                                                    in_dim, rows, ncol))
+        return y
+
     def norm_quant_q8(self, x, n: int, ncol: int, gain=None, eps: float = 1e-6, add=None,
                       want_y: bool = False):
         """Int8 activations of ``x`` [ncol][n]: returns (xq int8, xs (d, s) pairs[, y f32])."""

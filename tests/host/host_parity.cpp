@@ -619,7 +619,10 @@ void forge_matvec(Runner &r) {
         EXPECT(!rep.fromCache);
         EXPECT(!rep.candidates.empty());
         EXPECT(q40 || q6 || rep.candidates.size() == 2);                 // matrix-core and vector-ALU kernel
-        EXPECT(!q6 || rep.candidates.size() == (sh.cols == 4096 ? 3u : 2u));   // exact kernel (two waves, one wave a row), f64-sum kernel
+        // matrix-core kernel (built-in waves per row group, then 2 and 4 where they differ), dot4 kernel
+        // (two waves, one wave a row), f64-sum kernel
+        EXPECT(!q6 || rep.candidates.size() == (sh.cols == 4096 ? 6u : 4u));
+        EXPECT(!q6 || rep.candidates[0].schedule.family == 2u);
         EXPECT(!q40 || sh.cols < 1024 || rep.candidates.size() == 6);      // 3 depths x 2 grids, baseline first
         EXPECT(!q40 || sh.cols >= 1024 || rep.candidates.size() == 1);     // narrow rows: the built-in choice only
         for (const ForgeCandidate &c : rep.candidates) {

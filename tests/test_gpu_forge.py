@@ -97,7 +97,11 @@ def test_q6_k_candidates_pass_the_gate(ctx, rows, cols, expected):
     ref = O.q6_k_matvec_f64(w, rows, cols, x)
     dw, dx = dev(w), dev(x)
     cands = ctx.forge_candidates(capi.OP_Q6_K_GEMV, cols, rows)
-    assert [(c.family, c.rows_in_flight) for c in cands] == expected
+    # the matrix-core kernel first, with its built-in number of waves per row group, then with
+    # 2 and 4 where those differ; behind it the kernels it replaced as the built-in choice
+    listed = [(c.family, c.rows_in_flight) for c in cands]
+    assert listed[0][0] == 2 and listed[0][1] in (2, 4, 8, 16)
+    assert listed == [listed[0]] + [(2, n) for n in (2, 4) if n != listed[0][1]] + expected
     outs = []
     try:
         for s in cands:

@@ -323,6 +323,120 @@ def test_q6_k_config2_full_size_with_argmax(ctx):
     assert idx == O.argmax(got) and margin == O.top_margin(got)   # epilogue is exact on its input
 
 
+def q6k_ncol(ctx, w, x, rows, cols, ncol, gain=None, eps=1e-6):
+    y = torch.full((ncol, rows), float("nan"), device="cuda")
+    ctx.q6_k_gemv_ncol(dev(w), dev(x), cols, rows, ncol, gain=None if gain is None else dev(gain),
+                       eps=eps, y=y)
+    ctx.sync()
+    return y.cpu().numpy()
+
+
+@pytest.mark.parametrize("ncol", [1, 2, 3, 4, 5, 8, 16])
+@pytest.mark.parametrize("rows,cols", [(1, 256), (37, 1024), (64, 4096), (21, 4352), (9, 8192), (130, 2816)])
+def test_q6_k_ncol_shapes_with_rmsnorm(ctx, rows, cols, ncol):
+    """Q6_K applied to several f32 columns per weight read, RMSNorm fused in front: every
+    column against the FP64 oracle on the normalised activations, at the reference's 1e-4."""
+    w = O.synth_q6_k(rows * 5 + cols + ncol, rows * cols // 256)
+    x = O.normal(ncol * cols, 100 + rows + ncol).reshape(ncol, cols)
+    gain = O.normal(cols, 7 + ncol, 1.0, 0.1)
+    got = q6k_ncol(ctx, w, x, rows, cols, ncol, gain)
+    xn = H.rmsnorm_rows(x, gain)
+    for c in range(ncol):
+        assert O.max_rel_err(got[c], O.q6_k_matvec_f64(w, rows, cols, xn[c])) < TOL, c
+    plain = q6k_ncol(ctx, w, x, rows, cols, ncol)                # no norm
+    for c in range(ncol):
+        assert O.max_rel_err(plain[c], O.q6_k_matvec_f64(w, rows, cols, x[c])) < TOL, c
+    # the single-column entry point gives the same bits for column 0
+    assert np.array_equal(bits(q6_gemv(ctx, w, x[0], rows, cols)), bits(plain[0]))
+
+
+def test_q6_k_ncol_reference_fixture_and_hand_block(ctx):
+    """The reference's own wide-range 64 x 512 bytes (main.swift:1028-1085) in every column
+    position, and the hand-computed -315 block (main.swift:1091-1120) as one of four columns."""
+    w = H.swift_q6_k_blocks(555, 64 * 2)
+    x = np.stack([O.seeded_input(512, 1, 202 + c) for c in range(4)])
+    got = q6k_ncol(ctx, w, x, 64, 512, 4)
+    for c in range(4):
+        assert O.max_rel_err(got[c], O.q6_k_matvec_f64(w, 64, 512, x[c])) < TOL, c
+    block, xb = H.minus_315_block()
+    xs = np.stack([xb, np.zeros_like(xb), -xb, 2 * xb])
+    got = q6k_ncol(ctx, block, xs, 1, 256, 4)
+    assert got[:, 0].tolist() == [-315.0, 0.0, 315.0, -630.0]
+
+
+@pytest.mark.parametrize("ncol", [1, 4])
+@pytest.mark.parametrize("rows,cols", [(9000, 1024), (40000, 256), (5000, 8192)])
+def test_q6_k_ncol_many_rounds_per_workgroup(ctx, rows, cols, ncol):
+    """Tall matrices: a workgroup takes several rounds of row groups, and rows of one to 32
+    superblocks are shared by 2 to 16 waves."""
+    w = O.synth_q6_k(rows % 89 + ncol, rows * cols // 256)
+    x = O.normal(ncol * cols, rows % 13).reshape(ncol, cols)
+    got = q6k_ncol(ctx, w, x, rows, cols, ncol)
+    for c in range(ncol):
+        assert O.max_rel_err(got[c], O.q6_k_matvec_f64(w, rows, cols, x[c])) < TOL, c
+
+
+def test_q6_k_ncol_exact_sums_columns_and_scale(ctx):
+    """Nothing is rounded before the end: a column's bits do not depend on how many columns
+    travel with it, and scaling x by a power of two scales every output by exactly that power."""
+    rows, cols = 80, 4096
+    w = O.synth_q6_k(31, rows * cols // 256)
+    x = O.normal(8 * cols, 5).reshape(8, cols)
+    base = q6k_ncol(ctx, w, x, rows, cols, 8)
+    for n in (1, 2, 3, 5):
+        assert np.array_equal(bits(q6k_ncol(ctx, w, x[:n], rows, cols, n)), bits(base[:n])), n
+    for e in (-60, -20, 20, 60):
+        got = q6k_ncol(ctx, w, np.ldexp(x[:2], e).astype(np.float32), rows, cols, 2)
+        assert np.array_equal(bits(got), bits(np.ldexp(base[:2], e).astype(np.float32))), e
+
+
+def test_q6_k_ncol_mixed_magnitudes_and_non_finite(ctx):
+    """Superblocks of very different magnitude in one row carry their own power of two; a NaN
+    or an infinity in one column poisons that column only."""
+    rows, cols = 48, 4096
+    w = O.synth_q6_k(8, rows * cols // 256)
+    x = O.normal(3 * cols, 9).reshape(3, cols)
+    x[:, 256:512] *= 1e-6
+    x[:, 1024:1280] *= 3e4
+    x[1, 2048:2304] = 0.0
+    got = q6k_ncol(ctx, w, x, rows, cols, 3)
+    for c in range(3):
+        assert O.max_rel_err(got[c], O.q6_k_matvec_f64(w, rows, cols, x[c])) < TOL, c
+    for bad in (np.nan, np.inf, -np.inf):
+        xb = x.copy()
+        xb[1, 777] = bad
+        res = q6k_ncol(ctx, w, xb, rows, cols, 3)
+        assert np.isnan(res[1]).all(), bad
+        assert np.array_equal(bits(res[0]), bits(got[0])) and np.array_equal(bits(res[2]), bits(got[2]))
+
+
+def test_q6_k_ncol_weights_at_a_2_byte_offset_and_guards(ctx):
+    """GGUF aligns Q6_K tensors to two bytes only; odd geometry and operand counts are refused."""
+    from leviathan_amd import capi
+    from leviathan_amd.ops import LevError
+    rows, cols = 33, 2048
+    w = O.synth_q6_k(3, rows * cols // 256)
+    x = O.normal(2 * cols, 4).reshape(2, cols)
+    ref = q6k_ncol(ctx, w, x, rows, cols, 2)
+    for off in (2, 6, 210, 4098):
+        buf = np.concatenate([np.zeros(off, np.uint8), w])
+        y = ctx.q6_k_gemv_ncol(dev(buf), dev(x), cols, rows, 2, w_off=off)
+        ctx.sync()
+        assert np.array_equal(bits(y.cpu().numpy()), bits(ref)), off
+    wz = dev(np.zeros(210 * 4, np.uint8))
+    xz = dev(np.zeros(2 * 256, np.float32))
+    for kw, status in [
+        (dict(in_dim=100, rows=4, ncol=1), capi.BAD_DIMENSIONS),
+        (dict(in_dim=256, rows=5, ncol=1), capi.BAD_DIMENSIONS),
+        (dict(in_dim=256, rows=4, ncol=3), capi.WRONG_INPUT_COUNT),
+        (dict(in_dim=256, rows=4, ncol=0), capi.BAD_DIMENSIONS),
+        (dict(in_dim=256, rows=4, ncol=17), capi.BAD_DIMENSIONS),
+    ]:
+        with pytest.raises(LevError) as e:
+            ctx.q6_k_gemv_ncol(wz, xz, **kw)
+        assert e.value.status == status, kw
+
+
 def test_argmax_ties_lowest_index_and_columns(ctx):
     """rust/crates/lev-forge/src/ops.rs:508: lowest index on ties; margin = best - second."""
     v = np.full((3, 5000), -1.0, np.float32)
