@@ -45,7 +45,9 @@ struct lev_ctx {
     // words kTicketWord..+3: arrival counters of the router kernel, one per token,
     // zero between launches (the last workgroup to arrive resets its counter)
     int *d_flag = nullptr;
-    static constexpr uint32_t kFlagWords = 64, kTicketWord = 16;
+    // words kArgmaxTicketWord + 1024*k, k = 0..8: arrival counters of the greedy-token merge
+    // (4 KB apart: counters that share a cache line serialise in one L2 channel), zero between launches
+    static constexpr uint32_t kFlagWords = 10 * 1024, kTicketWord = 16, kArgmaxTicketWord = 1024;
     int *h_flag = nullptr;   // pinned
     // True between lev_hip_program_begin and lev_hip_program_end: the stream
     // is being captured, so nothing may allocate or synchronise.

@@ -542,7 +542,7 @@ uint32_t lev_q6_k_mfma_cols(const lev_ctx *ctx, uint32_t in_dim);
 uint32_t lev_q6_k_mfma_waves(const lev_ctx *ctx, uint32_t in_dim, uint32_t rows);
 hipError_t lev_q6_k_mfma_gemv_launch(lev_ctx *ctx, const uint8_t *w, const float *x, const float *gain,
                                      float eps, float *y, uint32_t in_dim, uint32_t rows, uint32_t ncol,
-                                     uint32_t waves, lev_f32x4 *partials, uint32_t *blocks_out);
+                                     uint32_t waves, lev_f32x4 *partials, uint32_t *d_argmax, float *d_margin);
 
 namespace {
 bool q6_mfma_usable(const lev_ctx *ctx, const uint8_t *w, const float *x, uint32_t in_dim) {
@@ -596,15 +596,9 @@ hipError_t lev_q6_k_gemv_argmax_launch(lev_ctx *ctx, const uint8_t *w, const flo
     const lev_schedule *sel = lev_selected(ctx, LEV_OP_Q6_K_GEMV, in_dim, rows, 1);
     const uint32_t family = sel ? sel->family : 2u;
     if (family == 2u && q6_mfma_usable(ctx, w, x, in_dim)) {
-        const bool top = d_argmax || d_margin;
-        uint32_t blocks = 0;
-        lev_f32x4 *partials = top ? static_cast<lev_f32x4 *>(ctx->argmax_partials) : nullptr;
-        hipError_t e = lev_q6_k_mfma_gemv_launch(ctx, w, x, nullptr, 0.f, y, in_dim, rows, 1,
-                                                 sel ? sel->rows_in_flight : 0u, partials, &blocks);
-        if (e != hipSuccess || !top) return e;
-        hipLaunchKernelGGL(argmax_partials_kernel, dim3(1), dim3(1024), 0, ctx->stream, partials, blocks,
-                           d_argmax, d_margin);
-        return hipGetLastError();
+        return lev_q6_k_mfma_gemv_launch(ctx, w, x, nullptr, 0.f, y, in_dim, rows, 1,
+                                         sel ? sel->rows_in_flight : 0u,
+                                         static_cast<lev_f32x4 *>(ctx->argmax_partials), d_argmax, d_margin);
     }
     const bool fast = q6_exact_usable(w, x, units) && family != 1u;
     if (!fast) {
@@ -686,7 +680,7 @@ extern "C" int lev_hip_q6_k_gemv_ncol(lev_ctx *ctx, const void *d_w, size_t w_by
         st = lev_hip_check(ctx,
                            lev_q6_k_mfma_gemv_launch(ctx, w, d_x + (uint64_t)c0 * in_dim, d_gain, eps,
                                                      d_y + (uint64_t)c0 * rows, in_dim, rows, nc, 0u, nullptr,
-                                                     nullptr),
+                                                     nullptr, nullptr),
                            "q6_k_gemv_ncol launch");
         if (st != LEV_OK) return st;
     }

@@ -120,7 +120,8 @@ template <int NC>
 __global__ void __launch_bounds__(kQThreads)
 q6_k_mfma_gemv(const uint8_t *__restrict__ w, const float *__restrict__ x, const float *__restrict__ gain,
                float eps, float *__restrict__ y, uint32_t cols, uint32_t rows, uint32_t ncol, uint32_t S,
-               uint32_t pb, double rcols, lev_f32x4 *__restrict__ partials) {
+               uint32_t pb, double rcols, lev_f32x4 *__restrict__ partials, uint32_t *__restrict__ tickets,
+               uint32_t *__restrict__ out_idx, float *__restrict__ out_margin) {
     using L = q6m_lds<NC>;
     constexpr uint32_t kLogNC = NC == 8 ? 3u : NC == 4 ? 2u : NC == 2 ? 1u : 0u;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -474,17 +475,67 @@ q6_k_mfma_gemv(const uint8_t *__restrict__ w, const float *__restrict__ x, const
     if (partials) {
         __shared__ float s_best[kQWaves], s_second[kQWaves];
         __shared__ uint32_t s_idx[kQWaves];
-        best = top2_wave(best);
-        if (lane == 0u) {
-            s_best[wave] = best.best;
-            s_second[wave] = best.second;
-            s_idx[wave] = best.idx;
+        // only the waves that stored outputs hold candidates; wave 0 finishes alone, so that no
+        // wave waits at a barrier for another one's stores
+        const uint32_t nred0 = (slots * 16u * NC + 63u) >> 6, nred = nred0 < (uint32_t)kQWaves ? nred0 : (uint32_t)kQWaves;
+        if (wave < nred) {
+            best = top2_wave(best);
+            if (lane == 0u) {
+                s_best[wave] = best.best;
+                s_second[wave] = best.second;
+                s_idx[wave] = best.idx;
+            }
         }
-        __syncthreads();
-        if (tid == 0u) {
-            top2 m{s_best[0], s_second[0], s_idx[0]};
-            for (int k = 1; k < kQWaves; ++k) m = top2_merge(m, top2{s_best[k], s_second[k], s_idx[k]});
-            partials[blockIdx.x] = lev_f32x4{m.best, m.second, __builtin_bit_cast(float, m.idx), 0.f};
+        lev_barrier_lds();
+        if (wave != 0u) return;
+        top2 m{kTop2Floor, kTop2Floor, 0xFFFFFFFFu};
+        if (lane < nred) m = top2{s_best[lane], s_second[lane], s_idx[lane]};
+        m = top2_wave(m);
+        if (!tickets) {
+            if (lane == 0u)
+                partials[blockIdx.x] = lev_f32x4{m.best, m.second, __builtin_bit_cast(float, m.idx), 0.f};
+            return;
+        }
+        // The last workgroup to finish merges the partials (a kernel of its own for that costs a
+        // launch and a cold round trip: 7 us behind a 25 us GEMV).  The partial goes out in
+        // device-scope stores, which go through to memory, and the arrival is counted once they
+        // have completed (a fence here would write back every dirty line of the L2, the rows of y
+        // included: 250 of those cost 12 us).  Arrivals are counted in eight groups (workgroup
+        // index mod 8, counters 4 KB apart, so that they do not queue up in one L2 channel); the
+        // last of each group arrives at a ninth counter.
+        uint32_t last = 0u;
+        if (lane == 0u) {
+            float *pf = reinterpret_cast<float *>(partials + blockIdx.x);
+            __hip_atomic_store(pf, m.best, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(pf + 1, m.second, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(pf + 2, __builtin_bit_cast(float, m.idx), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            const uint32_t grp = blockIdx.x & 7u, ngrp = gridDim.x < 8u ? gridDim.x : 8u;
+            const uint32_t in_grp = (gridDim.x - grp + 7u) >> 3;
+            if (__hip_atomic_fetch_add(&tickets[(1u + grp) * 1024u], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ==
+                in_grp - 1u) {
+                // nobody else touches the counter before the next launch
+                __hip_atomic_store(&tickets[(1u + grp) * 1024u], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (__hip_atomic_fetch_add(&tickets[0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == ngrp - 1u) {
+                    __hip_atomic_store(&tickets[0], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    last = 1u;
+                }
+            }
+        }
+        if (!__builtin_amdgcn_readfirstlane((int)last)) return;
+        top2 f{kTop2Floor, kTop2Floor, 0xFFFFFFFFu};
+        const float *pf = reinterpret_cast<const float *>(partials);
+        for (uint32_t i = lane; i < gridDim.x; i += 64u) {
+            // device-scope loads: the other workgroups' partials come from beyond this XCD's L2
+            const float b = __hip_atomic_load(pf + 4u * i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const float s2 = __hip_atomic_load(pf + 4u * i + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const float ib = __hip_atomic_load(pf + 4u * i + 2u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            f = top2_merge(f, top2{b, s2, __float_as_uint(ib)});
+        }
+        f = top2_wave(f);
+        if (lane == 0u) {
+            if (out_idx) out_idx[0] = f.idx == 0xFFFFFFFFu ? 0u : f.idx;   // nothing above -inf: first
+            if (out_margin) out_margin[0] = f.best - f.second;
         }
     }
 }
@@ -521,7 +572,7 @@ uint32_t q6m_waves_per_group(const lev_ctx *ctx, uint32_t cols, uint32_t rows) {
 template <int NC>
 hipError_t q6m_launch(lev_ctx *ctx, const uint8_t *w, const float *x, const float *gain, float eps, float *y,
                       uint32_t cols, uint32_t rows, uint32_t ncol, uint32_t waves, lev_f32x4 *partials,
-                      uint32_t *blocks_out) {
+                      uint32_t *d_argmax, float *d_margin) {
     const uint32_t pb = q6m_lds_bytes(cols, NC, 2u) <= q6m_lds_limit(ctx) ? 2u : 1u;
     const size_t lds = q6m_lds_bytes(cols, NC, pb);
     static size_t configured = 0;   // per instantiation: raise the dynamic LDS limit once per size
@@ -536,9 +587,9 @@ hipError_t q6m_launch(lev_ctx *ctx, const uint8_t *w, const float *x, const floa
     const uint32_t wgrounds = (ngroups + slots - 1u) / slots;
     uint32_t blocks = wgrounds < (uint32_t)ctx->num_cus ? wgrounds : (uint32_t)ctx->num_cus;
     if (partials && blocks > lev_ctx::kArgmaxPartials) blocks = lev_ctx::kArgmaxPartials;
-    if (blocks_out) *blocks_out = blocks;
+    uint32_t *tickets = partials ? reinterpret_cast<uint32_t *>(ctx->d_flag) + lev_ctx::kArgmaxTicketWord : nullptr;
     hipLaunchKernelGGL((q6_k_mfma_gemv<NC>), dim3(blocks), dim3(kQThreads), lds, ctx->stream, w, x, gain, eps,
-                       y, cols, rows, ncol, S, pb, 1.0 / (double)cols, partials);
+                       y, cols, rows, ncol, S, pb, 1.0 / (double)cols, partials, tickets, d_argmax, d_margin);
     return hipGetLastError();
 }
 
@@ -559,14 +610,17 @@ uint32_t lev_q6_k_mfma_waves(const lev_ctx *ctx, uint32_t in_dim, uint32_t rows)
 }
 
 // ncol <= lev_q6_k_mfma_cols(ctx, in_dim); w 2-byte, x and gain 16-byte aligned.  waves: 2, 4,
-// 8 or 16 waves per row group, 0 for the built-in choice.  partials (ncol == 1 only): one
-// top-two record per workgroup, *blocks_out of them.
+// 8 or 16 waves per row group, 0 for the built-in choice.  d_argmax / d_margin (ncol == 1
+// only, both may be NULL): the greedy token of the column, merged by the last workgroup to
+// finish from one top-two record per workgroup in `partials` (lev_ctx::kArgmaxPartials
+// records).
 hipError_t lev_q6_k_mfma_gemv_launch(lev_ctx *ctx, const uint8_t *w, const float *x, const float *gain,
                                      float eps, float *y, uint32_t in_dim, uint32_t rows, uint32_t ncol,
-                                     uint32_t waves, lev_f32x4 *partials, uint32_t *blocks_out) {
+                                     uint32_t waves, lev_f32x4 *partials, uint32_t *d_argmax, float *d_margin) {
+    if (!d_argmax && !d_margin) partials = nullptr;
     if (waves != 2u && waves != 4u && waves != 8u && waves != 16u) waves = 0u;
-    if (ncol > 4) return q6m_launch<8>(ctx, w, x, gain, eps, y, in_dim, rows, ncol, waves, partials, blocks_out);
-    if (ncol > 2) return q6m_launch<4>(ctx, w, x, gain, eps, y, in_dim, rows, ncol, waves, partials, blocks_out);
-    if (ncol > 1) return q6m_launch<2>(ctx, w, x, gain, eps, y, in_dim, rows, ncol, waves, partials, blocks_out);
-    return q6m_launch<1>(ctx, w, x, gain, eps, y, in_dim, rows, ncol, waves, partials, blocks_out);
+    if (ncol > 4) return q6m_launch<8>(ctx, w, x, gain, eps, y, in_dim, rows, ncol, waves, partials, d_argmax, d_margin);
+    if (ncol > 2) return q6m_launch<4>(ctx, w, x, gain, eps, y, in_dim, rows, ncol, waves, partials, d_argmax, d_margin);
+    if (ncol > 1) return q6m_launch<2>(ctx, w, x, gain, eps, y, in_dim, rows, ncol, waves, partials, d_argmax, d_margin);
+    return q6m_launch<1>(ctx, w, x, gain, eps, y, in_dim, rows, ncol, waves, partials, d_argmax, d_margin);
 }

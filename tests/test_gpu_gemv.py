@@ -437,6 +437,26 @@ def test_q6_k_ncol_weights_at_a_2_byte_offset_and_guards(ctx):
         assert e.value.status == status, kw
 
 
+def test_q6_k_greedy_token_merge_over_many_launches(ctx):
+    """The greedy token is merged inside the GEMV by the last workgroup to finish, from
+    per-workgroup records left in a buffer that outlives the launch: many launches in a row
+    with different activations, each checked against the launch's own logits (a record from an
+    earlier launch, or one not yet visible, would name another row or another margin)."""
+    rows, cols = 16400, 1024
+    w = dev(O.synth_q6_k(17, rows * cols // 256))
+    xs = torch.randn(60, cols, device="cuda", generator=torch.Generator(device="cuda").manual_seed(3))
+    outs = []
+    for i in range(60):
+        y, idx, mg = ctx.q6_k_gemv(w, xs[i].contiguous(), cols, rows, argmax=True)
+        outs.append((y, idx, mg))
+    ctx.sync()
+    for i, (y, idx, mg) in enumerate(outs):
+        top = torch.topk(y, 2)
+        ties = (y == top.values[0]).nonzero()
+        assert int(idx.item()) == int(ties[0].item()), i
+        assert float(mg.item()) == float(top.values[0] - top.values[1]), i
+
+
 def test_argmax_ties_lowest_index_and_columns(ctx):
     """rust/crates/lev-forge/src/ops.rs:508: lowest index on ties; margin = best - second."""
     v = np.full((3, 5000), -1.0, np.float32)
