@@ -332,6 +332,13 @@ def main():
             run_other("q6_k_gemv_32000x4096_no_argmax", lambda i: must(lib.lev_hip_q6_k_gemv(
                 c, ring6.data_ptr(), ring6.numel(), (i % 6) * nb6 * 210, x.data_ptr(), cols,
                 y6.data_ptr(), r6, cols, r6, None, None)), nb6 * 210 + cols * 4 + r6 * 4, 100, 20)
+            # the head on f32 activations, N columns per weight read
+            for n in (2, 4, 8):
+                xn = torch.randn(n, cols, device=dev, generator=gen)
+                yn = torch.empty(n, r6, device=dev)
+                run_other(f"q6_k_gemv_ncol_32000x4096_N{n}", lambda i: must(lib.lev_hip_q6_k_gemv_ncol(
+                    c, ring6.data_ptr(), ring6.numel(), (i % 6) * nb6 * 210, xn.data_ptr(), xn.numel(), None, 0.0,
+                    yn.data_ptr(), yn.numel(), cols, r6, n)), nb6 * 210 + n * (cols * 4 + r6 * 4), 100, 20)
             # the head on int8 activations, N columns per weight read (MTP verify)
             for n in (1, 4, 8):
                 xn = torch.randn(n, cols, device=dev, generator=gen)

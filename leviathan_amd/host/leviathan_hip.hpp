@@ -482,6 +482,42 @@ public:
               tensor);
     }
 
+    // ---- Builder::norm_quant + Builder::matvec on f32 activations, gpu.rs:295, 334-370 ----
+    // y[nb][rows] (from float index yOffset) = W rmsnorm(x[nb][inDim]) * gain for a Q4_K or
+    // Q6_K tensor, every column per one pass over the weights; no gain tensor: y = W x.
+    // Sums are formed without rounding, so a column does not depend on its companions.
+    void matvecCols(const std::string &tensor, const DeviceBuffer &x, int64_t nb, DeviceBuffer &y,
+                    const std::optional<std::string> &gainTensor = std::nullopt, int64_t yOffset = 0,
+                    std::optional<int64_t> maxRows = std::nullopt) {
+        const TensorRef &r = lookup(tensor);
+        if (r.type != GGMLTensorType::q4_K && r.type != GGMLTensorType::q6_K)
+            geometry(tensor + ": unsupported type for the multi-column matvec");
+        const float *g = nullptr;
+        if (gainTensor) {
+            auto it = ref_.find(*gainTensor);
+            if (it == ref_.end() || it->second.type != GGMLTensorType::float32 ||
+                it->second.inDim != r.inDim || it->second.end - it->second.offset != r.inDim * 4)
+                geometry("bad norm weight " + *gainTensor);
+            g = reinterpret_cast<const float *>(static_cast<const char *>(weights_.contents()) +
+                                                it->second.offset);
+        }
+        const int64_t blockBytes = bytesPerBlock(r.type);
+        const int64_t rows = std::min(r.outDim, maxRows.value_or(r.outDim));
+        int64_t count, outs, weightBytes, wEnd;
+        if (!(rows > 0 && r.inDim > 0 && r.inDim % 256 == 0 && nb > 0 && yOffset >= 0) ||
+            __builtin_mul_overflow(r.inDim, nb, &count) || __builtin_mul_overflow(rows, nb, &outs) ||
+            x.length < count * 4 || y.length < (yOffset + outs) * 4)
+            geometry("buffer extents violated for " + tensor);
+        if (__builtin_mul_overflow(rows, r.inDim / 256 * blockBytes, &weightBytes) ||
+            __builtin_add_overflow(r.offset, weightBytes, &wEnd) || wEnd > r.end || wEnd > mapEnd_)
+            geometry(tensor + ": weight bytes beyond tensor extent");
+        auto *kernel = r.type == GGMLTensorType::q4_K ? lev_hip_q4_k_gemv_ncol : lev_hip_q6_k_gemv_ncol;
+        check(kernel(ctx_, weights_.contents(), (size_t)weights_.length, (uint64_t)r.offset, x.floats(),
+                     (size_t)count, g, eps_, y.floats() + yOffset, (size_t)(y.length / 4 - yOffset),
+                     (uint32_t)r.inDim, (uint32_t)rows, (uint32_t)nb),
+              tensor);
+    }
+
     // ---- Gemma4.swift:3103 ----
     void geluUp(const DeviceBuffer &gu, DeviceBuffer &y, int64_t n) {
         if (n <= 0 || gu.length < 2 * n * 4 || y.length < n * 4)

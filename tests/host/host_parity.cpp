@@ -326,6 +326,55 @@ void runner_int8_path(Runner &r, const Model &m) {
     r.flushOpenSegment();
 }
 
+// F32-activation multi-column path: the RMSNorm of Builder::norm_quant fused in front of
+// Builder::matvec (rust/crates/lev-model/src/gpu.rs:295-370), every column per one pass over a
+// Q4_K tensor or the Q6_K head, gated at 1e-4 against the FP64 product on the CPU rmsnorm.
+void runner_f32_columns(Runner &r, const Model &m) {
+    const int H = Model::hidden, NB = 3, ROWS = 64;
+    std::vector<float> x((size_t)NB * H);
+    levo_fill_normal(81, 0.f, 1.f, x.data(), x.size());
+    DeviceBuffer dx = r.makeBuffer(x);
+    DeviceBuffer dy = r.makeBuffer((int64_t)NB * ROWS * 4), dl = r.makeBuffer((int64_t)NB * Model::vocab * 4);
+    const float *gain = reinterpret_cast<const float *>(m.at("blk.0.ffn_norm.weight"));
+    const TensorRef &t = m.table.at("blk.0.ffn_up.weight"), &o = m.table.at("output.weight");
+    r.matvecCols("blk.0.ffn_up.weight", dx, NB, dy, std::string("blk.0.ffn_norm.weight"));
+    r.matvecCols("output.weight", dx, NB, dl, std::string("blk.0.ffn_norm.weight"));
+    std::vector<float> y = r.read<float>(dy, (size_t)NB * ROWS), logits = r.read<float>(dl, (size_t)NB * Model::vocab);
+    for (int c = 0; c < NB; ++c) {
+        std::vector<float> xn(H);
+        levo_rmsnorm(x.data() + (size_t)c * H, gain, 1e-6f, H, xn.data());
+        std::vector<double> ref(ROWS), lref(Model::vocab);
+        EXPECT(levo_q4_k_matvec_f64(m.at("blk.0.ffn_up.weight"), (size_t)(t.end - t.offset), ROWS, H, xn.data(), H,
+                                    ref.data()) == 0);
+        EXPECT(levo_q6_k_matvec_f64(m.at("output.weight"), (size_t)(o.end - o.offset), Model::vocab, H, xn.data(), H,
+                                    lref.data()) == 0);
+        EXPECT(rel_err(std::vector<float>(y.begin() + (size_t)c * ROWS, y.begin() + (size_t)(c + 1) * ROWS), ref) < 1e-4);
+        EXPECT(rel_err(std::vector<float>(logits.begin() + (size_t)c * Model::vocab,
+                                          logits.begin() + (size_t)(c + 1) * Model::vocab), lref) < 1e-4);
+    }
+    // no gain: the plain product; one column alone gives the same bits as in company
+    DeviceBuffer d1 = r.makeBuffer((int64_t)Model::vocab * 4);
+    r.matvecCols("output.weight", dx, NB, dl);
+    r.matvecCols("output.weight", dx, 1, d1);
+    std::vector<float> all = r.read<float>(dl, (size_t)NB * Model::vocab), one = r.read<float>(d1, Model::vocab);
+    EXPECT(std::memcmp(all.data(), one.data(), (size_t)Model::vocab * 4) == 0);
+    std::vector<double> lref(Model::vocab);
+    EXPECT(levo_q6_k_matvec_f64(m.at("output.weight"), (size_t)(o.end - o.offset), Model::vocab, H, x.data(), H,
+                                lref.data()) == 0);
+    EXPECT(rel_err(one, lref) < 1e-4);
+    // and the single-column operator agrees bit for bit
+    DeviceBuffer ds = r.makeBuffer((int64_t)Model::vocab * 4);
+    r.matvec("output.weight", dx, H, ds, Model::vocab);
+    EXPECT(std::memcmp(r.read<float>(ds, Model::vocab).data(), one.data(), (size_t)Model::vocab * 4) == 0);
+    // a prefix of the rows, and the guards before any launch
+    r.matvecCols("blk.0.ffn_up.weight", dx, NB, dy, std::nullopt, 0, 16);
+    EXPECT(throws_geometry([&] { r.matvecCols("blk.0.attn_q.weight", dx, NB, dy); }));                 // Q4_0
+    EXPECT(throws_geometry([&] { r.matvecCols("blk.0.ffn_up.weight", dx, NB + 1, dy); }));             // x too small
+    EXPECT(throws_geometry([&] { r.matvecCols("blk.0.ffn_up.weight", dx, NB, dy, std::nullopt, 8); })); // y too small
+    EXPECT(throws_geometry([&] { r.matvecCols("blk.0.ffn_up.weight", dx, NB, dy, std::string("blk.0.attn_q.weight")); }));
+    r.flushOpenSegment();
+}
+
 void runner_elementwise(Runner &r, const Model &m) {
     const int H = Model::hidden, V = 3;
     std::vector<float> x((size_t)V * H);
@@ -806,6 +855,7 @@ int main(int argc, char **argv) {
         {"runner_matvec", [&] { runner_matvec(R(), model); }},
         {"runner_elementwise", [&] { runner_elementwise(R(), model); }},
         {"runner_int8_path", [&] { runner_int8_path(R(), model); }},
+        {"runner_f32_columns", [&] { runner_f32_columns(R(), model); }},
         {"runner_shared_expert", [&] { runner_shared_expert(R(), model); }},
         {"runner_moe", [&] { runner_moe(R(), model); }},
         {"runner_moe_hand_computed", [&] { runner_moe_hand_computed(R()); }},

@@ -12,7 +12,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 BIN = os.path.join(ROOT, "tests", "host", "build", "host_parity")
 
 CASES = ["q4_backend_2x32", "q4_backend_minus_16", "q4_backend_guards", "q6_backend_minus_315",
-         "q4_backend_seeded", "runner_matvec", "runner_elementwise", "runner_int8_path", "runner_shared_expert",
+         "q4_backend_seeded", "runner_matvec", "runner_elementwise", "runner_int8_path", "runner_f32_columns", "runner_shared_expert",
          "runner_moe",
          "runner_moe_hand_computed", "runner_gguf_file", "forge_matvec", "forge_moe_layer"]
 
