@@ -525,14 +525,17 @@ moe_scores_select_kernel(const float *__restrict__ wr, const float *__restrict__
         if (lane == 0) s_score[wave] = (float)acc;
     }
     lev_barrier_lds();
-    // One wave stores the workgroup's eight scores, makes them visible beyond this
-    // XCD (a fence writes the L2's dirty lines back: once per workgroup, not per
-    // wave) and takes the workgroup's arrival number.
+    // One wave stores the workgroup's eight scores with device-scope stores, which go
+    // through to memory, waits for them and takes the workgroup's arrival number (a
+    // fence in their place writes back every dirty line of the XCD's L2).
     if (wave == 0) {
         const uint32_t eo = blockIdx.x * 8u + lane;
-        if (lane < 8u && eo < experts) scores[(uint64_t)t * experts + eo] = s_score[lane];
-        __threadfence();
-        if (lane == 0) s_ticket = atomicAdd(&tickets[t], 1u);
+        if (lane < 8u && eo < experts)
+            __hip_atomic_store(&scores[(uint64_t)t * experts + eo], s_score[lane], __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if (lane == 0)
+            s_ticket = __hip_atomic_fetch_add(&tickets[t], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads();
     if (s_ticket != gridDim.x - 1u) return;

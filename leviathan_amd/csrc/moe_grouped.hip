@@ -286,6 +286,7 @@ moe_grouped_kernel(lev_moe_grouped_args a, uint32_t tiles_per_wg, const float *_
         }
         __syncthreads();
 
+        uint32_t cmax[4] = {0u, 0u, 0u, 0u};
         for (uint32_t tile = t0; tile < t1; ++tile) {
             lev_f32x4 y = {0.f, 0.f, 0.f, 0.f};
             for (uint32_t grp = 0; grp < ngrp; ++grp) {
@@ -360,18 +361,33 @@ moe_grouped_kernel(lev_moe_grouped_args a, uint32_t tiles_per_wg, const float *_
                         out[(uint64_t)p * out_rows + row] = v;
                     }
                     if (PAIRED) {
-                        // largest |act| of the pair: over the wave's 16 rows first, then one atomic per
-                        // column; the bit patterns of non-negative floats order as the floats do, and a
-                        // NaN ranks above every number (the down stage then leaves the row unscaled)
-                        uint32_t m = __float_as_uint(fabsf(v));
-#pragma unroll
-                        for (int off = 1; off < 16; off <<= 1) {
-                            const uint32_t o = (uint32_t)__shfl_xor((int)m, off);
-                            m = m > o ? m : o;
-                        }
-                        if (r == 0u && col < ncols && m != 0u) atomicMax(out_max + p, m);
+                        // running maximum of |act| per column over this wave's tiles: the bit patterns
+                        // of non-negative floats order as the floats do, and a NaN ranks above every
+                        // number (the down stage then leaves the row unscaled)
+                        const uint32_t m = __float_as_uint(fabsf(v));
+                        cmax[i] = m > cmax[i] ? m : cmax[i];
                     }
                 }
+            }
+        }
+        if (PAIRED && is_up) {
+            // largest |act| of each of the pass's pairs: over the wave's 16 rows by DPP, then one
+            // atomic per column and wave
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                uint32_t m = cmax[i];
+#define LEV_GRP_MAXSTEP(CTRL)                                                                          \
+                {                                                                                      \
+                    const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp((int)m, (int)m, CTRL, 0xF, 0xF, false); \
+                    m = o > m ? o : m;                                                                 \
+                }
+                LEV_GRP_MAXSTEP(0xB1);    // quad_perm [1,0,3,2]
+                LEV_GRP_MAXSTEP(0x4E);    // quad_perm [2,3,0,1]
+                LEV_GRP_MAXSTEP(0x141);   // row_half_mirror
+                LEV_GRP_MAXSTEP(0x140);   // row_mirror
+#undef LEV_GRP_MAXSTEP
+                const uint32_t col = 4u * g + (uint32_t)i;
+                if (r == 0u && col < ncols && m != 0u) atomicMax(out_max + s_pair[col], m);
             }
         }
     }
