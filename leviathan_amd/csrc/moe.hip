@@ -415,10 +415,13 @@ moe_scores_kernel(const float *__restrict__ wr, const float *__restrict__ x,
 
 // Many tokens: scores as a small f64 matrix product on the matrix cores
 // (v_mfma_f64_16x16x4_f64: exact products of f32 inputs, f64 sums, rounded to
-// f32 once).  Workgroup = a 16-token x 16-expert tile, its sixteen waves split
-// the hidden dimension (the loop is latency-bound: a short share per wave keeps
-// all of its loads in flight at once) and their partial tiles are added in
-// wave order.  The router
+// f32 once by the selection kernel).  A 16-token x 16-expert tile is shared by
+// kScoreSplit workgroups of four waves; the sixteen waves split the hidden
+// dimension (the loop is latency-bound: a short share per wave keeps all of its
+// loads in flight at once, and four workgroups a tile put 128 CUs instead of 32
+// to work at 64 tokens x 128 experts).  A workgroup adds its waves' partial
+// tiles in wave order and leaves the f64 sum in partials[split][token][expert];
+// moe_topk_kernel adds the kScoreSplit of them in order.  The router
 // and the activations are each read (tokens/16) resp. (experts/16) times instead
 // of once per (expert, 16 tokens).
 // Lane (i, kq) = (l % 16, l / 16) loads four consecutive floats of token row i
@@ -427,11 +430,14 @@ moe_scores_kernel(const float *__restrict__ wr, const float *__restrict__ x,
 // operands.  hidden % 256 == 0, rows 16-byte aligned.
 typedef double moe_f64x4 __attribute__((ext_vector_type(4)));
 
-__global__ void __launch_bounds__(1024)
-moe_scores_mfma_kernel(const float *__restrict__ wr, const float *__restrict__ x, float *__restrict__ scores,
+constexpr uint32_t kScoreSplit = 4;
+
+__global__ void __launch_bounds__(256)
+moe_scores_mfma_kernel(const float *__restrict__ wr, const float *__restrict__ x, double *__restrict__ partials,
                        uint32_t hidden, uint32_t experts, uint32_t tokens) {
-    __shared__ double part[16][256];
-    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    __shared__ double part[16 / kScoreSplit][256];
+    const uint32_t lane = threadIdx.x & 63u, lw = threadIdx.x >> 6;
+    const uint32_t wave = blockIdx.z * (16u / kScoreSplit) + lw;   // which sixteenth of the hidden dimension
     const uint32_t i = lane & 15u, kq = lane >> 4;
     const uint32_t e0 = blockIdx.x * 16u, t0 = blockIdx.y * 16u;
     const uint32_t tok = t0 + i < tokens ? t0 + i : tokens - 1u;       // rows past the end repeat the last one
@@ -451,26 +457,46 @@ moe_scores_mfma_kernel(const float *__restrict__ wr, const float *__restrict__ x
     }
     // D of the f64 16x16x4 product: register r of lane (i, kq) is row (token) 4*r + kq of column (expert) i
 #pragma unroll
-    for (int r = 0; r < 4; ++r) part[wave][(4u * (uint32_t)r + kq) * 16u + i] = acc[r];
+    for (int r = 0; r < 4; ++r) part[lw][(4u * (uint32_t)r + kq) * 16u + i] = acc[r];
     lev_barrier_lds();
     const uint32_t tt = (threadIdx.x >> 4) & 15u, ee = threadIdx.x & 15u;
-    if (threadIdx.x < 256u && t0 + tt < tokens && e0 + ee < experts) {
+    if (t0 + tt < tokens && e0 + ee < experts) {
         double total = part[0][threadIdx.x];
 #pragma unroll
-        for (int w = 1; w < 16; ++w) total += part[w][threadIdx.x];
-        scores[(uint64_t)(t0 + tt) * experts + e0 + ee] = (float)total;
+        for (uint32_t w = 1; w < 16u / kScoreSplit; ++w) total += part[w][threadIdx.x];
+        partials[((uint64_t)blockIdx.z * tokens + t0 + tt) * experts + e0 + ee] = total;
     }
 }
 
 // grid (tokens), 256 threads: selection for one token, written to global memory.
+// partials (optional): the scores arrive as kScoreSplit f64 partial sums per (token,
+// expert) from moe_scores_mfma_kernel; they are added in order, rounded to f32 once
+// and also stored in `scores`.
 template <int J>
 __global__ void __launch_bounds__(256)
-moe_topk_kernel(const float *__restrict__ scores, const float *__restrict__ expert_scale,
-                int32_t *__restrict__ ids, float *__restrict__ weights, int *__restrict__ flag,
-                uint32_t experts, uint32_t top_k) {
+moe_topk_kernel(float *__restrict__ scores, const double *__restrict__ partials,
+                const float *__restrict__ expert_scale, int32_t *__restrict__ ids,
+                float *__restrict__ weights, int *__restrict__ flag, uint32_t experts, uint32_t top_k,
+                uint32_t tokens) {
     extern __shared__ double s_router[];
     const uint32_t t = blockIdx.x;
-    const router_sel r = router_select_block<J>(scores + (uint64_t)t * experts, s_router, experts, top_k);
+    router_sel r;
+    if (partials) {
+        const uint32_t lane = threadIdx.x & 63u;
+        float sc[J];
+#pragma unroll
+        for (int j = 0; j < J; ++j) {
+            const uint32_t i = lane + 64u * j, ic = i < experts ? i : experts - 1u;
+            double total = partials[(uint64_t)t * experts + ic];
+#pragma unroll
+            for (uint32_t k = 1; k < kScoreSplit; ++k) total += partials[((uint64_t)k * tokens + t) * experts + ic];
+            sc[j] = (float)total;
+            if (threadIdx.x < 64u && i < experts) scores[(uint64_t)t * experts + i] = sc[j];
+        }
+        r = router_select_regs<J>(sc, s_router, experts, top_k, true, false);
+    } else {
+        r = router_select_block<J>(scores + (uint64_t)t * experts, s_router, experts, top_k);
+    }
     if (!r.ok && threadIdx.x == 0) atomicOr(flag, kFlagNonFiniteScore);
     if (threadIdx.x < top_k) {
         ids[(uint64_t)t * top_k + threadIdx.x] = r.ok ? (int32_t)r.sel_id[threadIdx.x] : (int32_t)threadIdx.x;
@@ -1070,22 +1096,30 @@ hipError_t run_experts(lev_ctx *ctx, const moe_args &a, const float *x, const gu
     return launch_down<4>(ctx, a, act, ids, weights, y, tokens);
 }
 
-// scratch layout: [scores f32[tokens*experts] | act f32[tokens*top_k*inter]]
+// scratch layout: [scores f32[tokens*experts] | f64 partial scores [kScoreSplit][tokens*experts] from
+// kScoresMfmaMinTokens tokens | act f32[tokens*top_k*inter] | grouped work area]
 struct moe_scratch {
     float *scores;
+    double *partials;   // nullptr below kScoresMfmaMinTokens tokens
     float *act;
     void *grouped;   // work area of the many-token path (grouped_bytes > 0)
 };
 
+size_t score_partial_bytes(uint32_t tokens, uint32_t experts) {
+    return tokens >= kScoresMfmaMinTokens ? (((size_t)kScoreSplit * tokens * experts * 8 + 255) & ~(size_t)255) : 0;
+}
+
 int get_scratch(lev_ctx *ctx, uint32_t tokens, uint32_t experts, uint32_t top_k, uint32_t inter,
                 moe_scratch *s, size_t grouped_bytes = 0) {
     size_t s_bytes = ((size_t)tokens * experts * 4 + 255) & ~(size_t)255;
+    size_t p_bytes = score_partial_bytes(tokens, experts);
     size_t a_bytes = ((size_t)tokens * top_k * inter * 4 + 255) & ~(size_t)255;
-    char *p = static_cast<char *>(lev_scratch(ctx, s_bytes + a_bytes + grouped_bytes));
+    char *p = static_cast<char *>(lev_scratch(ctx, s_bytes + p_bytes + a_bytes + grouped_bytes));
     if (!p) return lev_fail(ctx, LEV_ERR_EXCEEDS_WORKING_SET, "moe: scratch allocation failed");
     s->scores = reinterpret_cast<float *>(p);
-    s->act = reinterpret_cast<float *>(p + s_bytes);
-    s->grouped = p + s_bytes + a_bytes;
+    s->partials = p_bytes ? reinterpret_cast<double *>(p + s_bytes) : nullptr;
+    s->act = reinterpret_cast<float *>(p + s_bytes + p_bytes);
+    s->grouped = p + s_bytes + p_bytes + a_bytes;
     return LEV_OK;
 }
 
@@ -1108,12 +1142,15 @@ bool use_grouped(const lev_ctx *ctx, const moe_args &a, const float *x, uint32_t
            lev_moe_grouped_usable(ctx, grouped_args(a, tokens));
 }
 
-hipError_t run_scores(lev_ctx *ctx, const float *wr, const float *x, float *scores, uint32_t hidden,
-                      uint32_t experts, uint32_t tokens) {
-    if (tokens >= kScoresMfmaMinTokens && hidden % 256u == 0u &&
+// *in_partials: the scores were left as f64 partial sums in `partials` (for run_topk), not in `scores`.
+hipError_t run_scores(lev_ctx *ctx, const float *wr, const float *x, float *scores, double *partials,
+                      bool *in_partials, uint32_t hidden, uint32_t experts, uint32_t tokens) {
+    *in_partials = false;
+    if (partials && tokens >= kScoresMfmaMinTokens && hidden % 256u == 0u &&
         ((reinterpret_cast<uintptr_t>(wr) | reinterpret_cast<uintptr_t>(x)) & 15u) == 0u) {
-        hipLaunchKernelGGL(moe_scores_mfma_kernel, dim3((experts + 15u) / 16u, (tokens + 15u) / 16u), dim3(1024), 0,
-                           ctx->stream, wr, x, scores, hidden, experts, tokens);
+        hipLaunchKernelGGL(moe_scores_mfma_kernel, dim3((experts + 15u) / 16u, (tokens + 15u) / 16u, kScoreSplit),
+                           dim3(256), 0, ctx->stream, wr, x, partials, hidden, experts, tokens);
+        *in_partials = true;
         return hipGetLastError();
     }
     const int split = tokens <= 4u;
@@ -1139,11 +1176,11 @@ hipError_t run_scores_select(lev_ctx *ctx, const float *wr, const float *x, floa
     return hipGetLastError();
 }
 
-hipError_t run_topk(lev_ctx *ctx, const float *scores, const float *scale, int32_t *ids,
+hipError_t run_topk(lev_ctx *ctx, float *scores, const double *partials, const float *scale, int32_t *ids,
                     float *weights, uint32_t experts, uint32_t top_k, uint32_t tokens) {
 #define LEV_TOPK(J)                                                                               \
     hipLaunchKernelGGL((moe_topk_kernel<J>), dim3(tokens), dim3(256), router_lds_bytes(J), ctx->stream, \
-                       scores, scale, ids, weights, ctx->d_flag, experts, top_k)
+                       scores, partials, scale, ids, weights, ctx->d_flag, experts, top_k, tokens)
     if (experts <= 128u) LEV_TOPK(2);
     else if (experts <= 256u) LEV_TOPK(4);
     else if (experts <= 1024u) LEV_TOPK(16);
@@ -1173,17 +1210,21 @@ extern "C" int lev_hip_moe_route_topk(lev_ctx *ctx, const float *d_router_w, con
                         "moe_route_topk: hidden %u, experts %u, topK %u, tokens %u", hidden, experts,
                         top_k, tokens);
     float *scores = d_scores;
-    if (!scores) {
-        moe_scratch s;
+    moe_scratch s{nullptr, nullptr, nullptr, nullptr};
+    if (!scores || tokens >= kScoresMfmaMinTokens) {
         int st = get_scratch(ctx, tokens, experts, top_k, 0, &s);
         if (st != LEV_OK) return st;
-        scores = s.scores;
+        if (!scores) scores = s.scores;
     }
-    int st = lev_hip_check(ctx, run_scores(ctx, d_router_w, d_x, scores, hidden, experts, tokens),
+    bool in_partials = false;
+    int st = lev_hip_check(ctx,
+                           run_scores(ctx, d_router_w, d_x, scores, s.partials, &in_partials, hidden, experts,
+                                      tokens),
                            "moe router scores launch");
     if (st != LEV_OK) return st;
     return lev_hip_check(ctx,
-                         run_topk(ctx, scores, d_expert_scale, d_ids, d_weights, experts, top_k, tokens),
+                         run_topk(ctx, scores, in_partials ? s.partials : nullptr, d_expert_scale, d_ids,
+                                  d_weights, experts, top_k, tokens),
                          "moe router top-k launch");
 }
 
@@ -1245,6 +1286,7 @@ int moe_layer_impl(lev_ctx *ctx, const lev_moe_experts *pools, const float *d_ro
                             "moe_layer_noalloc: needs %zu bytes of scratch, the static buffer holds %zu",
                             s_bytes + a_bytes, fixed_bytes);
         s.scores = static_cast<float *>(fixed);
+        s.partials = nullptr;   // at most LEV_NOALLOC_MOE_MAX_TOKENS tokens: the f32 score kernel
         s.act = reinterpret_cast<float *>(static_cast<char *>(fixed) + s_bytes);
         s.grouped = nullptr;
     } else {
@@ -1268,7 +1310,10 @@ int moe_layer_impl(lev_ctx *ctx, const lev_moe_experts *pools, const float *d_ro
                            "moe router launch");
         if (st != LEV_OK) return st;
     } else {
-        st = lev_hip_check(ctx, run_scores(ctx, d_router_w, d_x, s.scores, a.hidden, a.experts, tokens),
+        bool in_partials = false;
+        st = lev_hip_check(ctx,
+                           run_scores(ctx, d_router_w, d_x, s.scores, s.partials, &in_partials, a.hidden,
+                                      a.experts, tokens),
                            "moe router scores launch");
         if (st != LEV_OK) return st;
         if (few && family == 1u) {
@@ -1276,8 +1321,8 @@ int moe_layer_impl(lev_ctx *ctx, const lev_moe_experts *pools, const float *d_ro
             rt = gu_route{nullptr, s.scores, d_expert_scale, d_ids, d_weights};
         } else {
             st = lev_hip_check(ctx,
-                               run_topk(ctx, s.scores, d_expert_scale, d_ids, d_weights, a.experts, top_k,
-                                        tokens),
+                               run_topk(ctx, s.scores, in_partials ? s.partials : nullptr, d_expert_scale, d_ids,
+                                        d_weights, a.experts, top_k, tokens),
                                "moe router top-k launch");
             if (st != LEV_OK) return st;
         }
