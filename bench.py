@@ -340,7 +340,7 @@ def main():
                     c, ring6.data_ptr(), ring6.numel(), (i % 6) * nb6 * 210, xn.data_ptr(), xn.numel(), None, 0.0,
                     yn.data_ptr(), yn.numel(), cols, r6, n)), nb6 * 210 + n * (cols * 4 + r6 * 4), 100, 20)
             # the head on int8 activations, N columns per weight read (MTP verify)
-            for n in (1, 4, 8):
+            for n in (1, 4, 8, 16):
                 xn = torch.randn(n, cols, device=dev, generator=gen)
                 yn = torch.empty(n, r6, device=dev)
                 xq = torch.empty(n, cols, dtype=torch.int8, device=dev)

@@ -97,6 +97,98 @@ __device__ __forceinline__ void q6m_issue(const uint8_t *__restrict__ w, uint64_
     }
 }
 
+// What a lane needs to turn a task's pieces into its matrix-core operands.
+// lane (r, g): weight row r of the task's 16, chunk g of the superblock (half hf = g/2,
+// j in {jb, jb + 2} with jb = g%2).  `odd`: the wave's superblocks are the odd ones.
+struct q6m_lane {
+    uint8_t *area;                // the wave's turn-round area
+    uint32_t lane, sel, maskq;
+    uint32_t rot[2];              // rotate right: bit pair jb + 2*nb of a qh byte to bits 6..7
+    uint32_t scoff[2];            // bit offset of scale 2*jb + lh in its dword
+    uint32_t at_ql[2], c3_ql[2], at_qh[2], c3_qh[2], at_sc[3], at_d;
+
+    __device__ __forceinline__ q6m_lane(uint8_t *area_all, uint32_t wave, uint32_t lane_, uint32_t odd)
+        : area(area_all + wave * kQAreaBytes), lane(lane_) {
+        const uint32_t r = lane & 15u, g = lane >> 4, hf = g >> 1, jb = g & 1u;
+        maskq = jb ? 0xCCCCCCCCu : 0x33333333u;   // the bit pairs jb and jb+2 of a qh byte
+        rot[0] = 26u + 2u * jb;
+        rot[1] = (30u + 2u * jb) & 31u;
+        scoff[0] = 16u * jb;
+        scoff[1] = 16u * jb + 8u;
+        // where (row r, piece P) of a task sits in the area: instruction r/4 wrote row r%4's
+        // pieces to lanes 16*(r%4) + (P + 4*(r%4)) % 16
+        auto piece_at = [&](uint32_t P) {
+            return (r >> 2) * kQAreaStride + (16u * (r & 3u) + ((P + 4u * (r & 3u)) & 15u)) * 16u;
+        };
+        // logical piece P: an even wave reads piece P; an odd one piece P+1 and, for its first
+        // two bytes, the last dword of piece P.  `sel` picks per byte from {next, previous} dword.
+        sel = odd ? 0x05040302u : 0x07060504u;
+        at_ql[0] = piece_at(2u * g + odd);
+        at_ql[1] = piece_at(2u * g + 1u + odd);
+        at_qh[0] = piece_at(8u + 2u * hf + odd);
+        at_qh[1] = piece_at(9u + 2u * hf + odd);
+        c3_ql[0] = piece_at(2u * g) + 12u;
+        c3_ql[1] = piece_at(2u * g + 1u) + 12u;
+        c3_qh[0] = piece_at(8u + 2u * hf) + 12u;
+        c3_qh[1] = piece_at(9u + 2u * hf) + 12u;
+        // the eight scale bytes 192 + 8*hf ..: three dwords A0..A2, the wanted two being
+        // {A1, A2} (even) or the bytes 2.. of {A0, A1, A2} (odd: stream position 206 + 8*hf)
+        at_sc[0] = odd ? (hf ? piece_at(13u) + 4u : piece_at(12u) + 12u) : piece_at(12u);
+        at_sc[1] = odd ? (hf ? piece_at(13u) + 8u : piece_at(13u)) : piece_at(12u) + 8u * hf;
+        at_sc[2] = odd ? (hf ? piece_at(13u) + 12u : piece_at(13u) + 4u) : piece_at(12u) + 8u * hf + 4u;
+        at_d = piece_at(13u) + 14u;
+    }
+
+    // B operands of the four MFMAs of a task (nb = nibble, lh = which 16 of the chunk's 32
+    // bytes): byte = nibble << 2 | bit pair << 6 with bit 7 flipped = 4*(q - 32) as int8.  The
+    // qh dwords are cleaned once (both pairs this lane uses survive, their top bits flipped);
+    // rotated so that the wanted pair sits in bits 6..7 the other one falls into bits 2..3,
+    // which the merge takes from the nibbles.  sc[nb][lh]: the int8 scale of the 16 weights.
+    __device__ __forceinline__ void operands(const q6m_regs &W, q6m_i4 (&B)[2][2], int (&sc)[2][2],
+                                             uint32_t &dbits) const {
+        // the task's pieces go round through the wave's area: written as loaded, read as
+        // (row r, chunk g) wants them.  One wave's LDS operations run in order.
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            *reinterpret_cast<q6m_i4 *>(area + (uint32_t)i * kQAreaStride + lane * 16u) = W.p[i];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        auto piece = [&](uint32_t at, uint32_t c3) {
+            const q6m_i4 n = *reinterpret_cast<const q6m_i4 *>(area + at);
+            const uint32_t prev = *reinterpret_cast<const uint32_t *>(area + c3);
+            return q6m_i4{(int)__builtin_amdgcn_perm((uint32_t)n.x, prev, sel),
+                          (int)__builtin_amdgcn_perm((uint32_t)n.y, (uint32_t)n.x, sel),
+                          (int)__builtin_amdgcn_perm((uint32_t)n.z, (uint32_t)n.y, sel),
+                          (int)__builtin_amdgcn_perm((uint32_t)n.w, (uint32_t)n.z, sel)};
+        };
+        const q6m_i4 ql[2] = {piece(at_ql[0], c3_ql[0]), piece(at_ql[1], c3_ql[1])};
+        const q6m_i4 qh[2] = {piece(at_qh[0], c3_qh[0]), piece(at_qh[1], c3_qh[1])};
+        const uint32_t sa0 = *reinterpret_cast<const uint32_t *>(area + at_sc[0]);
+        const uint32_t sa1 = *reinterpret_cast<const uint32_t *>(area + at_sc[1]);
+        const uint32_t sa2 = *reinterpret_cast<const uint32_t *>(area + at_sc[2]);
+        const uint32_t scw[2] = {__builtin_amdgcn_perm(sa1, sa0, sel), __builtin_amdgcn_perm(sa2, sa1, sel)};
+        dbits = *reinterpret_cast<const uint16_t *>(area + at_d);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();   // the reads are issued before the next task's writes
+#pragma unroll
+        for (int lh = 0; lh < 2; ++lh) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t qc = ((uint32_t)qh[lh][i] ^ 0xAAAAAAAAu) & maskq;
+#pragma unroll
+                for (int nb = 0; nb < 2; ++nb) {
+                    const uint32_t nib = nb ? (uint32_t)ql[lh][i] >> 2 : (uint32_t)ql[lh][i] << 2;
+                    const uint32_t top = __builtin_amdgcn_alignbit(qc, qc, rot[nb]);
+                    B[nb][lh][i] = (int)((nib & 0x3C3C3C3Cu) | (top & ~0x3C3C3C3Cu));
+                }
+            }
+#pragma unroll
+            for (int nb = 0; nb < 2; ++nb) sc[nb][lh] = __builtin_amdgcn_sbfe((int)scw[nb], scoff[lh], 8u);
+        }
+    }
+};
+
 // LDS, for SB superblocks and NC columns:
 //   dig  [NC][16*SB groups][4 planes][16 bytes]
 //   zero [512 bytes]
@@ -303,28 +395,7 @@ q6_k_mfma_gemv(const uint8_t *__restrict__ w, const float *__restrict__ x, const
     // ---- stream the weights ----
     const uint32_t hf = g >> 1, jb = g & 1u;
     const bool feeds = (r >> 2) == g;                      // this lane's A row belongs to its own lane group
-    const uint32_t maskq = jb ? 0xCCCCCCCCu : 0x33333333u;  // the bit pairs jb and jb+2 of a qh byte
-    const uint32_t rot[2] = {26u + 2u * jb, (30u + 2u * jb) & 31u};   // rotate right: pair jb + 2*nb to bits 6..7
-    const uint32_t scoff[2] = {16u * jb, 16u * jb + 8u};   // bit offset of scale 2*jb + lh in its dword
-    // where (row r, piece P) of a task sits in the wave's area: instruction r/4 wrote row r%4's
-    // pieces to lanes 16*(r%4) + (P + 4*(r%4)) % 16
-    uint8_t *area = area_all + wave * kQAreaBytes;
-    auto piece_at = [&](uint32_t P) {
-        return (r >> 2) * kQAreaStride + (16u * (r & 3u) + ((P + 4u * (r & 3u)) & 15u)) * 16u;
-    };
-    // logical piece P: an even wave reads piece P; an odd one piece P+1 and, for its first
-    // two bytes, the last dword of piece P.  `sel` picks per byte from {next, previous} dword.
-    const uint32_t sel = odd ? 0x05040302u : 0x07060504u;
-    const uint32_t at_ql[2] = {piece_at(2u * g + odd), piece_at(2u * g + 1u + odd)};
-    const uint32_t at_qh[2] = {piece_at(8u + 2u * hf + odd), piece_at(9u + 2u * hf + odd)};
-    const uint32_t c3_ql[2] = {piece_at(2u * g) + 12u, piece_at(2u * g + 1u) + 12u};
-    const uint32_t c3_qh[2] = {piece_at(8u + 2u * hf) + 12u, piece_at(9u + 2u * hf) + 12u};
-    // the eight scale bytes 192 + 8*hf ..: three dwords A0..A2, the wanted two being
-    // {A1, A2} (even) or the bytes 2.. of {A0, A1, A2} (odd: stream position 206 + 8*hf)
-    const uint32_t at_sc[3] = {odd ? (hf ? piece_at(13u) + 4u : piece_at(12u) + 12u) : piece_at(12u),
-                               odd ? (hf ? piece_at(13u) + 8u : piece_at(13u)) : piece_at(12u) + 8u * hf,
-                               odd ? (hf ? piece_at(13u) + 12u : piece_at(13u) + 4u) : piece_at(12u) + 8u * hf + 4u};
-    const uint32_t at_d = piece_at(13u) + 14u;
+    const q6m_lane L6(area_all, wave, lane, odd);
     double yacc[NC];
 #pragma unroll
     for (int q = 0; q < NC; ++q) yacc[q] = 0.0;
@@ -336,53 +407,10 @@ q6_k_mfma_gemv(const uint8_t *__restrict__ w, const float *__restrict__ x, const
         const uint32_t sbw = kpart + S * t;
         const bool live = sbw < SB;
         const uint32_t sb = live ? sbw : SB - 1u;
-        // B operands of the four MFMAs (nb = nibble, lh = which 16 of the chunk's 32 bytes): byte =
-        // nibble << 2 | bit pair << 6 with bit 7 flipped = 4*(q - 32) as int8.  The qh dwords are
-        // cleaned once (both pairs this lane uses survive, their top bits flipped); rotated so that
-        // the wanted pair sits in bits 6..7 the other one falls into bits 2..3, which the merge
-        // takes from the nibbles.
-        // the task's pieces go round through the wave's area: written as loaded, read as
-        // (row r, chunk g) wants them.  One wave's LDS operations run in order.
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-            *reinterpret_cast<q6m_i4 *>(area + (uint32_t)i * kQAreaStride + lane * 16u) = W.p[i];
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        auto piece = [&](uint32_t at, uint32_t c3) {
-            const q6m_i4 n = *reinterpret_cast<const q6m_i4 *>(area + at);
-            const uint32_t prev = *reinterpret_cast<const uint32_t *>(area + c3);
-            return q6m_i4{(int)__builtin_amdgcn_perm((uint32_t)n.x, prev, sel),
-                          (int)__builtin_amdgcn_perm((uint32_t)n.y, (uint32_t)n.x, sel),
-                          (int)__builtin_amdgcn_perm((uint32_t)n.z, (uint32_t)n.y, sel),
-                          (int)__builtin_amdgcn_perm((uint32_t)n.w, (uint32_t)n.z, sel)};
-        };
-        const q6m_i4 ql[2] = {piece(at_ql[0], c3_ql[0]), piece(at_ql[1], c3_ql[1])};
-        const q6m_i4 qh[2] = {piece(at_qh[0], c3_qh[0]), piece(at_qh[1], c3_qh[1])};
-        const uint32_t sa0 = *reinterpret_cast<const uint32_t *>(area + at_sc[0]);
-        const uint32_t sa1 = *reinterpret_cast<const uint32_t *>(area + at_sc[1]);
-        const uint32_t sa2 = *reinterpret_cast<const uint32_t *>(area + at_sc[2]);
-        const uint32_t scw[2] = {__builtin_amdgcn_perm(sa1, sa0, sel), __builtin_amdgcn_perm(sa2, sa1, sel)};
-        const uint32_t dbits = *reinterpret_cast<const uint16_t *>(area + at_d);
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();   // the reads are issued before the next task's writes
         q6m_i4 B[2][2];
         int sc[2][2];
-#pragma unroll
-        for (int lh = 0; lh < 2; ++lh) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const uint32_t qc = ((uint32_t)qh[lh][i] ^ 0xAAAAAAAAu) & maskq;
-#pragma unroll
-                for (int nb = 0; nb < 2; ++nb) {
-                    const uint32_t nib = nb ? (uint32_t)ql[lh][i] >> 2 : (uint32_t)ql[lh][i] << 2;
-                    const uint32_t top = __builtin_amdgcn_alignbit(qc, qc, rot[nb]);
-                    B[nb][lh][i] = (int)((nib & 0x3C3C3C3Cu) | (top & ~0x3C3C3C3Cu));
-                }
-            }
-#pragma unroll
-            for (int nb = 0; nb < 2; ++nb) sc[nb][lh] = __builtin_amdgcn_sbfe((int)scw[nb], scoff[lh], 8u);
-        }
+        uint32_t dbits;
+        L6.operands(W, B, sc, dbits);
         // a task past the wave's last superblock contributes nothing
         const double d = live ? (double)lev_f16_bits_to_f32(dbits) : 0.0;
         // lane (r, g) feeds A row r = 4*gs + p: plane p of group 16*sb + 8*hf + 2*jb (+ 4*nb + lh)
@@ -540,6 +568,192 @@ q6_k_mfma_gemv(const uint8_t *__restrict__ w, const float *__restrict__ x, const
     }
 }
 
+// ---------------------------------------------------------------------------
+// The same weight stream on int8 activations (q6k.q8.matvec, emit_q6k_q8,
+// lev-forge/src/q8.rs:330-447; oracle matvec_q6k_q8_f64, lev-cpu/src/lib.rs:333-337):
+// xq int8 [ncol][cols], xs (d, s) pairs per 32 activations.  A row 4*gs + c of an MFMA
+// holds the codes of column c (of a chunk of four) for the k-slots lane group gs
+// supplies, so one MFMA gives a lane the exact sums 4*(q-32)*xq over one 16-weight group
+// for four columns; the two halves of a 32-activation block take their int8 scales in
+// integers, then the block's activation scale in f32:
+//   y[c] += d * sum_blocks dx[c][block] * (sc_a * D_a[c] + sc_b * D_b[c]) / 4.
+// (The -32 of the codes is inside the operand, so the s of the pairs is not used.)
+// LDS: codes [NC][cols] as they come, dx [cols/32][NC] f32 (x 1/4), partial sums
+// [pb][16 waves][16 rows][NC] f32, the turn-round areas.
+// ---------------------------------------------------------------------------
+template <int NC>
+struct q6m_q8_lds {
+    static __host__ __device__ size_t total(uint32_t cols, uint32_t pb) {
+        return (size_t)NC * cols + kQZeroBytes + (size_t)(cols >> 5) * NC * 4u +
+               (size_t)pb * kQWaves * 16u * NC * 4u + (size_t)kQWaves * kQAreaBytes;
+    }
+};
+
+// NC: columns staged (4, 8 or 16; >= ncol).
+template <int NC>
+__global__ void __launch_bounds__(kQThreads)
+q6_k_mfma_gemv_q8(const uint8_t *__restrict__ w, const uint32_t *__restrict__ xq, const float *__restrict__ xs,
+                  float *__restrict__ y, uint32_t cols, uint32_t rows, uint32_t ncol, uint32_t S, uint32_t pb) {
+    constexpr int NCH = NC / 4;
+    constexpr uint32_t kLogNC = NC == 16 ? 4u : NC == 8 ? 3u : 2u;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const uint32_t SB = cols >> 8, nblk = cols >> 5;
+    uint8_t *dig = smem;
+    uint8_t *zero = smem + (size_t)NC * cols;
+    float *dxs = reinterpret_cast<float *>(zero + kQZeroBytes);
+    float *part = dxs + (size_t)nblk * NC;
+    uint8_t *area_all = reinterpret_cast<uint8_t *>(part + (size_t)pb * kQWaves * 16u * NC);
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t r = lane & 15u, g = lane >> 4;
+    const uint64_t row_bytes = (uint64_t)SB * 210u;
+    const uint32_t ngroups = (rows + 15u) >> 4;
+    const uint32_t slots = kQWaves / S;
+    const uint32_t slot = wave / S, kpart = wave % S;
+    const uint32_t tpr = (SB + S - 1u) / S;
+    const uint32_t wgrounds = (ngroups + slots - 1u) / slots;
+    const uint32_t nrounds = (wgrounds - blockIdx.x + gridDim.x - 1u) / gridDim.x;
+    const uint32_t ntasks = nrounds * tpr;
+    struct cursor {
+        uint32_t k, rd, t;
+    };
+    auto advance = [&](cursor &c) {
+        ++c.k;
+        if (++c.t == tpr) {
+            c.t = 0;
+            ++c.rd;
+        }
+    };
+    const uint32_t odd = kpart & 1u;
+    const int32_t poff = q6m_piece_offset(lane, odd), poff_even = q6m_piece_offset(lane, 0u);
+    auto group_of = [&](uint32_t rd, uint32_t sl) { return (rd * gridDim.x + blockIdx.x) * slots + sl; };
+    auto issue = [&](cursor &c, q6m_regs &W) {
+        const uint32_t sbw = kpart + S * c.t;
+        const bool real = c.k < ntasks && sbw < SB;
+        q6m_issue(w, row_bytes, real ? group_of(c.rd, slot) * 16u : 0u, rows, real ? sbw : 0u, lane,
+                  real ? poff : poff_even, W);
+        advance(c);
+    };
+    cursor ci{0u, 0u, 0u}, cc{0u, 0u, 0u};
+    q6m_regs W0, W1, W2;
+
+    // ---- stage the activations: the codes as they come, the block scales transposed ----
+    if (tid < kQZeroBytes / 4u) reinterpret_cast<uint32_t *>(zero)[tid] = 0u;
+    {
+        const lev_u32x4 *src = reinterpret_cast<const lev_u32x4 *>(xq);
+        lev_u32x4 *dst = reinterpret_cast<lev_u32x4 *>(dig);
+        const uint32_t n16 = ncol * (cols >> 4);
+        for (uint32_t i = tid; i < n16; i += kQThreads) dst[i] = src[i];
+        // columns of the layout beyond ncol: zero codes and scales (their outputs are never stored)
+        for (uint32_t i = n16 + tid; i < (uint32_t)NC * (cols >> 4); i += kQThreads) dst[i] = lev_u32x4{0u, 0u, 0u, 0u};
+        for (uint32_t i = tid; i < nblk * NC; i += kQThreads) {
+            const uint32_t c = i & (NC - 1u), b = i >> kLogNC;
+            // a quarter of the activation scale: the codes in the operand are 4*(q - 32)
+            dxs[i] = c < ncol ? 0.25f * xs[((uint64_t)c * nblk + b) * 2u] : 0.f;
+        }
+    }
+    lev_barrier_lds();
+    issue(ci, W0);
+
+    // ---- stream the weights ----
+    const uint32_t hf = g >> 1, jb = g & 1u;
+    const bool feeds = (r >> 2) == g;
+    const q6m_lane L6(area_all, wave, lane, odd);
+    float yacc[NCH][4];
+#pragma unroll
+    for (int ch = 0; ch < NCH; ++ch)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) yacc[ch][i] = 0.f;
+
+    uint32_t parity = 0;
+    auto compute = [&](cursor &c, const q6m_regs &W) {
+        const uint32_t rd = c.rd, t = c.t;
+        const uint32_t sbw = kpart + S * t;
+        const bool live = sbw < SB;
+        const uint32_t sb = live ? sbw : SB - 1u;
+        q6m_i4 B[2][2];
+        int sc[2][2];
+        uint32_t dbits;
+        L6.operands(W, B, sc, dbits);
+        const float d = live ? lev_f16_bits_to_f32(dbits) : 0.f;
+        // lane (r, g) feeds A row r = 4*gs + c: column 4*ch + r%4, the 16 codes of weight group
+        // 16*sb + 8*hf + 2*jb (+ 4*nb + lh) when gs == g, zeros otherwise
+        const uint32_t aoff = (r & 3u) * cols + (16u * sb + 8u * hf + 2u * jb) * 16u;
+        const uint32_t blk0 = 8u * sb + 4u * hf + jb;   // 32-activation block of nb = 0; nb = 1: + 2
+#pragma unroll
+        for (int ch = 0; ch < NCH; ++ch) {
+            const uint8_t *ab = feeds ? dig + (size_t)(4 * ch) * cols + aoff : zero;
+            float ysb[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int nb = 0; nb < 2; ++nb) {
+                const q6m_i4 A0 = *reinterpret_cast<const q6m_i4 *>(ab + (4 * nb) * 16);
+                const q6m_i4 A1 = *reinterpret_cast<const q6m_i4 *>(ab + (4 * nb + 1) * 16);
+                const lev_f32x4 dx = *reinterpret_cast<const lev_f32x4 *>(dxs + (size_t)(blk0 + 2u * nb) * NC + 4 * ch);
+                const q6m_i4 D0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A0, B[nb][0], q6m_i4{0, 0, 0, 0}, 0, 0, 0);
+                const q6m_i4 D1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A1, B[nb][1], q6m_i4{0, 0, 0, 0}, 0, 0, 0);
+                // |D| <= 16*128*127 < 2^18, |sc| <= 2^7: the sum of the two halves fits 32 bits
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    int E = __mul24(D0[i], sc[nb][0]);
+                    E += __mul24(D1[i], sc[nb][1]);
+                    ysb[i] = fmaf((float)E, dx[i], ysb[i]);
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) yacc[ch][i] = fmaf(d, ysb[i], yacc[ch][i]);
+        }
+
+        if (t + 1u == tpr) {   // workgroup-uniform: the round ends
+            float *pp = part + parity * (kQWaves * 16u * NC);
+            parity ^= pb - 1u;
+            // the four lane groups' shares of a row meet; lane group g keeps column 4*ch + g
+#pragma unroll
+            for (int ch = 0; ch < NCH; ++ch) {
+                float mine = 0.f;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    float v = yacc[ch][i];
+                    v += __shfl_xor(v, 16);
+                    v += __shfl_xor(v, 32);
+                    mine = g == (uint32_t)i ? v : mine;
+                    yacc[ch][i] = 0.f;
+                }
+                pp[(wave * 16u + r) * NC + 4u * (uint32_t)ch + g] = mine;
+            }
+            lev_barrier_lds();
+            for (uint32_t i = tid; i < slots * 16u * NC; i += kQThreads) {
+                const uint32_t rr = i & 15u, col = (i >> 4) & (NC - 1u), sl = i >> (4u + kLogNC);
+                const uint32_t row = group_of(rd, sl) * 16u + rr;
+                float sum = 0.f;
+                for (uint32_t k = 0; k < S; ++k) sum += pp[((sl * S + k) * 16u + rr) * NC + col];
+                if (col < ncol && row < rows) y[(uint64_t)col * rows + row] = sum;
+            }
+            if (pb == 1u) lev_barrier_lds();   // the one buffer is written again by the next round
+        }
+        advance(c);
+    };
+
+    issue(ci, W1);
+    issue(ci, W2);
+    while (true) {
+        compute(cc, W0);
+        __builtin_amdgcn_sched_barrier(0);
+        issue(ci, W0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (cc.k >= ntasks) break;
+        compute(cc, W1);
+        __builtin_amdgcn_sched_barrier(0);
+        issue(ci, W1);
+        __builtin_amdgcn_sched_barrier(0);
+        if (cc.k >= ntasks) break;
+        compute(cc, W2);
+        __builtin_amdgcn_sched_barrier(0);
+        issue(ci, W2);
+        __builtin_amdgcn_sched_barrier(0);
+        if (cc.k >= ntasks) break;
+    }
+}
+
 size_t q6m_lds_limit(const lev_ctx *ctx) {
     return ctx->props.sharedMemPerBlockOptin > ctx->props.sharedMemPerBlock ? ctx->props.sharedMemPerBlockOptin
                                                                             : ctx->props.sharedMemPerBlock;
@@ -623,4 +837,50 @@ hipError_t lev_q6_k_mfma_gemv_launch(lev_ctx *ctx, const uint8_t *w, const float
     if (ncol > 2) return q6m_launch<4>(ctx, w, x, gain, eps, y, in_dim, rows, ncol, waves, partials, d_argmax, d_margin);
     if (ncol > 1) return q6m_launch<2>(ctx, w, x, gain, eps, y, in_dim, rows, ncol, waves, partials, d_argmax, d_margin);
     return q6m_launch<1>(ctx, w, x, gain, eps, y, in_dim, rows, ncol, waves, partials, d_argmax, d_margin);
+}
+
+namespace {
+size_t q6m_q8_lds_bytes(uint32_t cols, uint32_t nc, uint32_t pb) {
+    return nc > 8u ? q6m_q8_lds<16>::total(cols, pb) : nc > 4u ? q6m_q8_lds<8>::total(cols, pb)
+                                                                 : q6m_q8_lds<4>::total(cols, pb);
+}
+
+template <int NC>
+hipError_t q6m_q8_launch(lev_ctx *ctx, const uint8_t *w, const uint32_t *xq, const float *xs, float *y,
+                         uint32_t cols, uint32_t rows, uint32_t ncol, uint32_t waves) {
+    const uint32_t pb = q6m_q8_lds_bytes(cols, NC, 2u) <= q6m_lds_limit(ctx) ? 2u : 1u;
+    const size_t lds = q6m_q8_lds_bytes(cols, NC, pb);
+    static size_t configured = 0;   // per instantiation: raise the dynamic LDS limit once per size
+    if (lds > 48 * 1024 && lds > configured) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&q6_k_mfma_gemv_q8<NC>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        configured = lds;
+    }
+    const uint32_t S = waves ? waves : q6m_waves_per_group(ctx, cols, rows);
+    const uint32_t slots = kQWaves / S, ngroups = (rows + 15u) / 16u;
+    const uint32_t wgrounds = (ngroups + slots - 1u) / slots;
+    const uint32_t blocks = wgrounds < (uint32_t)ctx->num_cus ? wgrounds : (uint32_t)ctx->num_cus;
+    hipLaunchKernelGGL((q6_k_mfma_gemv_q8<NC>), dim3(blocks), dim3(kQThreads), lds, ctx->stream, w, xq, xs, y,
+                       cols, rows, ncol, S, pb);
+    return hipGetLastError();
+}
+}  // namespace
+
+// Columns one launch of the int8-activation matrix-core kernel can take for this in_dim (0: not usable).
+uint32_t lev_q6_k_mfma_q8_cols(const lev_ctx *ctx, uint32_t in_dim) {
+    if (in_dim % 256u != 0u || in_dim == 0u) return 0;
+    const size_t limit = q6m_lds_limit(ctx);
+    for (uint32_t nc = 16; nc >= 4u; nc >>= 1)
+        if (q6m_q8_lds_bytes(in_dim, nc, 1u) <= limit) return nc;
+    return 0;
+}
+
+// ncol <= lev_q6_k_mfma_q8_cols(ctx, in_dim); w 2-byte, xq 16-byte, xs 8-byte aligned.
+hipError_t lev_q6_k_mfma_gemv_q8_launch(lev_ctx *ctx, const uint8_t *w, const uint32_t *xq, const float *xs,
+                                        float *y, uint32_t in_dim, uint32_t rows, uint32_t ncol, uint32_t waves) {
+    if (waves != 2u && waves != 4u && waves != 8u && waves != 16u) waves = 0u;
+    if (ncol > 8) return q6m_q8_launch<16>(ctx, w, xq, xs, y, in_dim, rows, ncol, waves);
+    if (ncol > 4) return q6m_q8_launch<8>(ctx, w, xq, xs, y, in_dim, rows, ncol, waves);
+    return q6m_q8_launch<4>(ctx, w, xq, xs, y, in_dim, rows, ncol, waves);
 }

@@ -868,23 +868,30 @@ static uint32_t q6_q8_cols_per_pass(const lev_ctx *ctx, uint32_t in_dim, uint32_
     return nc;
 }
 
+uint32_t lev_q6_k_mfma_q8_cols(const lev_ctx *ctx, uint32_t in_dim);
+hipError_t lev_q6_k_mfma_gemv_q8_launch(lev_ctx *ctx, const uint8_t *w, const uint32_t *xq, const float *xs,
+                                        float *y, uint32_t in_dim, uint32_t rows, uint32_t ncol, uint32_t waves);
+
 // Candidate schedules of a Q6_K x int8 GEMV shape, the built-in choice first
-// (q6k.matvec over int8 activations, lev-forge/src/q8.rs:328-447): a resident grid
-// or a workgroup per row tile, all columns in one pass over the weights or half
-// of them in each of two.
+// (q6k.matvec over int8 activations, lev-forge/src/q8.rs:328-447): the integer
+// matrix-core kernel (family 1; rows_in_flight = columns per pass over the weights),
+// then the dot4 kernel (family 0) with a resident grid or a workgroup per row tile,
+// all columns in one pass over the weights or half of them in each of two.
 uint32_t lev_q6_k_gemv_q8_candidates(const lev_ctx *ctx, uint32_t in_dim, uint32_t rows, uint32_t ncol,
                                      lev_schedule *out, uint32_t capacity) {
     (void)rows;
     const uint32_t all = q6_q8_cols_per_pass(ctx, in_dim, ncol);
+    const uint32_t mcols = lev_q6_k_mfma_q8_cols(ctx, in_dim);
     uint32_t n = 0;
-    auto add = [&](uint32_t cols, uint32_t persistent) {
-        if (n < capacity) out[n] = lev_schedule{LEV_OP_Q6_K_GEMV_Q8, 0u, cols, persistent};
+    auto add = [&](uint32_t family, uint32_t cols, uint32_t persistent) {
+        if (n < capacity) out[n] = lev_schedule{LEV_OP_Q6_K_GEMV_Q8, family, cols, persistent};
         ++n;
     };
-    if (all == 0) return 0;
-    add(all, 1u);
-    add(all, 0u);
-    if (all >= 2u) add(all / 2u, 1u);
+    if (mcols) add(1u, ncol < mcols ? ncol : mcols, 1u);
+    if (all == 0) return n;
+    add(0u, all, 1u);
+    add(0u, all, 0u);
+    if (all >= 2u) add(0u, all / 2u, 1u);
     return n;
 }
 
@@ -906,6 +913,21 @@ extern "C" int lev_hip_q6_k_gemv_q8(lev_ctx *ctx, const void *d_w, size_t w_byte
         (reinterpret_cast<uintptr_t>(d_xs) & 7u))
         return lev_fail(ctx, LEV_ERR_BAD_DIMENSIONS,
                         "q6_k_gemv_q8: weights must be 2-byte, xq 16-byte, xs 8-byte aligned");
+    const uint32_t *xq = reinterpret_cast<const uint32_t *>(d_xq);
+    // a schedule installed for this shape (lev_hip_forge_select) overrides the built-in choice
+    const lev_schedule *sel = lev_selected(ctx, LEV_OP_Q6_K_GEMV_Q8, in_dim, rows, ncol);
+    const uint32_t mcols = lev_q6_k_mfma_q8_cols(ctx, in_dim);
+    if (mcols && (!sel || sel->family == 1u)) {
+        // the integer matrix-core kernel: up to mcols columns per pass over the weights
+        for (uint32_t done = 0; done < ncol; done += mcols) {
+            const uint32_t nc = ncol - done < mcols ? ncol - done : mcols;
+            hipError_t e = lev_q6_k_mfma_gemv_q8_launch(ctx, w, xq + ((uint64_t)done * in_dim >> 2),
+                                                        d_xs + (uint64_t)done * (in_dim >> 5) * 2u,
+                                                        d_y + (uint64_t)done * rows, in_dim, rows, nc, 0u);
+            if (e != hipSuccess) return lev_hip_check(ctx, e, "q6_k_gemv_q8 launch");
+        }
+        return LEV_OK;
+    }
     const size_t limit = ctx->props.sharedMemPerBlockOptin > ctx->props.sharedMemPerBlock
                              ? ctx->props.sharedMemPerBlockOptin
                              : ctx->props.sharedMemPerBlock;
@@ -914,12 +936,10 @@ extern "C" int lev_hip_q6_k_gemv_q8(lev_ctx *ctx, const void *d_w, size_t w_byte
         return lev_fail(ctx, LEV_ERR_EXCEEDS_MODEL_WORKLOAD, "q6_k_gemv_q8: inDim %u does not fit the staging", in_dim);
     uint32_t fit = q6_q8_cols_per_pass(ctx, in_dim, ncol);
     bool persistent = true;
-    // a schedule installed for this shape (lev_hip_forge_select) overrides the built-in choice
-    if (const lev_schedule *sel = lev_selected(ctx, LEV_OP_Q6_K_GEMV_Q8, in_dim, rows, ncol)) {
+    if (sel) {
         if (sel->rows_in_flight >= 1u && sel->rows_in_flight < fit) fit = sel->rows_in_flight;
         persistent = sel->persistent != 0u;
     }
-    const uint32_t *xq = reinterpret_cast<const uint32_t *>(d_xq);
     uint32_t done = 0;
     while (done < ncol) {
         uint32_t nc = ncol - done;

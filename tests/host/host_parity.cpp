@@ -741,7 +741,7 @@ void forge_matvec(Runner &r) {
         for (const ForgeCandidate &c : rep.candidates) EXPECT(c.pass && c.maxRelErr < 1e-4);
         EXPECT(rep.selected >= 0);
     }
-    // the Q6_K head over int8 activations: grids and column passes, all the same bits
+    // the Q6_K head over int8 activations: the matrix-core kernel, then the dot4 kernel's grids and column passes
     for (int ncol : {1, 4}) {
         const int rows = 160, cols = 1024;
         std::vector<uint8_t> w((size_t)rows * cols / 256 * 210);
@@ -751,7 +751,8 @@ void forge_matvec(Runner &r) {
         opt.int8Activations = true;
         opt.rotateBytes = 8 << 20;
         ForgeReport rep = MatvecForge::forge(r, GGMLTensorType::q6_K, w, rows, cols, ncol, opt);
-        EXPECT(rep.op == LEV_OP_Q6_K_GEMV_Q8 && rep.candidates.size() == (ncol == 1 ? 2u : 3u));
+        EXPECT(rep.op == LEV_OP_Q6_K_GEMV_Q8 && rep.candidates.size() == (ncol == 1 ? 3u : 4u));
+        EXPECT(rep.candidates[0].schedule.family == 1u);
         for (const ForgeCandidate &c : rep.candidates) EXPECT(c.pass && c.maxRelErr < 1e-4 && c.medianUs > 0);
         EXPECT(rep.selected >= 0);
     }
