@@ -590,7 +590,9 @@ struct q6m_q8_lds {
 };
 
 // NC: columns staged (4, 8 or 16; >= ncol).
-template <int NC>
+// NC: columns staged (4, 8 or 16; >= ncol).  DEPTH: tasks in flight per wave (3; 2 at sixteen
+// columns, whose accumulators leave no registers for a third).
+template <int NC, int DEPTH>
 __global__ void __launch_bounds__(kQThreads)
 q6_k_mfma_gemv_q8(const uint8_t *__restrict__ w, const uint32_t *__restrict__ xq, const float *__restrict__ xs,
                   float *__restrict__ y, uint32_t cols, uint32_t rows, uint32_t ncol, uint32_t S, uint32_t pb) {
@@ -734,7 +736,7 @@ q6_k_mfma_gemv_q8(const uint8_t *__restrict__ w, const uint32_t *__restrict__ xq
     };
 
     issue(ci, W1);
-    issue(ci, W2);
+    if (DEPTH > 2) issue(ci, W2);
     while (true) {
         compute(cc, W0);
         __builtin_amdgcn_sched_barrier(0);
@@ -746,11 +748,13 @@ q6_k_mfma_gemv_q8(const uint8_t *__restrict__ w, const uint32_t *__restrict__ xq
         issue(ci, W1);
         __builtin_amdgcn_sched_barrier(0);
         if (cc.k >= ntasks) break;
-        compute(cc, W2);
-        __builtin_amdgcn_sched_barrier(0);
-        issue(ci, W2);
-        __builtin_amdgcn_sched_barrier(0);
-        if (cc.k >= ntasks) break;
+        if (DEPTH > 2) {
+            compute(cc, W2);
+            __builtin_amdgcn_sched_barrier(0);
+            issue(ci, W2);
+            __builtin_amdgcn_sched_barrier(0);
+            if (cc.k >= ntasks) break;
+        }
     }
 }
 
@@ -852,7 +856,7 @@ hipError_t q6m_q8_launch(lev_ctx *ctx, const uint8_t *w, const uint32_t *xq, con
     const size_t lds = q6m_q8_lds_bytes(cols, NC, pb);
     static size_t configured = 0;   // per instantiation: raise the dynamic LDS limit once per size
     if (lds > 48 * 1024 && lds > configured) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&q6_k_mfma_gemv_q8<NC>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&q6_k_mfma_gemv_q8<NC, (NC > 8 ? 2 : 3)>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
         configured = lds;
@@ -861,7 +865,7 @@ hipError_t q6m_q8_launch(lev_ctx *ctx, const uint8_t *w, const uint32_t *xq, con
     const uint32_t slots = kQWaves / S, ngroups = (rows + 15u) / 16u;
     const uint32_t wgrounds = (ngroups + slots - 1u) / slots;
     const uint32_t blocks = wgrounds < (uint32_t)ctx->num_cus ? wgrounds : (uint32_t)ctx->num_cus;
-    hipLaunchKernelGGL((q6_k_mfma_gemv_q8<NC>), dim3(blocks), dim3(kQThreads), lds, ctx->stream, w, xq, xs, y,
+    hipLaunchKernelGGL((q6_k_mfma_gemv_q8<NC, (NC > 8 ? 2 : 3)>), dim3(blocks), dim3(kQThreads), lds, ctx->stream, w, xq, xs, y,
                        cols, rows, ncol, S, pb);
     return hipGetLastError();
 }
