@@ -351,7 +351,7 @@ typedef struct lev_schedule {
     uint32_t family;         /* Q4_K: 1 = matrix-core kernel, 0 = vector-ALU (int8: dot4) kernel; Q4_0: 0;
                                 Q6_K: 2 = integer matrix-core kernel, 0 = digit-plane dot4 kernel (both exact),
                                 1 = one wave per row with f64 sums;
-                                Q6_K x int8: 0; MoE layer: who selects the experts: 1 = the gate/up workgroups
+                                Q6_K x int8: 1 = integer matrix-core kernel, 0 = dot4 kernel; MoE layer: who selects the experts: 1 = the gate/up workgroups
                                 themselves, 2 = the last workgroup of the router kernel to finish, 0 = a top-k
                                 kernel of its own ahead of them */
     uint32_t rows_in_flight; /* Q4_0: rows a wave keeps in flight (1, 2, 4; 0 = no variants for the shape);
