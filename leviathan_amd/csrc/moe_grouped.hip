@@ -39,9 +39,14 @@ namespace {
 
 constexpr int kGrpThreads = 1024;
 constexpr int kGrpWaves = kGrpThreads / LEV_WAVE;
-constexpr int kNC = 8;                 // token columns per pass
+constexpr int kNC = 12;                // token columns per pass (of the 16 an MFMA takes; the planes of 16 would not
+                                       // fit the LDS at hidden 2048).  An expert with more pairs takes another pass over
+                                       // its weights, and its workgroups that much longer than all the others: at 64
+                                       // tokens x top-8 over 128 experts one in fifty has more than 8 pairs (a layer then
+                                       // measured 172 us instead of 122), one in three thousand more than 12
 constexpr int kFlagBadExpertId = 1;    // same bit as the per-token kernels
 constexpr uint32_t kGrpScaleDw = 10;   // dwords per row of block scales in a wave's exchange area
+constexpr size_t kGrpStaticLds = (size_t)2 * (kGrpWaves / 2) * 16 * kNC * 4 + 1024;   // gate values, pair records
 
 typedef _Float16 g_h8 __attribute__((ext_vector_type(8)));
 typedef uint32_t g_u4 __attribute__((ext_vector_type(4)));
@@ -462,8 +467,8 @@ bool lev_moe_grouped_usable(const lev_ctx *ctx, const lev_moe_grouped_args &a) {
                              ? ctx->props.sharedMemPerBlockOptin
                              : ctx->props.sharedMemPerBlock;
     return a.hidden % 256u == 0u && a.inter % 256u == 0u && a.experts <= 4096u &&
-           (uint64_t)a.tokens * a.top_k <= (1u << 20) && grouped_lds(a.hidden, true) <= limit &&
-           grouped_lds(a.inter, false) <= limit;
+           (uint64_t)a.tokens * a.top_k <= (1u << 20) && grouped_lds(a.hidden, true) + kGrpStaticLds <= limit &&
+           grouped_lds(a.inter, false) + kGrpStaticLds <= limit;
 }
 
 // act: f32 [tokens*top_k][inter] (written here, read by the down stage).
