@@ -339,10 +339,17 @@ hipError_t lev_q4_k_mfma_gemv_launch(lev_ctx *ctx, const uint8_t *w, const float
 // matrix-core kernel forms every dot product without rounding and is the choice
 // wherever its activation staging fits; the vector-ALU kernel (f32 FMA chains)
 // takes the other shapes and stays a candidate for lev_hip_forge_select.
+uint32_t lev_q4_k_mfma_narrow_cols(const lev_ctx *ctx, uint32_t in_dim);
+
+// Whether the matrix-core family takes this shape: its four-columns-per-product kernel up to
+// in_dim 8192, its one- and two-column kernel up to in_dim 32768 / ncol.
+static bool q4k_mfma_serves(const lev_ctx *ctx, uint32_t in_dim, uint32_t ncol) {
+    return lev_q4_k_mfma_cols(ctx, in_dim) != 0u || ncol <= lev_q4_k_mfma_narrow_cols(ctx, in_dim);
+}
+
 static uint32_t q4k_builtin_family(const lev_ctx *ctx, uint32_t in_dim, uint32_t rows, uint32_t ncol) {
     (void)rows;
-    (void)ncol;
-    return lev_q4_k_mfma_cols(ctx, in_dim) == 0u ? 0u : 1u;
+    return q4k_mfma_serves(ctx, in_dim, ncol) ? 1u : 0u;
 }
 
 hipError_t lev_q4_k_gemv_launch(lev_ctx *ctx, const uint8_t *w, const float *x, const float *gain,
@@ -353,6 +360,9 @@ hipError_t lev_q4_k_gemv_launch(lev_ctx *ctx, const uint8_t *w, const float *x, 
     // a schedule installed for this shape (lev_hip_forge_select) overrides the built-in choice
     const lev_schedule *sel = lev_selected(ctx, LEV_OP_Q4_K_GEMV, in_dim, rows, ncol);
     const bool mfma = (sel ? sel->family : q4k_builtin_family(ctx, in_dim, rows, ncol)) == 1u;
+    // one column, or two of a row too wide for the four-column kernel: the narrow kernel
+    if (mfma && ncol <= lev_q4_k_mfma_narrow_cols(ctx, in_dim) && (ncol == 1u || lev_q4_k_mfma_cols(ctx, in_dim) < ncol))
+        return lev_q4_k_mfma_gemv_launch(ctx, w, x, gain, eps, y, in_dim, rows, ncol);
     const uint32_t mfma_cols = mfma ? lev_q4_k_mfma_cols(ctx, in_dim) : 0u;
     while (mfma_cols && done < ncol) {
         uint32_t nc = ncol - done < mfma_cols ? ncol - done : mfma_cols;
@@ -390,7 +400,7 @@ uint32_t lev_q4_k_gemv_candidates(const lev_ctx *ctx, uint32_t in_dim, uint32_t 
     uint32_t n = 0;
     if (n < capacity) out[n] = lev_schedule{LEV_OP_Q4_K_GEMV, first, 0u, 0u};
     ++n;
-    if (lev_q4_k_mfma_cols(ctx, in_dim) != 0u) {
+    if (q4k_mfma_serves(ctx, in_dim, ncol)) {
         if (n < capacity) out[n] = lev_schedule{LEV_OP_Q4_K_GEMV, 1u - first, 0u, 0u};
         ++n;
     }

@@ -40,10 +40,13 @@
 // A NaN or infinity in a column of x makes every output of that column NaN.
 #include "lev_common.hpp"
 
+#include <cstdlib>
+
 namespace {
 
 constexpr int kMThreads = 1024;
 constexpr int kMWaves = kMThreads / LEV_WAVE;
+constexpr uint32_t kNZeroBytes = 1024;   // what masked lanes of the narrow kernel read as their A operand
 
 typedef int lev_i4 __attribute__((ext_vector_type(4)));
 typedef uint32_t lev_u4 __attribute__((ext_vector_type(4)));
@@ -452,6 +455,372 @@ q4_k_mfma_gemv(const uint8_t *__restrict__ w, const float *__restrict__ x,
     }
 }
 
+// One or two columns: the same sums with half the matrix-core products and half the
+// multiply-adds.  v_mfma_i32_16x16x64_i8 takes 64 codes of 16 rows; lane group g
+// (l / 16) supplies the 16 codes of ONE half sub-block -- exactly the 16 bytes it
+// loaded (low or high nibbles), so nothing is exchanged between lanes -- and A row
+// 4*gs + p holds digit plane p of the elements lane group gs supplies and zeros
+// elsewhere: output row 4*gs + p is the plane sum over that half sub-block alone, in
+// a lane of the group that holds the sub-block's scale.  (With four columns per MFMA,
+// as above, three quarters of the lanes of a one-column launch multiply-add columns
+// that do not exist.)  The digit planes take 4 bytes per element and column, so rows
+// up to 32768 / NC wide are served.
+//   dig  [NC][16*SB groups of 16][4 planes][16 bytes]
+//   sx16 [NC][16*SB] i32                                sum of X per group of 16
+//   part [pb][wave][16 rows][NC] f64, psb [NC][SB] f64, inv [NC] f64, bad [NC] u32
+//   run  [NC][8*SB] f64 (RMSNorm), in the digit area
+template <int NC>
+struct q4k_narrow_lds {
+    static __host__ __device__ size_t dig_bytes(uint32_t cols) { return (size_t)NC * cols * 4u; }
+    static __host__ __device__ size_t total(uint32_t cols, uint32_t pb) {
+        return dig_bytes(cols) + kNZeroBytes + (size_t)NC * (cols >> 4) * 4u +
+               (size_t)pb * kMWaves * 16u * NC * 8u + (size_t)NC * (cols >> 8) * 8u + (size_t)NC * 12u + 8u;
+    }
+};
+
+template <int NC, bool SHORT>
+__global__ void __launch_bounds__(kMThreads)
+q4_k_mfma_gemv_narrow(const uint8_t *__restrict__ w, const float *__restrict__ x,
+               const float *__restrict__ gain, float eps, float *__restrict__ y, uint32_t cols,
+               uint32_t rows, uint32_t ncol, uint32_t pb, double rcols) {
+    using L = q4k_narrow_lds<NC>;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const uint32_t SB = cols >> 8, subs = cols >> 5;
+    uint8_t *dig = smem;
+    uint8_t *zero = smem + L::dig_bytes(cols);
+    double *part = reinterpret_cast<double *>(zero + kNZeroBytes);
+    double *psb = part + (size_t)pb * kMWaves * 16u * NC;
+    double *s_inv = psb + (size_t)SB * NC;
+    int32_t *sx16 = reinterpret_cast<int32_t *>(s_inv + NC);
+    uint32_t *s_bad = reinterpret_cast<uint32_t *>(sx16 + (size_t)NC * (cols >> 4));
+    double *run = reinterpret_cast<double *>(smem);
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+
+    // ---- geometry of the weight stream ----
+    const uint32_t r = lane & 15u, g = lane >> 4;
+    const uint64_t row_bytes = (uint64_t)SB * 144u;
+    const uint32_t ngroups = (rows + 15u) >> 4;
+    const uint32_t tpr = (SB + kMWaves - 1u) / kMWaves;    // tasks per row group and wave
+    const uint32_t ntasks = ((ngroups - blockIdx.x + gridDim.x - 1u) / gridDim.x) * tpr;
+    // A cursor walks the wave's tasks in order: row group rg (stride gridDim.x),
+    // within it superblock wave + 16*t for t < tpr.  A task past the end (or
+    // past the wave's last superblock) reads the first bytes of the matrix.
+    struct cursor {
+        uint32_t k, rg, t;
+    };
+    auto advance = [&](cursor &c) {
+        ++c.k;
+        if (++c.t == tpr) {
+            c.t = 0;
+            c.rg += gridDim.x;
+        }
+    };
+    auto issue = [&](cursor &c, q4k_regs &W) {
+        const uint32_t sbw = wave + kMWaves * c.t;
+        const bool real = c.k < ntasks && sbw < SB;
+        uint32_t row = c.rg * 16u + r;
+        row = row < rows ? row : rows - 1u;
+        q4k_issue(w, row_bytes, real ? row : 0u, real ? sbw : 0u, real ? g : 0u, W);
+        advance(c);
+    };
+    cursor ci{0u, blockIdx.x, 0u}, cc{0u, blockIdx.x, 0u};
+    q4k_regs W0, W1, W2;
+
+    // ---- stage the activations ----
+    // A thread takes runs of 8 consecutive elements (the 8 k-slots one lane
+    // feeds to one MFMA).  Slot q = tid + i*1024: the 32 runs of one superblock
+    // of one column sit in 32 adjacent lanes (q % 32), superblocks of the NC
+    // columns alternate (q / 32 % NC).  The loads are unconditional (clamped) so
+    // that they are in flight together; whole passes beyond the data are skipped.
+    constexpr int CH = 4;                                   // slots per thread: NC*cols/8 <= 4096
+    constexpr uint32_t kLogNC = NC == 8 ? 3u : NC == 4 ? 2u : NC == 2 ? 1u : 0u;
+    const uint32_t total_slots = (cols >> 3) * NC;
+    auto slot_of = [&](uint32_t q, uint32_t &c, uint32_t &k8) {
+        c = (q >> 5) & (NC - 1u);
+        k8 = ((q >> (5u + kLogNC)) << 5) | (q & 31u);
+        return q < total_slots && c < ncol;
+    };
+    lev_f32x4 va[CH], vb[CH];
+    {
+        lev_f32x4 ga[CH], gb[CH];
+#pragma unroll
+        for (int i = 0; i < CH; ++i) {
+            if ((uint32_t)i * kMThreads >= total_slots) break;   // workgroup-uniform
+            uint32_t c, k8;
+            if (!slot_of(tid + (uint32_t)i * kMThreads, c, k8)) c = 0u, k8 = 0u;
+            const lev_f32x4 *xp = reinterpret_cast<const lev_f32x4 *>(x + (uint64_t)c * cols) + 2u * k8;
+            va[i] = xp[0];
+            vb[i] = xp[1];
+            const lev_f32x4 *gp = reinterpret_cast<const lev_f32x4 *>(gain ? gain : x) + 2u * k8;
+            ga[i] = gp[0];
+            gb[i] = gp[1];
+        }
+        if (tid < (uint32_t)NC) s_bad[tid] = 0u;
+        if (tid < kNZeroBytes / 4u) reinterpret_cast<uint32_t *>(zero)[tid] = 0u;
+        // RMSNorm as the reference computes it (rmsnorm, rust/crates/lev-model/src/lib.rs:110-114):
+        // mean square and 1/sqrt in f64, then (f32)(x * inv) * gain
+        if (gain) {
+#pragma unroll
+            for (int i = 0; i < CH; ++i) {
+                if ((uint32_t)i * kMThreads >= total_slots) break;
+                uint32_t c, k8;
+                const bool real = slot_of(tid + (uint32_t)i * kMThreads, c, k8);
+                const lev_f32x4 a = va[i], b = vb[i];
+                double ss = (double)a.x * (double)a.x;
+                ss = fma((double)a.y, (double)a.y, ss); ss = fma((double)a.z, (double)a.z, ss);
+                ss = fma((double)a.w, (double)a.w, ss); ss = fma((double)b.x, (double)b.x, ss);
+                ss = fma((double)b.y, (double)b.y, ss); ss = fma((double)b.z, (double)b.z, ss);
+                ss = fma((double)b.w, (double)b.w, ss);
+                ss = lev_group_sum_f64<4>(ss);   // the four runs of a sub-block sit in four adjacent lanes
+                if (real && (k8 & 3u) == 3u) run[c * subs + (k8 >> 2)] = ss;
+            }
+        }
+        // every wave of the workgroup has its activations: a CU's memory pipeline is
+        // one queue, and weight loads of early waves would hold up the activation
+        // loads of late ones.  The first weights stream in while the digits are made.
+        lev_barrier_lds();
+        issue(ci, W0);
+        if constexpr (!SHORT) {
+            issue(ci, W1);
+            issue(ci, W2);
+        }
+        if (gain) {
+            // one wave per column adds the column's sums of squares
+            if (wave < ncol) {
+                double ss = 0.0;
+                for (uint32_t k = lane; k < subs; k += 64u) ss += run[wave * subs + k];
+                ss = lev_group_sum_f64<64>(ss);
+                // 1/sqrt(mean + eps): the hardware estimate and two Newton steps (full f64 accuracy)
+                const double a = fma(ss, rcols, (double)eps);
+                double rs = __builtin_amdgcn_rsq(a);
+                rs = rs * fma(-0.5 * a * rs, rs, 1.5);
+                rs = rs * fma(-0.5 * a * rs, rs, 1.5);
+                if (lane == 63u) s_inv[wave] = rs;
+            }
+            lev_barrier_lds();   // the sums (in the digit area) are dead from here
+#pragma unroll
+            for (int i = 0; i < CH; ++i) {
+                if ((uint32_t)i * kMThreads >= total_slots) break;
+                uint32_t c, k8;
+                const bool real = slot_of(tid + (uint32_t)i * kMThreads, c, k8);
+                const double inv = s_inv[real ? c : 0u];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    va[i][k] = (float)((double)va[i][k] * inv) * ga[i][k];
+                    vb[i][k] = (float)((double)vb[i][k] * inv) * gb[i][k];
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+        if ((uint32_t)i * kMThreads >= total_slots) break;
+        uint32_t c, k8;
+        const bool real = slot_of(tid + (uint32_t)i * kMThreads, c, k8);
+        const lev_f32x4 a = va[i], b = vb[i];
+        const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+        // largest magnitude of the superblock as an integer: NaN and infinity sort above every number
+        uint32_t mb = 0u;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const uint32_t bits = __float_as_uint(v[k]) & 0x7FFFFFFFu;
+            mb = bits > mb ? bits : mb;
+        }
+#define LEV_Q4K_MAXSTEP(CTRL)                                                                       \
+        {                                                                                          \
+            const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp((int)mb, (int)mb, CTRL, 0xF, 0xF, false); \
+            mb = o > mb ? o : mb;                                                                  \
+        }
+        LEV_Q4K_MAXSTEP(0xB1);    // quad_perm [1,0,3,2]
+        LEV_Q4K_MAXSTEP(0x4E);    // quad_perm [2,3,0,1]
+        LEV_Q4K_MAXSTEP(0x141);   // row_half_mirror
+        LEV_Q4K_MAXSTEP(0x140);   // row_mirror: all 16 lanes of a row hold the row's maximum
+#undef LEV_Q4K_MAXSTEP
+        {
+            const uint32_t o = (uint32_t)__builtin_amdgcn_ds_swizzle((int)mb, 0x401F);   // lane ^ 16
+            mb = o > mb ? o : mb;
+        }
+        uint32_t ex = mb >> 23;                             // biased exponent: |x| < 2^(ex-126)
+        if (real && ex == 255u) atomicOr(&s_bad[c], 1u);
+        ex = ex < 25u ? 25u : (ex > 254u ? 254u : ex);      // keeps both powers of two normal numbers
+        const float scale = __uint_as_float((278u - ex) << 23);   // 2^(151-ex): |x*scale| < 2^25
+        int sum = 0, X[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            X[k] = (int)rintf(v[k] * scale);
+            sum += X[k];
+        }
+        // balanced base-256 digits: adding 0x80 to each of the low three bytes carries
+        // into the next digit where a byte exceeds 127, and flipping bit 7 subtracts the
+        // 0x80 again, so the bytes of (X + 0x808080) ^ 0x808080 read as int8 are the
+        // digits.  A 4x4 byte transpose puts digit k of four neighbours into one dword.
+        uint32_t dw[4][2];                                  // dw[3] = highest digit
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            uint32_t Y[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) Y[k] = ((uint32_t)X[4 * h + k] + 0x00808080u) ^ 0x00808080u;
+            const uint32_t t0 = __builtin_amdgcn_perm(Y[1], Y[0], 0x05010400u);   // a0 b0 a1 b1
+            const uint32_t t1 = __builtin_amdgcn_perm(Y[1], Y[0], 0x07030602u);   // a2 b2 a3 b3
+            const uint32_t t2 = __builtin_amdgcn_perm(Y[3], Y[2], 0x05010400u);   // c0 d0 c1 d1
+            const uint32_t t3 = __builtin_amdgcn_perm(Y[3], Y[2], 0x07030602u);   // c2 d2 c3 d3
+            dw[0][h] = __builtin_amdgcn_perm(t2, t0, 0x05040100u);                // a0 b0 c0 d0
+            dw[1][h] = __builtin_amdgcn_perm(t2, t0, 0x07060302u);
+            dw[2][h] = __builtin_amdgcn_perm(t3, t1, 0x05040100u);
+            dw[3][h] = __builtin_amdgcn_perm(t3, t1, 0x07060302u);
+        }
+        sum += __builtin_amdgcn_update_dpp(0, sum, 0xB1, 0xF, 0xF, true);   // the two runs of a group of 16
+        if (real) {
+            // group of 16 = k8 / 2, this run its low or high 8 bytes of every plane
+            uint8_t *at = dig + (size_t)c * cols * 4u + (size_t)(k8 >> 1) * 64u + 8u * (k8 & 1u);
+#pragma unroll
+            for (int p = 0; p < 4; ++p) *reinterpret_cast<lev_u2 *>(at + 16 * p) = lev_u2{dw[p][0], dw[p][1]};
+            if (k8 & 1u) sx16[c * (cols >> 4) + (k8 >> 1)] = sum;
+            if ((k8 & 31u) == 31u) psb[c * SB + (k8 >> 5)] = __hiloint2double((int)((ex + 872u) << 20), 0);   // 2^(ex-151)
+        }
+    }
+    // columns of the layout beyond ncol hold no data: the lanes that read them
+    // only feed outputs that are never stored
+    lev_barrier_lds();
+
+    // ---- stream the weights ----
+    double yacc[NC];
+#pragma unroll
+    for (int q = 0; q < NC; ++q) yacc[q] = 0.0;
+    // lane (r, g): weight row r; its loads a and b are bytes [16*(g/2), +16) of chunks g%2 and
+    // 2 + g%2, i.e. for load i and nibble nb the half g/2 of sub-block 2*(2i + g%2) + nb
+    const uint32_t gh = g >> 1, gl = g & 1u;
+    const bool feeds = (r >> 2) == g;                       // this lane's A row belongs to its own lane group
+    const uint32_t a_lane = (4u * gl + gh) * 64u + 16u * (r & 3u);   // + (8i + 2nb) groups of 64 bytes
+
+    // One task: superblock (wave + 16*t) of the 16 rows of group rg.  After the
+    // last task of a row group the waves' partial sums meet in LDS.
+    uint32_t parity = 0;
+    auto compute = [&](cursor &c, const q4k_regs &W) {
+        const uint32_t rg = c.rg, t = c.t;
+        const uint32_t sbw = wave + kMWaves * t;
+        const bool live = sbw < SB;
+        const uint32_t sb = live ? sbw : SB - 1u;
+        // unpack_scale_min, lev-cpu/src/lib.rs:64-74: the eight scales and the eight mins as bytes
+        const uint32_t S0 = W.hdr.y, S1 = W.hdr.z, S2 = W.hdr.w;
+        const uint32_t sc_w[2] = {S0 & 0x3F3F3F3Fu, (S2 & 0x0F0F0F0Fu) | ((S0 >> 2) & 0x30303030u)};
+        const uint32_t mn_w[2] = {S1 & 0x3F3F3F3Fu, ((S2 >> 4) & 0x0F0F0F0Fu) | ((S1 >> 2) & 0x30303030u)};
+        // sub-block j = 4i + 2*gl + nb: byte 2*gl + nb of word i
+        int sc[2][2];
+        double mnd[2][2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int nb = 0; nb < 2; ++nb) {
+                sc[i][nb] = (int)__builtin_amdgcn_ubfe(sc_w[i], 16u * gl + 8u * (uint32_t)nb, 8u);
+                mnd[i][nb] = (double)__builtin_amdgcn_ubfe(mn_w[i], 16u * gl + 8u * (uint32_t)nb, 8u);
+            }
+        // B operands: the 16 code bytes as loaded, low or high nibbles
+        lev_i4 B[2][2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const lev_u4 v = i ? W.b : W.a;
+            B[i][0] = __builtin_bit_cast(lev_i4, v & 0x0F0F0F0Fu);
+            B[i][1] = __builtin_bit_cast(lev_i4, (v >> 4) & 0x0F0F0F0Fu);
+        }
+        // a task past the wave's last superblock contributes nothing
+        const double d = live ? (double)lev_f16_bits_to_f32(W.hdr.x & 0xFFFFu) : 0.0;
+        const double dmin = live ? (double)lev_f16_bits_to_f32(W.hdr.x >> 16) : 0.0;
+        const uint32_t goff = 16u * sb + 4u * gl + gh;        // group of 16 of (i, nb) = (0, 0); + 8i + 2nb
+#pragma unroll
+        for (int q = 0; q < NC; ++q) {
+            const uint8_t *ab = feeds ? dig + (size_t)q * cols * 4u + (size_t)sb * 1024u + a_lane : zero;
+            const int32_t *sxp = sx16 + (size_t)q * (cols >> 4) + goff;
+            int E[4] = {0, 0, 0, 0};
+            double acc2 = 0.0;
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+#pragma unroll
+                for (int nb = 0; nb < 2; ++nb) {
+                    const lev_i4 A = *reinterpret_cast<const lev_i4 *>(ab + (8 * i + 2 * nb) * 64);
+                    const lev_i4 D = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, B[i][nb], lev_i4{0, 0, 0, 0}, 0, 0, 0);
+                    // |D| <= 16*15*128 < 2^15, sc < 2^6: the four products per plane fit 32 bits with room
+#pragma unroll
+                    for (int p = 0; p < 4; ++p) {
+                        E[p] += __mul24(D[p], sc[i][nb]);
+                        asm("" : "+v"(E[p]));   // one multiply-add per plane: keeps the sums from being regrouped
+                    }
+                    acc2 = fma(mnd[i][nb], (double)sxp[8 * i + 2 * nb], acc2);
+                }
+            }
+            // plane 3 is the highest digit (at most 2 in magnitude)
+            const double hi = fma((double)E[3], 256.0, (double)E[2]);
+            const double lo = fma((double)E[1], 256.0, (double)E[0]);
+            const double dot = fma(hi, 65536.0, lo);
+            yacc[q] = fma(psb[q * SB + sb], fma(d, dot, -dmin * acc2), yacc[q]);
+        }
+
+        if (t + 1u == tpr) {   // workgroup-uniform
+            double *pp = part + parity * (kMWaves * 16u * NC);
+            parity ^= pb - 1u;
+#pragma unroll
+            for (int q = 0; q < NC; ++q) {
+                // the four lane groups hold the four quarters of the row's share
+                double s = yacc[q];
+                s += __shfl_xor(s, 16);
+                s += __shfl_xor(s, 32);
+                if (g == 0u) pp[(wave * 16u + r) * NC + q] = s;
+                yacc[q] = 0.0;
+            }
+            lev_barrier_lds();
+            if (tid < 16u * NC) {
+                const uint32_t col = tid >> 4, rr = tid & 15u, row = rg * 16u + rr;
+                double sum = 0.0;
+#pragma unroll
+                for (int kk = 0; kk < kMWaves; ++kk) sum += pp[((uint32_t)kk * 16u + rr) * NC + col];
+                if (col < ncol && row < rows)
+                    y[(uint64_t)col * rows + row] = s_bad[col] ? __builtin_nanf("") : (float)sum;
+            }
+            if (pb == 1u) lev_barrier_lds();   // the one buffer is written again by the next group
+        }
+        advance(c);
+    };
+
+    if constexpr (SHORT) {
+        // A wave that issues a load while the CU's memory queue is full waits until the
+        // queue drains: with all three tasks requested up front the waves sat in those
+        // waits while the digits were still to be made, and multiplied nothing until
+        // the last byte had arrived.  One task is requested before the digits, the
+        // next two each just ahead of the multiply that precedes their use.
+        issue(ci, W1);
+        __builtin_amdgcn_sched_barrier(0);
+        compute(cc, W0);
+        __builtin_amdgcn_sched_barrier(0);
+        issue(ci, W2);
+        __builtin_amdgcn_sched_barrier(0);
+        if (ntasks > 1u) compute(cc, W1);
+        if (ntasks > 2u) compute(cc, W2);
+        return;
+    }
+    // Three tasks in flight per wave.
+    // The scheduling barriers keep a refill's loads behind the compute that
+    // frees its registers: hoisted above it they would be younger than the
+    // data the compute waits for, and the wait would cover them too.
+    while (true) {
+        compute(cc, W0);
+        __builtin_amdgcn_sched_barrier(0);
+        issue(ci, W0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (cc.k >= ntasks) break;
+        compute(cc, W1);
+        __builtin_amdgcn_sched_barrier(0);
+        issue(ci, W1);
+        __builtin_amdgcn_sched_barrier(0);
+        if (cc.k >= ntasks) break;
+        compute(cc, W2);
+        __builtin_amdgcn_sched_barrier(0);
+        issue(ci, W2);
+        __builtin_amdgcn_sched_barrier(0);
+        if (cc.k >= ntasks) break;
+    }
+}
+
 size_t q4k_mfma_lds_bytes(uint32_t cols, uint32_t nc, uint32_t pb) {
     return nc > 4u ? q4k_lds<2>::total(cols >> 5, pb) : q4k_lds<1>::total(cols >> 5, pb);
 }
@@ -491,6 +860,40 @@ hipError_t launch_mfma(lev_ctx *ctx, const uint8_t *w, const float *x, const flo
     return launch_mfma_variant<NC, false>(ctx, w, x, gain, eps, y, cols, rows, ncol);
 }
 
+size_t q4k_narrow_lds_bytes(uint32_t cols, uint32_t nc, uint32_t pb) {
+    return nc > 1u ? q4k_narrow_lds<2>::total(cols, pb) : q4k_narrow_lds<1>::total(cols, pb);
+}
+
+template <int NC, bool SHORT>
+hipError_t launch_narrow_variant(lev_ctx *ctx, const uint8_t *w, const float *x, const float *gain, float eps,
+                                 float *y, uint32_t cols, uint32_t rows, uint32_t ncol) {
+    const uint32_t pb = q4k_narrow_lds_bytes(cols, NC, 2u) <= q4k_lds_limit(ctx) ? 2u : 1u;
+    const size_t lds = q4k_narrow_lds_bytes(cols, NC, pb);
+    static size_t configured = 0;   // per instantiation: raise the dynamic LDS limit once per size
+    if (lds > 48 * 1024 && lds > configured) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&q4_k_mfma_gemv_narrow<NC, SHORT>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        configured = lds;
+    }
+    const uint32_t groups = (rows + 15u) / 16u;
+    const uint32_t blocks = groups < (uint32_t)ctx->num_cus ? groups : (uint32_t)ctx->num_cus;
+    hipLaunchKernelGGL((q4_k_mfma_gemv_narrow<NC, SHORT>), dim3(blocks), dim3(kMThreads), lds, ctx->stream, w,
+                       x, gain, eps, y, cols, rows, ncol, pb, 1.0 / (double)cols);
+    return hipGetLastError();
+}
+
+template <int NC>
+hipError_t launch_narrow(lev_ctx *ctx, const uint8_t *w, const float *x, const float *gain, float eps,
+                         float *y, uint32_t cols, uint32_t rows, uint32_t ncol) {
+    const uint32_t groups = (rows + 15u) / 16u;
+    const uint32_t blocks = groups < (uint32_t)ctx->num_cus ? groups : (uint32_t)ctx->num_cus;
+    const uint32_t tpr = ((cols >> 8) + kMWaves - 1u) / kMWaves;
+    const uint32_t most = ((groups + blocks - 1u) / blocks) * tpr;   // tasks of the busiest wave
+    if (most <= 3u) return launch_narrow_variant<NC, true>(ctx, w, x, gain, eps, y, cols, rows, ncol);
+    return launch_narrow_variant<NC, false>(ctx, w, x, gain, eps, y, cols, rows, ncol);
+}
+
 }  // namespace
 
 // Columns one launch of the MFMA kernel can take for this in_dim (0: not usable).
@@ -503,10 +906,30 @@ uint32_t lev_q4_k_mfma_cols(const lev_ctx *ctx, uint32_t in_dim) {
     return nc;
 }
 
+// Columns the one- and two-column kernel can take for this in_dim (0: not usable).
+uint32_t lev_q4_k_mfma_narrow_cols(const lev_ctx *ctx, uint32_t in_dim) {
+    static const bool off = [] {
+        const char *e = getenv("LEV_Q4K_NARROW");   // LEV_Q4K_NARROW=0: four columns per product, for comparison
+        return e && e[0] == '0';
+    }();
+    if (off || in_dim % 256u != 0u || in_dim == 0u) return 0;
+    const size_t limit = q4k_lds_limit(ctx);
+    for (uint32_t nc = 2; nc >= 1u; --nc)
+        if ((uint64_t)nc * in_dim <= 32768u && q4k_narrow_lds_bytes(in_dim, nc, 1u) <= limit) return nc;
+    return 0;
+}
+
+// ncol <= lev_q4_k_mfma_narrow_cols(ctx, in_dim) (the narrow kernel) or
 // ncol <= lev_q4_k_mfma_cols(ctx, in_dim); w 16-byte aligned.
 hipError_t lev_q4_k_mfma_gemv_launch(lev_ctx *ctx, const uint8_t *w, const float *x, const float *gain,
                                      float eps, float *y, uint32_t in_dim, uint32_t rows,
                                      uint32_t ncol) {
+    // one column: the narrow kernel (9.1 us against 9.7 at 12288 x 4096); two columns: only where the
+    // four-column kernel's planes do not fit (it is the faster of the two there: 9.9 against 10.8 us)
+    if (ncol <= lev_q4_k_mfma_narrow_cols(ctx, in_dim) && (ncol == 1u || lev_q4_k_mfma_cols(ctx, in_dim) < ncol)) {
+        if (ncol > 1) return launch_narrow<2>(ctx, w, x, gain, eps, y, in_dim, rows, ncol);
+        return launch_narrow<1>(ctx, w, x, gain, eps, y, in_dim, rows, ncol);
+    }
     if (ncol > 4) return launch_mfma<8>(ctx, w, x, gain, eps, y, in_dim, rows, ncol);
     if (ncol > 2) return launch_mfma<4>(ctx, w, x, gain, eps, y, in_dim, rows, ncol);
     if (ncol > 1) return launch_mfma<2>(ctx, w, x, gain, eps, y, in_dim, rows, ncol);

@@ -569,6 +569,26 @@ def test_q4_k_exact_sums_do_not_depend_on_the_scale_of_x(ctx):
         assert np.array_equal(bits(got), bits(np.ldexp(base, e).astype(np.float32))), e
 
 
+@pytest.mark.parametrize("rows,cols,ncol", [(24, 12288, 1), (24, 12288, 2), (18, 16384, 2), (11, 32768, 1),
+                                            (3000, 1024, 1), (1, 256, 1), (70, 11008, 2)])
+def test_q4_k_one_and_two_columns_on_long_rows(ctx, rows, cols, ncol):
+    """One column, and two columns of a row too long for the four-column kernel's digit planes
+    (above 8192): the same integer sums, so the same contract and the same exact scaling by
+    powers of two; a column does not depend on its neighbour."""
+    w, x, gain = H.config3(rows, cols, ncol, seed=rows + cols % 101)
+    got = q4k_gemv(ctx, w, x, rows, cols, ncol, gain)
+    xn = H.rmsnorm_rows(x, gain)
+    for c in range(ncol):
+        assert O.max_rel_err(got[c], O.q4_k_matvec_f64(w, rows, cols, xn[c])) < TOL, c
+    plain = q4k_gemv(ctx, w, x, rows, cols, ncol)
+    for e in (-40, 33):
+        scaled = q4k_gemv(ctx, w, np.ldexp(x, e).astype(np.float32), rows, cols, ncol)
+        assert np.array_equal(bits(scaled), bits(np.ldexp(plain, e).astype(np.float32))), e
+    if ncol == 2:
+        alone = q4k_gemv(ctx, w, x[1:], rows, cols, 1)
+        assert np.array_equal(bits(alone[0]), bits(plain[1]))
+
+
 def test_q4_k_mixed_magnitudes_within_a_row(ctx):
     """Superblocks of very different magnitude in one row: each carries its own power of two."""
     rows, cols = 48, 4096
