@@ -430,9 +430,9 @@ def config4_q6(rows, cols, tokens, seed):
 
 
 @pytest.mark.parametrize("rows,cols,tokens", [(128, 256, 128), (64, 512, 32), (200, 1024, 37), (33, 256, 1),
-                                              # either side of the 128-row x 128-token workgroup tile
+                                              # either side of the 128-row x 256-token workgroup tile
                                               (129, 256, 129), (127, 512, 127), (256, 768, 256),
-                                              (300, 4096, 150)])
+                                              (300, 4096, 150), (97, 1280, 257), (260, 256, 300)])
 def test_q6_gemm_small_shapes_every_row(ctx, rows, cols, tokens):
     """coopmat.rs:333-425 against the gate of lev-cli main.rs:1201-1217 (W and X
     rounded to fp16, f64 accumulation), every row and token."""
