@@ -117,6 +117,7 @@ typedef _Float16 lev_f16x2 __attribute__((ext_vector_type(2)));
 // (Q4_0 and Q6_K blocks are 2-byte aligned; pairs of Q4_0 blocks 4-byte).
 struct __attribute__((packed, aligned(4))) lev_u32x4_a4 { uint32_t v[4]; };
 struct __attribute__((packed, aligned(4))) lev_u32_a4 { uint32_t v; };
+struct __attribute__((packed, aligned(4))) lev_u32x2_a4 { uint32_t v[2]; };
 struct __attribute__((packed, aligned(2))) lev_u32_a2 { uint32_t v; };
 struct __attribute__((packed, aligned(2))) lev_u16_a2 { uint16_t v; };
 

@@ -28,9 +28,13 @@
 //       (two MFMAs), x = hi + lo to 2^-22;
 //   the output lane of weight row n is the lane that holds row n's block scale
 //   d, so y += d * (A.B) needs no exchange.
-// A lane fetches a PAIR of blocks (36 bytes, as in the decode GEMV: wide loads,
-// whole rows contiguous per wave) and the four lanes of a row swap code bytes
-// through a small wave-private LDS area so that each MFMA sees one block.
+// A wave fetches the 144 bytes of eight blocks of each of its 16 rows as they lie
+// in memory, 16 bytes per lane with consecutive lanes on consecutive bytes of a row
+// (the L1 looks a 32-byte sector up once per four lanes that touch it: lanes on
+// different rows cost a lookup each, and with a block pair per lane the lookups,
+// not the bytes, kept the L1 busy for more than half of the kernel), parks them in
+// a small wave-private LDS area, and every lane reads from there the four code
+// bytes (both nibbles: eight weights) and the scale it multiplies.
 #include "moe_grouped.hpp"
 
 #include <cstdlib>
@@ -45,7 +49,10 @@ constexpr int kNC = 12;                // token columns per pass (of the 16 an M
                                        // tokens x top-8 over 128 experts one in fifty has more than 8 pairs (a layer then
                                        // measured 172 us instead of 122), one in three thousand more than 12
 constexpr int kFlagBadExpertId = 1;    // same bit as the per-token kernels
-constexpr uint32_t kGrpScaleDw = 10;   // dwords per row of block scales in a wave's exchange area
+constexpr uint32_t kGrpRowBytes = 152;        // a row of a wave's area: the 144 bytes of eight blocks + 8: 38 dwords,
+                                              // so that the 16 rows start in 16 different even banks of the 32
+constexpr uint32_t kGrpRawBytes = 16 * kGrpRowBytes;
+constexpr int kGrpLoads = 3;                  // 16-byte loads per lane and group: 16 rows x 144 bytes over 64 lanes
 constexpr size_t kGrpStaticLds = (size_t)2 * (kGrpWaves / 2) * 16 * kNC * 4 + 1024;   // gate values, pair records
 
 typedef _Float16 g_h8 __attribute__((ext_vector_type(8)));
@@ -55,8 +62,9 @@ typedef uint32_t g_u2 __attribute__((ext_vector_type(2)));
 // ---------------------------------------------------------------------------
 // Activation planes.  A row is scaled by the power of two that brings its maximum into [1, 2)
 // (zero, denormal and non-finite maxima: no scaling) and split into fp16 high and low halves;
-// inside each run of 8 elements the planes hold elements 0,2,1,3,4,6,5,7: the order in which
-// the masks of the matrix-core kernel deliver the code bytes of a dword pair.
+// run 4b + g of a row holds elements 4g, 4g+2, 4g+1, 4g+3, then 16+4g, 16+4g+2, 16+4g+1, 16+4g+3 of
+// block b: the weights in code bytes 4g..4g+3 of the block (low nibbles, then high nibbles), in the
+// order in which the masks of the matrix-core kernel deliver them.
 // ---------------------------------------------------------------------------
 struct grp_scale { float scale, unscale; };
 __device__ __forceinline__ grp_scale grp_row_scale(uint32_t max_bits) {
@@ -118,7 +126,7 @@ moe_group_kernel(const int32_t *__restrict__ ids, uint32_t pairs, uint32_t exper
         const float scale = grp_row_scale(__float_as_uint(m)).scale;
         for (uint32_t q = tid; q < runs; q += 1024u) {
             g_h8 h, l;
-            grp_split_run(s4[2u * q], s4[2u * q + 1u], scale, h, l);
+            grp_split_run(s4[8u * (q >> 2) + (q & 3u)], s4[8u * (q >> 2) + 4u + (q & 3u)], scale, h, l);
             *reinterpret_cast<g_h8 *>(xh + (uint64_t)t * hidden + 8u * q) = h;
             *reinterpret_cast<g_h8 *>(xl + (uint64_t)t * hidden + 8u * q) = l;
         }
@@ -164,10 +172,10 @@ moe_group_kernel(const int32_t *__restrict__ ids, uint32_t pairs, uint32_t exper
 // the pair's token (PAIRED: gate/up read x) or the pair itself (down reads act).
 // ---------------------------------------------------------------------------
 
-// the 8 code bytes a lane needs of one block -> B operand: fp16 integers n - 8.
-// sh = 0 for the lanes that take the low nibbles, 4 for the high nibbles; mask
-// and magic arrive in registers so that (v & mask) | magic is ONE v_and_or_b32.
-__device__ __forceinline__ g_h8 q4_0_operand(g_u2 codes, uint32_t sh, uint32_t mask, uint32_t magic) {
+// the 4 code bytes a lane takes of one block -> B operand: fp16 integers n - 8, low nibbles
+// of bytes (0, 2), (1, 3), then the high nibbles; mask and magic arrive in registers so that
+// (v & mask) | magic is ONE v_and_or_b32.
+__device__ __forceinline__ g_h8 q4_0_operand(uint32_t codes, uint32_t mask, uint32_t magic) {
     typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
     const f16x2 bias = {(_Float16)1032.0f, (_Float16)1032.0f};
     auto two = [&](uint32_t v) {
@@ -176,10 +184,10 @@ __device__ __forceinline__ g_h8 q4_0_operand(g_u2 codes, uint32_t sh, uint32_t m
         return __builtin_bit_cast(uint32_t, h - bias);
     };
     g_u4 bits;
-    bits.x = two(codes.x >> sh);
-    bits.y = two(codes.x >> (sh + 8u));
-    bits.z = two(codes.y >> sh);
-    bits.w = two(codes.y >> (sh + 8u));
+    bits.x = two(codes);
+    bits.y = two(codes >> 8);
+    bits.z = two(codes >> 4);
+    bits.w = two(codes >> 12);
     return __builtin_bit_cast(g_h8, bits);
 }
 
@@ -202,12 +210,10 @@ moe_grouped_kernel(lev_moe_grouped_args a, uint32_t tiles_per_wg, const float *_
     const uint32_t plane = runs * kNC * 8u;                      // halfs
     _Float16 *sxh = reinterpret_cast<_Float16 *>(smem);           // [run][col][8]
     _Float16 *sxl = sxh + plane;
-    // wave-private exchange area: 16 rows x (8 blocks x 4 dwords + 4 pad), then 16 rows of
-    // 8 scales + 2 pad (a stride of 8 dwords put rows r and r+8 into the same bank for every read)
-    uint32_t *xch = reinterpret_cast<uint32_t *>(sxl + plane);
-    constexpr uint32_t kRowDw = 36, kXchDw = 16 * kRowDw + 16 * kGrpScaleDw;
+    // wave-private area: the 144 bytes of a group of eight blocks of each of the wave's 16 rows (+ 8 of padding)
+    uint8_t *xch = reinterpret_cast<uint8_t *>(sxl + plane);
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-    uint32_t *area = xch + wave * kXchDw;
+    uint8_t *area = xch + wave * kGrpRawBytes;
     __shared__ int32_t s_pair[kNC];
     __shared__ float s_us[kNC], s_scale[kNC];
     __shared__ float s_gate[PAIRED ? 2 * (kGrpWaves / 2) * 16 * kNC : 1];   // [tile parity][tile row][col]
@@ -228,29 +234,40 @@ moe_grouped_kernel(lev_moe_grouped_args a, uint32_t tiles_per_wg, const float *_
     else
         mat = a.base + a.down_off + e * a.down_stride;
 
-    // groups of 8 blocks = 4 pairs; lane (r, g) fetches pair g of row r of a tile
+    // groups of 8 blocks = 144 bytes = nine 16-byte pieces per row; lane l fetches pieces l, l + 64
+    // and (lanes 0..15; the others repeat the last one) l + 128 of the 144 of a group, piece q being
+    // piece q % 9 of row q / 9, and parks it in that row of the wave's area (8-byte aligned: two
+    // halves; five 8-byte loads per lane instead measured 6 % slower)
     const uint32_t ngrp = nblk >> 3;
-    auto fetch = [&](uint32_t tile, uint32_t grp, uint32_t (&D)[9]) {
+    uint32_t prow[kGrpLoads], poff[kGrpLoads], pdst[kGrpLoads];
+#pragma unroll
+    for (int j = 0; j < kGrpLoads; ++j) {
+        const uint32_t q = lane + 64u * j < 143u ? lane + 64u * j : 143u;
+        prow[j] = q / 9u;
+        poff[j] = (q % 9u) * 16u;
+        pdst[j] = prow[j] * kGrpRowBytes + poff[j];
+    }
+    auto fetch = [&](uint32_t tile, uint32_t grp, g_u4 (&D)[kGrpLoads]) {
         const uint32_t tc = tile < t1 ? tile : t1 - 1u;          // past the end: any valid address
-        const uint32_t row = tc * tile_rows + wv * 16u + r;
-        const uint32_t rowc = row < out_rows ? row : out_rows - 1u;
-        const uint8_t *p = mat + rowc * row_bytes + (uint64_t)(grp * 4u + g) * 36u;
-        lev_u32x4_a4 v0 = *reinterpret_cast<const lev_u32x4_a4 *>(p);
-        lev_u32x4_a4 v1 = *reinterpret_cast<const lev_u32x4_a4 *>(p + 16);
-        lev_u32_a4 v2 = *reinterpret_cast<const lev_u32_a4 *>(p + 32);
-        D[0] = v0.v[0]; D[1] = v0.v[1]; D[2] = v0.v[2]; D[3] = v0.v[3];
-        D[4] = v1.v[0]; D[5] = v1.v[1]; D[6] = v1.v[2]; D[7] = v1.v[3];
-        D[8] = v2.v;
+        const uint32_t row0 = tc * tile_rows + wv * 16u;
+#pragma unroll
+        for (int j = 0; j < kGrpLoads; ++j) {
+            const uint32_t row = row0 + prow[j];
+            const uint32_t rowc = row < out_rows ? row : out_rows - 1u;
+            const lev_u32x4_a4 v =
+                *reinterpret_cast<const lev_u32x4_a4 *>(mat + rowc * row_bytes + (uint64_t)grp * 144u + poff[j]);
+            D[j] = g_u4{v.v[0], v.v[1], v.v[2], v.v[3]};
+        }
     };
-    const uint32_t nib_shift = 4u * (g >> 1);
     uint32_t k_mask = 0x000F000Fu, k_magic = 0x64006400u;
     asm("" : "+v"(k_mask), "+v"(k_magic));   // keep both in registers (see q4_0_operand)
+    const uint8_t *const my_row = area + r * kGrpRowBytes;    // this lane's weight row in the area
     const uint32_t colc = r < (uint32_t)kNC ? r : (uint32_t)kNC - 1u;   // A rows past kNC: any valid address
 
     for (uint32_t pass = 0; pass * kNC < n; ++pass) {
         const uint32_t ncols = n - pass * kNC < (uint32_t)kNC ? n - pass * kNC : (uint32_t)kNC;
         // the first weights are requested ahead of everything that only concerns the activations
-        uint32_t Dc[9], Dn[9];
+        g_u4 Dc[kGrpLoads], Dn[kGrpLoads];
         uint32_t ft = t0, fg = 0;                                 // the next group to request
         auto advance = [&] { if (++fg == ngrp) { fg = 0; ++ft; } };
         fetch(ft, fg, Dc);
@@ -282,8 +299,8 @@ moe_grouped_kernel(lev_moe_grouped_args a, uint32_t tiles_per_wg, const float *_
                     l = *reinterpret_cast<const g_h8 *>(src_l + at);
                 } else {
                     // act: split here, its row maximum was only complete when gate/up ended
-                    const lev_f32x4 *s4 = reinterpret_cast<const lev_f32x4 *>(src + (uint64_t)p * in_len + 8u * q);
-                    grp_split_run(s4[0], s4[1], s_scale[c], h, l);
+                    const lev_f32x4 *s4 = reinterpret_cast<const lev_f32x4 *>(src + (uint64_t)p * in_len);
+                    grp_split_run(s4[8u * (q >> 2) + (q & 3u)], s4[8u * (q >> 2) + 4u + (q & 3u)], s_scale[c], h, l);
                 }
                 *reinterpret_cast<g_h8 *>(sxh + (q * kNC + c) * 8u) = h;
                 *reinterpret_cast<g_h8 *>(sxl + (q * kNC + c) * 8u) = l;
@@ -300,20 +317,11 @@ moe_grouped_kernel(lev_moe_grouped_args a, uint32_t tiles_per_wg, const float *_
                 // unconditional (clamped past the end): no branch around loads
                 fetch(ft, fg, Dn);
                 advance();
-                // hand the pair's two blocks to the lanes that need them
-                {
-                    const uint32_t *D = Dc;
-                    g_u4 qa, qb;
-                    qa.x = __builtin_amdgcn_alignbit(D[1], D[0], 16);
-                    qa.y = __builtin_amdgcn_alignbit(D[2], D[1], 16);
-                    qa.z = __builtin_amdgcn_alignbit(D[3], D[2], 16);
-                    qa.w = __builtin_amdgcn_alignbit(D[4], D[3], 16);
-                    qb.x = D[5]; qb.y = D[6]; qb.z = D[7]; qb.w = D[8];
-                    *reinterpret_cast<g_u4 *>(area + r * kRowDw + (2u * g) * 4u) = qa;
-                    *reinterpret_cast<g_u4 *>(area + r * kRowDw + (2u * g + 1u) * 4u) = qb;
-                    typedef float f32x2 __attribute__((ext_vector_type(2)));
-                    *reinterpret_cast<f32x2 *>(area + 16 * kRowDw + r * kGrpScaleDw + 2u * g) =
-                        f32x2{lev_f16_bits_to_f32(D[0] & 0xFFFFu), lev_f16_bits_to_f32(D[4] >> 16)};
+                // park the group as it lies in memory
+#pragma unroll
+                for (int j = 0; j < kGrpLoads; ++j) {
+                    *reinterpret_cast<g_u2 *>(area + pdst[j]) = g_u2{Dc[j].x, Dc[j].y};
+                    *reinterpret_cast<g_u2 *>(area + pdst[j] + 8u) = g_u2{Dc[j].z, Dc[j].w};
                 }
                 // wave-private area: the hardware runs one wave's LDS accesses in order
                 __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -324,19 +332,27 @@ moe_grouped_kernel(lev_moe_grouped_args a, uint32_t tiles_per_wg, const float *_
                     const uint32_t at = (((grp * 8u + b) * 4u + g) * kNC + colc) * 8u;
                     const g_h8 Ah = *reinterpret_cast<const g_h8 *>(sxh + at);
                     const g_h8 Al = *reinterpret_cast<const g_h8 *>(sxl + at);
-                    const g_u2 codes = *reinterpret_cast<const g_u2 *>(area + r * kRowDw + b * 4u + 2u * (g & 1u));
-                    const float d = reinterpret_cast<const float *>(area + 16 * kRowDw)[r * kGrpScaleDw + b];
-                    const g_h8 B = q4_0_operand(codes, nib_shift, k_mask, k_magic);
+                    // code bytes 4g..4g+3 of block b start at byte 18 b + 2 + 4 g of the row's 144: on a
+                    // dword boundary for odd b, two bytes behind one for even b
+                    uint32_t codes;
+                    if (b & 1u) {
+                        codes = *reinterpret_cast<const uint32_t *>(my_row + 18u * b + 2u + 4u * g);
+                    } else {
+                        const lev_u32x2_a4 two_dw = *reinterpret_cast<const lev_u32x2_a4 *>(my_row + 18u * b + 4u * g);
+                        codes = __builtin_amdgcn_alignbit(two_dw.v[1], two_dw.v[0], 16);
+                    }
+                    const _Float16 d = *reinterpret_cast<const _Float16 *>(my_row + 18u * b);
+                    const g_h8 B = q4_0_operand(codes, k_mask, k_magic);
                     lev_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
                     acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ah, B, acc, 0, 0, 0);
                     acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(Al, B, acc, 0, 0, 0);
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) y[i] = fmaf(d, acc[i], y[i]);
+                    for (int i = 0; i < 4; ++i) y[i] = fmaf((float)d, acc[i], y[i]);
                 }
                 __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
                 __builtin_amdgcn_wave_barrier();   // reads done before the next group's writes
 #pragma unroll
-                for (int k = 0; k < 9; ++k) Dc[k] = Dn[k];
+                for (int k = 0; k < kGrpLoads; ++k) Dc[k] = Dn[k];
             }
 
             // output lane (r, g): weight row r of the tile, columns 4g..4g+3
@@ -438,7 +454,7 @@ grouped_layout layout_of(const lev_moe_grouped_args &a) {
 
 size_t grouped_lds(uint32_t in_len, bool paired) {
     (void)paired;
-    return (size_t)2 * (in_len / 8) * kNC * 16 + (size_t)kGrpWaves * (16 * 36 + 16 * kGrpScaleDw) * 4;
+    return (size_t)2 * (in_len / 8) * kNC * 16 + (size_t)kGrpWaves * kGrpRawBytes;
 }
 
 // Row tiles per workgroup.  A workgroup pays for its activation planes (a chain of dependent reads
