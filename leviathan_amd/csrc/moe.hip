@@ -447,13 +447,26 @@ moe_scores_mfma_kernel(const float *__restrict__ wr, const float *__restrict__ x
     const lev_f32x4 *wb = reinterpret_cast<const lev_f32x4 *>(wr + (uint64_t)exp * hidden + wave * span) + kq;
     moe_f64x4 acc = {0.0, 0.0, 0.0, 0.0};
     const uint32_t steps = span >> 4;
-#pragma unroll 8
-    for (uint32_t s = 0; s < steps; ++s) {
-        const lev_f32x4 a = xa[4u * s], b = wb[4u * s];
-        acc = __builtin_amdgcn_mfma_f64_16x16x4f64((double)a.x, (double)b.x, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f64_16x16x4f64((double)a.y, (double)b.y, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f64_16x16x4f64((double)a.z, (double)b.z, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f64_16x16x4f64((double)a.w, (double)b.w, acc, 0, 0, 0);
+    // four steps' operands are requested together (steps past the end repeat the last one with a zero
+    // activation: they add nothing)
+    for (uint32_t s0 = 0; s0 < steps; s0 += 4u) {
+        lev_f32x4 a[4], b[4];
+#pragma unroll
+        for (uint32_t j = 0; j < 4u; ++j) {
+            const uint32_t s = s0 + j < steps ? s0 + j : steps - 1u;
+            a[j] = xa[4u * s];
+            b[j] = wb[4u * s];
+        }
+#pragma unroll
+        for (uint32_t j = 0; j < 4u; ++j) {
+            const bool live = s0 + j < steps;
+            const lev_f32x4 aj = live ? a[j] : lev_f32x4{0.f, 0.f, 0.f, 0.f};
+            const lev_f32x4 bj = live ? b[j] : lev_f32x4{0.f, 0.f, 0.f, 0.f};
+            acc = __builtin_amdgcn_mfma_f64_16x16x4f64((double)aj.x, (double)bj.x, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f64_16x16x4f64((double)aj.y, (double)bj.y, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f64_16x16x4f64((double)aj.z, (double)bj.z, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f64_16x16x4f64((double)aj.w, (double)bj.w, acc, 0, 0, 0);
+        }
     }
     // D of the f64 16x16x4 product: register r of lane (i, kq) is row (token) 4*r + kq of column (expert) i
 #pragma unroll
