@@ -148,13 +148,34 @@ moe_group_kernel(const int32_t *__restrict__ ids, uint32_t pairs, uint32_t exper
     }
     if (bad_seen) atomicOr(flag, kFlagBadExpertId);
     __syncthreads();
-    // exclusive scan, every thread for its own experts (broadcast LDS reads;
-    // experts <= 4096, so at most a few thousand short iterations)
-    for (uint32_t e = tid; e <= experts; e += 1024u) {
-        int32_t run = 0;
-        for (uint32_t j = 0; j < e; ++j) run += s_cnt[j];
-        goff[e] = run;
-        if (e < experts) s_cur[e] = run;
+    // exclusive scan of the counts (experts <= 4096): thread i takes experts 4i..4i+3, the waves scan
+    // their threads' sums by shuffles and meet in LDS
+    {
+        __shared__ int32_t s_wave[16];
+        int32_t c4[4], local = 0;
+#pragma unroll
+        for (uint32_t k = 0; k < 4u; ++k) {
+            const uint32_t e = 4u * tid + k;
+            c4[k] = e < experts ? s_cnt[e] : 0;
+            local += c4[k];
+        }
+        int32_t incl = local;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int32_t o = __shfl_up(incl, off);
+            if ((int)(tid & 63u) >= off) incl += o;
+        }
+        if ((tid & 63u) == 63u) s_wave[tid >> 6] = incl;
+        __syncthreads();
+        int32_t run = incl - local;
+        for (uint32_t w = 0; w < (tid >> 6); ++w) run += s_wave[w];
+#pragma unroll
+        for (uint32_t k = 0; k < 4u; ++k) {
+            const uint32_t e = 4u * tid + k;
+            if (e <= experts) goff[e] = run;
+            if (e < experts) s_cur[e] = run;
+            run += c4[k];
+        }
     }
     __syncthreads();
     // The order of an expert's pairs in the list depends on the atomics; no
