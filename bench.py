@@ -307,6 +307,7 @@ def main():
 
         # ---------------------------------------------- Q4_0 large streaming
         if want("q4_0"):
+            torch.cuda.empty_cache()   # every family starts from fresh allocations, as when it runs alone
             rows2 = 32768
             nb2 = rows2 * cols // 32
             ring2 = make_q4_0(8 * nb2)
@@ -319,6 +320,7 @@ def main():
 
         # ------------------------------------------------------ Q6_K + argmax
         if want("q6_k"):
+            torch.cuda.empty_cache()
             r6, nb6 = 32000, 32000 * 4096 // 256
             ring6 = make_q6_k(6 * nb6)
             x = torch.randn(cols, device=dev, generator=gen)
@@ -369,6 +371,7 @@ def main():
 
         # ------------------------------------------- RMSNorm + Q4_K N columns
         if want("q4_k", "gemm"):
+            torch.cuda.empty_cache()
             r4, nb4 = 12288, 12288 * 4096 // 256
             ncopy4 = 20
             ring4 = make_q4_k(ncopy4 * nb4)
@@ -427,6 +430,9 @@ def main():
 
         # ------------------------------------------------------------- MoE
         if want("moe1", "moe64"):
+            # the blocks the earlier entries freed go back to the driver: the 1 GB of pools are then
+            # fresh allocations, as when this entry runs alone, not pieces of torch's cache
+            torch.cuda.empty_cache()
             hidden, inter, experts, top_k = 2048, 768, 128, 8
             gu = inter * (hidden // 32) * 18
             dn = hidden * (inter // 32) * 18
