@@ -217,7 +217,8 @@ int lev_hip_swiglu_quant_q8(lev_ctx *ctx, const float *d_gate, const float *d_up
 /* ---- prefill GEMM (Builder::matvec_rows with gemm, gpu.rs:345-355;
  * q4k gemm blocked, lev-forge/src/coopmat.rs:236-323) ----
  * x is fp16 [tokens][in_dim], y is f32 [tokens][rows]; W is dequantised to
- * fp16 tiles in LDS and multiplied on the matrix cores, f32 accumulate. */
+ * fp16 tiles in LDS and multiplied on the matrix cores, f32 accumulate.
+ * in_dim at most 4194304, tokens at most 1048576 (LEV_ERR_BAD_DIMENSIONS beyond). */
 int lev_hip_q4_k_gemm_prefill(lev_ctx *ctx, const void *d_w, size_t w_bytes, uint64_t w_off,
                               const uint16_t *d_x_f16, size_t x_count, float *d_y,
                               size_t y_capacity, uint32_t in_dim, uint32_t rows,
