@@ -465,6 +465,22 @@ def test_q6_gemm_lm_head_size_sampled_rows(ctx):
     assert np.array_equal(got2.view(np.uint32), (got * 2).view(np.uint32))
 
 
+def test_q6_gemm_token_tiles_taken_in_turn(ctx):
+    """More workgroup tiles than CUs with the row tiles alone nearly filling the chip: a workgroup
+    takes its rows' token tiles one after the other (three here, the last one ragged).  Every tile
+    is the product the kernel forms when that tile is the whole call, bit for bit, and sampled rows
+    meet the gate."""
+    rows, cols, tokens = 32000, 4096, 600
+    w, x = config4_q6(rows, cols, tokens, seed=16)
+    got = gemm6(ctx, w, x, rows, cols, tokens)
+    assert np.all(np.isfinite(got))
+    for lo, hi in ((0, 256), (256, 512), (512, 600)):
+        part = gemm6(ctx, w, x[lo:hi].copy(), rows, cols, hi - lo)
+        assert np.array_equal(part.view(np.uint32), got[lo:hi].view(np.uint32)), (lo, hi)
+    ref = O.q6_k_gemm_f16_oracle(w, rows, cols, x.view(np.uint16), tokens, 0, 97)
+    assert O.max_rel_err(got[:, 0::97], ref) < GEMM_TOL
+
+
 def test_q6_gemm_one_token_matches_the_gemv_within_rounding(ctx):
     """One token through the GEMM against the f64 GEMV oracle on the same fp16
     activations: the only difference is the fp16 rounding of W (2^-11 relative
