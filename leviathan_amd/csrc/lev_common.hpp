@@ -47,7 +47,8 @@ struct lev_ctx {
     int *d_flag = nullptr;
     // words kArgmaxTicketWord + 1024*k, k = 0..8: arrival counters of the greedy-token merge
     // (4 KB apart: counters that share a cache line serialise in one L2 channel), zero between launches
-    static constexpr uint32_t kFlagWords = 10 * 1024, kTicketWord = 16, kArgmaxTicketWord = 1024;
+    // word kSinkWord: where the read-only pass of lev_hip_prefetch would leave its (discarded) result
+    static constexpr uint32_t kFlagWords = 10 * 1024, kTicketWord = 16, kArgmaxTicketWord = 1024, kSinkWord = 8;
     int *h_flag = nullptr;   // pinned
     // True between lev_hip_program_begin and lev_hip_program_end: the stream
     // is being captured, so nothing may allocate or synchronise.
