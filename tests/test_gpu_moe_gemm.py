@@ -479,6 +479,15 @@ def test_q6_gemm_token_tiles_taken_in_turn(ctx):
         assert np.array_equal(part.view(np.uint32), got[lo:hi].view(np.uint32)), (lo, hi)
     ref = O.q6_k_gemm_f16_oracle(w, rows, cols, x.view(np.uint16), tokens, 0, 97)
     assert O.max_rel_err(got[:, 0::97], ref) < GEMM_TOL
+    # two token tiles side by side, four in turn (100 row tiles x 8 token tiles on 256 CUs)
+    rows, cols, tokens = 12800, 1024, 2000
+    w, x = config4_q6(rows, cols, tokens, seed=17)
+    got = gemm6(ctx, w, x, rows, cols, tokens)
+    for lo, hi in ((0, 256), (768, 1024), (1792, 2000)):
+        part = gemm6(ctx, w, x[lo:hi].copy(), rows, cols, hi - lo)
+        assert np.array_equal(part.view(np.uint32), got[lo:hi].view(np.uint32)), (lo, hi)
+    ref = O.q6_k_gemm_f16_oracle(w, rows, cols, x.view(np.uint16), tokens, 0, 211)
+    assert O.max_rel_err(got[:, 0::211], ref) < GEMM_TOL
 
 
 def test_q6_gemm_one_token_matches_the_gemv_within_rounding(ctx):
