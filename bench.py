@@ -305,32 +305,6 @@ def main():
             run_other("empty_kernel_launch", lambda i: must(lib.lev_hip_empty_launch(c)), 0, 1000, 100)
             del buf
 
-        # ---------------------------- the headline GEMV behind a prefetch of its weights
-        if want("q4_0", "prefetch"):
-            # Step i reads copy i + 1 with lev_hip_prefetch (a cold read-only pass: the bytes land in the
-            # memory-side cache) and multiplies copy i, which step i - 1 prefetched.  On one stream the
-            # two run one after the other, so the pair costs more than the cold GEMV alone; the second
-            # entry times the prefetch passes by themselves, and the difference is what the GEMV takes
-            # once something else has brought its weights into the cache.
-            torch.cuda.empty_cache()
-            ncopy_p = 64
-            ring_p = make_q4_0(ncopy_p * rows * cols // 32)
-            xp_ = torch.randn(cols, device=dev, generator=gen)
-            yp_ = torch.empty(rows, device=dev)
-
-            def pf(i):
-                must(lib.lev_hip_prefetch(c, ring_p.data_ptr() + ((i + 1) % ncopy_p) * q4_bytes_w, q4_bytes_w))
-
-            def pf_gemv(i):
-                pf(i)
-                must(lib.lev_hip_q4_0_gemv(c, ring_p.data_ptr(), ring_p.numel(), (i % ncopy_p) * q4_bytes_w,
-                                           xp_.data_ptr(), cols, yp_.data_ptr(), rows, cols, rows))
-            run_other("prefetch_9MiB_rotating", pf, q4_bytes_w, 2000, 100)
-            run_other("prefetch_then_q4_0_gemv_4096x4096", pf_gemv, q4_alg_bytes, 2000, 100)
-            pair, alone = others["prefetch_then_q4_0_gemv_4096x4096"], others["prefetch_9MiB_rotating"]
-            pair["gemv_on_prefetched_weights_us"] = pair["us_per_launch"] - alone["us_per_launch"]
-            del ring_p
-
         # ---------------------------------------------- Q4_0 large streaming
         if want("q4_0"):
             torch.cuda.empty_cache()   # every family starts from fresh allocations, as when it runs alone

@@ -132,16 +132,6 @@ int lev_hip_stream_read_probe(lev_ctx *ctx, const void *d_src, size_t bytes, uin
 /* Enqueues a kernel that does nothing: the launch-to-launch floor. */
 int lev_hip_empty_launch(lev_ctx *ctx);
 
-/* ---- warming the memory-side cache ----
- * No counterpart in the reference (its Metal and Vulkan backends have no such call).  Enqueues one
- * read-only pass over [d_mem, d_mem + bytes) on the context's stream, so that an operator that
- * follows finds those bytes in the 256 MB memory-side cache instead of in HBM (a 9 MiB weight
- * matrix is then read in 1.9 us instead of 3.1).  Nothing is written; any alignment; can be
- * recorded into a program one operator ahead of the operator that needs the bytes.  On one stream
- * the pass and the operators run one after the other: it pays where something else has to run
- * between the pass and the use anyway. */
-int lev_hip_prefetch(lev_ctx *ctx, const void *d_mem, size_t bytes);
-
 /* ---- dequantise (decodeBlock, Q4.swift:54; Q6.swift:23; dequant_block_f32,
  * lev-cpu/src/lib.rs:111): nblocks blocks of `type` -> f32, bit-exact ---- */
 int lev_hip_dequant(lev_ctx *ctx, int type, const void *d_w, size_t w_bytes, uint64_t w_off,
@@ -180,7 +170,11 @@ int lev_hip_q4_k_gemv_ncol(lev_ctx *ctx, const void *d_w, size_t w_bytes, uint64
  * with the same optional RMSNorm in front (d_gain == NULL skips it).  Same layouts as
  * lev_hip_q4_k_gemv_ncol: x is [ncol][in_dim], y[col*rows + row].  Sums are formed
  * without rounding, so a column's result does not depend on ncol.  Weights 2-byte
- * aligned (GGUF), x and gain 16-byte aligned, in_dim a multiple of 256. */
+ * aligned (GGUF), x and gain 16-byte aligned, in_dim a multiple of 256 and no wider
+ * than the activation staging of the matrix-core kernel holds in LDS (16384 on MI355X,
+ * never beyond 32768): wider rows are
+ * refused with LEV_ERR_EXCEEDS_MODEL_WORKLOAD and nothing is launched; lev_hip_q6_k_gemv
+ * takes them a column at a time. */
 int lev_hip_q6_k_gemv_ncol(lev_ctx *ctx, const void *d_w, size_t w_bytes, uint64_t w_off,
                            const float *d_x, size_t x_count, const float *d_gain, float eps,
                            float *d_y, size_t y_capacity, uint32_t in_dim, uint32_t rows,

@@ -82,7 +82,6 @@ SIGNATURES = {
     "lev_hip_buf_download": (_int, [_vp, _vp, _vp, _sz]),
     "lev_hip_stream_read_probe": (_int, [_vp, _vp, _sz, _vp, _u32]),
     "lev_hip_empty_launch": (_int, [_vp]),
-    "lev_hip_prefetch": (_int, [_vp, _vp, _sz]),
     "lev_hip_dequant": (_int, [_vp, _int, _vp, _sz, _u64, _u64, _vp, _sz]),
     "lev_hip_q4_0_gemv": (_int, [_vp, _vp, _sz, _u64, _vp, _sz, _vp, _sz, _u32, _u32]),
     "lev_hip_q6_k_gemv": (_int, [_vp, _vp, _sz, _u64, _vp, _sz, _vp, _sz, _u32, _u32, _vp, _vp]),

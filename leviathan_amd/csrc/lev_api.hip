@@ -389,26 +389,6 @@ extern "C" int lev_hip_stream_read_probe(lev_ctx *ctx, const void *d_src, size_t
     return lev_hip_check(ctx, hipGetLastError(), "probe launch");
 }
 
-extern "C" int lev_hip_prefetch(lev_ctx *ctx, const void *d_mem, size_t bytes) {
-    LEV_REQUIRE_CTX(ctx);
-    if (!d_mem || bytes == 0) return lev_fail(ctx, LEV_ERR_INVALID_ARGUMENT, "prefetch: nothing to read");
-    // whole 16-byte units inside the range (the cache works in lines: the edges come with them)
-    const uintptr_t lo = (reinterpret_cast<uintptr_t>(d_mem) + 15u) & ~(uintptr_t)15u;
-    const uintptr_t hi = (reinterpret_cast<uintptr_t>(d_mem) + bytes) & ~(uintptr_t)15u;
-    if (hi <= lo) return LEV_OK;
-    const uint64_t n16 = (uint64_t)(hi - lo) / 16u;
-    // four loads per thread in flight; at most eight workgroups per CU
-    uint64_t wgs = (n16 + 1023u) / 1024u;
-    const uint64_t cap = (uint64_t)ctx->num_cus * 8u;
-    if (wgs > cap) wgs = cap;
-    // the kernel's sink is a word of the flag block that nothing else reads (it is written only
-    // if the xor of everything read equals one particular value)
-    uint32_t *sink = reinterpret_cast<uint32_t *>(ctx->d_flag) + lev_ctx::kSinkWord;
-    hipLaunchKernelGGL(stream_read_kernel, dim3((uint32_t)wgs), dim3(256), 0, ctx->stream,
-                       reinterpret_cast<const lev_u32x4 *>(lo), n16, sink);
-    return lev_hip_check(ctx, hipGetLastError(), "prefetch launch");
-}
-
 extern "C" int lev_hip_empty_launch(lev_ctx *ctx) {
     LEV_REQUIRE_CTX(ctx);
     hipLaunchKernelGGL(empty_kernel, dim3(1), dim3(64), 0, ctx->stream);

@@ -47,8 +47,7 @@ struct lev_ctx {
     int *d_flag = nullptr;
     // words kArgmaxTicketWord + 1024*k, k = 0..8: arrival counters of the greedy-token merge
     // (4 KB apart: counters that share a cache line serialise in one L2 channel), zero between launches
-    // word kSinkWord: where the read-only pass of lev_hip_prefetch would leave its (discarded) result
-    static constexpr uint32_t kFlagWords = 10 * 1024, kTicketWord = 16, kArgmaxTicketWord = 1024, kSinkWord = 8;
+    static constexpr uint32_t kFlagWords = 10 * 1024, kTicketWord = 16, kArgmaxTicketWord = 1024;
     int *h_flag = nullptr;   // pinned
     // True between lev_hip_program_begin and lev_hip_program_end: the stream
     // is being captured, so nothing may allocate or synchronise.
@@ -182,6 +181,26 @@ __device__ __forceinline__ float lev_wave_sum_broadcast(float v) {
 __device__ __forceinline__ void lev_barrier_lds() {
     __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0); vmcnt and expcnt left open
     asm volatile("s_barrier" ::: "memory");
+}
+
+// Hand-over of a few words from one workgroup to whichever workgroup arrives last at a
+// counter, WITHOUT a release fence (on this chip a device-scope release writes back every
+// dirty line of the XCD's L2, the kernel's own outputs included).  The order is kept by three
+// properties of gfx942 / gfx950 hardware, not by the HIP memory model, so the code that uses
+// it is compiled for these targets only:
+//   1. a relaxed agent-scope atomic store is a store with sc1 set: it is written through the
+//      XCD's L2 to memory, and its completion is counted in vmcnt;
+//   2. `s_waitcnt vmcnt(0)` therefore returns only once those stores have reached memory; the
+//      relaxed agent-scope fetch_add that follows is issued after it (the asm statement is a
+//      compiler barrier for memory operations as well);
+//   3. a relaxed agent-scope atomic load is a load with sc1 set: it is served from memory, not
+//      from a line the reader's own L2 may still hold.
+// The last arriver sees the final count only after every other workgroup's stores completed.
+#if defined(__HIP_DEVICE_COMPILE__) && !defined(__gfx950__) && !defined(__gfx942__)
+#error "lev_publish_wait relies on gfx942/gfx950 store completion (vmcnt) and sc1 write-through semantics"
+#endif
+__device__ __forceinline__ void lev_publish_wait() {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
 // Overflow-safe tanh and gelu_tanh(g)*u exactly as the reference kernels

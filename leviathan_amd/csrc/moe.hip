@@ -572,13 +572,13 @@ moe_scores_select_kernel(const float *__restrict__ wr, const float *__restrict__
         if (lane < 8u && eo < experts)
             __hip_atomic_store(&scores[(uint64_t)t * experts + eo], s_score[lane], __ATOMIC_RELAXED,
                                __HIP_MEMORY_SCOPE_AGENT);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        lev_publish_wait();
         if (lane == 0)
             s_ticket = __hip_atomic_fetch_add(&tickets[t], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads();
     if (s_ticket != gridDim.x - 1u) return;
-    if (tid == 0) tickets[t] = 0u;
+    if (tid == 0) __hip_atomic_store(&tickets[t], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     // the other workgroups' scores are read with device-scope loads below
     float sc[J];
 #pragma unroll

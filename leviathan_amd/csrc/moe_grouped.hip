@@ -176,6 +176,8 @@ moe_group_kernel(const int32_t *__restrict__ ids, uint32_t pairs, uint32_t exper
             if (e < experts) s_cur[e] = run;
             run += c4[k];
         }
+        // 4096 experts: the total has no thread of its own (thread i owns 4i..4i+3 <= 4095)
+        if (4u * tid + 4u == experts && experts == 4096u) goff[experts] = run;
     }
     __syncthreads();
     // The order of an expert's pairs in the list depends on the atomics; no

@@ -537,7 +537,7 @@ q6_k_mfma_gemv(const uint8_t *__restrict__ w, const float *__restrict__ x, const
             __hip_atomic_store(pf, m.best, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             __hip_atomic_store(pf + 1, m.second, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             __hip_atomic_store(pf + 2, __builtin_bit_cast(float, m.idx), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            lev_publish_wait();
             const uint32_t grp = blockIdx.x & 7u, ngrp = gridDim.x < 8u ? gridDim.x : 8u;
             const uint32_t in_grp = (gridDim.x - grp + 7u) >> 3;
             if (__hip_atomic_fetch_add(&tickets[(1u + grp) * 1024u], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ==
@@ -775,8 +775,13 @@ size_t q6m_lds_bytes(uint32_t cols, uint32_t nc, uint32_t pb) {
 // Waves per row group.  The busiest workgroup runs ceil(rounds / grid) rounds of SB/S tasks:
 // the smallest S that makes that product smallest (fewer partial sums to add up).
 uint32_t q6m_waves_per_group(const lev_ctx *ctx, uint32_t cols, uint32_t rows) {
-    static const char *env = getenv("LEV_Q6_MFMA_WAVES");
-    if (env && atoi(env) > 1) return (uint32_t)atoi(env);
+    // LEV_Q6_MFMA_WAVES (experiments): only the values the kernel is built for; anything else is ignored
+    static const int forced = [] {
+        const char *env = getenv("LEV_Q6_MFMA_WAVES");
+        const int v = env ? atoi(env) : 0;
+        return v == 2 || v == 4 || v == 8 || v == 16 ? v : 0;
+    }();
+    if (forced) return (uint32_t)forced;
     const uint32_t SB = cols >> 8, ngroups = (rows + 15u) / 16u, cus = (uint32_t)ctx->num_cus;
     uint32_t best = 2, best_cost = 0xFFFFFFFFu;
     for (uint32_t s = 2; s <= (uint32_t)kQWaves; s <<= 1) {   // even: a wave's superblocks share their parity

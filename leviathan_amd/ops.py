@@ -76,14 +76,6 @@ class Context:
     def sync(self):
         self._check(self.lib.lev_hip_sync(self.ctx))
 
-    def prefetch(self, t, offset: int = 0, nbytes: int | None = None):
-        """One read-only pass over a byte range of a device tensor: warms the memory-side cache."""
-        total = t.numel() * t.element_size()
-        nbytes = total - offset if nbytes is None else nbytes
-        if offset < 0 or nbytes < 0 or offset + nbytes > total:
-            raise ValueError("prefetch: range outside the tensor")
-        self._check(self.lib.lev_hip_prefetch(self.ctx, t.data_ptr() + offset, nbytes))
-
     def device_name(self) -> str:
         buf = C.create_string_buffer(256)
         self._check(self.lib.lev_hip_device_name(self.ctx, buf, 256))

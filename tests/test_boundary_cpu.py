@@ -99,3 +99,35 @@ def test_product_code_never_touches_the_oracle():
                 text = open(os.path.join(dirpath, f)).read()
                 assert "lev_oracle" not in text and "import oracle" not in text \
                     and "from oracle" not in text, os.path.join(dirpath, f)
+
+
+def test_grouped_moe_offset_scan_writes_every_entry():
+    """The per-expert offsets of the grouped MoE path (moe_group_kernel): 1024 threads,
+    thread i owns experts 4i..4i+3 and writes goff[e] for e <= experts from its running
+    sum; at 4096 experts the total goff[4096] lies past the last thread's share and is
+    written by the thread that owns expert 4095.  Restated on the host for every expert
+    count: each of the experts+1 entries is written exactly once and equals the
+    exclusive prefix sum."""
+    import numpy as np
+    rng = np.random.default_rng(7)
+    for experts in list(range(1, 70)) + [255, 256, 257, 300, 1023, 1024, 1500, 4092, 4093, 4094, 4095, 4096]:
+        cnt = rng.integers(0, 5, experts)
+        goff = np.full(experts + 1, -1, np.int64)
+        writes = np.zeros(experts + 1, np.int64)
+        padded = np.zeros(4096, np.int64)
+        padded[:experts] = cnt
+        local = padded.reshape(1024, 4).sum(axis=1)
+        before = np.concatenate([[0], np.cumsum(local)[:-1]])            # what the shuffle scan leaves per thread
+        for tid in range(1024):
+            run = before[tid]
+            for k in range(4):
+                e = 4 * tid + k
+                if e <= experts:
+                    goff[e] = run
+                    writes[e] += 1
+                run += padded[e]
+            if 4 * tid + 4 == experts and experts == 4096:
+                goff[experts] = run
+                writes[experts] += 1
+        assert np.all(writes == 1), experts
+        assert np.array_equal(goff, np.concatenate([[0], np.cumsum(cnt)])), experts

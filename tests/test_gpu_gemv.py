@@ -376,6 +376,22 @@ def test_q6_k_ncol_many_rounds_per_workgroup(ctx, rows, cols, ncol):
         assert O.max_rel_err(got[c], O.q6_k_matvec_f64(w, rows, cols, x[c])) < TOL, c
 
 
+def test_q6_k_ncol_refuses_rows_wider_than_its_staging(ctx):
+    """in_dim beyond what the matrix-core kernel stages is refused before any launch
+    (exceedsModelWorkload); the single-column entry still serves the shape."""
+    from leviathan_amd import capi
+    from leviathan_amd.ops import LevError
+    rows, cols = 16, 40960
+    w = O.synth_q6_k(77, rows * cols // 256)
+    x = O.normal(2 * cols, 78).reshape(2, cols)
+    with pytest.raises(LevError) as e:
+        q6k_ncol(ctx, w, x, rows, cols, 2)
+    assert e.value.status == capi.EXCEEDS_MODEL_WORKLOAD
+    y = ctx.q6_k_gemv(dev(w), dev(x[0]), cols, rows)
+    ctx.sync()
+    assert O.max_rel_err(y.cpu().numpy(), O.q6_k_matvec_f64(w, rows, cols, x[0])) < TOL
+
+
 def test_q6_k_ncol_exact_sums_columns_and_scale(ctx):
     """Nothing is rounded before the end: a column's bits do not depend on how many columns
     travel with it, and scaling x by a power of two scales every output by exactly that power."""

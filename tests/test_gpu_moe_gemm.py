@@ -298,6 +298,30 @@ def test_moe_experts_vs_fp64(ctx, hidden, inter, experts, top_k, tokens):
         assert O.max_rel_err(y[t], ref["y"]) <= max(TOL / 2, 1.5 * O.max_rel_err(y32, ref["y"]))
 
 
+@pytest.mark.parametrize("experts", [300, 1500, 4096])
+def test_moe_grouped_path_many_experts(ctx, experts):
+    """Five tokens and up group the pairs by expert: the per-expert offsets are an
+    exclusive scan over up to 4096 counts, cut into four experts per thread and
+    sixteen waves.  Expert counts beyond one wave's 256, beyond several waves and
+    at the 4096 limit (whose total is the one entry past the last thread's share),
+    with the last expert and experts of every wave routed."""
+    hidden, inter, top_k, tokens = 256, 256, 4, 6
+    wr, pool, offs, x = H.config5(hidden, inter, experts, tokens, seed=experts)
+    rng = np.random.default_rng(experts)
+    ids = np.stack([rng.permutation(experts)[:top_k] for _ in range(tokens)]).astype(np.int32)
+    ids[0, 0], ids[1, 1], ids[2, 2] = experts - 1, 0, experts // 2
+    ids[3] = [experts - 1, experts - 2, 1, experts // 3]            # the last expert twice in the batch
+    for t in range(tokens):
+        assert len(set(ids[t].tolist())) == top_k
+    wts = rng.random((tokens, top_k)).astype(np.float32)
+    y, act = run_experts(ctx, pool, offs, hidden, inter, experts, x, ids, wts)
+    g, u, d = (pool[offs["gate_off"]:], pool[offs["up_off"]:], pool[offs["down_off"]:])
+    for t in range(tokens):
+        ref = O.moe_experts_f64(g, u, d, hidden, inter, ids[t], wts[t], x[t])
+        assert O.max_rel_err(act[t], ref["act"]) < TOL
+        assert O.max_rel_err(y[t], ref["y"]) < TOL
+
+
 def test_moe_rejects_bad_expert_ids(ctx):
     """MoEModelBinding.offsets (MoEModelBinding.swift:174-214): ids must be in
     range and distinct; nothing is written through a bad id."""

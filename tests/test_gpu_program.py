@@ -341,44 +341,3 @@ def test_shared_expert_ffn_recorded_program_matches_the_cpu_chain():
     with pytest.raises(ops.LevError):
         ctx.shared_expert_ffn(x, dfn, dgate, dup, ddown, dpn, hidden, 2112 - 32, bufs=bufs)   # up half unaligned
     ctx.close()
-
-
-def test_prefetch_reads_only_and_records():
-    """lev_hip_prefetch: a read-only pass over a byte range (any alignment, any length), eager or
-    recorded one operator ahead; it changes no byte, raises no flag, and the operator behind it
-    gives the bits it gives without it."""
-    from leviathan_amd import capi, ops
-    stream = torch.cuda.Stream()
-    ctx = ops.Context(0, stream=stream)
-    rows, cols = 64, 2048
-    copies = [O.synth_q4_0(30 + i, rows * cols // 32) for i in range(3)]
-    nb = copies[0].size
-    with torch.cuda.stream(stream):
-        ring = dev(np.concatenate(copies))
-        before = ring.clone()
-        x = dev(O.seeded_input(cols, 1, 9))
-        y = torch.empty(3, rows, device="cuda")
-        plain = [ctx.q4_0_gemv(ring, x, cols, rows, w_off=i * nb).clone() for i in range(3)]
-        ctx.sync()
-        # ranges of every alignment and size, also shorter than one 16-byte unit
-        for off, n in ((0, nb), (1, nb - 2), (7, 3), (nb, nb), (5, 16), (16, 15), (3 * nb - 1, 1)):
-            ctx.prefetch(ring, off, n)
-        ctx.sync()
-        assert torch.equal(ring, before)
-        ctx.program_begin()
-        for i in range(3):
-            ctx.prefetch(ring, ((i + 1) % 3) * nb, nb)        # the next operator's weights
-            ctx.q4_0_gemv(ring, x, cols, rows, y=y[i], w_off=i * nb)
-        prog = ctx.program_end()
-        for _ in range(3):
-            y.fill_(float("nan"))
-            prog.run()
-            ctx.sync()
-            for i in range(3):
-                assert torch.equal(y[i], plain[i]), i
-        assert torch.equal(ring, before)
-    for bad in ((None, 16), (ring.data_ptr(), 0)):
-        st = ctx.lib.lev_hip_prefetch(ctx.ctx, bad[0], bad[1])
-        assert st == capi.INVALID_ARGUMENT
-    with pytest.raises(ValueError):
-        ctx.prefetch(ring, 1, ring.numel())

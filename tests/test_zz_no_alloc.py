@@ -71,3 +71,64 @@ def test_noalloc_matches_allocating_entry_point_twice_in_a_row():
         ctx.sync()
     finally:
         ctx.close()
+
+
+def test_noalloc_first_call_on_a_fresh_context_allocates_nothing_and_records():
+    """The call is the FIRST thing a fresh context runs (its grow-on-demand scratch is still
+    empty): device free memory is the same before and after; it can be recorded into a
+    program on a context that never ran the shape, where the allocating entry point is
+    refused (exceedsWorkingSet: scratch cannot grow under capture); every replay gives
+    the bits of the allocating entry point."""
+    from leviathan_amd import capi, ops
+    hidden, inter, experts, top_k, tokens = 2048, 768, 128, 8, 2
+    wr, pool, offs, x = H.config5(hidden, inter, experts, tokens, seed=78)
+    pool_d, wr_d, x_d = dev(pool), dev(wr), dev(x)
+    pools = ops.Context.moe_pools(pool_d, hidden, inter, experts, offs["gate_off"], offs["up_off"], offs["down_off"])
+
+    def outputs():
+        return (torch.full((tokens, hidden), float("nan"), device="cuda"),
+                torch.full((tokens, top_k), -1, dtype=torch.int32, device="cuda"),
+                torch.full((tokens, top_k), float("nan"), device="cuda"))
+
+    ctx = ops.Context(0)
+    try:
+        y1, i1, w1 = outputs()
+        torch.cuda.synchronize()
+        free_before = torch.cuda.mem_get_info()[0]
+        ctx.moe_layer_q4_0(pools, wr_d, x_d, top_k, tokens, y=y1, ids=i1, weights=w1, noalloc=True)
+        ctx.sync()
+        assert torch.cuda.mem_get_info()[0] == free_before
+        first = (y1.cpu().numpy(), i1.cpu().numpy(), w1.cpu().numpy())
+        assert np.all(np.isfinite(first[0]))
+    finally:
+        ctx.close()
+
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        ctx = ops.Context(0, stream=stream)
+        try:
+            y2, i2, w2 = outputs()
+            torch.cuda.synchronize()
+            ctx.program_begin()
+            with pytest.raises(ops.LevError) as e:      # its scratch would have to be allocated under capture
+                ctx.moe_layer_q4_0(pools, wr_d, x_d, top_k, tokens, y=y2, ids=i2, weights=w2)
+            assert e.value.status == capi.EXCEEDS_WORKING_SET
+            ctx.moe_layer_q4_0(pools, wr_d, x_d, top_k, tokens, y=y2, ids=i2, weights=w2, noalloc=True)
+            prog = ctx.program_end()
+            for _ in range(3):
+                y2.fill_(float("nan"))
+                torch.cuda.synchronize()
+                prog.run()
+                ctx.sync()
+                assert np.array_equal(y2.cpu().numpy().view(np.uint32), first[0].view(np.uint32))
+                assert np.array_equal(i2.cpu().numpy(), first[1])
+                assert np.array_equal(w2.cpu().numpy().view(np.uint32), first[2].view(np.uint32))
+            prog.destroy()
+            # the allocating entry point outside a recording: the same bits
+            y3, i3, w3 = outputs()
+            ctx.moe_layer_q4_0(pools, wr_d, x_d, top_k, tokens, y=y3, ids=i3, weights=w3)
+            ctx.sync()
+            assert np.array_equal(y3.cpu().numpy().view(np.uint32), first[0].view(np.uint32))
+            assert np.array_equal(i3.cpu().numpy(), first[1])
+        finally:
+            ctx.close()
