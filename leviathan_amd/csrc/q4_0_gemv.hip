@@ -13,7 +13,7 @@
 //   - all R x 9 dword loads of a wave are issued before the first use, so a
 //     wave keeps R*2304 bytes in flight;
 //   - the L partial sums of a row are combined with DPP adds.
-#include "q4_0_device.hpp"
+#include "q4_0_mfma.hpp"
 
 namespace {
 
@@ -269,10 +269,25 @@ hipError_t launch_pairs(lev_ctx *ctx, const uint8_t *w, const float *x, float *y
 
 }  // namespace
 
+bool lev_q4_0_mfma_gemv_usable(const uint8_t *w, const float *x, uint32_t in_dim);
+hipError_t lev_q4_0_mfma_gemv_launch(lev_ctx *ctx, const uint8_t *w, const float *x, float *y, uint32_t in_dim,
+                                     uint32_t rows, int persistent);
+
 // Enqueue without argument checks (callers validated the geometry).
 hipError_t lev_q4_0_gemv_launch(lev_ctx *ctx, const uint8_t *w, const float *x, float *y,
                                 uint32_t in_dim, uint32_t rows) {
     const uint32_t nb = in_dim / 32u;
+    {
+        // a schedule installed for this shape (lev_hip_forge_select) overrides the built-in choice
+        const lev_schedule *sel = lev_selected(ctx, LEV_OP_Q4_0_GEMV, in_dim, rows, 1);
+        static const int env_mfma = [] {
+            const char *e = getenv("LEV_Q4_MFMA");   // experiments: 0 = vector-ALU kernels, 1 = matrix-core kernel
+            return e ? atoi(e) : -1;
+        }();
+        const bool usable = lev_q4_0_mfma_gemv_usable(w, x, in_dim);
+        if (usable && (sel ? sel->family == 1u : env_mfma != 0))
+            return lev_q4_0_mfma_gemv_launch(ctx, w, x, y, in_dim, rows, sel ? (int)sel->persistent : -1);
+    }
     const bool pairable = (nb % 2u == 0u) && ((reinterpret_cast<uintptr_t>(w) & 3u) == 0u) &&
                           (in_dim <= 32768u) && ((reinterpret_cast<uintptr_t>(x) & 15u) == 0u);
     if (!pairable) {
@@ -321,15 +336,24 @@ uint32_t lev_q4_0_gemv_candidates(const lev_ctx *ctx, uint32_t in_dim, uint32_t 
         const uint32_t rows_per_tile = kWaves * (LEV_WAVE / lanes) * r;
         return (rows + rows_per_tile - 1) / rows_per_tile > (uint32_t)ctx->num_cus * 4u ? 1u : 0u;
     };
-    lev_schedule all[8];
+    lev_schedule all[12];
     uint32_t n = 0;
     auto push = [&](uint32_t r, uint32_t p) {
         for (uint32_t i = 0; i < n; ++i)
-            if (all[i].rows_in_flight == r && all[i].persistent == p) return;
+            if (all[i].family == 0u && all[i].rows_in_flight == r && all[i].persistent == p) return;
         all[n++] = lev_schedule{LEV_OP_Q4_0_GEMV, 0u, r, p};
     };
+    // rows of whole 256-value tasks: the matrix-core kernel (family 1), the built-in choice, with
+    // one workgroup per round of row groups or a resident grid
+    if (in_dim % 256u == 0u && in_dim <= kLevQ4MfmaMaxInDim) {
+        const uint32_t ntask = in_dim >> 8, slots = ntask <= 16u ? 16u / ntask : 1u;
+        const uint32_t nrounds = ((rows + 15u) / 16u + slots - 1u) / slots;
+        const uint32_t builtin = nrounds <= (uint32_t)ctx->num_cus ? 0u : 1u;
+        all[n++] = lev_schedule{LEV_OP_Q4_0_GEMV, 1u, 0u, builtin};
+        all[n++] = lev_schedule{LEV_OP_Q4_0_GEMV, 1u, 0u, 1u - builtin};
+    }
     if (!family) {
-        push(0u, 0u);   // the built-in choice, which has no parameters here
+        push(0u, 0u);   // the vector-ALU kernel of the shape, which has no parameters here
     } else {
         push(base_r, is_persistent(base_r));
         for (uint32_t r : {1u, 2u, 4u})

@@ -672,8 +672,10 @@ void forge_matvec(Runner &r) {
         // (two waves, one wave a row), f64-sum kernel
         EXPECT(!q6 || rep.candidates.size() == (sh.cols == 4096 ? 6u : 4u));
         EXPECT(!q6 || rep.candidates[0].schedule.family == 2u);
-        EXPECT(!q40 || sh.cols < 1024 || rep.candidates.size() == 6);      // 3 depths x 2 grids, baseline first
-        EXPECT(!q40 || sh.cols >= 1024 || rep.candidates.size() == 1);     // narrow rows: the built-in choice only
+        // matrix-core kernel (two grids) first, then the vector-ALU kernels: 3 depths x 2 grids, or one for narrow rows
+        EXPECT(!q40 || sh.cols < 1024 || rep.candidates.size() == 8);
+        EXPECT(!q40 || sh.cols >= 1024 || rep.candidates.size() == 3);
+        EXPECT(!q40 || rep.candidates[0].schedule.family == 1u);
         for (const ForgeCandidate &c : rep.candidates) {
             EXPECT(c.pass);
             EXPECT(c.maxRelErr >= 0 && c.maxRelErr < 1e-4);
@@ -765,7 +767,7 @@ void forge_matvec(Runner &r) {
     uint32_t n = 0;
     EXPECT(lev_hip_forge_candidates(ctx, LEV_OP_Q4_K_GEMV, 100, 8, 1, nullptr, 0, &n) == LEV_ERR_BAD_DIMENSIONS);
     EXPECT(lev_hip_forge_candidates(ctx, LEV_OP_Q4_0_GEMV, 4096, 8, 2, nullptr, 0, &n) == LEV_ERR_BAD_DIMENSIONS);
-    EXPECT(lev_hip_forge_candidates(ctx, LEV_OP_Q4_0_GEMV, 4096, 512, 1, nullptr, 0, &n) == LEV_OK && n == 6);
+    EXPECT(lev_hip_forge_candidates(ctx, LEV_OP_Q4_0_GEMV, 4096, 512, 1, nullptr, 0, &n) == LEV_OK && n == 8);
 }
 
 // MoELoweringForge.forge (MoELowering.swift:1896-1985) on the test model's layer 0

@@ -31,8 +31,8 @@ def dev(a):
     return torch.from_numpy(np.ascontiguousarray(a)).cuda()
 
 
-@pytest.mark.parametrize("rows,cols,expected", [(4096, 4096, 6), (300, 2048, 6), (40000, 4096, 6),
-                                                (512, 1088, 6), (64, 256, 1), (16, 8192, 1)])
+@pytest.mark.parametrize("rows,cols,expected", [(4096, 4096, 8), (300, 2048, 8), (40000, 4096, 8),
+                                                (512, 1088, 6), (64, 256, 3), (16, 8192, 3), (16, 16384, 1)])
 def test_q4_0_candidates_pass_the_gate_and_agree_bitwise(ctx, rows, cols, expected):
     from leviathan_amd import capi
     w = O.synth_q4_0(rows + cols, rows * cols // 32, 0.02)
@@ -42,9 +42,14 @@ def test_q4_0_candidates_pass_the_gate_and_agree_bitwise(ctx, rows, cols, expect
     cands = ctx.forge_candidates(capi.OP_Q4_0_GEMV, cols, rows)
     assert len(cands) == expected
     assert len({c.key() for c in cands}) == len(cands)
+    # rows of whole 256-value tasks up to 8192 wide: the matrix-core kernel (family 1) first, with one
+    # workgroup per round of row groups or a resident grid; behind it the vector-ALU kernels (family 0)
+    mfma = cols % 256 == 0 and cols <= 8192
+    assert [c.family for c in cands[:2]] == ([1, 1] if mfma else [0, 0][:len(cands)])
     builtin = ctx.q4_0_gemv(dw, dx, cols, rows).cpu().numpy()
     ctx.sync()
     assert O.max_rel_err(builtin, ref) < GATE
+    outs = {}
     try:
         for i, s in enumerate(cands):
             ctx.forge_select(cols, rows, s)
@@ -53,10 +58,14 @@ def test_q4_0_candidates_pass_the_gate_and_agree_bitwise(ctx, rows, cols, expect
             ctx.sync()
             got = y.cpu().numpy()
             assert O.max_rel_err(got, ref) < GATE, s.key()
-            # a row is summed by the same lanes in the same order whatever the tiling
-            assert np.array_equal(got.view(np.uint32), builtin.view(np.uint32)), s.key()
+            # within a family a row is summed by the same lanes in the same order whatever the tiling
+            first = outs.setdefault(s.family, got)
+            assert np.array_equal(got.view(np.uint32), first.view(np.uint32)), s.key()
     finally:
         ctx.forge_clear(capi.OP_Q4_0_GEMV, cols, rows)
+    assert np.array_equal(builtin.view(np.uint32), outs[cands[0].family].view(np.uint32))
+    if len(outs) > 1:   # two different kernels: a selection really switches
+        assert not np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
 
 
 @pytest.mark.parametrize("rows,cols,ncol", [(1024, 4096, 1), (512, 1024, 3), (96, 256, 8), (256, 4096, 16)])

@@ -376,6 +376,46 @@ def test_q6_k_ncol_many_rounds_per_workgroup(ctx, rows, cols, ncol):
         assert O.max_rel_err(got[c], O.q6_k_matvec_f64(w, rows, cols, x[c])) < TOL, c
 
 
+@pytest.mark.parametrize("rows,cols", [(16, 256), (5, 256), (100, 768), (33, 1280), (257, 2048), (48, 3072),
+                                       (4096 + 7, 4096), (64, 5120), (40, 8192), (9000, 512), (5000, 4096)])
+def test_q4_0_matrix_core_kernel_shapes(ctx, rows, cols):
+    """Rows of whole 256-value tasks up to 8192 wide run on the integer matrix cores: 1 to 32 tasks
+    a row (one or two a wave; 16 / tasks row groups a round when a row has fewer than 16), row
+    counts that are no multiple of 16, grids of one round per workgroup and resident grids that
+    walk many rounds.  Gate: the reference's 1e-4 against the FP64 oracle; the integer sums are
+    exact, so the error stays near f32 rounding."""
+    w = O.synth_q4_0(rows * 3 + cols, rows * cols // 32, 0.02)
+    x = O.normal(cols, rows + cols)
+    y = torch.full((rows,), float("nan"), device="cuda")
+    ctx.q4_0_gemv(dev(w), dev(x), cols, rows, y=y)
+    ctx.sync()
+    err = O.max_rel_err(y.cpu().numpy(), O.q4_0_matvec_f64(w, rows, cols, x))
+    assert err < 2e-5, err
+
+
+def test_q4_0_matrix_core_kernel_scale_and_non_finite(ctx):
+    """Activations are scaled per pair of blocks by a power of two: scaling x by 2^k scales every
+    output by exactly 2^k; pairs of very different magnitude keep their own scale; a NaN or an
+    infinity anywhere in x makes every output NaN (every row multiplies every activation)."""
+    rows, cols = 64, 2048
+    w = O.synth_q4_0(5, rows * cols // 32, 0.02)
+    x = O.normal(cols, 6)
+    base = ctx.q4_0_gemv(dev(w), dev(x), cols, rows).cpu().numpy()
+    for e in (-40, -9, 13, 60):
+        got = ctx.q4_0_gemv(dev(w), dev(np.ldexp(x, e).astype(np.float32)), cols, rows).cpu().numpy()
+        assert np.array_equal(bits(got), bits(np.ldexp(base, e).astype(np.float32))), e
+    x2 = x.copy()
+    x2[64:128] *= 1e-7
+    x2[1024:1088] *= 3e5
+    got = ctx.q4_0_gemv(dev(w), dev(x2), cols, rows).cpu().numpy()
+    assert O.max_rel_err(got, O.q4_0_matvec_f64(w, rows, cols, x2)) < 2e-5
+    for bad in (np.nan, np.inf, -np.inf):
+        x3 = x.copy()
+        x3[777] = bad
+        got = ctx.q4_0_gemv(dev(w), dev(x3), cols, rows).cpu().numpy()
+        assert np.all(np.isnan(got)), bad
+
+
 def test_q6_k_ncol_refuses_rows_wider_than_its_staging(ctx):
     """in_dim beyond what the matrix-core kernel stages is refused before any launch
     (exceedsModelWorkload); the single-column entry still serves the shape."""
