@@ -353,18 +353,20 @@ int lev_hip_q6_k_matvec_reporting(const uint8_t *blocks, size_t blocks_count, in
 #define LEV_OP_MOE_LAYER_Q4_0 6u
 typedef struct lev_schedule {
     uint32_t op;             /* LEV_OP_* */
-    uint32_t family;         /* Q4_K: 1 = matrix-core kernel, 0 = vector-ALU (int8: dot4) kernel; Q4_0: 0;
+    uint32_t family;         /* Q4_K: 1 = matrix-core kernel, 0 = vector-ALU (int8: dot4) kernel; Q4_0: 1 = integer
+                                matrix-core kernel (rows of whole 256-value tasks up to 8192 wide), 0 = vector-ALU kernels;
                                 Q6_K: 2 = integer matrix-core kernel, 0 = digit-plane dot4 kernel (both exact),
                                 1 = one wave per row with f64 sums;
                                 Q6_K x int8: 1 = integer matrix-core kernel, 0 = dot4 kernel; MoE layer: who selects the experts: 1 = the gate/up workgroups
                                 themselves, 2 = the last workgroup of the router kernel to finish, 0 = a top-k
                                 kernel of its own ahead of them */
-    uint32_t rows_in_flight; /* Q4_0: rows a wave keeps in flight (1, 2, 4; 0 = no variants for the shape);
+    uint32_t rows_in_flight; /* Q4_0 family 0: rows a wave keeps in flight (1, 2, 4; 0 = no variants for the shape);
                                 Q6_K: waves that share a row (family 0: 1, 2) or a group of 16 rows (family 2:
                                 2, 4, 8, 16); Q6_K x int8: columns per pass over the
                                 weights; MoE layer: gate/up workgroups aimed at per CU (1, 2, 4) */
     uint32_t persistent;     /* Q4_0, Q6_K x int8: 0 = one workgroup per row tile, 1 = resident grid walking
-                                the tiles */
+                                the tiles; MoE layer: 0 = expert kernels on the integer matrix cores where the
+                                shape allows, 1 = vector-ALU expert kernels */
 } lev_schedule;
 /* Writes min(*count, capacity) candidates; *count is the full number. */
 int lev_hip_forge_candidates(lev_ctx *ctx, uint32_t op, uint32_t in_dim, uint32_t rows,

@@ -18,7 +18,7 @@
 //      workgroup's tile of outputs; partial results meet in LDS and are merged
 //      IN SLOT ORDER in f32, as the reference's axpy chain does.
 #include "moe_grouped.hpp"
-#include "q4_0_device.hpp"
+#include "q4_0_mfma.hpp"
 
 namespace {
 
@@ -315,6 +315,103 @@ __device__ router_sel router_select_regs(const float (&sc)[J], void *lds, uint32
     }
     lev_barrier_lds();
     return out;
+}
+
+// The same selection run by ONE wave with no exchange at all, for kernels in which a single
+// wave ranks the scores while the others of the workgroup do something else: the wave holds all
+// scores (lane l keeps experts j*64 + l) and extracts minima of the integer keys round by round
+// (see router_select_regs).  all == false: returns the expert of `slot` after slot + 1 rounds.
+// all == true: lists the top_k winners and their probabilities in sel_id / sel_p (LDS, the layout
+// of router_select_regs) and returns the expert of `slot`.
+// Returns kRouteNotFinite when a score is not finite, kRouteNeedsBlock when the integer keys do
+// not order the probabilities (exp saturating or running into denormals): the caller then runs
+// the workgroup-wide selection.
+constexpr uint32_t kRouteNotFinite = 0xFFFFFFFFu, kRouteNeedsBlock = 0xFFFFFFFEu;
+
+template <int J>
+__device__ uint32_t router_select_wave(const float (&sc)[J], void *lds, uint32_t experts, uint32_t top_k,
+                                       uint32_t slot, bool all) {
+    constexpr uint32_t padded = 64u * J;
+    uint64_t *table = static_cast<uint64_t *>(lds);
+    double *sel_p = reinterpret_cast<double *>(table + padded);
+    uint32_t *rank = reinterpret_cast<uint32_t *>(sel_p + 64);
+    uint32_t *sel_id = rank + padded;
+    const uint32_t lane = threadIdx.x & 63u;
+    float mx = -INFINITY;
+    bool finite = true;
+#pragma unroll
+    for (int j = 0; j < J; ++j) {
+        finite = finite && isfinite(sc[j]);
+        mx = fmaxf(mx, sc[j]);
+    }
+    mx = wave_max_f32(mx);
+    if (__any(!finite)) return kRouteNotFinite;
+    uint32_t dk[J];
+    bool plain = true;
+#pragma unroll
+    for (int j = 0; j < J; ++j) {
+        const bool valid = lane + 64u * j < experts;
+        const float d = sc[j] - mx;
+        plain = plain && (!valid || d == 0.f || (d <= -1e-6f && d >= -690.f));
+        dk[j] = valid ? __float_as_uint(d) & 0x7FFFFFFFu : 0xFFFFFFFFu;
+    }
+    if (__any(!plain)) return kRouteNeedsBlock;
+    double p[J];
+    if (all) {
+        double sum = 0.0;
+#pragma unroll
+        for (int j = 0; j < J; ++j) {
+            const bool valid = lane + 64u * j < experts;
+            p[j] = valid ? exp((double)(sc[j] - mx)) : 0.0;   // subtraction in f32, exp in f64
+            sum += p[j];
+        }
+        sum = wave_sum_f64(sum);
+#pragma unroll
+        for (int j = 0; j < J; ++j) p[j] = lane + 64u * j < experts ? p[j] / sum : 0.0;
+    }
+    const uint32_t rounds = all ? top_k : slot + 1u;
+    uint32_t mine = 0xFFFFFFFFu;
+    for (uint32_t rnd = 0; rnd < rounds; ++rnd) {
+        uint32_t m = dk[0];
+#pragma unroll
+        for (int j = 1; j < J; ++j) m = dk[j] < m ? dk[j] : m;
+#define LEV_MOE_MINSTEP(CTRL, ROWS)                                                                \
+        {                                                                                          \
+            const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp((int)m, (int)m, CTRL, ROWS, 0xF, false); \
+            m = o < m ? o : m;                                                                     \
+        }
+        LEV_MOE_MINSTEP(0xB1, 0xF)
+        LEV_MOE_MINSTEP(0x4E, 0xF)
+        LEV_MOE_MINSTEP(0x141, 0xF)
+        LEV_MOE_MINSTEP(0x140, 0xF)
+        LEV_MOE_MINSTEP(0x142, 0xA)
+        LEV_MOE_MINSTEP(0x143, 0xC)
+#undef LEV_MOE_MINSTEP
+        const uint32_t best = (uint32_t)__builtin_amdgcn_readlane((int)m, 63);
+        uint32_t wl = 0, wj = 0;
+        bool seen = false;
+#pragma unroll
+        for (int j = 0; j < J; ++j) {   // ascending j, lowest lane: the lowest index among equals
+            const unsigned long long hit = __ballot(dk[j] == best);
+            if (!seen && hit != 0ull) {
+                wl = (uint32_t)__builtin_ctzll(hit);
+                wj = (uint32_t)j;
+                seen = true;
+            }
+        }
+        const uint32_t found = wl + 64u * wj;
+        if (rnd == slot) mine = found;
+#pragma unroll
+        for (int j = 0; j < J; ++j) {
+            const bool here = lane == wl && wj == (uint32_t)j;
+            if (all && here) {
+                sel_id[rnd] = found;
+                sel_p[rnd] = p[j];
+            }
+            dk[j] = here ? 0xFFFFFFFFu : dk[j];
+        }
+    }
+    return mine;
 }
 
 // Renormalised weight of selection slot k (Gemma4.swift:3808-3810): the sum
@@ -888,6 +985,262 @@ moe_down_kernel(moe_args a, const float *__restrict__ act, const int32_t *__rest
 }
 
 // ---------------------------------------------------------------------------
+// gate/up and down on the integer matrix cores (q4_0_mfma.hpp), up to four tokens.
+// A task is 16 rows x 256 activations; a wave stages the activations of its own tasks in LDS of
+// its own (no workgroup barrier in front of the products) and keeps the operands in registers.
+// ---------------------------------------------------------------------------
+
+constexpr int kMmWaves = 8;
+constexpr int kMmThreads = kMmWaves * LEV_WAVE;
+constexpr uint32_t kGumPartBytes = 2u * 2u * kMmWaves * 16u * 4u;   // [round parity][gate, up][wave][row] f32
+
+__host__ __device__ constexpr size_t mm_areas_bytes(uint32_t tpw) {
+    return (size_t)kMmWaves * (tpw * kQ4mTaskArea + kQ4mZeroBytes);
+}
+
+// grid (chunks, top_k, tokens), 8 waves.  Wave w multiplies the column tasks w*TPW.. of gate row
+// group i AND of up row group i (the same operands); the eight partial sums of a row meet in LDS
+// and wave 0 writes act = gelu_tanh(g) * u.  A workgroup takes rows_per_block rows in groups of 16
+// with the next group's weights in flight.
+// ROUTE > 0 (experts <= 64*ROUTE): the expert comes from this token's router scores, ranked by
+// wave 0 alone while the other waves' activation requests are on their way (every workgroup of a
+// token repeats the selection, which costs less than a kernel boundary; one wave ranking costs an
+// eighth of the vector instructions of eight); the first workgroup of a token publishes ids and
+// weights.  Otherwise the ids are read from `ids`.
+// LDS: part | expert word | task areas | router area (ROUTE > 0)
+template <int TPW, int ROUTE>
+__global__ void __launch_bounds__(kMmThreads)
+moe_gate_up_mfma(moe_args a, const float *__restrict__ x, const int32_t *ids, const float *__restrict__ scores,
+                 const float *__restrict__ expert_scale, int32_t *ids_out, float *weights_out,
+                 float *__restrict__ act, int *__restrict__ flag, uint32_t rows_per_block) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    const uint32_t slot = blockIdx.y, t = blockIdx.z;
+    const uint32_t ntask = a.hidden >> 8;
+    const uint32_t t_first = wave * TPW;
+    const float *xt = x + (uint64_t)t * a.hidden;
+
+    // request order = return order: the scores (the expert, and with it every weight address,
+    // hangs on them) first, the activations behind them
+    float sc[ROUTE > 0 ? ROUTE : 1];
+    if constexpr (ROUTE > 0) {
+        if (wave == 0u) router_load_scores<ROUTE>(scores + (uint64_t)t * a.experts, a.experts, sc);
+    }
+    lev_f32x4 v[TPW];
+#pragma unroll
+    for (int k = 0; k < TPW; ++k) {
+        const uint32_t T = t_first + k < ntask ? t_first + k : ntask - 1u;
+        v[k] = reinterpret_cast<const lev_f32x4 *>(xt)[64u * T + lane];
+    }
+
+    uint32_t *s_e = reinterpret_cast<uint32_t *>(smem + kGumPartBytes);
+    uint8_t *area = smem + kGumPartBytes + 16u + (size_t)wave * (TPW * kQ4mTaskArea + kQ4mZeroBytes);
+    uint8_t *zero = area + TPW * kQ4mTaskArea;
+    void *rl = smem + kGumPartBytes + 16u + mm_areas_bytes(TPW);
+    uint32_t e;
+    bool ok = true;
+    const bool publisher = ROUTE > 0 && blockIdx.x == 0 && slot == 0;
+    if constexpr (ROUTE > 0) {
+        // (all eight waves ranking a share of the keys each was measured as well: the layer takes 0.5 us
+        // longer, the 16 waves of a CU then queue for its four vector pipelines)
+        if (wave == 0u) {
+            const uint32_t got = router_select_wave<ROUTE>(sc, rl, a.experts, a.top_k, slot, publisher);
+            if (lane == 0u) s_e[0] = got;
+        }
+        lev_barrier_lds();
+        e = s_e[0];
+        if (e == kRouteNeedsBlock) {   // workgroup-uniform and rare: the workgroup ranks the probabilities together
+            const router_sel r = router_select_block<ROUTE>(scores + (uint64_t)t * a.experts, rl, a.experts,
+                                                            a.top_k, publisher);
+            e = r.ok ? r.sel_id[slot] : kRouteNotFinite;
+        }
+        ok = e != kRouteNotFinite;
+        if (!ok) e = slot;
+    } else {
+        const int32_t *tids = ids + (uint64_t)t * a.top_k;
+        if (!expert_ids_ok(tids, a.top_k, slot, a.experts, &e)) {
+            if (tid == 0) atomicOr(flag, kFlagBadExpertId);
+            return;
+        }
+    }
+    e = (uint32_t)__builtin_amdgcn_readfirstlane((int)e);
+    const uint64_t row_bytes = (uint64_t)(a.hidden >> 6) * 36u;
+    const uint8_t *gbase = a.base + a.gate_off + e * a.gate_stride;
+    const uint8_t *ubase = a.base + a.up_off + e * a.up_stride;
+    const uint32_t i_begin = blockIdx.x * rows_per_block;
+    const uint32_t i_end = min(i_begin + rows_per_block, a.inter);
+    const uint32_t lrow = lane >> 2;                              // fetch order: lane = 4 * row + pair
+    auto issue = [&](uint32_t i0, uint32_t (&Dg)[TPW][9], uint32_t (&Du)[TPW][9]) {
+        uint32_t row = i0 + lrow;
+        row = row < i_end ? row : i_end - 1u;
+        const uint64_t off = (uint64_t)row * row_bytes;
+#pragma unroll
+        for (int k = 0; k < TPW; ++k) {
+            const uint32_t T = t_first + k < ntask ? t_first + k : ntask - 1u;
+            q4m_load_task(gbase + off, 4u * T, Dg[k]);
+            q4m_load_task(ubase + off, 4u * T, Du[k]);
+        }
+    };
+    uint32_t Ga[TPW][9], Ua[TPW][9];
+    uint32_t i0 = i_begin;
+    issue(i0, Ga, Ua);
+
+    // ---- while the weights are on their way ----
+    if constexpr (ROUTE > 0) {
+        if (publisher) {
+            constexpr uint32_t padded = 64u * ROUTE;
+            uint64_t *table = static_cast<uint64_t *>(rl);
+            double *sel_p = reinterpret_cast<double *>(table + padded);
+            uint32_t *sel_id = reinterpret_cast<uint32_t *>(sel_p + 64) + padded;
+            const router_sel r{sel_p, sel_id, ok, 0xFFFFFFFFu};
+            if (!ok && tid == 0) atomicOr(flag, kFlagNonFiniteScore);
+            if (tid < a.top_k) {
+                ids_out[(uint64_t)t * a.top_k + tid] = ok ? (int32_t)sel_id[tid] : (int32_t)tid;
+                weights_out[(uint64_t)t * a.top_k + tid] = ok ? router_weight(r, expert_scale, a.top_k, tid) : 0.f;
+            }
+        }
+    }
+    const uint32_t r16 = lane & 15u, q = lane >> 4;
+    uint32_t pw = (wave * 16u + lane) * 4u;                       // byte offsets into `part`: gate, then up at + 512
+    uint32_t pr = (q * 16u + r16) * 4u;                           // wave 0: lane (r, q) adds waves q and q + 4
+    float *arow = act + ((uint64_t)t * a.top_k + slot) * a.inter;
+    q4m_pin(pw);
+    q4m_pin(pr);
+    if (lane < kQ4mZeroBytes / 4u) reinterpret_cast<uint32_t *>(zero)[lane] = 0u;
+    q4m_operand op[TPW];
+#pragma unroll
+    for (int k = 0; k < TPW; ++k) q4m_stage_task(v[k], area + k * kQ4mTaskArea, zero, t_first + k < ntask, op[k]);
+    __builtin_amdgcn_sched_barrier(0);
+
+    auto finish = [&](uint32_t i_here, const uint32_t (&Dg)[TPW][9], const uint32_t (&Du)[TPW][9]) {
+        float vg = 0.f, vu = 0.f;
+#pragma unroll
+        for (int k = 0; k < TPW; ++k) {
+            uint32_t W[9];
+            q4m_turn_task(Dg[k], W);
+            vg += q4m_task_dot(W, op[k]);
+            q4m_turn_task(Du[k], W);
+            vu += q4m_task_dot(W, op[k]);
+        }
+        vg = q4m_row_sum(vg);
+        vu = q4m_row_sum(vu);
+        if (lane < 16u) {
+            *reinterpret_cast<float *>(smem + pw) = vg;
+            *reinterpret_cast<float *>(smem + pw + kMmWaves * 16u * 4u) = vu;
+        }
+        lev_barrier_lds();
+        if (wave == 0u) {
+            const float *pp = reinterpret_cast<const float *>(smem + pr);
+            const float g0 = pp[0], g1 = pp[64], u0 = pp[128], u1 = pp[192];
+            const float g = q4m_row_sum(g0 + g1), u = q4m_row_sum(u0 + u1);
+            if (q == 0u && i_here + r16 < i_end) arow[i_here + r16] = lev_gelu_up_value(g, u);
+        }
+        pw ^= kGumPartBytes / 2u;                                 // the other half of `part` next round
+        pr ^= kGumPartBytes / 2u;
+    };
+    if (rows_per_block <= 16u) {   // one group per workgroup: nothing to prefetch
+        finish(i0, Ga, Ua);
+        return;
+    }
+    // unconditional (clamped) prefetch: a branch around the loads would make the compiler wait
+    // for them before the current group is multiplied
+    uint32_t Gb[TPW][9], Ub[TPW][9];
+    while (true) {
+        uint32_t next = i0 + 16u;
+        issue(next < i_end ? next : i0, Gb, Ub);
+        finish(i0, Ga, Ua);
+        if (next >= i_end) break;
+        i0 = next;
+        next = i0 + 16u;
+        issue(next < i_end ? next : i0, Ga, Ua);
+        finish(i0, Gb, Ub);
+        if (next >= i_end) break;
+        i0 = next;
+    }
+}
+
+// grid (row tiles of `tile` <= 16 rows, tokens), 8 waves.  Wave s takes slots s, s + 8, ...: the
+// whole reduction (TPW tasks, inter <= 256*TPW) of the tile's rows against the slot's activations,
+// which it stages for itself; the per-slot results meet in LDS and are merged IN SLOT ORDER in
+// f32, as the reference's axpy chain does.
+// LDS: partial [top_k][16] f32 | w_slot [64] f32 | task areas
+template <int TPW>
+__global__ void __launch_bounds__(kMmThreads)
+moe_down_mfma(moe_args a, const float *__restrict__ act, const int32_t *__restrict__ ids,
+              const float *__restrict__ weights, float *__restrict__ y, int *__restrict__ flag, uint32_t tile) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    const uint32_t t = blockIdx.y;
+    const uint32_t ntask = a.inter >> 8;
+    const uint32_t row_begin = blockIdx.x * tile;
+    const uint32_t row_end = min(row_begin + tile, a.hidden);
+    float *partial = reinterpret_cast<float *>(smem);                       // [top_k][16]
+    float *w_slot = partial + a.top_k * 16u;
+    uint8_t *area = smem + (size_t)a.top_k * 64u + 256u + (size_t)wave * (TPW * kQ4mTaskArea + kQ4mZeroBytes);
+    uint8_t *zero = area + TPW * kQ4mTaskArea;
+    const int32_t *tids = ids + (uint64_t)t * a.top_k;
+    const uint64_t row_bytes = (uint64_t)(a.inter >> 6) * 36u;
+    // the routing weights are requested now and parked in LDS for the merge at the end
+    const float w_mine = weights[(uint64_t)t * a.top_k + (lane < a.top_k ? lane : a.top_k - 1u)];
+    if (lane < kQ4mZeroBytes / 4u) reinterpret_cast<uint32_t *>(zero)[lane] = 0u;
+    uint32_t lr = row_begin + (lane >> 2);                                   // fetch order: lane = 4 * row + pair
+    lr = lr < row_end ? lr : row_end - 1u;
+
+    bool bad = false;
+    for (uint32_t slot = wave; slot < a.top_k; slot += kMmWaves) {
+        // request order = return order: the ids (the weight addresses hang on them) first, then
+        // this slot's activations
+        const int32_t ids_mine = expert_ids_request(tids, a.top_k);
+        const float *av = act + ((uint64_t)t * a.top_k + slot) * a.inter;
+        lev_f32x4 v[TPW];
+#pragma unroll
+        for (int k = 0; k < TPW; ++k) {
+            const uint32_t T = (uint32_t)k < ntask ? (uint32_t)k : ntask - 1u;
+            v[k] = reinterpret_cast<const lev_f32x4 *>(av)[64u * T + lane];
+        }
+        uint32_t e;
+        if (!expert_ids_verdict(ids_mine, a.top_k, slot, a.experts, &e)) {
+            bad = true;
+            if (lane < 16u) partial[slot * 16u + lane] = 0.f;
+            continue;
+        }
+        e = (uint32_t)__builtin_amdgcn_readfirstlane((int)e);
+        const uint8_t *rowp = a.base + a.down_off + e * a.down_stride + (uint64_t)lr * row_bytes;
+        uint32_t D[TPW][9];
+#pragma unroll
+        for (int k = 0; k < TPW; ++k) {
+            const uint32_t T = (uint32_t)k < ntask ? (uint32_t)k : ntask - 1u;
+            q4m_load_task(rowp, 4u * T, D[k]);
+        }
+        // the slot's activations become operands while its weights are on their way
+        q4m_operand op[TPW];
+#pragma unroll
+        for (int k = 0; k < TPW; ++k) q4m_stage_task(v[k], area + k * kQ4mTaskArea, zero, (uint32_t)k < ntask, op[k]);
+        __builtin_amdgcn_sched_barrier(0);
+        float val = 0.f;
+#pragma unroll
+        for (int k = 0; k < TPW; ++k) {
+            uint32_t W[9];
+            q4m_turn_task(D[k], W);
+            val += q4m_task_dot(W, op[k]);
+        }
+        val = q4m_row_sum(val);
+        if (lane < 16u) partial[slot * 16u + lane] = val;
+    }
+    if (bad && lane == 0) atomicOr(flag, kFlagBadExpertId);
+    if (wave == 0u && lane < a.top_k) w_slot[lane] = w_mine;
+    lev_barrier_lds();
+    // ordered merge: y = sum over slots, in slot order, of w_slot * dn[slot]
+    if (tid < 16u && row_begin + tid < row_end) {
+        float accum = 0.f;
+        for (uint32_t slot = 0; slot < a.top_k; ++slot) accum = fmaf(w_slot[slot], partial[slot * 16u + tid], accum);
+        y[(uint64_t)t * a.hidden + row_begin + tid] = accum;
+    }
+}
+
+// ---------------------------------------------------------------------------
 // generic expert path (odd block counts, unaligned pools, very long rows):
 // one wave per output row, 16-bit loads, activations through the cache.
 // ---------------------------------------------------------------------------
@@ -1033,6 +1386,61 @@ hipError_t launch_down(lev_ctx *ctx, const moe_args &a, const float *act, const 
     return hipGetLastError();
 }
 
+// Shapes the matrix-core expert kernels take: rows of whole 256-value tasks, at most two tasks a
+// wave for gate/up (the hidden dimension is split over the eight waves), at most four for down
+// (a wave reduces over the whole intermediate dimension).
+bool gate_up_mfma_ok(const moe_args &a) { return a.hidden % 256u == 0u && a.hidden <= 4096u; }
+bool down_mfma_ok(const moe_args &a) { return a.inter % 256u == 0u && a.inter <= 1024u; }
+
+hipError_t launch_gate_up_mfma(lev_ctx *ctx, const moe_args &a, const float *x, const gu_route &rt,
+                               float *act, uint32_t tokens, uint32_t per_cu) {
+    const uint64_t slots = (uint64_t)a.top_k * tokens;
+    uint32_t want = (uint32_t)(((uint64_t)ctx->num_cus * per_cu + slots - 1) / slots);
+    if (want < 1) want = 1;
+    const uint32_t rows_per_block = (a.inter + want - 1) / want;
+    const uint32_t chunks = (a.inter + rows_per_block - 1) / rows_per_block;
+    const uint32_t tpw = a.hidden > 2048u ? 2u : 1u;
+    const uint32_t route = rt.ids ? 0u : a.experts <= 128u ? 2u : 4u;      // callers keep experts <= kRouteInKernelMax
+    const size_t lds = kGumPartBytes + 16u + mm_areas_bytes(tpw) + (route ? router_lds_bytes(route) + 8u : 0u);
+    const dim3 grid(chunks, a.top_k, tokens);
+#define LEV_GUM(TPW, ROUTE)                                                                          \
+    hipLaunchKernelGGL((moe_gate_up_mfma<TPW, ROUTE>), grid, dim3(kMmThreads), lds, ctx->stream, a, x, rt.ids,   \
+                       rt.scores, rt.expert_scale, rt.ids_out, rt.weights_out, act, ctx->d_flag, rows_per_block)
+    if (tpw == 1u) {
+        if (route == 0u) LEV_GUM(1, 0);
+        else if (route == 2u) LEV_GUM(1, 2);
+        else LEV_GUM(1, 4);
+    } else {
+        if (route == 0u) LEV_GUM(2, 0);
+        else if (route == 2u) LEV_GUM(2, 2);
+        else LEV_GUM(2, 4);
+    }
+#undef LEV_GUM
+    return hipGetLastError();
+}
+
+hipError_t launch_down_mfma(lev_ctx *ctx, const moe_args &a, const float *act, const int32_t *ids,
+                            const float *weights, float *y, uint32_t tokens) {
+    // one workgroup per CU at one token; a tile is at most the 16 rows of a task
+    uint32_t want_tiles = (uint32_t)(((uint64_t)ctx->num_cus + tokens - 1) / tokens);
+    if (want_tiles < 1) want_tiles = 1;
+    uint32_t tile = (a.hidden + want_tiles - 1) / want_tiles;
+    tile = tile < 4u ? 4u : tile > 16u ? 16u : tile;
+    const uint32_t tiles = (a.hidden + tile - 1) / tile;
+    const uint32_t tpw = (a.inter + 255u) / 256u;
+    const size_t lds = (size_t)a.top_k * 64u + 256u + mm_areas_bytes(tpw);
+    const dim3 grid(tiles, tokens);
+#define LEV_DNM(TPW)                                                                                 \
+    hipLaunchKernelGGL((moe_down_mfma<TPW>), grid, dim3(kMmThreads), lds, ctx->stream, a, act, ids, weights, y, \
+                       ctx->d_flag, tile)
+    if (tpw == 1u) LEV_DNM(1);
+    else if (tpw == 2u) LEV_DNM(2);
+    else if (tpw == 3u) LEV_DNM(3);
+    else LEV_DNM(4);
+#undef LEV_DNM
+    return hipGetLastError();
+}
+
 int check_pools(lev_ctx *ctx, const lev_moe_experts *p, uint32_t top_k, uint32_t tokens,
                 moe_args *out) {
     if (!p || !p->d_base) return lev_fail(ctx, LEV_ERR_INVALID_ARGUMENT, "moe: null pools");
@@ -1085,7 +1493,7 @@ bool experts_fast(const moe_args &a, const float *x) {
 // fast path: callers test experts_fast() first.
 hipError_t run_experts(lev_ctx *ctx, const moe_args &a, const float *x, const gu_route &rt,
                        const int32_t *ids, const float *weights, float *y, float *act,
-                       uint32_t tokens, bool fast, uint32_t gu_per_cu = 2u) {
+                       uint32_t tokens, bool fast, uint32_t gu_per_cu = 2u, bool matrix_cores = true) {
     hipError_t e;
     if (!fast) {
         hipLaunchKernelGGL(moe_gate_up_generic, dim3((a.inter + 3) / 4, a.top_k, tokens), dim3(256), 0,
@@ -1098,9 +1506,16 @@ hipError_t run_experts(lev_ctx *ctx, const moe_args &a, const float *x, const gu
     // One row pair per wave and step: what a wave does after its last byte has
     // landed is issued at one instruction per eight cycles whatever else runs
     // on the SIMD, so many short waves finish sooner than few long ones.
-    if (a.hidden <= 2048u) e = launch_gate_up<1, 1, 1>(ctx, a, x, rt, act, tokens, gu_per_cu);
+    static const bool env_mfma = [] {
+        const char *v = getenv("LEV_MOE_MFMA");   // LEV_MOE_MFMA=0: the vector-ALU expert kernels, for comparison
+        return !(v && v[0] == '0');
+    }();
+    const bool mfma = matrix_cores && env_mfma;
+    if (mfma && gate_up_mfma_ok(a)) e = launch_gate_up_mfma(ctx, a, x, rt, act, tokens, gu_per_cu);
+    else if (a.hidden <= 2048u) e = launch_gate_up<1, 1, 1>(ctx, a, x, rt, act, tokens, gu_per_cu);
     else e = launch_gate_up<2, 1, 2>(ctx, a, x, rt, act, tokens, gu_per_cu);
     if (e != hipSuccess) return e;
+    if (mfma && down_mfma_ok(a)) return launch_down_mfma(ctx, a, act, ids, weights, y, tokens);
     const uint32_t dp = a.inter / 64u;
     if (dp > 32) return launch_down<64>(ctx, a, act, ids, weights, y, tokens);
     if (dp > 16) return launch_down<32>(ctx, a, act, ids, weights, y, tokens);
@@ -1314,6 +1729,7 @@ int moe_layer_impl(lev_ctx *ctx, const lev_moe_experts *pools, const float *d_ro
                                            : nullptr;
     const uint32_t family = sel ? sel->family : 1u;
     const uint32_t gu_per_cu = sel && sel->rows_in_flight ? sel->rows_in_flight : 2u;
+    const bool matrix_cores = !(sel && sel->persistent);   // schedule field `persistent` = 1: the vector-ALU expert kernels
     const bool few = fast && tokens <= 4u && a.experts <= kRouteInKernelMax;
     if (few && family == 2u) {
         // few tokens: the router kernel's last workgroup selects the experts
@@ -1346,7 +1762,7 @@ int moe_layer_impl(lev_ctx *ctx, const lev_moe_experts *pools, const float *d_ro
                                                     d_y, s.act, s.grouped),
                              "moe grouped experts launch");
     return lev_hip_check(ctx,
-                         run_experts(ctx, a, d_x, rt, d_ids, d_weights, d_y, s.act, tokens, fast, gu_per_cu),
+                         run_experts(ctx, a, d_x, rt, d_ids, d_weights, d_y, s.act, tokens, fast, gu_per_cu, matrix_cores),
                          "moe experts launch");
 }
 
@@ -1378,6 +1794,10 @@ uint32_t lev_moe_layer_candidates(const lev_ctx *ctx, uint32_t hidden, uint32_t 
     add(1u, 4u);
     add(2u, 2u);
     add(0u, 2u);
+    // the expert kernels on the vector ALU (f32 FMA chains) instead of the integer matrix cores, the
+    // built-in choice wherever rows are whole 256-value tasks: same routing, sums rounded differently
+    if (n < capacity) out[n] = lev_schedule{LEV_OP_MOE_LAYER_Q4_0, 1u, 2u, 1u};
+    ++n;
     return n;
 }
 

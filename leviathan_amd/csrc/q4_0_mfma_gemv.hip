@@ -24,15 +24,6 @@ __host__ __device__ constexpr size_t q4m_gemv_lds(uint32_t tpw) {
     return 2u * kQ4mWaves * 16u * 4u + (size_t)kQ4mWaves * (tpw * kQ4mTaskArea + kQ4mZeroBytes);
 }
 
-// Keeps a value that the tail of a round needs (an LDS address, an output pointer) computed where
-// it is written: between the load requests and the first wait, where instructions cost nothing.
-// Left to itself the compiler sinks such arithmetic to its use, behind the barrier, where every
-// instruction is on the critical path of the launch.
-template <typename T>
-__device__ __forceinline__ void q4m_pin(T &v) {
-    asm volatile("" : "+v"(v));
-}
-
 // wave -> (slot, position in the slot) as 4-bit entries of two 64-bit kernel arguments: a division
 // in front of the first load would cost some thirty instructions.
 // SINGLE: the grid covers every round once: straight-line code, nothing to prefetch.

@@ -781,10 +781,10 @@ void forge_moe_layer(Runner &r, const Model &m) {
         opt.timed = 5;
         opt.rotateBytes = 4 << 20;
         ForgeReport rep = MoELayerForge::forge(r, m.bytes, m.binding, router, tokens, opt);
-        EXPECT(rep.op == LEV_OP_MOE_LAYER_Q4_0 && rep.candidates.size() == 5);
+        EXPECT(rep.op == LEV_OP_MOE_LAYER_Q4_0 && rep.candidates.size() == 6);
         EXPECT(rep.candidates[0].schedule.family == 1u && rep.candidates[0].schedule.rows_in_flight == 2u);
         for (const ForgeCandidate &c : rep.candidates) EXPECT(c.pass && c.maxRelErr >= 0 && c.maxRelErr < 1e-4 && c.medianUs > 0);
-        EXPECT(rep.selected >= 0 && rep.selected < 5);
+        EXPECT(rep.selected >= 0 && rep.selected < 6);
         if (rep.selected > 0)
             EXPECT(rep.candidates[(size_t)rep.selected].medianUs < 0.98 * rep.candidates[0].medianUs);
         ForgeOptions strict = opt;

@@ -172,7 +172,8 @@ def test_moe_layer_candidates_pass_the_gate_and_agree_bitwise(ctx, hidden, inter
     dwr, dx = dev(wr), dev(x)
     g, u, d = (pool[offs["gate_off"]:], pool[offs["up_off"]:], pool[offs["down_off"]:])
     cands = ctx.forge_candidates(capi.OP_MOE_LAYER_Q4_0, hidden, inter, tokens)
-    assert [(c.family, c.rows_in_flight) for c in cands] == [(1, 2), (1, 1), (1, 4), (2, 2), (0, 2)]
+    assert [(c.family, c.rows_in_flight, c.persistent) for c in cands] == [(1, 2, 0), (1, 1, 0), (1, 4, 0), (2, 2, 0),
+                                                                           (0, 2, 0), (1, 2, 1)]
     outs = []
     try:
         for s in cands:
@@ -185,8 +186,12 @@ def test_moe_layer_candidates_pass_the_gate_and_agree_bitwise(ctx, hidden, inter
                 ref_ids, ref_w = O.router_topk(scores, top_k, None)
                 H.check_moe_layer_token(outs[-1][0][t], outs[-1][1][t], outs[-1][2][t], ref_ids, ref_w, g, u, d,
                                         hidden, inter, x[t], GATE)
-            for a, b in zip(outs[-1], outs[0]):
-                assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), s.key()
+            # same routing whatever the schedule; the same expert kernels give the same bits; the
+            # vector-ALU kernels (persistent = 1) round their sums differently
+            assert np.array_equal(outs[-1][1], outs[0][1]) and np.array_equal(outs[-1][2].view(np.uint32),
+                                                                              outs[0][2].view(np.uint32))
+            if s.persistent == 0:
+                assert np.array_equal(outs[-1][0].view(np.uint32), outs[0][0].view(np.uint32)), s.key()
     finally:
         ctx.forge_clear(capi.OP_MOE_LAYER_Q4_0, hidden, inter, tokens)
     with pytest.raises(ops.LevError):
