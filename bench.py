@@ -164,6 +164,22 @@ def main():
         if tag is not None:
             eager_ms[tag] = {"host_launched": eager, "program": program, "host_kept_ahead": host_ahead,
                              "used": "program" if use_program else "host_launched"}
+            # spread, as the reference reports its timings (median of 11 samples,
+            # rust/crates/lev-vulkan/src/lib.rs:683-704): the same region eleven more times, each behind
+            # its own cache flush; `ms_per_step` stays the one region above
+            samples = []
+            es = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(11)]
+            for a_ev, b_ev in es:
+                for _ in range(4):
+                    flush_caches()
+                a_ev.record(stream)
+                for i in range(steps):
+                    fn(warmup + i)
+                b_ev.record(stream)
+            torch.cuda.synchronize()
+            samples = sorted(a_ev.elapsed_time(b_ev) / steps for a_ev, b_ev in es)
+            eager_ms[tag]["samples"] = {"n": len(samples), "steps_each": steps, "median_ms": samples[len(samples) // 2],
+                                        "min_ms": samples[0], "max_ms": samples[-1], "launched": "host"}
         return program if use_program else eager
 
     def rand_bytes(n):
@@ -252,6 +268,29 @@ def main():
         result["check"] = check
         del ring
 
+    def cpu_matvec_baseline(label, call, alg_bytes, what):
+        """The reference's CPU GEMV of a configuration on this host's cores: single thread, then
+        the rows split over the cores as Model::matvec does (lev-model/src/lib.rs:184-199); a
+        bounded sample of about 3 s each, as GB/s of the configuration's algorithmic bytes."""
+        ncores = os.cpu_count() or 1
+        threads = min(ncores, 64)
+        out = {}
+        for nthreads, key, budget in ((0, "single_thread", 3.0), (threads, "row_parallel", 3.0)):
+            n, t0 = 0, time.perf_counter()
+            while True:
+                call(nthreads)
+                n += 1
+                dt = time.perf_counter() - t0
+                if dt >= budget:
+                    break
+            out[key] = {"value": alg_bytes * n / dt / 1e9, "unit": "GB/s", "cores": max(nthreads, 1),
+                        "ms_per_gemv": dt / n * 1e3, "sample": f"{n} GEMVs"}
+        out["kind"] = "port"
+        out["what"] = what
+        cpu_others[label] = out
+
+    cpu_others = {}
+
     def run_other(name, fn, alg_bytes, steps, warmup, extra=None):
         ms = timed(fn, steps, warmup)
         entry = {"us_per_launch": ms * 1e3, "algorithmic_bytes": alg_bytes,
@@ -334,6 +373,15 @@ def main():
             run_other("q6_k_gemv_32000x4096_no_argmax", lambda i: must(lib.lev_hip_q6_k_gemv(
                 c, ring6.data_ptr(), ring6.numel(), (i % 6) * nb6 * 210, x.data_ptr(), cols,
                 y6.data_ptr(), r6, cols, r6, None, None)), nb6 * 210 + cols * 4 + r6 * 4, 100, 20)
+            if not args.skip_cpu:
+                import oracle as O                              # cpu_baseline leg only
+                w6h = ring6[:nb6 * 210].cpu().numpy()
+                x6h = x.cpu().numpy()
+                cpu_matvec_baseline("q6_k_gemv_32000x4096", lambda nt: O.q6_k_matvec_f32(w6h, r6, cols, x6h, threads=nt),
+                                    nb6 * 210 + cols * 4 + r6 * 4,
+                                    "C restatement of matvec_q6k_f32 (lev-cpu/src/lib.rs:261-276: dequantise a superblock "
+                                    "to f32, ascending f32 sum), gcc -O3, no FMA contraction, no fast-math")
+                del w6h
             # the head on f32 activations, N columns per weight read
             for n in (2, 4, 8):
                 xn = torch.randn(n, cols, device=dev, generator=gen)
@@ -384,6 +432,18 @@ def main():
                     c, ring4.data_ptr(), ring4.numel(), (i % ncopy4) * nb4 * 144, xn.data_ptr(),
                     xn.numel(), gain.data_ptr(), 1e-6, yn.data_ptr(), yn.numel(), cols, r4, n)),
                     nb4 * 144 + cols * 4 + n * (cols * 4 + r4 * 4), 200, 20)
+            if not args.skip_cpu:
+                import oracle as O                              # cpu_baseline leg only
+                w4h = ring4[:nb4 * 144].cpu().numpy()
+                x4h = torch.randn(cols, generator=torch.Generator().manual_seed(3)).numpy()
+                g4h = gain.cpu().numpy()
+
+                def c3_cpu(nt):
+                    O.q4_k_matvec_f32(w4h, r4, cols, O.rmsnorm(x4h, g4h, 1e-6), threads=nt)
+                cpu_matvec_baseline("rmsnorm_q4_k_gemv_12288x4096_N1", c3_cpu, nb4 * 144 + cols * 4 + cols * 4 + r4 * 4,
+                                    "C restatement of rmsnorm (lev-model/src/lib.rs:110-114) + matvec_q4k_f32 "
+                                    "(lev-cpu/src/lib.rs:158-175), one column, gcc -O3, no FMA contraction, no fast-math")
+                del w4h
             # int8-activation path: RMSNorm+quantise, then the integer-dot GEMV
             # (timed together, as the reference's vk-q8 command times quantize + matvec)
             for n in (1, 2, 4, 8, 16):
@@ -543,6 +603,8 @@ def main():
     moe1 = others.get("moe_layer_q4_0_T1", {})
     if result.get("cpu_baseline") is not None and "cpu_moe" in result:
         result["cpu_baseline"]["moe_layer_T1"] = result["cpu_moe"]
+    if result.get("cpu_baseline") is not None:
+        result["cpu_baseline"].update(cpu_others)
     line = {
         "metric": "Q4 GEMV achieved HBM GB/s (% of 8 TB/s); MoE layer us/token at T=1",
         "value": achieved,
@@ -555,6 +617,7 @@ def main():
         "ms_per_step": result["ms_per_step"],
         "ms_per_step_host_launched": eager_ms.get("q4_0", {}).get("host_launched"),
         "ms_per_step_program": eager_ms.get("q4_0", {}).get("program"),
+        "ms_per_step_samples": eager_ms.get("q4_0", {}).get("samples"),
         "timing": "HIP events on the launch stream around exactly `steps` steps, enqueued behind a read-only "
                   "1 GiB cache flush that is still running when they are enqueued (cold HBM, no host latency "
                   "inside the timed region); `ms_per_step` is the " + str(eager_ms.get("q4_0", {}).get("used")) +
@@ -572,7 +635,7 @@ def main():
                    "in_dim": cols, "out_rows": rows, "algorithmic_bytes_per_step": q4_alg_bytes},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": measured_traffic_bytes(),
-                     "kernel": "q4_0_gemv_tile<64,1,2,true>",
+                     "kernel": "q4_0_mfma_gemv<1,true>",
                      "note": "achieved = 9,469,952 B / mean launch-to-launch time of the timed "
                              "region (HIP events on the launch stream)"},
         "cpu_baseline": result.get("cpu_baseline"),

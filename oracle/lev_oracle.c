@@ -451,23 +451,43 @@ int levo_q6_k_matvec_f64(const uint8_t *w, size_t w_bytes, int64_t out_dim, int6
 }
 
 /* Rust matvec_q6k_f32, lev-cpu lib.rs:261-276 (shape errors :246-259) */
-int levo_q6_k_matvec_f32(const uint8_t *w, size_t w_bytes, int64_t rows, int64_t cols,
-                         const float *x, size_t x_count, float *y) {
-    if (cols == 0 || cols % 256 != 0 || rows < 0) return LEVO_BAD_DIMENSIONS;
-    int64_t row_bytes = cols / 256 * 210, expected;
-    if (mul_overflow_i64(rows, row_bytes, &expected) || (int64_t)w_bytes != expected)
-        return LEVO_BAD_DIMENSIONS;
-    if ((int64_t)x_count != cols) return LEVO_WRONG_INPUT_COUNT;
+static int q6_k_rows_f32(const uint8_t *w, int64_t bpr, const float *x, float *y, int64_t row0, int64_t row1) {
+    const int64_t row_bytes = bpr * 210;
     float tmp[256];
-    for (int64_t r = 0; r < rows; r++) {
+    for (int64_t r = row0; r < row1; r++) {
         float sum = 0.0f;
-        for (int64_t b = 0; b < cols / 256; b++) {
+        for (int64_t b = 0; b < bpr; b++) {
             levo_q6_k_dequant_block_f32(w + r * row_bytes + b * 210, tmp);
             for (int i = 0; i < 256; i++) sum += tmp[i] * x[b * 256 + i];
         }
         y[r] = sum;
     }
     return LEVO_OK;
+}
+
+static int q6_k_check_shape_f32(size_t w_bytes, int64_t rows, int64_t cols, size_t x_count) {
+    if (cols == 0 || cols % 256 != 0 || rows < 0) return LEVO_BAD_DIMENSIONS;
+    int64_t row_bytes = cols / 256 * 210, expected;
+    if (mul_overflow_i64(rows, row_bytes, &expected) || (int64_t)w_bytes != expected)
+        return LEVO_BAD_DIMENSIONS;
+    if ((int64_t)x_count != cols) return LEVO_WRONG_INPUT_COUNT;
+    return LEVO_OK;
+}
+
+int levo_q6_k_matvec_f32(const uint8_t *w, size_t w_bytes, int64_t rows, int64_t cols,
+                         const float *x, size_t x_count, float *y) {
+    int st = q6_k_check_shape_f32(w_bytes, rows, cols, x_count);
+    if (st) return st;
+    return q6_k_rows_f32(w, cols / 256, x, y, 0, rows);
+}
+
+/* the same rows split over threads, as Model::matvec does (lev-model lib.rs:184-199) */
+int levo_q6_k_matvec_f32_mt(const uint8_t *w, size_t w_bytes, int64_t rows, int64_t cols,
+                            const float *x, size_t x_count, float *y, int threads) {
+    int st = q6_k_check_shape_f32(w_bytes, rows, cols, x_count);
+    if (st) return st;
+    if (rows == 0) return LEVO_OK;
+    return run_rows_mt(q6_k_rows_f32, w, cols / 256, x, y, rows, threads);
 }
 
 /* ------------------------------------------------------------------ */

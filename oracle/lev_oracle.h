@@ -112,6 +112,10 @@ int levo_q6_k_matvec_f64(const uint8_t *w, size_t w_bytes, int64_t out_dim,
 /* Rust matvec_q6k_f32: pure f32, ascending. */
 int levo_q6_k_matvec_f32(const uint8_t *w, size_t w_bytes, int64_t out_dim,
                          int64_t in_dim, const float *x, size_t x_count, float *y);
+/* ... with the rows split over `threads` threads (Model::matvec, lev-model lib.rs:184-199). */
+int levo_q6_k_matvec_f32_mt(const uint8_t *w, size_t w_bytes, int64_t out_dim,
+                            int64_t in_dim, const float *x, size_t x_count, float *y,
+                            int threads);
 
 /* ---- Q4_K (rust/crates/lev-cpu/src/lib.rs:62-195, test packer :380-394) ---- */
 void levo_q4_k_unpack_scale_min(int j, const uint8_t *scales12, uint8_t *sc, uint8_t *mn);

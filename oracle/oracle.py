@@ -224,6 +224,7 @@ _q6_ref = _sig("levo_q6_k_matvec_ref", C.c_int, *_mv_args, _f32p)
 _q6_ref_mt = _sig("levo_q6_k_matvec_ref_mt", C.c_int, *_mv_args, _f32p, C.c_int)
 _q6_f64 = _sig("levo_q6_k_matvec_f64", C.c_int, *_mv_args, _f64p)
 _q6_f32 = _sig("levo_q6_k_matvec_f32", C.c_int, *_mv_args, _f32p)
+_q6_f32_mt = _sig("levo_q6_k_matvec_f32_mt", C.c_int, *_mv_args, _f32p, C.c_int)
 
 
 def q6_k_decode_block(block) -> np.ndarray:
@@ -274,7 +275,9 @@ def q6_k_matvec_f64(w, out_dim, in_dim, x) -> np.ndarray:
     return _matvec(_q6_f64, w, out_dim, in_dim, x, np.float64)
 
 
-def q6_k_matvec_f32(w, rows, cols, x) -> np.ndarray:
+def q6_k_matvec_f32(w, rows, cols, x, threads: int = 0) -> np.ndarray:
+    if threads > 0:
+        return _matvec(_q6_f32_mt, w, rows, cols, x, np.float32, threads)
     return _matvec(_q6_f32, w, rows, cols, x, np.float32)
 
 

@@ -281,6 +281,11 @@ def test_q6_k_brute_force():
     assert np.allclose(O.q6_k_matvec_f64(w, rows, cols, x), want, rtol=1e-12, atol=1e-12)
     assert np.array_equal(O.q6_k_matvec_ref(w, rows, cols, x),
                           O.q6_k_matvec_ref(w, rows, cols, x, threads=2))
+    # the Rust f32 GEMV split over threads (Model::matvec, lev-model lib.rs:184-199): a row's sum does not
+    # depend on which thread forms it, and stays within f32 rounding of the dense f64 product
+    f32 = O.q6_k_matvec_f32(w, rows, cols, x)
+    assert np.array_equal(f32, O.q6_k_matvec_f32(w, rows, cols, x, threads=3))
+    assert np.allclose(f32, want, rtol=1e-4, atol=1e-4)
 
 
 # --------------------------------------------------------------------------
