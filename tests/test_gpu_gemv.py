@@ -645,6 +645,29 @@ def test_q4_k_one_and_two_columns_on_long_rows(ctx, rows, cols, ncol):
         assert np.array_equal(bits(alone[0]), bits(plain[1]))
 
 
+@pytest.mark.parametrize("rows,cols", [(50, 3072), (33, 3840), (100, 2048), (11205, 512), (4099, 4096), (16, 768),
+                                       (257, 1280)])
+def test_q4_k_one_column_kernel_shapes(ctx, rows, cols):
+    """One column of at most sixteen superblocks: a wave per superblock column.  Rows of fewer
+    superblocks share a round between several row groups (2048: two, 512: eight), widths that do
+    not divide sixteen leave waves idle (3072, 3840, 768, 1280), tall matrices take many rounds per
+    workgroup; the column is the same bits as the first of two columns through the wider kernel."""
+    w, x, gain = H.config3(rows, cols, 2, seed=rows % 89 + cols // 256)
+    got = q4k_gemv(ctx, w, x[:1], rows, cols, 1, gain)
+    xn = H.rmsnorm_rows(x, gain)
+    assert O.max_rel_err(got[0], O.q4_k_matvec_f64(w, rows, cols, xn[0])) < TOL
+    both = q4k_gemv(ctx, w, x, rows, cols, 2, gain)
+    assert np.array_equal(bits(got[0]), bits(both[0]))
+    plain = q4k_gemv(ctx, w, x[:1], rows, cols, 1)
+    assert O.max_rel_err(plain[0], O.q4_k_matvec_f64(w, rows, cols, x[0])) < TOL
+    for e in (-50, 41):
+        scaled = q4k_gemv(ctx, w, np.ldexp(x[:1], e).astype(np.float32), rows, cols, 1)
+        assert np.array_equal(bits(scaled), bits(np.ldexp(plain, e).astype(np.float32))), e
+    xb = x[:1].copy()
+    xb[0, cols - 3] = np.inf
+    assert np.isnan(q4k_gemv(ctx, w, xb, rows, cols, 1, gain)).all()
+
+
 def test_q4_k_mixed_magnitudes_within_a_row(ctx):
     """Superblocks of very different magnitude in one row: each carries its own power of two."""
     rows, cols = 48, 4096
