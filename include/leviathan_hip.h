@@ -82,7 +82,8 @@ typedef struct lev_evidence {
 
 /* ---- library ---- */
 
-/* ABI version of this header (bumped on any signature change). */
+/* ABI version of this header (bumped on any signature change; 2: without lev_hip_prefetch, Q4_0 GEMV
+ * schedules of family 1, MoE schedules with `persistent`). */
 int lev_hip_abi_version(void);
 const char *lev_hip_status_name(int status);
 

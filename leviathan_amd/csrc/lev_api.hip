@@ -68,7 +68,7 @@ hipError_t lev_zero_async(lev_ctx *ctx, void *d_ptr, size_t bytes) {
     return hipGetLastError();
 }
 
-extern "C" int lev_hip_abi_version(void) { return 1; }
+extern "C" int lev_hip_abi_version(void) { return 2; }
 
 extern "C" const char *lev_hip_status_name(int status) {
     switch (status) {

@@ -44,7 +44,7 @@ def test_ctypes_signatures_cover_the_header():
 def test_library_loads_and_reports_without_a_gpu():
     from leviathan_amd import capi
     lib = capi.load()
-    assert lib.lev_hip_abi_version() == 1
+    assert lib.lev_hip_abi_version() == 2
     assert lib.lev_hip_status_name(0) == b"ok"
     assert lib.lev_hip_status_name(capi.BAD_DIMENSIONS) == b"badDimensions"
     assert lib.lev_hip_status_name(capi.NON_FINITE_SCALE) == b"nonFiniteScale"
