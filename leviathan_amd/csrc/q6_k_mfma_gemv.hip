@@ -43,9 +43,11 @@
 // pieces rotated by 4 per row and a 16-byte skew per instruction keep both sides
 // free of bank conflicts).
 //
-// Workgroup = 16 waves.  S waves share a group of 16 rows (each takes 1/S of the
-// row's superblocks), 16/S row groups per workgroup and round; the partial sums of
-// a round meet in LDS.  A NaN or infinity in a column of x makes every output of
+// Workgroup = 16 waves.  Several columns (q6_k_mfma_gemv): S waves share a group of 16
+// rows (each takes 1/S of the row's superblocks), 16/S row groups per workgroup and
+// round; the digit planes of every column are staged once per workgroup; the partial
+// sums of a round meet in LDS.  One column of at most sixteen superblocks
+// (q6_k_mfma_gemv_one): a wave per superblock column, see there.  A NaN or infinity in a column of x makes every output of
 // that column NaN.
 #include "lev_common.hpp"
 #include "top2.hpp"
@@ -107,8 +109,10 @@ struct q6m_lane {
     uint32_t scoff[2];            // bit offset of scale 2*jb + lh in its dword
     uint32_t at_ql[2], c3_ql[2], at_qh[2], c3_qh[2], at_sc[3], at_d;
 
-    __device__ __forceinline__ q6m_lane(uint8_t *area_all, uint32_t wave, uint32_t lane_, uint32_t odd)
-        : area(area_all + wave * kQAreaBytes), lane(lane_) {
+    // area_all + wave * stride: the wave's turn-round area (kQAreaBytes of it)
+    __device__ __forceinline__ q6m_lane(uint8_t *area_all, uint32_t wave, uint32_t lane_, uint32_t odd,
+                                        uint32_t stride = kQAreaBytes)
+        : area(area_all + wave * stride), lane(lane_) {
         const uint32_t r = lane & 15u, g = lane >> 4, hf = g >> 1, jb = g & 1u;
         maskq = jb ? 0xCCCCCCCCu : 0x33333333u;   // the bit pairs jb and jb+2 of a qh byte
         rot[0] = 26u + 2u * jb;
@@ -205,6 +209,88 @@ struct q6m_lds {
                (size_t)pb * kQWaves * 16u * NC * 8u + (size_t)NC * 16u + (size_t)kQWaves * kQAreaBytes;
     }
 };
+
+// The greedy token behind one column: `best` is the running top two of the rows this thread
+// stored (waves 0 .. nred-1 hold candidates).  Every thread of the workgroup calls it.
+__device__ __forceinline__ void q6m_greedy_token(top2 best, uint32_t nred, lev_f32x4 *__restrict__ partials,
+                                                 uint32_t *__restrict__ tickets, uint32_t *__restrict__ out_idx,
+                                                 float *__restrict__ out_margin) {
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    __shared__ float s_best[kQWaves], s_second[kQWaves];
+    __shared__ uint32_t s_idx[kQWaves];
+    // only the waves that stored outputs hold candidates; wave 0 finishes alone, so that no
+    // wave waits at a barrier for another one's stores
+    if (wave < nred) {
+        best = top2_wave(best);
+        if (lane == 0u) {
+            s_best[wave] = best.best;
+            s_second[wave] = best.second;
+            s_idx[wave] = best.idx;
+        }
+    }
+    lev_barrier_lds();
+    if (wave != 0u) return;
+    top2 m{s_best[0], s_second[0], s_idx[0]};
+    if (nred > 1u) {   // workgroup-uniform
+        m = top2{kTop2Floor, kTop2Floor, 0xFFFFFFFFu};
+        if (lane < nred) m = top2{s_best[lane], s_second[lane], s_idx[lane]};
+        m = top2_wave(m);
+    }
+    if (!tickets) {
+        if (lane == 0u)
+            partials[blockIdx.x] = lev_f32x4{m.best, m.second, __builtin_bit_cast(float, m.idx), 0.f};
+        return;
+    }
+    // The last workgroup to finish merges the partials (a kernel of its own for that costs a
+    // launch and a cold round trip: 7 us behind a 25 us GEMV).  The partial goes out in
+    // device-scope stores, which go through to memory, and the arrival is counted once they
+    // have completed (a fence here would write back every dirty line of the L2, the rows of y
+    // included: 250 of those cost 12 us).  Arrivals are counted in eight groups (workgroup
+    // index mod 8, counters 4 KB apart, so that they do not queue up in one L2 channel); the
+    // last of each group arrives at a ninth counter.
+    uint32_t last = 0u;
+    if (lane == 0u) {
+        float *pf = reinterpret_cast<float *>(partials + blockIdx.x);
+        __hip_atomic_store(pf, m.best, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(pf + 1, m.second, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(pf + 2, __builtin_bit_cast(float, m.idx), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        lev_publish_wait();
+        const uint32_t grp = blockIdx.x & 7u, ngrp = gridDim.x < 8u ? gridDim.x : 8u;
+        const uint32_t in_grp = (gridDim.x - grp + 7u) >> 3;
+        if (__hip_atomic_fetch_add(&tickets[(1u + grp) * 1024u], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ==
+            in_grp - 1u) {
+            // nobody else touches the counter before the next launch
+            __hip_atomic_store(&tickets[(1u + grp) * 1024u], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (__hip_atomic_fetch_add(&tickets[0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == ngrp - 1u) {
+                __hip_atomic_store(&tickets[0], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                last = 1u;
+            }
+        }
+    }
+    if (!__builtin_amdgcn_readfirstlane((int)last)) return;
+    top2 f{kTop2Floor, kTop2Floor, 0xFFFFFFFFu};
+    const float *pf = reinterpret_cast<const float *>(partials);
+    // device-scope loads: the other workgroups' partials come from beyond this XCD's L2.  Four
+    // records a lane are requested together (256 workgroups: one trip to memory, not four)
+    for (uint32_t i0 = lane; i0 < gridDim.x; i0 += 256u) {
+        float b[4], s2[4], ib[4];
+#pragma unroll
+        for (uint32_t u = 0; u < 4u; ++u) {
+            const uint32_t i = i0 + 64u * u < gridDim.x ? i0 + 64u * u : i0;
+            b[u] = __hip_atomic_load(pf + 4u * i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            s2[u] = __hip_atomic_load(pf + 4u * i + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            ib[u] = __hip_atomic_load(pf + 4u * i + 2u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < 4u; ++u)   // (a request past the end repeated the lane's first record: not merged again)
+            if (i0 + 64u * u < gridDim.x) f = top2_merge(f, top2{b[u], s2[u], __float_as_uint(ib[u])});
+    }
+    f = top2_wave(f);
+    if (lane == 0u) {
+        if (out_idx) out_idx[0] = f.idx == 0xFFFFFFFFu ? 0u : f.idx;   // nothing above -inf: first
+        if (out_margin) out_margin[0] = f.best - f.second;
+    }
+}
 
 // NC: columns staged (1, 2, 4 or 8; >= ncol).  S: waves per row group (2..16, a
 // power of two).  partials (optional, ncol == 1): the workgroup's top two outputs.
@@ -501,71 +587,271 @@ q6_k_mfma_gemv(const uint8_t *__restrict__ w, const float *__restrict__ x, const
     }
 
     if (partials) {
-        __shared__ float s_best[kQWaves], s_second[kQWaves];
-        __shared__ uint32_t s_idx[kQWaves];
-        // only the waves that stored outputs hold candidates; wave 0 finishes alone, so that no
-        // wave waits at a barrier for another one's stores
-        const uint32_t nred0 = (slots * 16u * NC + 63u) >> 6, nred = nred0 < (uint32_t)kQWaves ? nred0 : (uint32_t)kQWaves;
-        if (wave < nred) {
-            best = top2_wave(best);
-            if (lane == 0u) {
-                s_best[wave] = best.best;
-                s_second[wave] = best.second;
-                s_idx[wave] = best.idx;
-            }
-        }
+        const uint32_t nred0 = (slots * 16u * NC + 63u) >> 6;
+        q6m_greedy_token(best, nred0 < (uint32_t)kQWaves ? nred0 : (uint32_t)kQWaves, partials, tickets, out_idx, out_margin);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// One column, rows of at most sixteen superblocks: a wave per superblock COLUMN of the matrix.
+// The wave stages the 256 activations of its column by itself (1 KB of LDS nobody else
+// touches), keeps the A operands of its four MFMAs in registers and walks the row groups
+// with the next group's weights in flight; the partial sums of a row meet in LDS behind ONE
+// barrier per round, nothing but the RMSNorm's sum of squares crosses waves before the
+// products.  The arithmetic, the fetch and the turn-round are those of q6_k_mfma_gemv (a
+// wave's superblocks are all even or all odd here as well: it has one).
+// LDS: part [2][16 waves][16 rows] f64 | sums of squares [16] f64 | per wave: turn-round area,
+// digit planes [16 groups][4 planes][16 B], a zero strip.
+// ---------------------------------------------------------------------------
+constexpr uint32_t kQ1PartBytes = 2u * kQWaves * 16u * 8u;
+constexpr uint32_t kQ1NormBytes = kQWaves * 8u;
+constexpr uint32_t kQ1DigBytes = 1024u, kQ1ZeroBytes = 16u;
+constexpr uint32_t kQ1WaveBytes = kQAreaBytes + kQ1DigBytes + kQ1ZeroBytes;
+__host__ __device__ constexpr size_t q6m_one_lds() {
+    return kQ1PartBytes + kQ1NormBytes + (size_t)kQWaves * kQ1WaveBytes;
+}
+
+// Sum over lanes l, l ^ 16, l ^ 32, l ^ 48 in every lane, in f64, by row swaps.
+__device__ __forceinline__ double q6m_row_sum(double v) {
+    uint32_t lo = (uint32_t)__double2loint(v), hi = (uint32_t)__double2hiint(v);
+    auto a0 = __builtin_amdgcn_permlane32_swap(lo, lo, false, false);
+    auto a1 = __builtin_amdgcn_permlane32_swap(hi, hi, false, false);
+    v = __hiloint2double((int)a1[0], (int)a0[0]) + __hiloint2double((int)a1[1], (int)a0[1]);
+    lo = (uint32_t)__double2loint(v);
+    hi = (uint32_t)__double2hiint(v);
+    a0 = __builtin_amdgcn_permlane16_swap(lo, lo, false, false);
+    a1 = __builtin_amdgcn_permlane16_swap(hi, hi, false, false);
+    return __hiloint2double((int)a1[0], (int)a0[0]) + __hiloint2double((int)a1[1], (int)a0[1]);
+}
+
+template <typename T>
+__device__ __forceinline__ void q6m_pin(T &v) {
+    asm volatile("" : "+v"(v));
+}
+
+// wave -> (slot, superblock) as 4-bit entries of two 64-bit kernel arguments (no division in
+// front of the first load).  NORM: RMSNorm (gain != nullptr) in front.
+template <bool NORM>
+__global__ void __launch_bounds__(kQThreads)
+q6_k_mfma_gemv_one(const uint8_t *__restrict__ w, const float *__restrict__ x, const float *__restrict__ gain,
+                   float eps, float *__restrict__ y, uint32_t cols, uint32_t rows, uint32_t wpr, uint32_t slots,
+                   uint64_t slot_of_wave, uint64_t pos_of_wave, double rcols, lev_f32x4 *__restrict__ partials,
+                   uint32_t *__restrict__ tickets, uint32_t *__restrict__ out_idx, float *__restrict__ out_margin) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    const uint32_t slot = (uint32_t)(slot_of_wave >> (4u * wave)) & 15u;   // idle waves: slot >= slots
+    const uint32_t sb = (uint32_t)(pos_of_wave >> (4u * wave)) & 15u;      // the wave's superblock column
+    const uint32_t SB = cols >> 8;
+
+    // the wave's activations first ...
+    lev_f32x4 v = reinterpret_cast<const lev_f32x4 *>(x)[64u * sb + lane];
+    lev_f32x4 gn;
+    if (NORM) gn = reinterpret_cast<const lev_f32x4 *>(gain)[64u * sb + lane];
+    const bool active = slot < slots;
+    const uint64_t row_bytes = (uint64_t)SB * 210u;
+    const uint32_t ngroups = (rows + 15u) >> 4;
+    const uint32_t nrounds = (ngroups + slots - 1u) / slots;     // rounds of `slots` row groups
+    const uint32_t odd = sb & 1u;
+    const int32_t poff = q6m_piece_offset(lane, odd);
+    auto issue = [&](uint32_t round_block, q6m_regs &W) {
+        uint32_t rg = round_block * slots + (active ? slot : 0u);
+        rg = rg < ngroups ? rg : ngroups - 1u;
+        q6m_issue(w, row_bytes, rg * 16u, rows, sb, lane, poff, W);
+    };
+    q6m_regs Wa, Wb;
+    uint32_t rb = blockIdx.x;
+    // ... and the first row group's weights; with RMSNorm in front only once every wave's request
+    // for its activations is in the CU's memory queue (a short load queued behind other waves'
+    // long ones waits for them, and every wave waits for every wave's activations there)
+    if (NORM) {
+        __builtin_amdgcn_sched_barrier(0);
+        asm volatile("s_barrier" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    issue(rb, Wa);
+
+    // ---- everything the tail of a round needs, while the loads are on their way ----
+    double *norm = reinterpret_cast<double *>(smem + kQ1PartBytes);
+    uint8_t *wave_lds = smem + kQ1PartBytes + kQ1NormBytes + (size_t)wave * kQ1WaveBytes;
+    uint8_t *dig = wave_lds + kQAreaBytes, *zero = dig + kQ1DigBytes;
+    const uint32_t r = lane & 15u, q = lane >> 4;
+    uint32_t pw = (wave * 16u + lane) * 8u;
+    // wave s < slots adds the wpr partial sums of slot s: lane (r, q) reads waves q, q + 4, q + 8, q + 12
+    uint32_t pr = (((wave < slots ? wave : 0u) * wpr + q) * 16u + r) * 8u;
+    uint32_t k0 = q < wpr ? 1u : 0u, k1 = q + 4u < wpr ? 1u : 0u, k2 = q + 8u < wpr ? 1u : 0u,
+             k3 = q + 12u < wpr ? 1u : 0u;
+    uint32_t orow = (rb * slots + wave) * 16u + r;
+    const uint32_t orow_step = gridDim.x * slots * 16u;
+    const bool writer = wave < slots && q == 0u;
+    uint32_t stores = writer && orow < rows ? 1u : 0u;
+    uint64_t yp = reinterpret_cast<uint64_t>(y + orow);
+    q6m_pin(pw);
+    q6m_pin(pr);
+    q6m_pin(k0);
+    q6m_pin(k1);
+    q6m_pin(k2);
+    q6m_pin(k3);
+    q6m_pin(stores);
+    q6m_pin(yp);
+
+    if (NORM) {
+        // RMSNorm as the reference computes it: mean square and 1/sqrt in f64, then (f32)(x * inv) * gain
+        double ss = (double)v.x * (double)v.x;
+        ss = fma((double)v.y, (double)v.y, ss);
+        ss = fma((double)v.z, (double)v.z, ss);
+        ss = fma((double)v.w, (double)v.w, ss);
+        ss = lev_group_sum_f64<64>(ss);                        // lane 63 holds the wave's sum
+        if (lane == 63u) norm[wave] = ss;
         lev_barrier_lds();
-        if (wave != 0u) return;
-        top2 m{kTop2Floor, kTop2Floor, 0xFFFFFFFFu};
-        if (lane < nred) m = top2{s_best[lane], s_second[lane], s_idx[lane]};
-        m = top2_wave(m);
-        if (!tickets) {
-            if (lane == 0u)
-                partials[blockIdx.x] = lev_f32x4{m.best, m.second, __builtin_bit_cast(float, m.idx), 0.f};
-            return;
+        // the waves of slot 0 cover the row once; sixteen reads in flight together, added in order
+        double nk[kQWaves];
+#pragma unroll
+        for (int k = 0; k < kQWaves; ++k) nk[k] = norm[k];
+        double tot = nk[0];
+#pragma unroll
+        for (int k = 1; k < kQWaves; ++k) tot += (uint32_t)k < wpr ? nk[k] : 0.0;
+        const double a = fma(tot, rcols, (double)eps);
+        double rs = __builtin_amdgcn_rsq(a);
+        rs = rs * fma(-0.5 * a * rs, rs, 1.5);
+        rs = rs * fma(-0.5 * a * rs, rs, 1.5);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) v[k] = (float)((double)v[k] * rs) * gn[k];
+    }
+
+    // ---- the wave's digit planes and its A operands ----
+    double ps;                                                 // 2^(e - 2): undoes the scaling and the 4 of the codes
+    q6m_i4 A[2][2];
+    {
+        uint32_t mb = 0u;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const uint32_t bits = __float_as_uint(v[k]) & 0x7FFFFFFFu;
+            mb = bits > mb ? bits : mb;
         }
-        // The last workgroup to finish merges the partials (a kernel of its own for that costs a
-        // launch and a cold round trip: 7 us behind a 25 us GEMV).  The partial goes out in
-        // device-scope stores, which go through to memory, and the arrival is counted once they
-        // have completed (a fence here would write back every dirty line of the L2, the rows of y
-        // included: 250 of those cost 12 us).  Arrivals are counted in eight groups (workgroup
-        // index mod 8, counters 4 KB apart, so that they do not queue up in one L2 channel); the
-        // last of each group arrives at a ninth counter.
-        uint32_t last = 0u;
-        if (lane == 0u) {
-            float *pf = reinterpret_cast<float *>(partials + blockIdx.x);
-            __hip_atomic_store(pf, m.best, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(pf + 1, m.second, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(pf + 2, __builtin_bit_cast(float, m.idx), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            lev_publish_wait();
-            const uint32_t grp = blockIdx.x & 7u, ngrp = gridDim.x < 8u ? gridDim.x : 8u;
-            const uint32_t in_grp = (gridDim.x - grp + 7u) >> 3;
-            if (__hip_atomic_fetch_add(&tickets[(1u + grp) * 1024u], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ==
-                in_grp - 1u) {
-                // nobody else touches the counter before the next launch
-                __hip_atomic_store(&tickets[(1u + grp) * 1024u], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                if (__hip_atomic_fetch_add(&tickets[0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == ngrp - 1u) {
-                    __hip_atomic_store(&tickets[0], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    last = 1u;
+#define LEV_Q6M_MAXSTEP(CTRL)                                                                           \
+        {                                                                                              \
+            const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp((int)mb, (int)mb, CTRL, 0xF, 0xF, false); \
+            mb = o > mb ? o : mb;                                                                      \
+        }
+        LEV_Q6M_MAXSTEP(0xB1);
+        LEV_Q6M_MAXSTEP(0x4E);
+        LEV_Q6M_MAXSTEP(0x141);
+        LEV_Q6M_MAXSTEP(0x140);
+#undef LEV_Q6M_MAXSTEP
+        {
+            const auto s0 = __builtin_amdgcn_permlane32_swap(mb, mb, false, false);
+            mb = s0[0] > s0[1] ? s0[0] : s0[1];
+            const auto s1 = __builtin_amdgcn_permlane16_swap(mb, mb, false, false);
+            mb = s1[0] > s1[1] ? s1[0] : s1[1];
+        }
+        uint32_t ex = mb >> 23;                             // biased exponent: |x| < 2^(ex-126)
+        const bool bad = ex == 255u;                        // NaN or infinity in the superblock
+        ex = ex < 30u ? 30u : (ex > 254u ? 254u : ex);      // keeps both powers of two normal numbers
+        const float scale = __uint_as_float((283u - ex) << 23);   // 2^(156-ex): |x*scale| < 2^30
+        ps = !active ? 0.0 : bad ? (double)__builtin_nanf("") : __hiloint2double((int)((ex + 865u) << 20), 0);   // 2^(ex-158)
+        uint32_t Y[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int X = (int)rintf(v[k] * scale);
+            Y[k] = ((uint32_t)X + 0x00808080u) ^ 0x00808080u;   // bytes = balanced base-256 digits
+        }
+        const uint32_t t0 = __builtin_amdgcn_perm(Y[1], Y[0], 0x05010400u);
+        const uint32_t t1 = __builtin_amdgcn_perm(Y[1], Y[0], 0x07030602u);
+        const uint32_t t2 = __builtin_amdgcn_perm(Y[3], Y[2], 0x05010400u);
+        const uint32_t t3 = __builtin_amdgcn_perm(Y[3], Y[2], 0x07030602u);
+        const uint32_t dw[4] = {__builtin_amdgcn_perm(t2, t0, 0x05040100u), __builtin_amdgcn_perm(t2, t0, 0x07060302u),
+                                __builtin_amdgcn_perm(t3, t1, 0x05040100u), __builtin_amdgcn_perm(t3, t1, 0x07060302u)};
+        // group lane/4, plane p at +16p, the lane's four elements at +4*(lane%4)
+        uint8_t *at = dig + (lane >> 2) * 64u + 4u * (lane & 3u);
+#pragma unroll
+        for (int p = 0; p < 4; ++p) *reinterpret_cast<uint32_t *>(at + 16 * p) = dw[p];
+        if (lane < kQ1ZeroBytes / 4u) reinterpret_cast<uint32_t *>(zero)[lane] = 0u;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        // lane (r, g) feeds A row r = 4*gs + p: plane p of group 8*hf + 2*jb (+ 4*nb + lh) when gs == g,
+        // zeros otherwise
+        const uint32_t hf = q >> 1, jb = q & 1u;
+        const bool feeds = active && (r >> 2) == q;
+        const uint8_t *ab = feeds ? dig + (8u * hf + 2u * jb) * 64u + 16u * (r & 3u) : zero;
+        const uint32_t hs = feeds ? 64u : 0u;
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+            for (int lh = 0; lh < 2; ++lh) A[nb][lh] = *reinterpret_cast<const q6m_i4 *>(ab + (4 * nb + lh) * hs);
+    }
+    const q6m_lane L6(smem + kQ1PartBytes + kQ1NormBytes, wave, lane, odd, kQ1WaveBytes);
+    // the operands are read back before the wait for the weights, not behind it
+    __builtin_amdgcn_sched_barrier(0);
+
+    top2 best{kTop2Floor, kTop2Floor, 0xFFFFFFFFu};
+    auto finish = [&](const q6m_regs &W) {
+        q6m_i4 B[2][2];
+        int sc[2][2];
+        uint32_t dbits;
+        L6.operands(W, B, sc, dbits);
+        int E[4] = {0, 0, 0, 0};
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb) {
+#pragma unroll
+            for (int lh = 0; lh < 2; ++lh) {
+                const q6m_i4 D = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[nb][lh], B[nb][lh], q6m_i4{0, 0, 0, 0}, 0, 0, 0);
+                // |D| <= 16*128*128 = 2^18, |sc| <= 2^7: four products per plane stay below 2^27
+#pragma unroll
+                for (int p = 0; p < 4; ++p) {
+                    E[p] += __mul24(D[p], sc[nb][lh]);
+                    asm("" : "+v"(E[p]));   // one multiply-add per plane: keeps the sums from being regrouped
                 }
             }
         }
-        if (!__builtin_amdgcn_readfirstlane((int)last)) return;
-        top2 f{kTop2Floor, kTop2Floor, 0xFFFFFFFFu};
-        const float *pf = reinterpret_cast<const float *>(partials);
-        for (uint32_t i = lane; i < gridDim.x; i += 64u) {
-            // device-scope loads: the other workgroups' partials come from beyond this XCD's L2
-            const float b = __hip_atomic_load(pf + 4u * i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            const float s2 = __hip_atomic_load(pf + 4u * i + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            const float ib = __hip_atomic_load(pf + 4u * i + 2u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            f = top2_merge(f, top2{b, s2, __float_as_uint(ib)});
+        const double hi = fma((double)E[3], 256.0, (double)E[2]);
+        const double lo = fma((double)E[1], 256.0, (double)E[0]);
+        const double dot = fma(hi, 65536.0, lo);
+        double val = (ps * (double)lev_f16_bits_to_f32(dbits)) * dot;
+        val = q6m_row_sum(val);
+        if (lane < 16u) *reinterpret_cast<double *>(smem + pw) = val;
+        lev_barrier_lds();
+        if (wave < slots) {
+            const double *pp = reinterpret_cast<const double *>(smem + pr);
+            const double p0 = pp[0], p1 = pp[64], p2 = pp[128], p3 = pp[192];   // four reads in flight together
+            double s = ((k0 ? p0 : 0.0) + (k1 ? p1 : 0.0)) + ((k2 ? p2 : 0.0) + (k3 ? p3 : 0.0));
+            s = q6m_row_sum(s);
+            if (stores) {
+                const float out = (float)s;
+                *reinterpret_cast<__attribute__((address_space(1))) float *>(yp) = out;
+                // running top two of the rows this lane finishes (rows ascend, so a tie keeps the
+                // earlier, lower index)
+                if (out > best.best) {
+                    best.second = best.best;
+                    best.best = out;
+                    best.idx = orow;
+                } else if (out > best.second) {
+                    best.second = out;
+                }
+            }
         }
-        f = top2_wave(f);
-        if (lane == 0u) {
-            if (out_idx) out_idx[0] = f.idx == 0xFFFFFFFFu ? 0u : f.idx;   // nothing above -inf: first
-            if (out_margin) out_margin[0] = f.best - f.second;
-        }
+        pw ^= kQWaves * 16u * 8u;                              // the other half of `part` next round
+        pr ^= kQWaves * 16u * 8u;
+        orow += orow_step;
+        yp += (uint64_t)orow_step * 4u;
+        stores = writer && orow < rows ? 1u : 0u;
+    };
+    // Unconditional (clamped) prefetch, one round ahead (a branch around the loads would make the
+    // compiler wait for them before the current group is multiplied).
+    while (true) {
+        uint32_t next = rb + gridDim.x;
+        issue(next < nrounds ? next : rb, Wb);
+        finish(Wa);
+        if (next >= nrounds) break;
+        rb = next;
+        next = rb + gridDim.x;
+        issue(next < nrounds ? next : rb, Wa);
+        finish(Wb);
+        if (next >= nrounds) break;
+        rb = next;
     }
+    if (partials) q6m_greedy_token(best, slots, partials, tickets, out_idx, out_margin);
 }
 
 // ---------------------------------------------------------------------------
@@ -816,6 +1102,34 @@ hipError_t q6m_launch(lev_ctx *ctx, const uint8_t *w, const float *x, const floa
     return hipGetLastError();
 }
 
+template <bool NORM>
+hipError_t q6m_one_launch(lev_ctx *ctx, const uint8_t *w, const float *x, const float *gain, float eps, float *y,
+                          uint32_t cols, uint32_t rows, lev_f32x4 *partials, uint32_t *d_argmax, float *d_margin) {
+    const uint32_t wpr = cols >> 8, slots = (uint32_t)kQWaves / wpr;
+    const uint32_t ngroups = (rows + 15u) / 16u;
+    const uint32_t nrounds = (ngroups + slots - 1u) / slots;
+    uint64_t slot_of_wave = 0, pos_of_wave = 0;
+    for (uint32_t wv = 0; wv < (uint32_t)kQWaves; ++wv) {
+        slot_of_wave |= (uint64_t)(wv / wpr > 15u ? 15u : wv / wpr) << (4u * wv);
+        pos_of_wave |= (uint64_t)(wv % wpr) << (4u * wv);
+    }
+    constexpr size_t lds = q6m_one_lds();
+    static bool configured = false;   // per instantiation: raise the dynamic LDS limit once
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&q6_k_mfma_gemv_one<NORM>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        configured = true;
+    }
+    uint32_t blocks = nrounds < (uint32_t)ctx->num_cus ? nrounds : (uint32_t)ctx->num_cus;
+    if (partials && blocks > lev_ctx::kArgmaxPartials) blocks = lev_ctx::kArgmaxPartials;
+    uint32_t *tickets = partials ? reinterpret_cast<uint32_t *>(ctx->d_flag) + lev_ctx::kArgmaxTicketWord : nullptr;
+    hipLaunchKernelGGL((q6_k_mfma_gemv_one<NORM>), dim3(blocks), dim3(kQThreads), lds, ctx->stream, w, x, gain, eps, y,
+                       cols, rows, wpr, slots, slot_of_wave, pos_of_wave, 1.0 / (double)cols, partials, tickets,
+                       d_argmax, d_margin);
+    return hipGetLastError();
+}
+
 }  // namespace
 
 // Columns one launch of the matrix-core kernel can take for this in_dim (0: not usable).
@@ -842,6 +1156,16 @@ hipError_t lev_q6_k_mfma_gemv_launch(lev_ctx *ctx, const uint8_t *w, const float
                                      uint32_t waves, lev_f32x4 *partials, uint32_t *d_argmax, float *d_margin) {
     if (!d_argmax && !d_margin) partials = nullptr;
     if (waves != 2u && waves != 4u && waves != 8u && waves != 16u) waves = 0u;
+    // one column of at most sixteen superblocks, no number of waves per row group asked for: a
+    // wave per superblock column
+    static const bool one_off = [] {
+        const char *e = getenv("LEV_Q6K_ONE");   // LEV_Q6K_ONE=0: the several-column kernel at one column too, for comparison
+        return e && e[0] == '0';
+    }();
+    if (ncol == 1u && waves == 0u && !one_off && in_dim <= 4096u) {
+        if (gain) return q6m_one_launch<true>(ctx, w, x, gain, eps, y, in_dim, rows, partials, d_argmax, d_margin);
+        return q6m_one_launch<false>(ctx, w, x, gain, eps, y, in_dim, rows, partials, d_argmax, d_margin);
+    }
     if (ncol > 4) return q6m_launch<8>(ctx, w, x, gain, eps, y, in_dim, rows, ncol, waves, partials, d_argmax, d_margin);
     if (ncol > 2) return q6m_launch<4>(ctx, w, x, gain, eps, y, in_dim, rows, ncol, waves, partials, d_argmax, d_margin);
     if (ncol > 1) return q6m_launch<2>(ctx, w, x, gain, eps, y, in_dim, rows, ncol, waves, partials, d_argmax, d_margin);

@@ -350,6 +350,34 @@ def test_q6_k_ncol_shapes_with_rmsnorm(ctx, rows, cols, ncol):
     assert np.array_equal(bits(q6_gemv(ctx, w, x[0], rows, cols)), bits(plain[0]))
 
 
+@pytest.mark.parametrize("rows,cols", [(50, 3072), (33, 3840), (100, 2048), (9001, 512), (4099, 4096), (16, 768),
+                                       (257, 1280)])
+def test_q6_k_one_column_kernel_shapes(ctx, rows, cols):
+    """One column of at most sixteen superblocks: a wave per superblock column.  Narrow rows share
+    a round between several row groups, widths that do not divide sixteen leave waves idle, tall
+    matrices take many rounds per workgroup (the greedy token then merges many rounds' rows per
+    lane); the column is the same bits as the first of two through the several-column kernel,
+    with and without RMSNorm, and scaling x by a power of two scales y by exactly that power."""
+    w = O.synth_q6_k(rows % 97 + cols, rows * cols // 256)
+    x = O.normal(2 * cols, 300 + rows % 50).reshape(2, cols)
+    gain = O.normal(cols, 9, 1.0, 0.1)
+    got, idx, margin = q6_gemv(ctx, w, x[0], rows, cols, argmax=True)
+    assert O.max_rel_err(got, O.q6_k_matvec_f64(w, rows, cols, x[0])) < TOL
+    assert idx == O.argmax(got) and margin == O.top_margin(got)
+    both = q6k_ncol(ctx, w, x, rows, cols, 2)
+    assert np.array_equal(bits(got), bits(both[0]))
+    normed = q6k_ncol(ctx, w, x[:1], rows, cols, 1, gain)
+    xn = H.rmsnorm_rows(x, gain)
+    assert O.max_rel_err(normed[0], O.q6_k_matvec_f64(w, rows, cols, xn[0])) < TOL
+    assert np.array_equal(bits(normed[0]), bits(q6k_ncol(ctx, w, x, rows, cols, 2, gain)[0]))
+    for e in (-45, 37):
+        scaled = q6_gemv(ctx, w, np.ldexp(x[0], e).astype(np.float32), rows, cols)
+        assert np.array_equal(bits(scaled), bits(np.ldexp(got, e).astype(np.float32))), e
+    xb = x[0].copy()
+    xb[cols - 5] = np.nan
+    assert np.isnan(q6_gemv(ctx, w, xb, rows, cols)).all()
+
+
 def test_q6_k_ncol_reference_fixture_and_hand_block(ctx):
     """The reference's own wide-range 64 x 512 bytes (main.swift:1028-1085) in every column
     position, and the hand-computed -315 block (main.swift:1091-1120) as one of four columns."""
