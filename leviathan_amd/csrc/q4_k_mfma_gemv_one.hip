@@ -284,13 +284,10 @@ q4_k_mfma_gemv_one(const uint8_t *__restrict__ w, const float *__restrict__ x, c
         ss = lev_group_sum_f64<64>(ss);                        // lane 63 holds the wave's sum
         if (lane == 63u) norm[wave] = ss;
         lev_barrier_lds();
-        // the waves of slot 0 cover the row once; sixteen reads in flight together, added in order
-        double nk[kOneWaves];
-#pragma unroll
-        for (int k = 0; k < kOneWaves; ++k) nk[k] = norm[k];
-        double tot = nk[0];
-#pragma unroll
-        for (int k = 1; k < kOneWaves; ++k) tot += (uint32_t)k < wpr ? nk[k] : 0.0;
+        // the waves of slot 0 cover the row once: lane k of every row of 16 lanes takes wave k's
+        // sum, and the row adds them up (every lane ends with the total)
+        const double mine = norm[r];
+        const double tot = lev_group_sum_f64<16>(r < wpr ? mine : 0.0);
         // 1/sqrt(mean + eps): the hardware estimate and two Newton steps (full f64 accuracy)
         const double a = fma(tot, rcols, (double)eps);
         double rs = __builtin_amdgcn_rsq(a);

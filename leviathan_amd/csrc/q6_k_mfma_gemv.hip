@@ -600,15 +600,16 @@ q6_k_mfma_gemv(const uint8_t *__restrict__ w, const float *__restrict__ x, const
 // barrier per round, nothing but the RMSNorm's sum of squares crosses waves before the
 // products.  The arithmetic, the fetch and the turn-round are those of q6_k_mfma_gemv (a
 // wave's superblocks are all even or all odd here as well: it has one).
-// LDS: part [2][16 waves][16 rows] f64 | sums of squares [16] f64 | per wave: turn-round area,
-// digit planes [16 groups][4 planes][16 B], a zero strip.
+// Two columns go through it as well (a column costs four MFMAs and the recombination again).
+// LDS: part [2][16 waves][16 rows][NC] f64 | sums of squares [NC][16] f64 | per wave: turn-round
+// area, digit planes [NC][16 groups][4 planes][16 B], a zero strip.
 // ---------------------------------------------------------------------------
-constexpr uint32_t kQ1PartBytes = 2u * kQWaves * 16u * 8u;
-constexpr uint32_t kQ1NormBytes = kQWaves * 8u;
 constexpr uint32_t kQ1DigBytes = 1024u, kQ1ZeroBytes = 16u;
-constexpr uint32_t kQ1WaveBytes = kQAreaBytes + kQ1DigBytes + kQ1ZeroBytes;
-__host__ __device__ constexpr size_t q6m_one_lds() {
-    return kQ1PartBytes + kQ1NormBytes + (size_t)kQWaves * kQ1WaveBytes;
+__host__ __device__ constexpr uint32_t q6m_one_part_bytes(uint32_t nc) { return 2u * kQWaves * 16u * 8u * nc; }
+__host__ __device__ constexpr uint32_t q6m_one_norm_bytes(uint32_t nc) { return kQWaves * 8u * nc; }
+__host__ __device__ constexpr uint32_t q6m_one_wave_bytes(uint32_t nc) { return kQAreaBytes + nc * kQ1DigBytes + kQ1ZeroBytes; }
+__host__ __device__ constexpr size_t q6m_one_lds(uint32_t nc) {
+    return q6m_one_part_bytes(nc) + q6m_one_norm_bytes(nc) + (size_t)kQWaves * q6m_one_wave_bytes(nc);
 }
 
 // Sum over lanes l, l ^ 16, l ^ 32, l ^ 48 in every lane, in f64, by row swaps.
@@ -630,13 +631,17 @@ __device__ __forceinline__ void q6m_pin(T &v) {
 }
 
 // wave -> (slot, superblock) as 4-bit entries of two 64-bit kernel arguments (no division in
-// front of the first load).  NORM: RMSNorm (gain != nullptr) in front.
-template <bool NORM>
+// front of the first load).  NC: columns staged (1 or 2; >= ncol); one column keeps its A
+// operands in registers, several read them from the wave's planes at every product.
+// NORM: RMSNorm (gain != nullptr) in front.  partials (optional, ncol == 1): the greedy token.
+template <int NC, bool NORM>
 __global__ void __launch_bounds__(kQThreads)
 q6_k_mfma_gemv_one(const uint8_t *__restrict__ w, const float *__restrict__ x, const float *__restrict__ gain,
-                   float eps, float *__restrict__ y, uint32_t cols, uint32_t rows, uint32_t wpr, uint32_t slots,
-                   uint64_t slot_of_wave, uint64_t pos_of_wave, double rcols, lev_f32x4 *__restrict__ partials,
-                   uint32_t *__restrict__ tickets, uint32_t *__restrict__ out_idx, float *__restrict__ out_margin) {
+                   float eps, float *__restrict__ y, uint32_t cols, uint32_t rows, uint32_t ncol, uint32_t wpr,
+                   uint32_t slots, uint64_t slot_of_wave, uint64_t pos_of_wave, double rcols,
+                   lev_f32x4 *__restrict__ partials, uint32_t *__restrict__ tickets, uint32_t *__restrict__ out_idx,
+                   float *__restrict__ out_margin) {
+    constexpr uint32_t kPart = q6m_one_part_bytes(NC), kNorm = q6m_one_norm_bytes(NC), kWave = q6m_one_wave_bytes(NC);
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
@@ -644,8 +649,13 @@ q6_k_mfma_gemv_one(const uint8_t *__restrict__ w, const float *__restrict__ x, c
     const uint32_t sb = (uint32_t)(pos_of_wave >> (4u * wave)) & 15u;      // the wave's superblock column
     const uint32_t SB = cols >> 8;
 
-    // the wave's activations first ...
-    lev_f32x4 v = reinterpret_cast<const lev_f32x4 *>(x)[64u * sb + lane];
+    // the wave's activations first (columns of the layout beyond ncol repeat the last one: never stored) ...
+    lev_f32x4 v[NC];
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+        const uint32_t cc = (uint32_t)c < ncol ? (uint32_t)c : ncol - 1u;
+        v[c] = reinterpret_cast<const lev_f32x4 *>(x + (uint64_t)cc * cols)[64u * sb + lane];
+    }
     lev_f32x4 gn;
     if (NORM) gn = reinterpret_cast<const lev_f32x4 *>(gain)[64u * sb + lane];
     const bool active = slot < slots;
@@ -672,13 +682,13 @@ q6_k_mfma_gemv_one(const uint8_t *__restrict__ w, const float *__restrict__ x, c
     issue(rb, Wa);
 
     // ---- everything the tail of a round needs, while the loads are on their way ----
-    double *norm = reinterpret_cast<double *>(smem + kQ1PartBytes);
-    uint8_t *wave_lds = smem + kQ1PartBytes + kQ1NormBytes + (size_t)wave * kQ1WaveBytes;
-    uint8_t *dig = wave_lds + kQAreaBytes, *zero = dig + kQ1DigBytes;
+    double *norm = reinterpret_cast<double *>(smem + kPart);
+    uint8_t *wave_lds = smem + kPart + kNorm + (size_t)wave * kWave;
+    uint8_t *dig = wave_lds + kQAreaBytes, *zero = dig + NC * kQ1DigBytes;
     const uint32_t r = lane & 15u, q = lane >> 4;
-    uint32_t pw = (wave * 16u + lane) * 8u;
+    uint32_t pw = ((wave * 16u + lane) * NC) * 8u;
     // wave s < slots adds the wpr partial sums of slot s: lane (r, q) reads waves q, q + 4, q + 8, q + 12
-    uint32_t pr = (((wave < slots ? wave : 0u) * wpr + q) * 16u + r) * 8u;
+    uint32_t pr = ((((wave < slots ? wave : 0u) * wpr + q) * 16u + r) * NC) * 8u;
     uint32_t k0 = q < wpr ? 1u : 0u, k1 = q + 4u < wpr ? 1u : 0u, k2 = q + 8u < wpr ? 1u : 0u,
              k3 = q + 12u < wpr ? 1u : 0u;
     uint32_t orow = (rb * slots + wave) * 16u + r;
@@ -697,36 +707,39 @@ q6_k_mfma_gemv_one(const uint8_t *__restrict__ w, const float *__restrict__ x, c
 
     if (NORM) {
         // RMSNorm as the reference computes it: mean square and 1/sqrt in f64, then (f32)(x * inv) * gain
-        double ss = (double)v.x * (double)v.x;
-        ss = fma((double)v.y, (double)v.y, ss);
-        ss = fma((double)v.z, (double)v.z, ss);
-        ss = fma((double)v.w, (double)v.w, ss);
-        ss = lev_group_sum_f64<64>(ss);                        // lane 63 holds the wave's sum
-        if (lane == 63u) norm[wave] = ss;
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            double ss = (double)v[c].x * (double)v[c].x;
+            ss = fma((double)v[c].y, (double)v[c].y, ss);
+            ss = fma((double)v[c].z, (double)v[c].z, ss);
+            ss = fma((double)v[c].w, (double)v[c].w, ss);
+            ss = lev_group_sum_f64<64>(ss);                    // lane 63 holds the wave's sum
+            if (lane == 63u) norm[c * kQWaves + wave] = ss;
+        }
         lev_barrier_lds();
-        // the waves of slot 0 cover the row once; sixteen reads in flight together, added in order
-        double nk[kQWaves];
 #pragma unroll
-        for (int k = 0; k < kQWaves; ++k) nk[k] = norm[k];
-        double tot = nk[0];
+        for (int c = 0; c < NC; ++c) {
+            // the waves of slot 0 cover the row once: lane k of every row of 16 lanes takes wave k's
+            // sum, and the row adds them up (every lane ends with the total)
+            const double mine = norm[c * kQWaves + r];
+            const double tot = lev_group_sum_f64<16>(r < wpr ? mine : 0.0);
+            const double a = fma(tot, rcols, (double)eps);
+            double rs = __builtin_amdgcn_rsq(a);
+            rs = rs * fma(-0.5 * a * rs, rs, 1.5);
+            rs = rs * fma(-0.5 * a * rs, rs, 1.5);
 #pragma unroll
-        for (int k = 1; k < kQWaves; ++k) tot += (uint32_t)k < wpr ? nk[k] : 0.0;
-        const double a = fma(tot, rcols, (double)eps);
-        double rs = __builtin_amdgcn_rsq(a);
-        rs = rs * fma(-0.5 * a * rs, rs, 1.5);
-        rs = rs * fma(-0.5 * a * rs, rs, 1.5);
-#pragma unroll
-        for (int k = 0; k < 4; ++k) v[k] = (float)((double)v[k] * rs) * gn[k];
+            for (int k = 0; k < 4; ++k) v[c][k] = (float)((double)v[c][k] * rs) * gn[k];
+        }
     }
 
-    // ---- the wave's digit planes and its A operands ----
-    double ps;                                                 // 2^(e - 2): undoes the scaling and the 4 of the codes
-    q6m_i4 A[2][2];
-    {
+    // ---- the wave's digit planes (and, at one column, its A operands) ----
+    double ps[NC];                                             // 2^(e - 2): undoes the scaling and the 4 of the codes
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
         uint32_t mb = 0u;
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
-            const uint32_t bits = __float_as_uint(v[k]) & 0x7FFFFFFFu;
+            const uint32_t bits = __float_as_uint(v[c][k]) & 0x7FFFFFFFu;
             mb = bits > mb ? bits : mb;
         }
 #define LEV_Q6M_MAXSTEP(CTRL)                                                                           \
@@ -749,11 +762,11 @@ q6_k_mfma_gemv_one(const uint8_t *__restrict__ w, const float *__restrict__ x, c
         const bool bad = ex == 255u;                        // NaN or infinity in the superblock
         ex = ex < 30u ? 30u : (ex > 254u ? 254u : ex);      // keeps both powers of two normal numbers
         const float scale = __uint_as_float((283u - ex) << 23);   // 2^(156-ex): |x*scale| < 2^30
-        ps = !active ? 0.0 : bad ? (double)__builtin_nanf("") : __hiloint2double((int)((ex + 865u) << 20), 0);   // 2^(ex-158)
+        ps[c] = !active ? 0.0 : bad ? (double)__builtin_nanf("") : __hiloint2double((int)((ex + 865u) << 20), 0);   // 2^(ex-158)
         uint32_t Y[4];
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
-            const int X = (int)rintf(v[k] * scale);
+            const int X = (int)rintf(v[c][k] * scale);
             Y[k] = ((uint32_t)X + 0x00808080u) ^ 0x00808080u;   // bytes = balanced base-256 digits
         }
         const uint32_t t0 = __builtin_amdgcn_perm(Y[1], Y[0], 0x05010400u);
@@ -763,25 +776,28 @@ q6_k_mfma_gemv_one(const uint8_t *__restrict__ w, const float *__restrict__ x, c
         const uint32_t dw[4] = {__builtin_amdgcn_perm(t2, t0, 0x05040100u), __builtin_amdgcn_perm(t2, t0, 0x07060302u),
                                 __builtin_amdgcn_perm(t3, t1, 0x05040100u), __builtin_amdgcn_perm(t3, t1, 0x07060302u)};
         // group lane/4, plane p at +16p, the lane's four elements at +4*(lane%4)
-        uint8_t *at = dig + (lane >> 2) * 64u + 4u * (lane & 3u);
+        uint8_t *at = dig + c * kQ1DigBytes + (lane >> 2) * 64u + 4u * (lane & 3u);
 #pragma unroll
         for (int p = 0; p < 4; ++p) *reinterpret_cast<uint32_t *>(at + 16 * p) = dw[p];
-        if (lane < kQ1ZeroBytes / 4u) reinterpret_cast<uint32_t *>(zero)[lane] = 0u;
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        // lane (r, g) feeds A row r = 4*gs + p: plane p of group 8*hf + 2*jb (+ 4*nb + lh) when gs == g,
-        // zeros otherwise
-        const uint32_t hf = q >> 1, jb = q & 1u;
-        const bool feeds = active && (r >> 2) == q;
-        const uint8_t *ab = feeds ? dig + (8u * hf + 2u * jb) * 64u + 16u * (r & 3u) : zero;
-        const uint32_t hs = feeds ? 64u : 0u;
+    }
+    if (lane < kQ1ZeroBytes / 4u) reinterpret_cast<uint32_t *>(zero)[lane] = 0u;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    // lane (r, g) feeds A row r = 4*gs + p: plane p of group 8*hf + 2*jb (+ 4*nb + lh) when gs == g,
+    // zeros otherwise
+    const uint32_t hf = q >> 1, jb = q & 1u;
+    const bool feeds = active && (r >> 2) == q;
+    const uint8_t *ab = feeds ? dig + (8u * hf + 2u * jb) * 64u + 16u * (r & 3u) : zero;
+    const uint32_t hs = feeds ? 64u : 0u, cs = feeds ? kQ1DigBytes : 0u;
+    q6m_i4 A1[2][2];
+    if (NC == 1) {
 #pragma unroll
         for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
-            for (int lh = 0; lh < 2; ++lh) A[nb][lh] = *reinterpret_cast<const q6m_i4 *>(ab + (4 * nb + lh) * hs);
+            for (int lh = 0; lh < 2; ++lh) A1[nb][lh] = *reinterpret_cast<const q6m_i4 *>(ab + (4 * nb + lh) * hs);
     }
-    const q6m_lane L6(smem + kQ1PartBytes + kQ1NormBytes, wave, lane, odd, kQ1WaveBytes);
+    const q6m_lane L6(smem + kPart + kNorm, wave, lane, odd, kWave);
     // the operands are read back before the wait for the weights, not behind it
     __builtin_amdgcn_sched_barrier(0);
 
@@ -791,48 +807,62 @@ q6_k_mfma_gemv_one(const uint8_t *__restrict__ w, const float *__restrict__ x, c
         int sc[2][2];
         uint32_t dbits;
         L6.operands(W, B, sc, dbits);
-        int E[4] = {0, 0, 0, 0};
+        const double d = (double)lev_f16_bits_to_f32(dbits);
+        double val[NC];
 #pragma unroll
-        for (int nb = 0; nb < 2; ++nb) {
+        for (int c = 0; c < NC; ++c) {
+            int E[4] = {0, 0, 0, 0};
 #pragma unroll
-            for (int lh = 0; lh < 2; ++lh) {
-                const q6m_i4 D = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[nb][lh], B[nb][lh], q6m_i4{0, 0, 0, 0}, 0, 0, 0);
-                // |D| <= 16*128*128 = 2^18, |sc| <= 2^7: four products per plane stay below 2^27
+            for (int nb = 0; nb < 2; ++nb) {
 #pragma unroll
-                for (int p = 0; p < 4; ++p) {
-                    E[p] += __mul24(D[p], sc[nb][lh]);
-                    asm("" : "+v"(E[p]));   // one multiply-add per plane: keeps the sums from being regrouped
+                for (int lh = 0; lh < 2; ++lh) {
+                    const q6m_i4 A = NC == 1 ? A1[nb][lh]
+                                             : *reinterpret_cast<const q6m_i4 *>(ab + c * cs + (4 * nb + lh) * hs);
+                    const q6m_i4 D = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, B[nb][lh], q6m_i4{0, 0, 0, 0}, 0, 0, 0);
+                    // |D| <= 16*128*128 = 2^18, |sc| <= 2^7: four products per plane stay below 2^27
+#pragma unroll
+                    for (int p = 0; p < 4; ++p) {
+                        E[p] += __mul24(D[p], sc[nb][lh]);
+                        asm("" : "+v"(E[p]));   // one multiply-add per plane: keeps the sums from being regrouped
+                    }
                 }
             }
+            const double hi = fma((double)E[3], 256.0, (double)E[2]);
+            const double lo = fma((double)E[1], 256.0, (double)E[0]);
+            const double dot = fma(hi, 65536.0, lo);
+            val[c] = q6m_row_sum((ps[c] * d) * dot);
         }
-        const double hi = fma((double)E[3], 256.0, (double)E[2]);
-        const double lo = fma((double)E[1], 256.0, (double)E[0]);
-        const double dot = fma(hi, 65536.0, lo);
-        double val = (ps * (double)lev_f16_bits_to_f32(dbits)) * dot;
-        val = q6m_row_sum(val);
-        if (lane < 16u) *reinterpret_cast<double *>(smem + pw) = val;
+        if (lane < 16u) {
+#pragma unroll
+            for (int c = 0; c < NC; ++c) *reinterpret_cast<double *>(smem + pw + 8 * c) = val[c];
+        }
         lev_barrier_lds();
         if (wave < slots) {
             const double *pp = reinterpret_cast<const double *>(smem + pr);
-            const double p0 = pp[0], p1 = pp[64], p2 = pp[128], p3 = pp[192];   // four reads in flight together
-            double s = ((k0 ? p0 : 0.0) + (k1 ? p1 : 0.0)) + ((k2 ? p2 : 0.0) + (k3 ? p3 : 0.0));
-            s = q6m_row_sum(s);
-            if (stores) {
-                const float out = (float)s;
-                *reinterpret_cast<__attribute__((address_space(1))) float *>(yp) = out;
-                // running top two of the rows this lane finishes (rows ascend, so a tie keeps the
-                // earlier, lower index)
-                if (out > best.best) {
-                    best.second = best.best;
-                    best.best = out;
-                    best.idx = orow;
-                } else if (out > best.second) {
-                    best.second = out;
+#pragma unroll
+            for (int c = 0; c < NC; ++c) {
+                const double p0 = pp[c], p1 = pp[64 * NC + c], p2 = pp[128 * NC + c], p3 = pp[192 * NC + c];
+                double s = ((k0 ? p0 : 0.0) + (k1 ? p1 : 0.0)) + ((k2 ? p2 : 0.0) + (k3 ? p3 : 0.0));
+                s = q6m_row_sum(s);
+                if (stores && (uint32_t)c < ncol) {
+                    const float out = (float)s;
+                    *reinterpret_cast<__attribute__((address_space(1))) float *>(yp + (uint64_t)c * rows * 4u) = out;
+                    if (NC == 1) {
+                        // running top two of the rows this lane finishes (rows ascend, so a tie keeps
+                        // the earlier, lower index)
+                        if (out > best.best) {
+                            best.second = best.best;
+                            best.best = out;
+                            best.idx = orow;
+                        } else if (out > best.second) {
+                            best.second = out;
+                        }
+                    }
                 }
             }
         }
-        pw ^= kQWaves * 16u * 8u;                              // the other half of `part` next round
-        pr ^= kQWaves * 16u * 8u;
+        pw ^= kQWaves * 16u * 8u * NC;                         // the other half of `part` next round
+        pr ^= kQWaves * 16u * 8u * NC;
         orow += orow_step;
         yp += (uint64_t)orow_step * 4u;
         stores = writer && orow < rows ? 1u : 0u;
@@ -851,7 +881,7 @@ q6_k_mfma_gemv_one(const uint8_t *__restrict__ w, const float *__restrict__ x, c
         if (next >= nrounds) break;
         rb = next;
     }
-    if (partials) q6m_greedy_token(best, slots, partials, tickets, out_idx, out_margin);
+    if (NC == 1 && partials) q6m_greedy_token(best, slots, partials, tickets, out_idx, out_margin);
 }
 
 // ---------------------------------------------------------------------------
@@ -1102,9 +1132,10 @@ hipError_t q6m_launch(lev_ctx *ctx, const uint8_t *w, const float *x, const floa
     return hipGetLastError();
 }
 
-template <bool NORM>
+template <int NC, bool NORM>
 hipError_t q6m_one_launch(lev_ctx *ctx, const uint8_t *w, const float *x, const float *gain, float eps, float *y,
-                          uint32_t cols, uint32_t rows, lev_f32x4 *partials, uint32_t *d_argmax, float *d_margin) {
+                          uint32_t cols, uint32_t rows, uint32_t ncol, lev_f32x4 *partials, uint32_t *d_argmax,
+                          float *d_margin) {
     const uint32_t wpr = cols >> 8, slots = (uint32_t)kQWaves / wpr;
     const uint32_t ngroups = (rows + 15u) / 16u;
     const uint32_t nrounds = (ngroups + slots - 1u) / slots;
@@ -1113,21 +1144,30 @@ hipError_t q6m_one_launch(lev_ctx *ctx, const uint8_t *w, const float *x, const 
         slot_of_wave |= (uint64_t)(wv / wpr > 15u ? 15u : wv / wpr) << (4u * wv);
         pos_of_wave |= (uint64_t)(wv % wpr) << (4u * wv);
     }
-    constexpr size_t lds = q6m_one_lds();
+    constexpr size_t lds = q6m_one_lds(NC);
     static bool configured = false;   // per instantiation: raise the dynamic LDS limit once
     if (!configured) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&q6_k_mfma_gemv_one<NORM>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&q6_k_mfma_gemv_one<NC, NORM>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
         configured = true;
     }
+    if (NC != 1) partials = nullptr;
     uint32_t blocks = nrounds < (uint32_t)ctx->num_cus ? nrounds : (uint32_t)ctx->num_cus;
     if (partials && blocks > lev_ctx::kArgmaxPartials) blocks = lev_ctx::kArgmaxPartials;
     uint32_t *tickets = partials ? reinterpret_cast<uint32_t *>(ctx->d_flag) + lev_ctx::kArgmaxTicketWord : nullptr;
-    hipLaunchKernelGGL((q6_k_mfma_gemv_one<NORM>), dim3(blocks), dim3(kQThreads), lds, ctx->stream, w, x, gain, eps, y,
-                       cols, rows, wpr, slots, slot_of_wave, pos_of_wave, 1.0 / (double)cols, partials, tickets,
-                       d_argmax, d_margin);
+    hipLaunchKernelGGL((q6_k_mfma_gemv_one<NC, NORM>), dim3(blocks), dim3(kQThreads), lds, ctx->stream, w, x, gain,
+                       eps, y, cols, rows, ncol, wpr, slots, slot_of_wave, pos_of_wave, 1.0 / (double)cols, partials,
+                       tickets, d_argmax, d_margin);
     return hipGetLastError();
+}
+
+template <int NC>
+hipError_t q6m_one_launch_nc(lev_ctx *ctx, const uint8_t *w, const float *x, const float *gain, float eps, float *y,
+                             uint32_t cols, uint32_t rows, uint32_t ncol, lev_f32x4 *partials, uint32_t *d_argmax,
+                             float *d_margin) {
+    if (gain) return q6m_one_launch<NC, true>(ctx, w, x, gain, eps, y, cols, rows, ncol, partials, d_argmax, d_margin);
+    return q6m_one_launch<NC, false>(ctx, w, x, gain, eps, y, cols, rows, ncol, partials, d_argmax, d_margin);
 }
 
 }  // namespace
@@ -1156,15 +1196,17 @@ hipError_t lev_q6_k_mfma_gemv_launch(lev_ctx *ctx, const uint8_t *w, const float
                                      uint32_t waves, lev_f32x4 *partials, uint32_t *d_argmax, float *d_margin) {
     if (!d_argmax && !d_margin) partials = nullptr;
     if (waves != 2u && waves != 4u && waves != 8u && waves != 16u) waves = 0u;
-    // one column of at most sixteen superblocks, no number of waves per row group asked for: a
-    // wave per superblock column
+    // one or two columns of at most sixteen superblocks, no number of waves per row group asked
+    // for: a wave per superblock column (four columns measured 31.5 us at 32000 x 4096 either way:
+    // a column costs its products and recombination again, and the several-column kernel stages
+    // the planes once per workgroup)
     static const bool one_off = [] {
         const char *e = getenv("LEV_Q6K_ONE");   // LEV_Q6K_ONE=0: the several-column kernel at one column too, for comparison
         return e && e[0] == '0';
     }();
-    if (ncol == 1u && waves == 0u && !one_off && in_dim <= 4096u) {
-        if (gain) return q6m_one_launch<true>(ctx, w, x, gain, eps, y, in_dim, rows, partials, d_argmax, d_margin);
-        return q6m_one_launch<false>(ctx, w, x, gain, eps, y, in_dim, rows, partials, d_argmax, d_margin);
+    if (ncol <= 2u && waves == 0u && !one_off && in_dim <= 4096u) {
+        if (ncol > 1u) return q6m_one_launch_nc<2>(ctx, w, x, gain, eps, y, in_dim, rows, ncol, partials, d_argmax, d_margin);
+        return q6m_one_launch_nc<1>(ctx, w, x, gain, eps, y, in_dim, rows, ncol, partials, d_argmax, d_margin);
     }
     if (ncol > 4) return q6m_launch<8>(ctx, w, x, gain, eps, y, in_dim, rows, ncol, waves, partials, d_argmax, d_margin);
     if (ncol > 2) return q6m_launch<4>(ctx, w, x, gain, eps, y, in_dim, rows, ncol, waves, partials, d_argmax, d_margin);
