@@ -919,9 +919,9 @@ uint32_t lev_q4_k_mfma_narrow_cols(const lev_ctx *ctx, uint32_t in_dim) {
     return 0;
 }
 
-bool lev_q4_k_mfma_one_usable(const uint8_t *w, const float *x, const float *gain, uint32_t in_dim);
+bool lev_q4_k_mfma_one_usable(const uint8_t *w, const float *x, const float *gain, uint32_t in_dim, uint32_t ncol);
 hipError_t lev_q4_k_mfma_one_launch(lev_ctx *ctx, const uint8_t *w, const float *x, const float *gain, float eps,
-                                    float *y, uint32_t in_dim, uint32_t rows);
+                                    float *y, uint32_t in_dim, uint32_t rows, uint32_t ncol);
 
 // ncol <= lev_q4_k_mfma_narrow_cols(ctx, in_dim) (the narrow kernel) or
 // ncol <= lev_q4_k_mfma_cols(ctx, in_dim); w 16-byte aligned.
@@ -933,8 +933,8 @@ hipError_t lev_q4_k_mfma_gemv_launch(lev_ctx *ctx, const uint8_t *w, const float
         const char *e = getenv("LEV_Q4K_ONE");   // LEV_Q4K_ONE=0: the narrow kernel at one column too, for comparison
         return e && e[0] == '0';
     }();
-    if (ncol == 1u && !one_off && lev_q4_k_mfma_one_usable(w, x, gain, in_dim))
-        return lev_q4_k_mfma_one_launch(ctx, w, x, gain, eps, y, in_dim, rows);
+    if (!one_off && lev_q4_k_mfma_one_usable(w, x, gain, in_dim, ncol))
+        return lev_q4_k_mfma_one_launch(ctx, w, x, gain, eps, y, in_dim, rows, ncol);
     // one column of a longer row: the narrow kernel (9.1 us against 9.7 at 12288 x 4096); two columns: only where the
     // four-column kernel's planes do not fit (it is the faster of the two there: 9.9 against 10.8 us)
     if (ncol <= lev_q4_k_mfma_narrow_cols(ctx, in_dim) && (ncol == 1u || lev_q4_k_mfma_cols(ctx, in_dim) < ncol)) {

@@ -34,16 +34,17 @@ namespace {
 
 constexpr int kOneWaves = 16;
 constexpr int kOneThreads = kOneWaves * LEV_WAVE;
-constexpr uint32_t kOnePartBytes = 2u * kOneWaves * 16u * 8u;   // [2][16 waves][16 rows] f64
-constexpr uint32_t kOneNormBytes = kOneWaves * 8u;             // a sum of squares per wave
-constexpr uint32_t kOneWaveBytes = kQ4mTaskArea + kQ4mZeroBytes;   // per wave: the staging area of its activations, a zero strip
-
-__host__ __device__ constexpr size_t q4k_one_lds() {
-    return kOnePartBytes + kOneNormBytes + (size_t)kOneWaves * kOneWaveBytes;
+// LDS for NC columns: part [2][16 waves][16 rows][NC] f64 | sums of squares [NC][16] f64 | per
+// wave: NC staging areas of its activations, a zero strip
+__host__ __device__ constexpr uint32_t q4k_one_part_bytes(uint32_t nc) { return 2u * kOneWaves * 16u * 8u * nc; }
+__host__ __device__ constexpr uint32_t q4k_one_norm_bytes(uint32_t nc) { return kOneWaves * 8u * nc; }
+__host__ __device__ constexpr uint32_t q4k_one_wave_bytes(uint32_t nc) { return nc * kQ4mTaskArea + kQ4mZeroBytes; }
+__host__ __device__ constexpr size_t q4k_one_lds(uint32_t nc) {
+    return q4k_one_part_bytes(nc) + q4k_one_norm_bytes(nc) + (size_t)kOneWaves * q4k_one_wave_bytes(nc);
 }
 
-struct q4k_one_operand {
-    lev_i32x4 a[4];     // digit planes of elements 16h .. 16h+15 of the lane group's 64 (zeros outside the group's rows)
+// What a lane keeps of one column of its wave's 256 activations besides the digit planes.
+struct q4k_one_column {
     int c1[4];          // 128 * (sum of plane p's digits over the high sub-block): undoes the -8 of its codes
     double sx0, sx1;    // sum of X over the low / high sub-block
     double ps;          // 2^(e - 4): undoes the scaling and the 16 of the codes; 0 for an idle wave, NaN for bad input
@@ -51,9 +52,9 @@ struct q4k_one_operand {
 
 #define LEV_Q4K1_DPP(v, CTRL) __builtin_amdgcn_update_dpp(0, (v), (CTRL), 0xF, 0xF, true)
 
-// Stages the wave's 256 activations (lane i: elements 4i .. 4i+3) and reads the lane's operands back.
-__device__ __forceinline__ void q4k_one_stage(const lev_f32x4 v, uint8_t *area, uint8_t *zero, bool live,
-                                              q4k_one_operand &op) {
+// Stages the wave's 256 activations of one column (lane i: elements 4i .. 4i+3) as digit planes
+// [chunk 4][plane 4][half 4][16 B] in `area` (1 KB, the wave's own).
+__device__ __forceinline__ void q4k_one_stage(const lev_f32x4 v, uint8_t *area, bool live, q4k_one_column &op) {
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t r = lane & 15u, g = lane >> 4;
     uint32_t mb = 0u;
@@ -129,17 +130,6 @@ __device__ __forceinline__ void q4k_one_stage(const lev_f32x4 v, uint8_t *area, 
     uint8_t *at = area + g * 256u + (r >> 2) * 16u + (r & 3u) * 4u;
 #pragma unroll
     for (int p = 0; p < 4; ++p) *reinterpret_cast<uint32_t *>(at + 64 * p) = dw[p];
-    if (lane < kQ4mZeroBytes / 4u) reinterpret_cast<uint32_t *>(zero)[lane] = 0u;
-    // the area belongs to this wave alone: LDS runs a wave's accesses in order, the fences only
-    // keep the compiler from moving the reads above the writes
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    const bool feeds = live && (r >> 2) == g;                  // A row r belongs to lane group r / 4
-    const uint8_t *ab = feeds ? area + g * 256u + (r & 3u) * 64u : zero;
-    const uint32_t hs = feeds ? 16u : 0u;
-#pragma unroll
-    for (int h = 0; h < 4; ++h) op.a[h] = *reinterpret_cast<const lev_i32x4 *>(ab + h * hs);
 }
 
 // Sum over lanes l, l ^ 16, l ^ 32, l ^ 48 in every lane, in f64, by row swaps.
@@ -155,11 +145,18 @@ __device__ __forceinline__ double q4k_one_row_sum(double v) {
     return __hiloint2double((int)a1[0], (int)a0[0]) + __hiloint2double((int)a1[1], (int)a0[1]);
 }
 
-// Contribution of chunk g of row r (hdr: the superblock's first 16 bytes, c: the chunk's 32 code
-// bytes) to the row's dot product.
-__device__ __forceinline__ double q4k_one_dot(const lev_i32x4 hdr, const lev_i32x4 ca, const lev_i32x4 cb,
-                                              const q4k_one_operand &op, uint32_t g) {
+// Chunk g of row r as the products want it (hdr: the superblock's first 16 bytes, ca / cb: the
+// chunk's 32 code bytes).
+struct q4k_one_weights {
+    lev_i32x4 la, lb, ha, hb;   // B operands: low nibbles as q, high nibbles as 16 * (q - 8)
+    int sc0, sc1;               // scales of sub-blocks 2g (x 16: the high sub-block's codes carry a 16) and 2g + 1
+    double m0, m1, d, dmin;
+};
+
+__device__ __forceinline__ q4k_one_weights q4k_one_unpack(const lev_i32x4 hdr, const lev_i32x4 ca, const lev_i32x4 cb,
+                                                          uint32_t g) {
     typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+    q4k_one_weights W;
     // unpack_scale_min (lev-cpu/src/lib.rs:64-74), four sub-blocks a word; this lane wants sub-blocks
     // 2g and 2g + 1: bytes 2 * (g % 2) and + 1 of word g / 2
     const uint32_t S0 = (uint32_t)hdr[1], S1 = (uint32_t)hdr[2], S2 = (uint32_t)hdr[3];
@@ -170,40 +167,49 @@ __device__ __forceinline__ double q4k_one_dot(const lev_i32x4 hdr, const lev_i32
     const uint32_t scw = (sc_hi & up) | (sc_lo & ~up);
     const uint32_t mnw = (mn_hi & up) | (mn_lo & ~up);
     const uint32_t sh = 16u * (g & 1u);
-    const int sc0 = (int)__builtin_amdgcn_ubfe(scw, sh, 8u) * 16;        // the high sub-block's codes carry a 16
-    const int sc1 = (int)__builtin_amdgcn_ubfe(scw, sh + 8u, 8u);
-    const double m0 = (double)__builtin_amdgcn_ubfe(mnw, sh, 8u);
-    const double m1 = (double)__builtin_amdgcn_ubfe(mnw, sh + 8u, 8u);
+    W.sc0 = (int)__builtin_amdgcn_ubfe(scw, sh, 8u) * 16;
+    W.sc1 = (int)__builtin_amdgcn_ubfe(scw, sh + 8u, 8u);
+    W.m0 = (double)__builtin_amdgcn_ubfe(mnw, sh, 8u);
+    W.m1 = (double)__builtin_amdgcn_ubfe(mnw, sh + 8u, 8u);
     const u4 qa = __builtin_bit_cast(u4, ca), qb = __builtin_bit_cast(u4, cb);
-    const lev_i32x4 la = __builtin_bit_cast(lev_i32x4, qa & 0x0F0F0F0Fu);
-    const lev_i32x4 lb = __builtin_bit_cast(lev_i32x4, qb & 0x0F0F0F0Fu);
-    const lev_i32x4 ha = __builtin_bit_cast(lev_i32x4, (qa & 0xF0F0F0F0u) ^ 0x80808080u);
-    const lev_i32x4 hb = __builtin_bit_cast(lev_i32x4, (qb & 0xF0F0F0F0u) ^ 0x80808080u);
-    lev_i32x4 d0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(op.a[0], la, lev_i32x4{0, 0, 0, 0}, 0, 0, 0);
-    lev_i32x4 d1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(op.a[2], ha, lev_i32x4{0, 0, 0, 0}, 0, 0, 0);
-    d0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(op.a[1], lb, d0, 0, 0, 0);
-    d1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(op.a[3], hb, d1, 0, 0, 0);
+    W.la = __builtin_bit_cast(lev_i32x4, qa & 0x0F0F0F0Fu);
+    W.lb = __builtin_bit_cast(lev_i32x4, qb & 0x0F0F0F0Fu);
+    W.ha = __builtin_bit_cast(lev_i32x4, (qa & 0xF0F0F0F0u) ^ 0x80808080u);
+    W.hb = __builtin_bit_cast(lev_i32x4, (qb & 0xF0F0F0F0u) ^ 0x80808080u);
+    W.d = (double)lev_f16_bits_to_f32((uint32_t)hdr[0] & 0xFFFFu);
+    W.dmin = (double)lev_f16_bits_to_f32((uint32_t)hdr[0] >> 16);
+    return W;
+}
+
+// Contribution of the chunk to the row's dot product with one column (a: the column's A operands,
+// elements 16h .. 16h+15 of the lane group's 64, zeros outside the group's rows).
+__device__ __forceinline__ double q4k_one_dot(const q4k_one_weights &W, const lev_i32x4 (&a)[4], const q4k_one_column &op) {
+    lev_i32x4 d0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[0], W.la, lev_i32x4{0, 0, 0, 0}, 0, 0, 0);
+    lev_i32x4 d1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[2], W.ha, lev_i32x4{0, 0, 0, 0}, 0, 0, 0);
+    d0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[1], W.lb, d0, 0, 0, 0);
+    d1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[3], W.hb, d1, 0, 0, 0);
     // |d0| < 2^16, |d1 + c1| < 2^20, scales below 2^10: every product and sum fits 32 bits
     int E[4];
 #pragma unroll
-    for (int p = 0; p < 4; ++p) E[p] = __mul24(d0[p], sc0) + __mul24(d1[p] + op.c1[p], sc1);
+    for (int p = 0; p < 4; ++p) E[p] = __mul24(d0[p], W.sc0) + __mul24(d1[p] + op.c1[p], W.sc1);
     // plane 3 is the highest digit (at most 2 in magnitude): E[3] * 256 + E[2] stays below 2^29
     const double hi = (double)(E[3] * 256 + E[2]);
     const double lo = fma((double)E[1], 256.0, (double)E[0]);
     const double dot = fma(hi, 65536.0, lo);                             // 16 * sum_j sc_j sum_k q_k X_k
-    const double mins = fma(m1, op.sx1, m0 * op.sx0) * 16.0;
-    const double d = (double)lev_f16_bits_to_f32((uint32_t)hdr[0] & 0xFFFFu);
-    const double dmin = (double)lev_f16_bits_to_f32((uint32_t)hdr[0] >> 16);
-    return op.ps * fma(d, dot, -dmin * mins);
+    const double mins = fma(W.m1, op.sx1, W.m0 * op.sx0) * 16.0;
+    return op.ps * fma(W.d, dot, -W.dmin * mins);
 }
 
 // wave -> (slot, superblock) as 4-bit entries of two 64-bit kernel arguments (no division in
-// front of the first load).  NORM: RMSNorm (gain != nullptr) in front.
-template <bool NORM>
+// front of the first load).  NC: columns staged (1, 2 or 4; >= ncol): one column keeps its A
+// operands in registers, several read them from the wave's planes at every product.
+// NORM: RMSNorm (gain != nullptr) in front.
+template <int NC, bool NORM>
 __global__ void __launch_bounds__(kOneThreads)
 q4_k_mfma_gemv_one(const uint8_t *__restrict__ w, const float *__restrict__ x, const float *__restrict__ gain,
-                   float eps, float *__restrict__ y, uint32_t cols, uint32_t rows, uint32_t wpr, uint32_t slots,
-                   uint64_t slot_of_wave, uint64_t pos_of_wave, double rcols) {
+                   float eps, float *__restrict__ y, uint32_t cols, uint32_t rows, uint32_t ncol, uint32_t wpr,
+                   uint32_t slots, uint64_t slot_of_wave, uint64_t pos_of_wave, double rcols) {
+    constexpr uint32_t kPart = q4k_one_part_bytes(NC), kNorm = q4k_one_norm_bytes(NC), kWave = q4k_one_wave_bytes(NC);
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
@@ -211,16 +217,22 @@ q4_k_mfma_gemv_one(const uint8_t *__restrict__ w, const float *__restrict__ x, c
     const uint32_t sb = (uint32_t)(pos_of_wave >> (4u * wave)) & 15u;      // the wave's superblock column
     const uint32_t SB = cols >> 8;
 
-    // the wave's activations first (short, mostly L2 hits) ...
-    lev_f32x4 v = reinterpret_cast<const lev_f32x4 *>(x)[64u * sb + lane];
+    // the wave's activations first (short, mostly L2 hits; columns of the layout beyond ncol
+    // repeat the last one and are never stored) ...
+    lev_f32x4 v[NC];
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+        const uint32_t cc = (uint32_t)c < ncol ? (uint32_t)c : ncol - 1u;
+        v[c] = reinterpret_cast<const lev_f32x4 *>(x + (uint64_t)cc * cols)[64u * sb + lane];
+    }
     lev_f32x4 gn;
     if (NORM) gn = reinterpret_cast<const lev_f32x4 *>(gain)[64u * sb + lane];
-    // ... the first two row groups' weights right behind them
+    // ... the first row group's weights right behind them
     const bool active = slot < slots;
     const uint64_t row_bytes = (uint64_t)SB * 144u;
     const uint32_t ngroups = (rows + 15u) >> 4;
     const uint32_t nrounds = (ngroups + slots - 1u) / slots;     // rounds of `slots` row groups
-    const uint32_t lrow = lane >> 2;                             // fetch order: lane = 4 * row + quarter
+    const uint32_t lrow = lane >> 2;                             // fetch order: lane = 4 * row + chunk
     auto issue = [&](uint32_t round_block, uint32_t (&D)[9]) {
         uint32_t rg = round_block * slots + (active ? slot : 0u);
         rg = rg < ngroups ? rg : ngroups - 1u;
@@ -237,7 +249,7 @@ q4_k_mfma_gemv_one(const uint8_t *__restrict__ w, const float *__restrict__ x, c
         D[1] = a.x; D[2] = a.y; D[3] = a.z; D[4] = a.w;
         D[5] = b.x; D[6] = b.y; D[7] = b.z; D[8] = b.w;
     };
-    uint32_t Da[9], Db[9];
+    uint32_t D[9];
     uint32_t rb = blockIdx.x;
     if (NORM) {
         // A CU's memory pipeline is one queue: without this barrier the activations of the last
@@ -247,17 +259,18 @@ q4_k_mfma_gemv_one(const uint8_t *__restrict__ w, const float *__restrict__ x, c
         asm volatile("s_barrier" ::: "memory");
         __builtin_amdgcn_sched_barrier(0);
     }
-    issue(rb, Da);
+    issue(rb, D);
 
     // ---- everything the tail of a round needs, while the loads are on their way ----
-    double *norm = reinterpret_cast<double *>(smem + kOnePartBytes);
-    uint8_t *area = smem + kOnePartBytes + kOneNormBytes + (size_t)wave * kOneWaveBytes;
+    double *norm = reinterpret_cast<double *>(smem + kPart);
+    uint8_t *area = smem + kPart + kNorm + (size_t)wave * kWave;
+    uint8_t *zero = area + NC * kQ4mTaskArea;
     const uint32_t r = lane & 15u, q = lane >> 4;
     // byte offsets into the workgroup's LDS, not pointers (an address that has been through an
     // integer register is no longer known to be LDS)
-    uint32_t pw = (wave * 16u + lane) * 8u;
+    uint32_t pw = ((wave * 16u + lane) * NC) * 8u;
     // wave s < slots adds the wpr partial sums of slot s: lane (r, q) reads waves q, q + 4, q + 8, q + 12
-    uint32_t pr = (((wave < slots ? wave : 0u) * wpr + q) * 16u + r) * 8u;
+    uint32_t pr = ((((wave < slots ? wave : 0u) * wpr + q) * 16u + r) * NC) * 8u;
     uint32_t k0 = q < wpr ? 1u : 0u, k1 = q + 4u < wpr ? 1u : 0u, k2 = q + 8u < wpr ? 1u : 0u,
              k3 = q + 12u < wpr ? 1u : 0u;
     uint32_t orow = (rb * slots + wave) * 16u + r;
@@ -277,31 +290,58 @@ q4_k_mfma_gemv_one(const uint8_t *__restrict__ w, const float *__restrict__ x, c
     if (NORM) {
         // RMSNorm as the reference computes it (rmsnorm, rust/crates/lev-model/src/lib.rs:110-114):
         // mean square and 1/sqrt in f64, then (f32)(x * inv) * gain
-        double ss = (double)v.x * (double)v.x;
-        ss = fma((double)v.y, (double)v.y, ss);
-        ss = fma((double)v.z, (double)v.z, ss);
-        ss = fma((double)v.w, (double)v.w, ss);
-        ss = lev_group_sum_f64<64>(ss);                        // lane 63 holds the wave's sum
-        if (lane == 63u) norm[wave] = ss;
-        lev_barrier_lds();
-        // the waves of slot 0 cover the row once: lane k of every row of 16 lanes takes wave k's
-        // sum, and the row adds them up (every lane ends with the total)
-        const double mine = norm[r];
-        const double tot = lev_group_sum_f64<16>(r < wpr ? mine : 0.0);
-        // 1/sqrt(mean + eps): the hardware estimate and two Newton steps (full f64 accuracy)
-        const double a = fma(tot, rcols, (double)eps);
-        double rs = __builtin_amdgcn_rsq(a);
-        rs = rs * fma(-0.5 * a * rs, rs, 1.5);
-        rs = rs * fma(-0.5 * a * rs, rs, 1.5);
 #pragma unroll
-        for (int k = 0; k < 4; ++k) v[k] = (float)((double)v[k] * rs) * gn[k];
+        for (int c = 0; c < NC; ++c) {
+            double ss = (double)v[c].x * (double)v[c].x;
+            ss = fma((double)v[c].y, (double)v[c].y, ss);
+            ss = fma((double)v[c].z, (double)v[c].z, ss);
+            ss = fma((double)v[c].w, (double)v[c].w, ss);
+            ss = lev_group_sum_f64<64>(ss);                    // lane 63 holds the wave's sum
+            if (lane == 63u) norm[c * kOneWaves + wave] = ss;
+        }
+        lev_barrier_lds();
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            // the waves of slot 0 cover the row once: lane k of every row of 16 lanes takes wave k's
+            // sum, and the row adds them up (every lane ends with the total)
+            const double mine = norm[c * kOneWaves + r];
+            const double tot = lev_group_sum_f64<16>(r < wpr ? mine : 0.0);
+            // 1/sqrt(mean + eps): the hardware estimate and two Newton steps (full f64 accuracy)
+            const double a = fma(tot, rcols, (double)eps);
+            double rs = __builtin_amdgcn_rsq(a);
+            rs = rs * fma(-0.5 * a * rs, rs, 1.5);
+            rs = rs * fma(-0.5 * a * rs, rs, 1.5);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) v[c][k] = (float)((double)v[c][k] * rs) * gn[k];
+        }
     }
-    q4k_one_operand op;
-    q4k_one_stage(v, area, area + kQ4mTaskArea, active, op);
+    q4k_one_column op[NC];
+#pragma unroll
+    for (int c = 0; c < NC; ++c) q4k_one_stage(v[c], area + c * kQ4mTaskArea, active, op[c]);
+    if (lane < kQ4mZeroBytes / 4u) reinterpret_cast<uint32_t *>(zero)[lane] = 0u;
+    // the areas belong to this wave alone: LDS runs a wave's accesses in order, the fences only
+    // keep the compiler from moving the reads above the writes
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const bool feeds = active && (r >> 2) == q;                // A row r belongs to lane group r / 4
+    const uint8_t *ab = feeds ? area + q * 256u + (r & 3u) * 64u : zero;
+    const uint32_t hs = feeds ? 16u : 0u, cs = feeds ? kQ4mTaskArea : 0u;
+    lev_i32x4 a1[4];
+    if (NC == 1) {
+#pragma unroll
+        for (int h = 0; h < 4; ++h) a1[h] = *reinterpret_cast<const lev_i32x4 *>(ab + h * hs);
+    }
     // the operands are read back before the wait for the weights, not behind it
     __builtin_amdgcn_sched_barrier(0);
 
-    auto finish = [&](const uint32_t (&D)[9]) {
+    // A round: the fetched dwords go to the lanes that multiply them, and the registers they came
+    // in take the NEXT round's request at once (one round ahead and no more: with a second round
+    // requested before the first is multiplied the same matrix streams in slower, 8.4 us against
+    // 7.9 at 12288 x 4096; a workgroup walking adjacent rounds instead of rounds a grid apart: 8.1).
+    // The request is unconditional (clamped): a branch around the loads would make the compiler
+    // wait for them before the current group is multiplied.
+    auto round = [&](uint32_t next_block) {
         // lane (r, q) <- lane 4r + q for the chunk, lanes 4r .. 4r + 3 for the header's four dwords
         lev_i32x4 hdr, ca, cb;
 #pragma unroll
@@ -312,45 +352,58 @@ q4_k_mfma_gemv_one(const uint8_t *__restrict__ w, const float *__restrict__ x, c
             ca[k] = __builtin_amdgcn_ds_bpermute(src, (int)D[1 + k]);
             cb[k] = __builtin_amdgcn_ds_bpermute(src, (int)D[5 + k]);
         }
-        double val = q4k_one_dot(hdr, ca, cb, op, q);
-        val = q4k_one_row_sum(val);
-        if (lane < 16u) *reinterpret_cast<double *>(smem + pw) = val;
+        // (the scheduling barriers keep the request where it is written: sunk below the products
+        // it would no longer run ahead of anything)
+        __builtin_amdgcn_sched_barrier(0);
+        issue(next_block, D);
+        __builtin_amdgcn_sched_barrier(0);
+        const q4k_one_weights W = q4k_one_unpack(hdr, ca, cb, q);
+        double val[NC];
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            if (NC == 1) {
+                val[c] = q4k_one_dot(W, a1, op[c]);
+            } else {
+                lev_i32x4 a[4];
+#pragma unroll
+                for (int h = 0; h < 4; ++h) a[h] = *reinterpret_cast<const lev_i32x4 *>(ab + c * cs + h * hs);
+                val[c] = q4k_one_dot(W, a, op[c]);
+            }
+            val[c] = q4k_one_row_sum(val[c]);
+        }
+        if (lane < 16u) {
+#pragma unroll
+            for (int c = 0; c < NC; ++c) *reinterpret_cast<double *>(smem + pw + 8 * c) = val[c];
+        }
         lev_barrier_lds();
         if (wave < slots) {
             const double *pp = reinterpret_cast<const double *>(smem + pr);
-            const double p0 = pp[0], p1 = pp[64], p2 = pp[128], p3 = pp[192];   // four reads in flight together
-            double s = ((k0 ? p0 : 0.0) + (k1 ? p1 : 0.0)) + ((k2 ? p2 : 0.0) + (k3 ? p3 : 0.0));
-            s = q4k_one_row_sum(s);
-            if (stores) *reinterpret_cast<__attribute__((address_space(1))) float *>(yp) = (float)s;
+#pragma unroll
+            for (int c = 0; c < NC; ++c) {
+                const double p0 = pp[c], p1 = pp[64 * NC + c], p2 = pp[128 * NC + c], p3 = pp[192 * NC + c];
+                double s = ((k0 ? p0 : 0.0) + (k1 ? p1 : 0.0)) + ((k2 ? p2 : 0.0) + (k3 ? p3 : 0.0));
+                s = q4k_one_row_sum(s);
+                if (stores && (uint32_t)c < ncol)
+                    *reinterpret_cast<__attribute__((address_space(1))) float *>(yp + (uint64_t)c * rows * 4u) = (float)s;
+            }
         }
-        pw ^= kOneWaves * 16u * 8u;                            // the other half of `part` next round
-        pr ^= kOneWaves * 16u * 8u;
+        pw ^= kOneWaves * 16u * 8u * NC;                       // the other half of `part` next round
+        pr ^= kOneWaves * 16u * 8u * NC;
         orow += orow_step;
         yp += (uint64_t)orow_step * 4u;
         stores = writer && orow < rows ? 1u : 0u;
     };
-    // Unconditional (clamped) prefetch: a branch around the loads would make the compiler wait
-    // for them before the current group is multiplied.  One round ahead and no more: with a
-    // second round requested before the first is multiplied the same matrix streams in slower
-    // (8.4 us against 7.9 at 12288 x 4096; a workgroup walking adjacent rounds instead of rounds a
-    // grid apart: 8.1).
     while (true) {
-        uint32_t next = rb + gridDim.x;
-        issue(next < nrounds ? next : rb, Db);
-        finish(Da);
-        if (next >= nrounds) break;
-        rb = next;
-        next = rb + gridDim.x;
-        issue(next < nrounds ? next : rb, Da);
-        finish(Db);
+        const uint32_t next = rb + gridDim.x;
+        round(next < nrounds ? next : rb);
         if (next >= nrounds) break;
         rb = next;
     }
 }
 
-template <bool NORM>
+template <int NC, bool NORM>
 hipError_t launch_one(lev_ctx *ctx, const uint8_t *w, const float *x, const float *gain, float eps, float *y,
-                      uint32_t cols, uint32_t rows) {
+                      uint32_t cols, uint32_t rows, uint32_t ncol) {
     const uint32_t wpr = cols >> 8, slots = (uint32_t)kOneWaves / wpr;
     const uint32_t ngroups = (rows + 15u) / 16u;
     const uint32_t nrounds = (ngroups + slots - 1u) / slots;
@@ -359,24 +412,44 @@ hipError_t launch_one(lev_ctx *ctx, const uint8_t *w, const float *x, const floa
         slot_of_wave |= (uint64_t)(wv / wpr > 15u ? 15u : wv / wpr) << (4u * wv);
         pos_of_wave |= (uint64_t)(wv % wpr) << (4u * wv);
     }
+    constexpr size_t lds = q4k_one_lds(NC);
+    if (lds > 48u * 1024u) {
+        static bool configured = false;   // per instantiation: raise the dynamic LDS limit once
+        if (!configured) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&q4_k_mfma_gemv_one<NC, NORM>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (e != hipSuccess) return e;
+            configured = true;
+        }
+    }
     const uint32_t cus = (uint32_t)ctx->num_cus;
     const uint32_t blocks = nrounds < cus ? nrounds : cus;
-    static_assert(q4k_one_lds() <= 48u * 1024u, "fits the default dynamic LDS limit");
-    hipLaunchKernelGGL((q4_k_mfma_gemv_one<NORM>), dim3(blocks), dim3(kOneThreads), q4k_one_lds(), ctx->stream, w, x,
-                       gain, eps, y, cols, rows, wpr, slots, slot_of_wave, pos_of_wave, 1.0 / (double)cols);
+    hipLaunchKernelGGL((q4_k_mfma_gemv_one<NC, NORM>), dim3(blocks), dim3(kOneThreads), lds, ctx->stream, w, x, gain,
+                       eps, y, cols, rows, ncol, wpr, slots, slot_of_wave, pos_of_wave, 1.0 / (double)cols);
     return hipGetLastError();
+}
+
+template <int NC>
+hipError_t launch_one_nc(lev_ctx *ctx, const uint8_t *w, const float *x, const float *gain, float eps, float *y,
+                         uint32_t cols, uint32_t rows, uint32_t ncol) {
+    if (gain) return launch_one<NC, true>(ctx, w, x, gain, eps, y, cols, rows, ncol);
+    return launch_one<NC, false>(ctx, w, x, gain, eps, y, cols, rows, ncol);
 }
 
 }  // namespace
 
-// Shapes the one-column kernel takes: rows of one to sixteen whole superblocks.
-bool lev_q4_k_mfma_one_usable(const uint8_t *w, const float *x, const float *gain, uint32_t in_dim) {
-    return in_dim % 256u == 0u && in_dim != 0u && in_dim <= 4096u && (reinterpret_cast<uintptr_t>(w) & 3u) == 0u &&
+// Shapes the kernel takes: one column, rows of one to sixteen whole superblocks.  (The kernel is
+// written for NC columns, and two and four were measured at 12288 x 4096: 10.1 and 14.8 us against
+// the 9.9 and 11.3 of q4_k_mfma_gemv, whose products carry four columns each.  Here a column costs
+// its four products and some 75 vector instructions a round again, and with sixteen waves a CU
+// the instruction count of a round, not the weight stream, then sets the time.)
+bool lev_q4_k_mfma_one_usable(const uint8_t *w, const float *x, const float *gain, uint32_t in_dim, uint32_t ncol) {
+    return ncol == 1u && in_dim % 256u == 0u && in_dim != 0u && in_dim <= 4096u &&
+           (reinterpret_cast<uintptr_t>(w) & 3u) == 0u &&
            ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(gain)) & 15u) == 0u;
 }
 
 hipError_t lev_q4_k_mfma_one_launch(lev_ctx *ctx, const uint8_t *w, const float *x, const float *gain, float eps,
-                                    float *y, uint32_t in_dim, uint32_t rows) {
-    if (gain) return launch_one<true>(ctx, w, x, gain, eps, y, in_dim, rows);
-    return launch_one<false>(ctx, w, x, gain, eps, y, in_dim, rows);
+                                    float *y, uint32_t in_dim, uint32_t rows, uint32_t ncol) {
+    return launch_one_nc<1>(ctx, w, x, gain, eps, y, in_dim, rows, ncol);
 }

@@ -869,14 +869,20 @@ q6_k_mfma_gemv_one(const uint8_t *__restrict__ w, const float *__restrict__ x, c
     };
     // Unconditional (clamped) prefetch, one round ahead (a branch around the loads would make the
     // compiler wait for them before the current group is multiplied).
+    // (The scheduling barriers keep the requests where they are written: sunk below the products
+    // of the round in hand they would no longer run ahead of anything.)
     while (true) {
         uint32_t next = rb + gridDim.x;
+        __builtin_amdgcn_sched_barrier(0);
         issue(next < nrounds ? next : rb, Wb);
+        __builtin_amdgcn_sched_barrier(0);
         finish(Wa);
         if (next >= nrounds) break;
         rb = next;
         next = rb + gridDim.x;
+        __builtin_amdgcn_sched_barrier(0);
         issue(next < nrounds ? next : rb, Wa);
+        __builtin_amdgcn_sched_barrier(0);
         finish(Wb);
         if (next >= nrounds) break;
         rb = next;
