@@ -1080,6 +1080,177 @@ q6_k_mfma_gemv_q8(const uint8_t *__restrict__ w, const uint32_t *__restrict__ xq
     }
 }
 
+// ---------------------------------------------------------------------------
+// Int8 activations, up to eight columns, rows of at most sixteen superblocks: a wave per
+// superblock COLUMN of the matrix, as q6_k_mfma_gemv_one.  The A operands are the activation
+// codes as they lie in memory (16 consecutive codes of one column), so a lane loads the ones of
+// its wave's superblock straight into registers, with the quarter activation scales of its
+// blocks beside them: nothing is staged in LDS but the turn-round of the weights and the
+// partial sums of a round.
+// LDS: part [2][16 waves][16 rows][NC] f32 | per wave: the turn-round area.
+// ---------------------------------------------------------------------------
+__host__ __device__ constexpr uint32_t q6m_q8_one_part_bytes(uint32_t nc) { return 2u * kQWaves * 16u * 4u * nc; }
+__host__ __device__ constexpr size_t q6m_q8_one_lds(uint32_t nc) {
+    return q6m_q8_one_part_bytes(nc) + (size_t)kQWaves * kQAreaBytes;
+}
+
+// NC: columns staged (4 or 8; >= ncol).
+template <int NC>
+__global__ void __launch_bounds__(kQThreads)
+q6_k_mfma_gemv_q8_one(const uint8_t *__restrict__ w, const uint32_t *__restrict__ xq, const float *__restrict__ xs,
+                      float *__restrict__ y, uint32_t cols, uint32_t rows, uint32_t ncol, uint32_t wpr, uint32_t slots,
+                      uint64_t slot_of_wave, uint64_t pos_of_wave) {
+    constexpr int NCH = NC / 4;
+    constexpr uint32_t kPart = q6m_q8_one_part_bytes(NC);
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    const uint32_t slot = (uint32_t)(slot_of_wave >> (4u * wave)) & 15u;   // idle waves: slot >= slots
+    const uint32_t sb = (uint32_t)(pos_of_wave >> (4u * wave)) & 15u;      // the wave's superblock column
+    const uint32_t SB = cols >> 8, nblk = cols >> 5;
+    const uint32_t r = lane & 15u, q = lane >> 4;
+    const uint32_t hf = q >> 1, jb = q & 1u;
+    const bool active = slot < slots;
+
+    // the wave's activations first: lane (r, g) feeds A row r = 4*gs + c, i.e. column 4*ch + r%4,
+    // the 16 codes of weight group 16*sb + 8*hf + 2*jb (+ 4*nb + lh), when gs == g, zeros
+    // otherwise (columns of the layout beyond ncol repeat the last one and are never stored)
+    q6m_i4 A[NCH][2][2];
+    float dx[NCH][2][4];   // a quarter of the activation scale (the codes in the operand are 4*(q - 32)) of block nb, column 4*ch + i
+    const uint32_t blk0 = 8u * sb + 4u * hf + jb;   // 32-activation block of nb = 0; nb = 1: + 2
+#pragma unroll
+    for (int ch = 0; ch < NCH; ++ch) {
+        const uint32_t ca = 4u * (uint32_t)ch + (r & 3u);
+        const uint8_t *xa = reinterpret_cast<const uint8_t *>(xq) + (uint64_t)(ca < ncol ? ca : ncol - 1u) * cols +
+                            256u * sb + (8u * hf + 2u * jb) * 16u;
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb) {
+#pragma unroll
+            for (int lh = 0; lh < 2; ++lh) A[ch][nb][lh] = *reinterpret_cast<const q6m_i4 *>(xa + (4 * nb + lh) * 16);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t ci = 4u * (uint32_t)ch + (uint32_t)i;
+                dx[ch][nb][i] = xs[((uint64_t)(ci < ncol ? ci : ncol - 1u) * nblk + blk0 + 2u * (uint32_t)nb) * 2u];
+            }
+        }
+    }
+    // ... the first row group's weights right behind them
+    const uint64_t row_bytes = (uint64_t)SB * 210u;
+    const uint32_t ngroups = (rows + 15u) >> 4;
+    const uint32_t nrounds = (ngroups + slots - 1u) / slots;     // rounds of `slots` row groups
+    const uint32_t odd = sb & 1u;
+    const int32_t poff = q6m_piece_offset(lane, odd);
+    auto issue = [&](uint32_t round_block, q6m_regs &W) {
+        uint32_t rg = round_block * slots + (active ? slot : 0u);
+        rg = rg < ngroups ? rg : ngroups - 1u;
+        q6m_issue(w, row_bytes, rg * 16u, rows, sb, lane, poff, W);
+    };
+    q6m_regs Wa, Wb;
+    uint32_t rb = blockIdx.x;
+    issue(rb, Wa);
+
+    // ---- everything the tail of a round needs, while the loads are on their way ----
+    uint32_t pw = ((wave * 16u + r) * NC + q) * 4u;              // lane (r, q): row r, column q (+ 4 per chunk)
+    uint32_t pr = ((((wave < slots ? wave : 0u) * wpr) * 16u + r) * NC + q) * 4u;
+    uint32_t orow = (rb * slots + wave) * 16u + r;
+    const uint32_t orow_step = gridDim.x * slots * 16u;
+    const bool writer = wave < slots;
+    uint32_t stores = writer && orow < rows ? 1u : 0u;
+    uint64_t yp = reinterpret_cast<uint64_t>(y + (uint64_t)q * rows + orow);
+    q6m_pin(pw);
+    q6m_pin(pr);
+    q6m_pin(stores);
+    q6m_pin(yp);
+    const bool feeds = active && (r >> 2) == q;
+#pragma unroll
+    for (int ch = 0; ch < NCH; ++ch)
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb) {
+#pragma unroll
+            for (int lh = 0; lh < 2; ++lh) A[ch][nb][lh] = feeds ? A[ch][nb][lh] : q6m_i4{0, 0, 0, 0};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) dx[ch][nb][i] *= active ? 0.25f : 0.f;
+        }
+    const q6m_lane L6(smem + kPart, wave, lane, odd);
+    __builtin_amdgcn_sched_barrier(0);
+
+    auto finish = [&](const q6m_regs &W) {
+        q6m_i4 B[2][2];
+        int sc[2][2];
+        uint32_t dbits;
+        L6.operands(W, B, sc, dbits);
+        const float d = lev_f16_bits_to_f32(dbits);
+#pragma unroll
+        for (int ch = 0; ch < NCH; ++ch) {
+            float v[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int nb = 0; nb < 2; ++nb) {
+                const q6m_i4 D0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[ch][nb][0], B[nb][0], q6m_i4{0, 0, 0, 0}, 0, 0, 0);
+                const q6m_i4 D1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[ch][nb][1], B[nb][1], q6m_i4{0, 0, 0, 0}, 0, 0, 0);
+                // |D| <= 16*128*127 < 2^18, |sc| <= 2^7: the sum of the two halves fits 32 bits
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    int E = __mul24(D0[i], sc[nb][0]);
+                    E += __mul24(D1[i], sc[nb][1]);
+                    v[i] = fmaf((float)E, dx[ch][nb][i], v[i]);
+                }
+            }
+            // the four lane groups' shares of a row meet, lane group g keeping column 4*ch + g: two
+            // exchanges between the halves of the wave, one between the rows of a half
+            {
+                auto s02 = __builtin_amdgcn_permlane32_swap(__float_as_uint(v[0]), __float_as_uint(v[2]), false, false);
+                auto s13 = __builtin_amdgcn_permlane32_swap(__float_as_uint(v[1]), __float_as_uint(v[3]), false, false);
+                // lower half: columns 0 and 1 (own + the upper half's); upper half: columns 2 and 3
+                const float a = __uint_as_float(s02[0]) + __uint_as_float(s02[1]);
+                const float b = __uint_as_float(s13[0]) + __uint_as_float(s13[1]);
+                auto sab = __builtin_amdgcn_permlane16_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+                const float mine = __uint_as_float(sab[0]) + __uint_as_float(sab[1]);
+                *reinterpret_cast<float *>(smem + pw + 16 * ch) = d * mine;
+            }
+        }
+        lev_barrier_lds();
+        if (wave < slots) {
+            const float *pp = reinterpret_cast<const float *>(smem + pr);
+#pragma unroll
+            for (int ch = 0; ch < NCH; ++ch) {
+                // the slot's waves in order, four chains added at the end (sixteen reads in flight)
+                float s4[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int k = 0; k < kQWaves; ++k) {
+                    const float pk = pp[k * 16 * NC + 4 * ch];
+                    s4[k & 3] += (uint32_t)k < wpr ? pk : 0.f;
+                }
+                const float s = (s4[0] + s4[1]) + (s4[2] + s4[3]);
+                if (stores && 4u * (uint32_t)ch + q < ncol)
+                    *reinterpret_cast<__attribute__((address_space(1))) float *>(yp + (uint64_t)(4 * ch) * rows * 4u) = s;
+            }
+        }
+        pw ^= kQWaves * 16u * 4u * NC;                         // the other half of `part` next round
+        pr ^= kQWaves * 16u * 4u * NC;
+        orow += orow_step;
+        yp += (uint64_t)orow_step * 4u;
+        stores = writer && orow < rows ? 1u : 0u;
+    };
+    // Unconditional (clamped) prefetch, one round ahead; the scheduling barriers keep the requests
+    // where they are written.
+    while (true) {
+        uint32_t next = rb + gridDim.x;
+        __builtin_amdgcn_sched_barrier(0);
+        issue(next < nrounds ? next : rb, Wb);
+        __builtin_amdgcn_sched_barrier(0);
+        finish(Wa);
+        if (next >= nrounds) break;
+        rb = next;
+        next = rb + gridDim.x;
+        __builtin_amdgcn_sched_barrier(0);
+        issue(next < nrounds ? next : rb, Wa);
+        __builtin_amdgcn_sched_barrier(0);
+        finish(Wb);
+        if (next >= nrounds) break;
+        rb = next;
+    }
+}
+
 size_t q6m_lds_limit(const lev_ctx *ctx) {
     return ctx->props.sharedMemPerBlockOptin > ctx->props.sharedMemPerBlock ? ctx->props.sharedMemPerBlockOptin
                                                                             : ctx->props.sharedMemPerBlock;
@@ -1257,10 +1428,47 @@ uint32_t lev_q6_k_mfma_q8_cols(const lev_ctx *ctx, uint32_t in_dim) {
     return 0;
 }
 
+namespace {
+template <int NC>
+hipError_t q6m_q8_one_launch(lev_ctx *ctx, const uint8_t *w, const uint32_t *xq, const float *xs, float *y,
+                             uint32_t cols, uint32_t rows, uint32_t ncol) {
+    const uint32_t wpr = cols >> 8, slots = (uint32_t)kQWaves / wpr;
+    const uint32_t ngroups = (rows + 15u) / 16u;
+    const uint32_t nrounds = (ngroups + slots - 1u) / slots;
+    uint64_t slot_of_wave = 0, pos_of_wave = 0;
+    for (uint32_t wv = 0; wv < (uint32_t)kQWaves; ++wv) {
+        slot_of_wave |= (uint64_t)(wv / wpr > 15u ? 15u : wv / wpr) << (4u * wv);
+        pos_of_wave |= (uint64_t)(wv % wpr) << (4u * wv);
+    }
+    constexpr size_t lds = q6m_q8_one_lds(NC);
+    static bool configured = false;   // per instantiation: raise the dynamic LDS limit once
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&q6_k_mfma_gemv_q8_one<NC>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        configured = true;
+    }
+    const uint32_t blocks = nrounds < (uint32_t)ctx->num_cus ? nrounds : (uint32_t)ctx->num_cus;
+    hipLaunchKernelGGL((q6_k_mfma_gemv_q8_one<NC>), dim3(blocks), dim3(kQThreads), lds, ctx->stream, w, xq, xs, y,
+                       cols, rows, ncol, wpr, slots, slot_of_wave, pos_of_wave);
+    return hipGetLastError();
+}
+}  // namespace
+
 // ncol <= lev_q6_k_mfma_q8_cols(ctx, in_dim); w 2-byte, xq 16-byte, xs 8-byte aligned.
 hipError_t lev_q6_k_mfma_gemv_q8_launch(lev_ctx *ctx, const uint8_t *w, const uint32_t *xq, const float *xs,
                                         float *y, uint32_t in_dim, uint32_t rows, uint32_t ncol, uint32_t waves) {
     if (waves != 2u && waves != 4u && waves != 8u && waves != 16u) waves = 0u;
+    // up to eight columns of at most sixteen superblocks, no number of waves per row group asked
+    // for: a wave per superblock column
+    static const bool one_off = [] {
+        const char *e = getenv("LEV_Q6K_ONE");
+        return e && e[0] == '0';
+    }();
+    if (ncol <= 8u && waves == 0u && !one_off && in_dim <= 4096u) {
+        if (ncol > 4u) return q6m_q8_one_launch<8>(ctx, w, xq, xs, y, in_dim, rows, ncol);
+        return q6m_q8_one_launch<4>(ctx, w, xq, xs, y, in_dim, rows, ncol);
+    }
     if (ncol > 8) return q6m_q8_launch<16>(ctx, w, xq, xs, y, in_dim, rows, ncol, waves);
     if (ncol > 4) return q6m_q8_launch<8>(ctx, w, xq, xs, y, in_dim, rows, ncol, waves);
     return q6m_q8_launch<4>(ctx, w, xq, xs, y, in_dim, rows, ncol, waves);
