@@ -708,6 +708,224 @@ q4_k_q8_mfma(const uint8_t *__restrict__ w, const uint8_t *__restrict__ xq, cons
     }
 }
 
+// ---------------------------------------------------------------------------
+// Up to four columns, rows of at most sixteen superblocks, in the shape of the f32 one-column
+// kernel (q4_k_mfma_gemv_one.hip): a wave owns ONE superblock column of the matrix.  Lane (r, g)
+// multiplies chunk g (32 code bytes: low nibbles = sub-block 2g, high = 2g+1) of row r by four
+// v_mfma_i32_16x16x64_i8; A row 4g + c holds the 16 activation codes of column c (of a chunk of
+// four columns) that lane group g multiplies, zeros elsewhere, so the four accumulator registers
+// of a lane are the exact sums q * xq of its own sub-block for four columns.  The A operands are
+// the activation codes as they lie in memory, so a lane loads them straight into registers, with
+// the scales and sums of its two blocks beside them: nothing is staged in LDS, no barrier stands
+// in front of the products.  The wave walks the row groups with the next group's weights in
+// flight; the partial sums of a row meet in LDS behind one barrier per round.
+// Weights: lane 4*row + c fetches dword c of the superblock's header and the 32 aligned bytes of
+// chunk c (a quad reads the row's 144 contiguous bytes); one lane permutation per dword hands them
+// to lane (row, c).
+// LDS: part [2][16 waves][16 rows][NC] f32.
+// ---------------------------------------------------------------------------
+__host__ __device__ constexpr uint32_t q8m_one_part_bytes(uint32_t nc) { return 2u * kMWaves * 16u * 4u * nc; }
+
+template <typename T>
+__device__ __forceinline__ void q8m_pin(T &v) {
+    asm volatile("" : "+v"(v));
+}
+
+// NC: columns staged (a multiple of 4, >= ncol; 4 is what is built).
+template <int NC>
+__global__ void __launch_bounds__(kMThreads)
+q4_k_q8_mfma_one(const uint8_t *__restrict__ w, const uint8_t *__restrict__ xq, const float *__restrict__ xs,
+                 float *__restrict__ y, uint32_t cols, uint32_t rows, uint32_t ncol, uint32_t wpr, uint32_t slots,
+                 uint64_t slot_of_wave, uint64_t pos_of_wave) {
+    constexpr int NCH = NC / 4;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    const uint32_t slot = (uint32_t)(slot_of_wave >> (4u * wave)) & 15u;   // idle waves: slot >= slots
+    const uint32_t sb = (uint32_t)(pos_of_wave >> (4u * wave)) & 15u;      // the wave's superblock column
+    const uint32_t SB = cols >> 8, nblk = cols >> 5;
+    const uint32_t r = lane & 15u, g = lane >> 4;
+    const bool active = slot < slots;
+
+    // The first row group's weights are requested first: they come from HBM, the activations
+    // (L2 hits) queue behind them and are back long before.
+    const uint64_t row_bytes = (uint64_t)SB * 144u;
+    const uint32_t ngroups = (rows + 15u) >> 4;
+    const uint32_t nrounds = (ngroups + slots - 1u) / slots;     // rounds of `slots` row groups
+    const uint32_t lrow = lane >> 2, lc = lane & 3u;             // fetch order: lane = 4 * row + chunk
+    auto issue = [&](uint32_t round_block, uint32_t (&D)[9]) {
+        uint32_t rg = round_block * slots + (active ? slot : 0u);
+        rg = rg < ngroups ? rg : ngroups - 1u;
+        uint32_t row = rg * 16u + lrow;
+        row = row < rows ? row : rows - 1u;
+        const uint8_t *p = w + (uint64_t)row * row_bytes + (uint64_t)sb * 144u;
+        D[0] = *reinterpret_cast<const uint32_t *>(p + 4u * lc);
+        const lev_u32x4 a = *reinterpret_cast<const lev_u32x4 *>(p + 16u + 32u * lc);
+        const lev_u32x4 b = *reinterpret_cast<const lev_u32x4 *>(p + 32u + 32u * lc);
+        D[1] = a.x; D[2] = a.y; D[3] = a.z; D[4] = a.w;
+        D[5] = b.x; D[6] = b.y; D[7] = b.z; D[8] = b.w;
+    };
+    uint32_t D[9];
+    uint32_t rb = blockIdx.x;
+    issue(rb, D);
+    __builtin_amdgcn_sched_barrier(0);
+
+    // the wave's activations: lane (r, g) feeds A row r = 4*gs + c, i.e. column 4*ch + r%4, the 16
+    // codes 64g + 16h .. of the superblock (h = 0, 1: sub-block 2g; 2, 3: sub-block 2g+1), when
+    // gs == g, zeros otherwise (columns beyond ncol repeat the last one: their scales are zeroed)
+    lev_i32x4 A[NCH][4];
+    float dxa[NCH][4], dxb[NCH][4], sa[NCH][4], sbm[NCH][4];     // scale and sum of blocks 2g and 2g+1, column 4*ch + i
+#pragma unroll
+    for (int ch = 0; ch < NCH; ++ch) {
+        const uint32_t ca = 4u * (uint32_t)ch + (r & 3u);
+        const uint8_t *xa = xq + (uint64_t)(ca < ncol ? ca : ncol - 1u) * cols + 256u * sb + 64u * g;
+#pragma unroll
+        for (int h = 0; h < 4; ++h) A[ch][h] = *reinterpret_cast<const lev_i32x4 *>(xa + 16 * h);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t ci = 4u * (uint32_t)ch + (uint32_t)i;
+            const lev_f32x4 t = *reinterpret_cast<const lev_f32x4 *>(
+                xs + ((uint64_t)(ci < ncol ? ci : ncol - 1u) * nblk + 8u * sb + 2u * g) * 2u);
+            const bool on = active && ci < ncol;
+            dxa[ch][i] = on ? t.x : 0.f;
+            sa[ch][i] = on ? t.y : 0.f;
+            dxb[ch][i] = on ? t.z : 0.f;
+            sbm[ch][i] = on ? t.w : 0.f;
+        }
+    }
+
+    // ---- everything the tail of a round needs, while the loads are on their way ----
+    // byte offsets into the workgroup's LDS, not pointers
+    uint32_t pw = ((wave * 16u + r) * NC + g) * 4u;              // lane (r, g): row r, column g (+ 4 per chunk)
+    uint32_t pr = ((((wave < slots ? wave : 0u) * wpr) * 16u + r) * NC + g) * 4u;
+    uint32_t orow = (rb * slots + wave) * 16u + r;
+    const uint32_t orow_step = gridDim.x * slots * 16u;
+    const bool writer = wave < slots;
+    uint32_t stores = writer && orow < rows ? 1u : 0u;
+    uint64_t yp = reinterpret_cast<uint64_t>(y + (uint64_t)g * rows + orow);
+    q8m_pin(pw);
+    q8m_pin(pr);
+    q8m_pin(stores);
+    q8m_pin(yp);
+    {
+        const bool feeds = active && (r >> 2) == g;
+#pragma unroll
+        for (int ch = 0; ch < NCH; ++ch)
+#pragma unroll
+            for (int h = 0; h < 4; ++h) A[ch][h] = feeds ? A[ch][h] : lev_i32x4{0, 0, 0, 0};
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    // A round: the fetched dwords go to the lanes that multiply them, and the registers they came
+    // in take the NEXT round's request at once (unconditional, clamped: a branch around the loads
+    // would make the compiler wait for them before the current group is multiplied).
+    auto round = [&](uint32_t next_block) {
+        // lane (r, g) <- lane 4r + g for the chunk, lanes 4r .. 4r + 3 for the header's four dwords
+        uint32_t hdr[4];
+        lev_u32x4 ca, cb;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) hdr[k] = (uint32_t)__builtin_amdgcn_ds_bpermute((int)(16u * r + 4u * k), (int)D[0]);
+        const int src = (int)((4u * r + g) * 4u);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            ca[k] = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)D[1 + k]);
+            cb[k] = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)D[5 + k]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        issue(next_block, D);
+        __builtin_amdgcn_sched_barrier(0);
+        // unpack_scale_min (lev-cpu/src/lib.rs:64-74), four sub-blocks a word; this lane wants sub-blocks
+        // 2g and 2g + 1: bytes 2 * (g % 2) and + 1 of word g / 2 (both words are formed and one is
+        // kept by a bit select: a conditional here becomes a branch)
+        const uint32_t S0 = hdr[1], S1 = hdr[2], S2 = hdr[3];
+        const uint32_t up = g >= 2u ? ~0u : 0u;
+        const uint32_t sc_hi = (S2 & 0x0F0F0F0Fu) | ((S0 >> 2) & 0x30303030u), sc_lo = S0 & 0x3F3F3F3Fu;
+        const uint32_t mn_hi = ((S2 >> 4) & 0x0F0F0F0Fu) | ((S1 >> 2) & 0x30303030u), mn_lo = S1 & 0x3F3F3F3Fu;
+        const uint32_t scw = (sc_hi & up) | (sc_lo & ~up);
+        const uint32_t mnw = (mn_hi & up) | (mn_lo & ~up);
+        const uint32_t sh = 16u * (g & 1u);
+        const float d = lev_f16_bits_to_f32(hdr[0] & 0xFFFFu);
+        const float dmin = lev_f16_bits_to_f32(hdr[0] >> 16);
+        const float sca = d * (float)__builtin_amdgcn_ubfe(scw, sh, 8u);
+        const float scb = d * (float)__builtin_amdgcn_ubfe(scw, sh + 8u, 8u);
+        const float mna = dmin * (float)__builtin_amdgcn_ubfe(mnw, sh, 8u);
+        const float mnb = dmin * (float)__builtin_amdgcn_ubfe(mnw, sh + 8u, 8u);
+        const lev_i32x4 la = __builtin_bit_cast(lev_i32x4, ca & 0x0F0F0F0Fu);
+        const lev_i32x4 lb = __builtin_bit_cast(lev_i32x4, cb & 0x0F0F0F0Fu);
+        const lev_i32x4 ha = __builtin_bit_cast(lev_i32x4, (ca >> 4) & 0x0F0F0F0Fu);
+        const lev_i32x4 hb = __builtin_bit_cast(lev_i32x4, (cb >> 4) & 0x0F0F0F0Fu);
+#pragma unroll
+        for (int ch = 0; ch < NCH; ++ch) {
+            lev_i32x4 d0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[ch][0], la, lev_i32x4{0, 0, 0, 0}, 0, 0, 0);
+            lev_i32x4 d1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[ch][2], ha, lev_i32x4{0, 0, 0, 0}, 0, 0, 0);
+            d0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[ch][1], lb, d0, 0, 0, 0);
+            d1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[ch][3], hb, d1, 0, 0, 0);
+            float v[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                // y += d*sc_j*dx_j*idot - dmin*m_j*s_j for the lane's two sub-blocks
+                float t = fmaf(sca, dxa[ch][i] * (float)d0[i], -mna * sa[ch][i]);
+                t = fmaf(scb, dxb[ch][i] * (float)d1[i], t);
+                v[i] = fmaf(-mnb, sbm[ch][i], t);
+            }
+            // the four lane groups' shares of a row meet, lane group g keeping column 4*ch + g: two
+            // exchanges between the halves of the wave, one between the rows of a half
+            auto s02 = __builtin_amdgcn_permlane32_swap(__float_as_uint(v[0]), __float_as_uint(v[2]), false, false);
+            auto s13 = __builtin_amdgcn_permlane32_swap(__float_as_uint(v[1]), __float_as_uint(v[3]), false, false);
+            const float a = __uint_as_float(s02[0]) + __uint_as_float(s02[1]);
+            const float b = __uint_as_float(s13[0]) + __uint_as_float(s13[1]);
+            auto sab = __builtin_amdgcn_permlane16_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+            *reinterpret_cast<float *>(smem + pw + 16 * ch) = __uint_as_float(sab[0]) + __uint_as_float(sab[1]);
+        }
+        lev_barrier_lds();
+        if (wave < slots) {
+            const float *pp = reinterpret_cast<const float *>(smem + pr);
+#pragma unroll
+            for (int ch = 0; ch < NCH; ++ch) {
+                // the slot's waves in order, four chains added at the end (sixteen reads in flight)
+                float s4[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int k = 0; k < kMWaves; ++k) {
+                    const float pk = pp[k * 16 * NC + 4 * ch];
+                    s4[k & 3] += (uint32_t)k < wpr ? pk : 0.f;
+                }
+                const float s = (s4[0] + s4[1]) + (s4[2] + s4[3]);
+                if (stores && 4u * (uint32_t)ch + g < ncol)
+                    *reinterpret_cast<__attribute__((address_space(1))) float *>(yp + (uint64_t)(4 * ch) * rows * 4u) = s;
+            }
+        }
+        pw ^= kMWaves * 16u * 4u * NC;                          // the other half of `part` next round
+        pr ^= kMWaves * 16u * 4u * NC;
+        orow += orow_step;
+        yp += (uint64_t)orow_step * 4u;
+        stores = writer && orow < rows ? 1u : 0u;
+    };
+    while (true) {
+        const uint32_t next = rb + gridDim.x;
+        round(next < nrounds ? next : rb);
+        if (next >= nrounds) break;
+        rb = next;
+    }
+}
+
+template <int NC>
+hipError_t launch_q8m_one(lev_ctx *ctx, const uint8_t *w, const uint8_t *xq, const float *xs, float *y,
+                          uint32_t cols, uint32_t rows, uint32_t ncol) {
+    const uint32_t wpr = cols >> 8, slots = (uint32_t)kMWaves / wpr;
+    const uint32_t ngroups = (rows + 15u) / 16u;
+    const uint32_t nrounds = (ngroups + slots - 1u) / slots;
+    uint64_t slot_of_wave = 0, pos_of_wave = 0;
+    for (uint32_t wv = 0; wv < (uint32_t)kMWaves; ++wv) {
+        slot_of_wave |= (uint64_t)(wv / wpr > 15u ? 15u : wv / wpr) << (4u * wv);
+        pos_of_wave |= (uint64_t)(wv % wpr) << (4u * wv);
+    }
+    const uint32_t blocks = nrounds < (uint32_t)ctx->num_cus ? nrounds : (uint32_t)ctx->num_cus;
+    static_assert(q8m_one_part_bytes(NC) <= 48u * 1024u, "fits the default dynamic LDS limit");
+    hipLaunchKernelGGL((q4_k_q8_mfma_one<NC>), dim3(blocks), dim3(kMThreads), q8m_one_part_bytes(NC), ctx->stream, w,
+                       xq, xs, y, cols, rows, ncol, wpr, slots, slot_of_wave, pos_of_wave);
+    return hipGetLastError();
+}
+
 size_t q8m_lds_bytes(uint32_t cols, uint32_t ncl) {
     return (size_t)cols * ncl + (size_t)2 * (cols >> 5) * ncl * 4 + (size_t)2 * kMWaves * 16 * ncl * 4;
 }
@@ -784,7 +1002,9 @@ uint32_t lev_q4_k_gemv_q8_candidates(const lev_ctx *ctx, uint32_t in_dim, uint32
                                      lev_schedule *out, uint32_t capacity) {
     (void)rows;
     const bool has_mfma = q8m_cols(ctx, in_dim) != 0u;
-    const uint32_t first = has_mfma && ncol >= kQ8MfmaMinCols ? 1u : 0u;
+    // built-in: the matrix cores for every column count of rows up to 4096 wide (a wave per
+    // superblock column up to four columns), from kQ8MfmaMinCols columns for wider rows
+    const uint32_t first = has_mfma && (ncol >= kQ8MfmaMinCols || in_dim <= 4096u) ? 1u : 0u;
     uint32_t n = 0;
     if (n < capacity) out[n] = lev_schedule{LEV_OP_Q4_K_GEMV_Q8, first, 0u, 0u};
     ++n;
@@ -821,7 +1041,14 @@ extern "C" int lev_hip_q4_k_gemv_q8(lev_ctx *ctx, const void *d_w, size_t w_byte
     // overrides it.
     const uint32_t mcols = q8m_cols(ctx, in_dim);
     const lev_schedule *sel = lev_selected(ctx, LEV_OP_Q4_K_GEMV_Q8, in_dim, rows, ncol);
-    const bool mfma = mcols != 0u && (sel ? sel->family == 1u : ncol >= kQ8MfmaMinCols);
+    const bool mfma = mcols != 0u && (sel ? sel->family == 1u : (ncol >= kQ8MfmaMinCols || in_dim <= 4096u));
+    // rows of at most sixteen superblocks: the matrix-core kernel with a wave per superblock column,
+    // for every column count (a schedule of family 0 still selects the dot4 kernel)
+    static const bool one_off = [] {
+        const char *e = getenv("LEV_Q4K_Q8_ONE");   // LEV_Q4K_Q8_ONE=0: the kernels below, for comparison
+        return e && e[0] == '0';
+    }();
+    const bool mfma_one = !one_off && in_dim <= 4096u && mfma;
     uint32_t done = 0;
     while (done < ncol) {
         uint32_t nc = ncol - done;
@@ -829,7 +1056,12 @@ extern "C" int lev_hip_q4_k_gemv_q8(lev_ctx *ctx, const void *d_w, size_t w_byte
         const float *xsc = d_xs + (uint64_t)done * (in_dim >> 5) * 2u;
         float *yc = d_y + (uint64_t)done * rows;
         hipError_t e;
-        if (mfma) {
+        if (mfma_one && nc <= 4u) {
+            // up to four columns (eight through it measured 11.9 us at 12288 x 4096, what the
+            // sixteen-column kernel below takes for eight as well)
+            if (nc > 4u) nc = 4u;
+            e = launch_q8m_one<4>(ctx, w, reinterpret_cast<const uint8_t *>(xqc), xsc, yc, in_dim, rows, nc);
+        } else if (mfma) {
             if (nc > mcols) nc = mcols;
             const uint8_t *xb = reinterpret_cast<const uint8_t *>(xqc);
             if (mcols == 16u) e = launch_q8m<16>(ctx, w, xb, xsc, yc, in_dim, rows, nc);

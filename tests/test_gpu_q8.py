@@ -183,15 +183,16 @@ def test_q4_k_q8_shapes(ctx, rows, cols, ncol):
 @pytest.mark.parametrize("rows,cols,ncol", [(37, 1024, 1), (130, 4352, 3), (20, 12288, 8), (64, 4096, 16),
                                             (5000, 4096, 12), (16, 16384, 5), (40, 28672, 4)])
 def test_q4_k_q8_both_kernels_every_column_count(ctx, rows, cols, ncol, family):
-    """A forge selection pins the kernel: family 1 the integer matrix-core kernel
-    (built-in choice from 4 columns), 0 the dot4 kernel (built-in below); both meet
-    the gate everywhere.  5000 rows give a wave more than three tasks (the looping
+    """A forge selection pins the kernel: family 1 the integer matrix-core kernels
+    (built-in choice from 4 columns, and for every column count of rows up to 4096 wide, where
+    a wave per superblock column serves up to four columns), 0 the dot4 kernel (built-in for
+    fewer columns of wider rows); both meet the gate everywhere.  5000 rows give a wave more than three tasks (the looping
     variant); 28672 columns exceed the unrolled staging of the matrix-core kernel
     (its tail loops)."""
     from leviathan_amd import capi
     cands = ctx.forge_candidates(capi.OP_Q4_K_GEMV_Q8, cols, rows, ncol)
     assert sorted(c.family for c in cands) == [0, 1]
-    assert cands[0].family == (1 if ncol >= 4 else 0)          # candidate 0 is the built-in choice
+    assert cands[0].family == (1 if ncol >= 4 or cols <= 4096 else 0)          # candidate 0 is the built-in choice
     ctx.forge_select(cols, rows, [c for c in cands if c.family == family][0], ncol)
     try:
         w, x, gain = H.config3(rows, cols, ncol, seed=rows + ncol)
