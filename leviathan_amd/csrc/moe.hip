@@ -1235,7 +1235,19 @@ moe_down_mfma(moe_args a, const float *__restrict__ act, const int32_t *__restri
     // ordered merge: y = sum over slots, in slot order, of w_slot * dn[slot]
     if (tid < 16u && row_begin + tid < row_end) {
         float accum = 0.f;
-        for (uint32_t slot = 0; slot < a.top_k; ++slot) accum = fmaf(w_slot[slot], partial[slot * 16u + tid], accum);
+        // eight slots' reads in flight together, the multiply-adds in slot order behind them
+        for (uint32_t s0 = 0; s0 < a.top_k; s0 += 8u) {
+            float pv[8], wv[8];
+#pragma unroll
+            for (uint32_t u = 0; u < 8u; ++u) {
+                const uint32_t slot = s0 + u < a.top_k ? s0 + u : a.top_k - 1u;
+                pv[u] = partial[slot * 16u + tid];
+                wv[u] = w_slot[slot];
+            }
+#pragma unroll
+            for (uint32_t u = 0; u < 8u; ++u)
+                if (s0 + u < a.top_k) accum = fmaf(wv[u], pv[u], accum);
+        }
         y[(uint64_t)t * a.hidden + row_begin + tid] = accum;
     }
 }
