@@ -363,7 +363,8 @@ typedef struct lev_schedule {
                                 kernel of its own ahead of them */
     uint32_t rows_in_flight; /* Q4_0 family 0: rows a wave keeps in flight (1, 2, 4; 0 = no variants for the shape);
                                 Q6_K: waves that share a row (family 0: 1, 2) or a group of 16 rows (family 2:
-                                2, 4, 8, 16); Q6_K x int8: columns per pass over the
+                                2, 4, 8, 16; 0 = a wave per superblock column, for rows up to 4096 wide);
+                                Q6_K x int8: columns per pass over the
                                 weights; MoE layer: gate/up workgroups aimed at per CU (1, 2, 4) */
     uint32_t persistent;     /* Q4_0, Q6_K x int8: 0 = one workgroup per row tile, 1 = resident grid walking
                                 the tiles; MoE layer: 0 = expert kernels on the integer matrix cores where the

@@ -573,6 +573,9 @@ uint32_t lev_q6_k_gemv_candidates(const lev_ctx *ctx, uint32_t in_dim, uint32_t 
         ++n;
     };
     if (lev_q6_k_mfma_cols(ctx, in_dim) >= 1u) {
+        // rows of at most sixteen superblocks: a wave per superblock column (schedule field 0 waves
+        // per row group), the built-in choice there; then the several-column kernel at one column
+        if (in_dim <= 4096u) add(2u, 0u);
         const uint32_t builtin = lev_q6_k_mfma_waves(ctx, in_dim, rows);
         add(2u, builtin);
         if (builtin != 2u) add(2u, 2u);

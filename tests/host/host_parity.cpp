@@ -668,10 +668,11 @@ void forge_matvec(Runner &r) {
         EXPECT(!rep.fromCache);
         EXPECT(!rep.candidates.empty());
         EXPECT(q40 || q6 || rep.candidates.size() == 2);                 // matrix-core and vector-ALU kernel
-        // matrix-core kernel (built-in waves per row group, then 2 and 4 where they differ), dot4 kernel
-        // (two waves, one wave a row), f64-sum kernel
-        EXPECT(!q6 || rep.candidates.size() == (sh.cols == 4096 ? 6u : 4u));
-        EXPECT(!q6 || rep.candidates[0].schedule.family == 2u);
+        // matrix-core kernels (a wave per superblock column for these rows of at most sixteen superblocks, then
+        // the several-column kernel with its built-in waves per row group, then 2 and 4 where they differ), dot4
+        // kernel (two waves, one wave a row), f64-sum kernel
+        EXPECT(!q6 || rep.candidates.size() == (sh.cols == 4096 ? 7u : 5u));
+        EXPECT(!q6 || (rep.candidates[0].schedule.family == 2u && rep.candidates[0].schedule.rows_in_flight == 0u));
         // matrix-core kernel (two grids) first, then the vector-ALU kernels: 3 depths x 2 grids, or one for narrow rows
         EXPECT(!q40 || sh.cols < 1024 || rep.candidates.size() == 8);
         EXPECT(!q40 || sh.cols >= 1024 || rep.candidates.size() == 3);
