@@ -183,6 +183,45 @@ __device__ __forceinline__ void lev_barrier_lds() {
     asm volatile("s_barrier" ::: "memory");
 }
 
+// ---- shared by the kernels in which a wave owns one column block of the matrix (a Q4_0 task,
+// a Q4_K or Q6_K superblock column) and `wpr` waves of a workgroup of 16 cover a row ----
+
+// Sum over lanes l, l ^ 16, l ^ 32, l ^ 48 (the four lane groups of a matrix-core row), in every
+// lane, in f64, by two row swaps per dword: no LDS.
+__device__ __forceinline__ double lev_row_sum_f64(double v) {
+    uint32_t lo = (uint32_t)__double2loint(v), hi = (uint32_t)__double2hiint(v);
+    auto a0 = __builtin_amdgcn_permlane32_swap(lo, lo, false, false);
+    auto a1 = __builtin_amdgcn_permlane32_swap(hi, hi, false, false);
+    v = __hiloint2double((int)a1[0], (int)a0[0]) + __hiloint2double((int)a1[1], (int)a0[1]);
+    lo = (uint32_t)__double2loint(v);
+    hi = (uint32_t)__double2hiint(v);
+    a0 = __builtin_amdgcn_permlane16_swap(lo, lo, false, false);
+    a1 = __builtin_amdgcn_permlane16_swap(hi, hi, false, false);
+    return __hiloint2double((int)a1[0], (int)a0[0]) + __hiloint2double((int)a1[1], (int)a0[1]);
+}
+
+// Keeps a value that the tail of a round needs (an LDS offset, an output pointer, a mask)
+// computed where it is written: between the load requests and the first wait, where
+// instructions cost nothing.  Left to itself the compiler sinks such arithmetic to its use,
+// behind the barrier, where every instruction is on the critical path of the launch.
+template <typename T>
+__device__ __forceinline__ void lev_pin(T &v) {
+    asm volatile("" : "+v"(v));
+}
+
+// wave -> (slot, position in the slot) as 4-bit entries of two 64-bit kernel arguments, for 16
+// waves of which `wpr` (1..16) share a group of rows: a division in front of a kernel's first
+// load would cost some thirty instructions.  Waves beyond the last whole slot get slot 15 or the
+// first unused one (>= 16 / wpr): idle.
+inline void lev_wave_tables(uint32_t wpr, uint64_t *slot_of_wave, uint64_t *pos_of_wave) {
+    *slot_of_wave = 0;
+    *pos_of_wave = 0;
+    for (uint32_t wv = 0; wv < 16u; ++wv) {
+        *slot_of_wave |= (uint64_t)(wv / wpr > 15u ? 15u : wv / wpr) << (4u * wv);
+        *pos_of_wave |= (uint64_t)(wv % wpr) << (4u * wv);
+    }
+}
+
 // Hand-over of a few words from one workgroup to whichever workgroup arrives last at a
 // counter, WITHOUT a release fence (on this chip a device-scope release writes back every
 // dirty line of the XCD's L2, the kernel's own outputs included).  The order is kept by three

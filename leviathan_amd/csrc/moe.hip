@@ -1105,8 +1105,8 @@ moe_gate_up_mfma(moe_args a, const float *__restrict__ x, const int32_t *ids, co
     uint32_t pw = (wave * 16u + lane) * 4u;                       // byte offsets into `part`: gate, then up at + 512
     uint32_t pr = (q * 16u + r16) * 4u;                           // wave 0: lane (r, q) adds waves q and q + 4
     float *arow = act + ((uint64_t)t * a.top_k + slot) * a.inter;
-    q4m_pin(pw);
-    q4m_pin(pr);
+    lev_pin(pw);
+    lev_pin(pr);
     if (lane < kQ4mZeroBytes / 4u) reinterpret_cast<uint32_t *>(zero)[lane] = 0u;
     q4m_operand op[TPW];
 #pragma unroll

@@ -153,12 +153,3 @@ __device__ __forceinline__ float q4m_row_sum(float v) {
     return __uint_as_float(s1[0]) + __uint_as_float(s1[1]);
 }
 
-// Keeps a value that the tail of a round needs (an LDS address, an output pointer) computed where
-// it is written: between the load requests and the first wait, where instructions cost nothing.
-// Left to itself the compiler sinks such arithmetic to its use, behind the barrier, where every
-// instruction is on the critical path of the launch.
-template <typename T>
-__device__ __forceinline__ void q4m_pin(T &v) {
-    asm volatile("" : "+v"(v));
-}
-

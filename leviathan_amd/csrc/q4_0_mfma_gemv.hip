@@ -24,8 +24,7 @@ __host__ __device__ constexpr size_t q4m_gemv_lds(uint32_t tpw) {
     return 2u * kQ4mWaves * 16u * 4u + (size_t)kQ4mWaves * (tpw * kQ4mTaskArea + kQ4mZeroBytes);
 }
 
-// wave -> (slot, position in the slot) as 4-bit entries of two 64-bit kernel arguments: a division
-// in front of the first load would cost some thirty instructions.
+// wave -> (slot, position in the slot): 4-bit entries of two 64-bit kernel arguments (lev_wave_tables).
 // SINGLE: the grid covers every round once: straight-line code, nothing to prefetch.
 template <int TPW, bool SINGLE>
 __global__ void __launch_bounds__(kQ4mThreads)
@@ -88,14 +87,14 @@ q4_0_mfma_gemv(const uint8_t *__restrict__ w, const float *__restrict__ x, float
     const bool writer = wave < slots && q == 0u;
     uint32_t stores = writer && orow < rows ? 1u : 0u;
     uint64_t yp = reinterpret_cast<uint64_t>(y + orow);        // (the pointer argument is read here, not behind the barrier)
-    q4m_pin(pw);
-    q4m_pin(pr);
-    q4m_pin(k0);
-    q4m_pin(k1);
-    q4m_pin(k2);
-    q4m_pin(k3);
-    q4m_pin(stores);
-    q4m_pin(yp);
+    lev_pin(pw);
+    lev_pin(pr);
+    lev_pin(k0);
+    lev_pin(k1);
+    lev_pin(k2);
+    lev_pin(k3);
+    lev_pin(stores);
+    lev_pin(yp);
 
     if (lane < kQ4mZeroBytes / 4u) reinterpret_cast<uint32_t *>(zero)[lane] = 0u;
     q4m_operand op[TPW];
@@ -160,11 +159,8 @@ hipError_t launch(lev_ctx *ctx, const uint8_t *w, const float *x, float *y, uint
     const uint32_t ngroups = (rows + 15u) / 16u;
     const uint32_t nrounds = (ngroups + slots - 1u) / slots;
     const size_t lds = q4m_gemv_lds(TPW);
-    uint64_t slot_of_wave = 0, pos_of_wave = 0;
-    for (uint32_t wv = 0; wv < (uint32_t)kQ4mWaves; ++wv) {
-        slot_of_wave |= (uint64_t)(wv / wpr > 15u ? 15u : wv / wpr) << (4u * wv);
-        pos_of_wave |= (uint64_t)(wv % wpr) << (4u * wv);
-    }
+    uint64_t slot_of_wave, pos_of_wave;
+    lev_wave_tables(wpr, &slot_of_wave, &pos_of_wave);
     // built-in choice (persistent < 0): one workgroup per round while every round has a CU of its own
     const uint32_t cus = (uint32_t)ctx->num_cus;
     const bool single = persistent < 0 ? nrounds <= cus : persistent == 0;

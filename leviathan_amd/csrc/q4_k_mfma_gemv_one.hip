@@ -132,19 +132,6 @@ __device__ __forceinline__ void q4k_one_stage(const lev_f32x4 v, uint8_t *area, 
     for (int p = 0; p < 4; ++p) *reinterpret_cast<uint32_t *>(at + 64 * p) = dw[p];
 }
 
-// Sum over lanes l, l ^ 16, l ^ 32, l ^ 48 in every lane, in f64, by row swaps.
-__device__ __forceinline__ double q4k_one_row_sum(double v) {
-    uint32_t lo = (uint32_t)__double2loint(v), hi = (uint32_t)__double2hiint(v);
-    auto a0 = __builtin_amdgcn_permlane32_swap(lo, lo, false, false);
-    auto a1 = __builtin_amdgcn_permlane32_swap(hi, hi, false, false);
-    v = __hiloint2double((int)a1[0], (int)a0[0]) + __hiloint2double((int)a1[1], (int)a0[1]);
-    lo = (uint32_t)__double2loint(v);
-    hi = (uint32_t)__double2hiint(v);
-    a0 = __builtin_amdgcn_permlane16_swap(lo, lo, false, false);
-    a1 = __builtin_amdgcn_permlane16_swap(hi, hi, false, false);
-    return __hiloint2double((int)a1[0], (int)a0[0]) + __hiloint2double((int)a1[1], (int)a0[1]);
-}
-
 // Chunk g of row r as the products want it (hdr: the superblock's first 16 bytes, ca / cb: the
 // chunk's 32 code bytes).
 struct q4k_one_weights {
@@ -278,14 +265,14 @@ q4_k_mfma_gemv_one(const uint8_t *__restrict__ w, const float *__restrict__ x, c
     const bool writer = wave < slots && q == 0u;
     uint32_t stores = writer && orow < rows ? 1u : 0u;
     uint64_t yp = reinterpret_cast<uint64_t>(y + orow);
-    q4m_pin(pw);
-    q4m_pin(pr);
-    q4m_pin(k0);
-    q4m_pin(k1);
-    q4m_pin(k2);
-    q4m_pin(k3);
-    q4m_pin(stores);
-    q4m_pin(yp);
+    lev_pin(pw);
+    lev_pin(pr);
+    lev_pin(k0);
+    lev_pin(k1);
+    lev_pin(k2);
+    lev_pin(k3);
+    lev_pin(stores);
+    lev_pin(yp);
 
     if (NORM) {
         // RMSNorm as the reference computes it (rmsnorm, rust/crates/lev-model/src/lib.rs:110-114):
@@ -369,7 +356,7 @@ q4_k_mfma_gemv_one(const uint8_t *__restrict__ w, const float *__restrict__ x, c
                 for (int h = 0; h < 4; ++h) a[h] = *reinterpret_cast<const lev_i32x4 *>(ab + c * cs + h * hs);
                 val[c] = q4k_one_dot(W, a, op[c]);
             }
-            val[c] = q4k_one_row_sum(val[c]);
+            val[c] = lev_row_sum_f64(val[c]);
         }
         if (lane < 16u) {
 #pragma unroll
@@ -382,7 +369,7 @@ q4_k_mfma_gemv_one(const uint8_t *__restrict__ w, const float *__restrict__ x, c
             for (int c = 0; c < NC; ++c) {
                 const double p0 = pp[c], p1 = pp[64 * NC + c], p2 = pp[128 * NC + c], p3 = pp[192 * NC + c];
                 double s = ((k0 ? p0 : 0.0) + (k1 ? p1 : 0.0)) + ((k2 ? p2 : 0.0) + (k3 ? p3 : 0.0));
-                s = q4k_one_row_sum(s);
+                s = lev_row_sum_f64(s);
                 if (stores && (uint32_t)c < ncol)
                     *reinterpret_cast<__attribute__((address_space(1))) float *>(yp + (uint64_t)c * rows * 4u) = (float)s;
             }
@@ -407,11 +394,8 @@ hipError_t launch_one(lev_ctx *ctx, const uint8_t *w, const float *x, const floa
     const uint32_t wpr = cols >> 8, slots = (uint32_t)kOneWaves / wpr;
     const uint32_t ngroups = (rows + 15u) / 16u;
     const uint32_t nrounds = (ngroups + slots - 1u) / slots;
-    uint64_t slot_of_wave = 0, pos_of_wave = 0;
-    for (uint32_t wv = 0; wv < (uint32_t)kOneWaves; ++wv) {
-        slot_of_wave |= (uint64_t)(wv / wpr > 15u ? 15u : wv / wpr) << (4u * wv);
-        pos_of_wave |= (uint64_t)(wv % wpr) << (4u * wv);
-    }
+    uint64_t slot_of_wave, pos_of_wave;
+    lev_wave_tables(wpr, &slot_of_wave, &pos_of_wave);
     constexpr size_t lds = q4k_one_lds(NC);
     if (lds > 48u * 1024u) {
         static bool configured = false;   // per instantiation: raise the dynamic LDS limit once

@@ -612,24 +612,6 @@ __host__ __device__ constexpr size_t q6m_one_lds(uint32_t nc) {
     return q6m_one_part_bytes(nc) + q6m_one_norm_bytes(nc) + (size_t)kQWaves * q6m_one_wave_bytes(nc);
 }
 
-// Sum over lanes l, l ^ 16, l ^ 32, l ^ 48 in every lane, in f64, by row swaps.
-__device__ __forceinline__ double q6m_row_sum(double v) {
-    uint32_t lo = (uint32_t)__double2loint(v), hi = (uint32_t)__double2hiint(v);
-    auto a0 = __builtin_amdgcn_permlane32_swap(lo, lo, false, false);
-    auto a1 = __builtin_amdgcn_permlane32_swap(hi, hi, false, false);
-    v = __hiloint2double((int)a1[0], (int)a0[0]) + __hiloint2double((int)a1[1], (int)a0[1]);
-    lo = (uint32_t)__double2loint(v);
-    hi = (uint32_t)__double2hiint(v);
-    a0 = __builtin_amdgcn_permlane16_swap(lo, lo, false, false);
-    a1 = __builtin_amdgcn_permlane16_swap(hi, hi, false, false);
-    return __hiloint2double((int)a1[0], (int)a0[0]) + __hiloint2double((int)a1[1], (int)a0[1]);
-}
-
-template <typename T>
-__device__ __forceinline__ void q6m_pin(T &v) {
-    asm volatile("" : "+v"(v));
-}
-
 // wave -> (slot, superblock) as 4-bit entries of two 64-bit kernel arguments (no division in
 // front of the first load).  NC: columns staged (1 or 2; >= ncol); one column keeps its A
 // operands in registers, several read them from the wave's planes at every product.
@@ -696,14 +678,14 @@ q6_k_mfma_gemv_one(const uint8_t *__restrict__ w, const float *__restrict__ x, c
     const bool writer = wave < slots && q == 0u;
     uint32_t stores = writer && orow < rows ? 1u : 0u;
     uint64_t yp = reinterpret_cast<uint64_t>(y + orow);
-    q6m_pin(pw);
-    q6m_pin(pr);
-    q6m_pin(k0);
-    q6m_pin(k1);
-    q6m_pin(k2);
-    q6m_pin(k3);
-    q6m_pin(stores);
-    q6m_pin(yp);
+    lev_pin(pw);
+    lev_pin(pr);
+    lev_pin(k0);
+    lev_pin(k1);
+    lev_pin(k2);
+    lev_pin(k3);
+    lev_pin(stores);
+    lev_pin(yp);
 
     if (NORM) {
         // RMSNorm as the reference computes it: mean square and 1/sqrt in f64, then (f32)(x * inv) * gain
@@ -830,7 +812,7 @@ q6_k_mfma_gemv_one(const uint8_t *__restrict__ w, const float *__restrict__ x, c
             const double hi = fma((double)E[3], 256.0, (double)E[2]);
             const double lo = fma((double)E[1], 256.0, (double)E[0]);
             const double dot = fma(hi, 65536.0, lo);
-            val[c] = q6m_row_sum((ps[c] * d) * dot);
+            val[c] = lev_row_sum_f64((ps[c] * d) * dot);
         }
         if (lane < 16u) {
 #pragma unroll
@@ -843,7 +825,7 @@ q6_k_mfma_gemv_one(const uint8_t *__restrict__ w, const float *__restrict__ x, c
             for (int c = 0; c < NC; ++c) {
                 const double p0 = pp[c], p1 = pp[64 * NC + c], p2 = pp[128 * NC + c], p3 = pp[192 * NC + c];
                 double s = ((k0 ? p0 : 0.0) + (k1 ? p1 : 0.0)) + ((k2 ? p2 : 0.0) + (k3 ? p3 : 0.0));
-                s = q6m_row_sum(s);
+                s = lev_row_sum_f64(s);
                 if (stores && (uint32_t)c < ncol) {
                     const float out = (float)s;
                     *reinterpret_cast<__attribute__((address_space(1))) float *>(yp + (uint64_t)c * rows * 4u) = out;
@@ -1157,10 +1139,10 @@ q6_k_mfma_gemv_q8_one(const uint8_t *__restrict__ w, const uint32_t *__restrict_
     const bool writer = wave < slots;
     uint32_t stores = writer && orow < rows ? 1u : 0u;
     uint64_t yp = reinterpret_cast<uint64_t>(y + (uint64_t)q * rows + orow);
-    q6m_pin(pw);
-    q6m_pin(pr);
-    q6m_pin(stores);
-    q6m_pin(yp);
+    lev_pin(pw);
+    lev_pin(pr);
+    lev_pin(stores);
+    lev_pin(yp);
     const bool feeds = active && (r >> 2) == q;
 #pragma unroll
     for (int ch = 0; ch < NCH; ++ch)
@@ -1316,11 +1298,8 @@ hipError_t q6m_one_launch(lev_ctx *ctx, const uint8_t *w, const float *x, const 
     const uint32_t wpr = cols >> 8, slots = (uint32_t)kQWaves / wpr;
     const uint32_t ngroups = (rows + 15u) / 16u;
     const uint32_t nrounds = (ngroups + slots - 1u) / slots;
-    uint64_t slot_of_wave = 0, pos_of_wave = 0;
-    for (uint32_t wv = 0; wv < (uint32_t)kQWaves; ++wv) {
-        slot_of_wave |= (uint64_t)(wv / wpr > 15u ? 15u : wv / wpr) << (4u * wv);
-        pos_of_wave |= (uint64_t)(wv % wpr) << (4u * wv);
-    }
+    uint64_t slot_of_wave, pos_of_wave;
+    lev_wave_tables(wpr, &slot_of_wave, &pos_of_wave);
     constexpr size_t lds = q6m_one_lds(NC);
     static bool configured = false;   // per instantiation: raise the dynamic LDS limit once
     if (!configured) {
@@ -1435,11 +1414,8 @@ hipError_t q6m_q8_one_launch(lev_ctx *ctx, const uint8_t *w, const uint32_t *xq,
     const uint32_t wpr = cols >> 8, slots = (uint32_t)kQWaves / wpr;
     const uint32_t ngroups = (rows + 15u) / 16u;
     const uint32_t nrounds = (ngroups + slots - 1u) / slots;
-    uint64_t slot_of_wave = 0, pos_of_wave = 0;
-    for (uint32_t wv = 0; wv < (uint32_t)kQWaves; ++wv) {
-        slot_of_wave |= (uint64_t)(wv / wpr > 15u ? 15u : wv / wpr) << (4u * wv);
-        pos_of_wave |= (uint64_t)(wv % wpr) << (4u * wv);
-    }
+    uint64_t slot_of_wave, pos_of_wave;
+    lev_wave_tables(wpr, &slot_of_wave, &pos_of_wave);
     constexpr size_t lds = q6m_q8_one_lds(NC);
     static bool configured = false;   // per instantiation: raise the dynamic LDS limit once
     if (!configured) {

@@ -726,11 +726,6 @@ q4_k_q8_mfma(const uint8_t *__restrict__ w, const uint8_t *__restrict__ xq, cons
 // ---------------------------------------------------------------------------
 __host__ __device__ constexpr uint32_t q8m_one_part_bytes(uint32_t nc) { return 2u * kMWaves * 16u * 4u * nc; }
 
-template <typename T>
-__device__ __forceinline__ void q8m_pin(T &v) {
-    asm volatile("" : "+v"(v));
-}
-
 // NC: columns staged (a multiple of 4, >= ncol; 4 is what is built).
 template <int NC>
 __global__ void __launch_bounds__(kMThreads)
@@ -803,10 +798,10 @@ q4_k_q8_mfma_one(const uint8_t *__restrict__ w, const uint8_t *__restrict__ xq, 
     const bool writer = wave < slots;
     uint32_t stores = writer && orow < rows ? 1u : 0u;
     uint64_t yp = reinterpret_cast<uint64_t>(y + (uint64_t)g * rows + orow);
-    q8m_pin(pw);
-    q8m_pin(pr);
-    q8m_pin(stores);
-    q8m_pin(yp);
+    lev_pin(pw);
+    lev_pin(pr);
+    lev_pin(stores);
+    lev_pin(yp);
     {
         const bool feeds = active && (r >> 2) == g;
 #pragma unroll
@@ -914,11 +909,8 @@ hipError_t launch_q8m_one(lev_ctx *ctx, const uint8_t *w, const uint8_t *xq, con
     const uint32_t wpr = cols >> 8, slots = (uint32_t)kMWaves / wpr;
     const uint32_t ngroups = (rows + 15u) / 16u;
     const uint32_t nrounds = (ngroups + slots - 1u) / slots;
-    uint64_t slot_of_wave = 0, pos_of_wave = 0;
-    for (uint32_t wv = 0; wv < (uint32_t)kMWaves; ++wv) {
-        slot_of_wave |= (uint64_t)(wv / wpr > 15u ? 15u : wv / wpr) << (4u * wv);
-        pos_of_wave |= (uint64_t)(wv % wpr) << (4u * wv);
-    }
+    uint64_t slot_of_wave, pos_of_wave;
+    lev_wave_tables(wpr, &slot_of_wave, &pos_of_wave);
     const uint32_t blocks = nrounds < (uint32_t)ctx->num_cus ? nrounds : (uint32_t)ctx->num_cus;
     static_assert(q8m_one_part_bytes(NC) <= 48u * 1024u, "fits the default dynamic LDS limit");
     hipLaunchKernelGGL((q4_k_q8_mfma_one<NC>), dim3(blocks), dim3(kMThreads), q8m_one_part_bytes(NC), ctx->stream, w,
