@@ -200,6 +200,19 @@ __device__ __forceinline__ double lev_row_sum_f64(double v) {
     return __hiloint2double((int)a1[0], (int)a0[0]) + __hiloint2double((int)a1[1], (int)a0[1]);
 }
 
+// Four values per lane whose sums over lanes l, l ^ 16, l ^ 32, l ^ 48 are wanted: lane group
+// g = lane / 16 gets the sum of v[g], by two exchanges between the halves of the wave and one
+// between the rows of a half (three swaps for four sums; the additions pair the lane groups as
+// lev_row_sum_f64 does: (g, g ^ 2) first, then (g, g ^ 1)).
+__device__ __forceinline__ float lev_lanegroup_sums4(const float v[4]) {
+    const auto s02 = __builtin_amdgcn_permlane32_swap(__float_as_uint(v[0]), __float_as_uint(v[2]), false, false);
+    const auto s13 = __builtin_amdgcn_permlane32_swap(__float_as_uint(v[1]), __float_as_uint(v[3]), false, false);
+    const float a = __uint_as_float(s02[0]) + __uint_as_float(s02[1]);
+    const float b = __uint_as_float(s13[0]) + __uint_as_float(s13[1]);
+    const auto sab = __builtin_amdgcn_permlane16_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+    return __uint_as_float(sab[0]) + __uint_as_float(sab[1]);
+}
+
 // Keeps a value that the tail of a round needs (an LDS offset, an output pointer, a mask)
 // computed where it is written: between the load requests and the first wait, where
 // instructions cost nothing.  Left to itself the compiler sinks such arithmetic to its use,

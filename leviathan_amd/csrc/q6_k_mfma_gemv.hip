@@ -1177,18 +1177,8 @@ q6_k_mfma_gemv_q8_one(const uint8_t *__restrict__ w, const uint32_t *__restrict_
                     v[i] = fmaf((float)E, dx[ch][nb][i], v[i]);
                 }
             }
-            // the four lane groups' shares of a row meet, lane group g keeping column 4*ch + g: two
-            // exchanges between the halves of the wave, one between the rows of a half
-            {
-                auto s02 = __builtin_amdgcn_permlane32_swap(__float_as_uint(v[0]), __float_as_uint(v[2]), false, false);
-                auto s13 = __builtin_amdgcn_permlane32_swap(__float_as_uint(v[1]), __float_as_uint(v[3]), false, false);
-                // lower half: columns 0 and 1 (own + the upper half's); upper half: columns 2 and 3
-                const float a = __uint_as_float(s02[0]) + __uint_as_float(s02[1]);
-                const float b = __uint_as_float(s13[0]) + __uint_as_float(s13[1]);
-                auto sab = __builtin_amdgcn_permlane16_swap(__float_as_uint(a), __float_as_uint(b), false, false);
-                const float mine = __uint_as_float(sab[0]) + __uint_as_float(sab[1]);
-                *reinterpret_cast<float *>(smem + pw + 16 * ch) = d * mine;
-            }
+            // the four lane groups' shares of a row meet, lane group g keeping column 4*ch + g
+            *reinterpret_cast<float *>(smem + pw + 16 * ch) = d * lev_lanegroup_sums4(v);
         }
         lev_barrier_lds();
         if (wave < slots) {

@@ -863,14 +863,8 @@ q4_k_q8_mfma_one(const uint8_t *__restrict__ w, const uint8_t *__restrict__ xq, 
                 t = fmaf(scb, dxb[ch][i] * (float)d1[i], t);
                 v[i] = fmaf(-mnb, sbm[ch][i], t);
             }
-            // the four lane groups' shares of a row meet, lane group g keeping column 4*ch + g: two
-            // exchanges between the halves of the wave, one between the rows of a half
-            auto s02 = __builtin_amdgcn_permlane32_swap(__float_as_uint(v[0]), __float_as_uint(v[2]), false, false);
-            auto s13 = __builtin_amdgcn_permlane32_swap(__float_as_uint(v[1]), __float_as_uint(v[3]), false, false);
-            const float a = __uint_as_float(s02[0]) + __uint_as_float(s02[1]);
-            const float b = __uint_as_float(s13[0]) + __uint_as_float(s13[1]);
-            auto sab = __builtin_amdgcn_permlane16_swap(__float_as_uint(a), __float_as_uint(b), false, false);
-            *reinterpret_cast<float *>(smem + pw + 16 * ch) = __uint_as_float(sab[0]) + __uint_as_float(sab[1]);
+            // the four lane groups' shares of a row meet, lane group g keeping column 4*ch + g
+            *reinterpret_cast<float *>(smem + pw + 16 * ch) = lev_lanegroup_sums4(v);
         }
         lev_barrier_lds();
         if (wave < slots) {
