@@ -245,9 +245,12 @@ __device__ __forceinline__ void q6m_greedy_token(top2 best, uint32_t nred, lev_f
     // launch and a cold round trip: 7 us behind a 25 us GEMV).  The partial goes out in
     // device-scope stores, which go through to memory, and the arrival is counted once they
     // have completed (a fence here would write back every dirty line of the L2, the rows of y
-    // included: 250 of those cost 12 us).  Arrivals are counted in eight groups (workgroup
-    // index mod 8, counters 4 KB apart, so that they do not queue up in one L2 channel); the
-    // last of each group arrives at a ninth counter.
+    // included: 250 of those cost 12 us).  Arrivals are counted in four groups (workgroup
+    // index mod 4, counters 4 KB apart: arrivals at one word are served one after the other, some
+    // ten nanoseconds each, and the workgroups of a resident grid finish within a microsecond of
+    // each other); the last of each group arrives at a fifth counter.  (Eight groups: 0.4 us
+    // slower at 250 workgroups, the second level then waits for more stragglers; one: the same
+    // as four there, and a queue of 250 in the worst case.)
     uint32_t last = 0u;
     if (lane == 0u) {
         float *pf = reinterpret_cast<float *>(partials + blockIdx.x);
@@ -255,8 +258,9 @@ __device__ __forceinline__ void q6m_greedy_token(top2 best, uint32_t nred, lev_f
         __hip_atomic_store(pf + 1, m.second, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __hip_atomic_store(pf + 2, __builtin_bit_cast(float, m.idx), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         lev_publish_wait();
-        const uint32_t grp = blockIdx.x & 7u, ngrp = gridDim.x < 8u ? gridDim.x : 8u;
-        const uint32_t in_grp = (gridDim.x - grp + 7u) >> 3;
+        constexpr uint32_t G = 4u;
+        const uint32_t grp = blockIdx.x % G, ngrp = gridDim.x < G ? gridDim.x : G;
+        const uint32_t in_grp = (gridDim.x - grp + G - 1u) / G;
         if (__hip_atomic_fetch_add(&tickets[(1u + grp) * 1024u], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ==
             in_grp - 1u) {
             // nobody else touches the counter before the next launch
