@@ -438,19 +438,47 @@ moe_grouped_kernel(lev_moe_grouped_args a, uint32_t tiles_per_wg, const float *_
 }
 
 // 4. merge in slot order (g4_axpy chain, Gemma4.swift:2171-2175); dropped pairs add nothing.
+// grid (ceil(hidden / 1024), tokens), 256 threads, four outputs a thread.  Eight slots' rows are
+// requested together (a row of a dropped pair was never written: it is read all the same, so that
+// no load waits behind a branch, and replaced by zeros), the multiply-adds follow in slot order.
 __global__ void __launch_bounds__(256)
 moe_merge_kernel(const float *__restrict__ dn, const float *__restrict__ weights,
                  const uint8_t *__restrict__ valid, float *__restrict__ y, uint32_t hidden,
                  uint32_t top_k) {
-    const uint32_t t = blockIdx.y, h = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t t = blockIdx.y, h = (blockIdx.x * 256u + threadIdx.x) * 4u;
     if (h >= hidden) return;
-    float acc = 0.f;
-    for (uint32_t k = 0; k < top_k; ++k) {
-        const uint32_t p = t * top_k + k;
-        const float v = valid[p] ? dn[(uint64_t)p * hidden + h] : 0.f;
-        acc = fmaf(weights[p], v, acc);
+    const bool whole = h + 4u <= hidden && (hidden & 3u) == 0u;   // (hidden is a multiple of 256 on this path)
+    lev_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (uint32_t k0 = 0; k0 < top_k; k0 += 8u) {
+        lev_f32x4 v[8];
+        float w[8];
+        bool ok[8];
+#pragma unroll
+        for (uint32_t u = 0; u < 8u; ++u) {
+            const uint32_t p = t * top_k + (k0 + u < top_k ? k0 + u : top_k - 1u);
+            const float *row = dn + (uint64_t)p * hidden + h;
+            if (whole) {
+                v[u] = *reinterpret_cast<const lev_f32x4 *>(row);
+            } else {
+#pragma unroll
+                for (uint32_t c = 0; c < 4u; ++c) v[u][c] = h + c < hidden ? row[c] : 0.f;
+            }
+            w[u] = weights[p];
+            ok[u] = valid[p] != 0 && k0 + u < top_k;
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < 8u; ++u) {
+            if (k0 + u >= top_k) break;
+            const lev_f32x4 vu = ok[u] ? v[u] : lev_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (uint32_t c = 0; c < 4u; ++c) acc[c] = fmaf(w[u], vu[c], acc[c]);
+        }
     }
-    y[(uint64_t)t * hidden + h] = acc;
+    if (whole) {
+        *reinterpret_cast<lev_f32x4 *>(y + (uint64_t)t * hidden + h) = acc;
+    } else {
+        for (uint32_t c = 0; c < 4u && h + c < hidden; ++c) y[(uint64_t)t * hidden + h + c] = acc[c];
+    }
 }
 
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
@@ -555,7 +583,7 @@ hipError_t lev_moe_grouped_launch(lev_ctx *ctx, const lev_moe_grouped_args &a, c
     hipLaunchKernelGGL((moe_grouped_kernel<false>), dim3((tiles_dn + tpw_dn - 1) / tpw_dn, a.experts),
                        dim3(kGrpThreads), lds_dn, ctx->stream, a, tpw_dn, act, nullptr, nullptr, amax, goff, glist, dn, nullptr);
     if ((e = hipGetLastError()) != hipSuccess) return e;
-    hipLaunchKernelGGL(moe_merge_kernel, dim3((a.hidden + 255) / 256, a.tokens), dim3(256), 0, ctx->stream,
+    hipLaunchKernelGGL(moe_merge_kernel, dim3((a.hidden + 1023) / 1024, a.tokens), dim3(256), 0, ctx->stream,
                        dn, weights, valid, y, a.hidden, a.top_k);
     return hipGetLastError();
 }
