@@ -322,6 +322,55 @@ def test_moe_grouped_path_many_experts(ctx, experts):
         assert O.max_rel_err(y[t], ref["y"]) < TOL
 
 
+@pytest.mark.parametrize("experts", [16, 1500])
+def test_moe_grouped_path_many_tokens(ctx, experts):
+    """2100 tokens through the grouped path: with 16 experts every expert takes many passes of
+    twelve columns over its weights, with 1500 the scan over the expert counts crosses waves and
+    most experts hold a handful of pairs.  Sampled tokens against the FP64 chain, and the first 64
+    tokens as a batch of their own bit for bit (a pair's result does not depend on the batch)."""
+    hidden, inter, top_k, tokens = 256, 256, 4, 2100
+    wr, pool, offs, x = H.config5(hidden, inter, experts, tokens, seed=experts + 7)
+    rng = np.random.default_rng(experts + 7)
+    ids = np.stack([rng.permutation(experts)[:top_k] for _ in range(tokens)]).astype(np.int32)
+    ids[0, 0], ids[1, 1] = experts - 1, 0
+    wts = rng.random((tokens, top_k)).astype(np.float32)
+    y, act = run_experts(ctx, pool, offs, hidden, inter, experts, x, ids, wts)
+    g, u, d = (pool[offs["gate_off"]:], pool[offs["up_off"]:], pool[offs["down_off"]:])
+    for t in list(range(0, tokens, 97)) + [1, tokens - 1]:
+        ref = O.moe_experts_f64(g, u, d, hidden, inter, ids[t], wts[t], x[t])
+        assert O.max_rel_err(act[t], ref["act"]) < TOL
+        assert O.max_rel_err(y[t], ref["y"]) < TOL
+    y64, act64 = run_experts(ctx, pool, offs, hidden, inter, experts, x[:64], ids[:64], wts[:64])
+    assert np.array_equal(y64.view(np.uint32), y[:64].view(np.uint32))
+    assert np.array_equal(act64.view(np.uint32), act[:64].view(np.uint32))
+
+
+def test_moe_grouped_path_rejects_bad_expert_ids(ctx):
+    """The same rule on the many-token path: a pair whose id is out of range or repeats another
+    slot of its token is dropped (it adds nothing to its token) and reported; the other tokens
+    are computed."""
+    from leviathan_amd import capi, ops
+    from leviathan_amd.ops import LevError
+    hidden, inter, experts, top_k, tokens = 256, 256, 8, 2, 6
+    wr, pool, offs, x = H.config5(hidden, inter, experts, tokens, seed=11)
+    good = np.array([[0, 1], [2, 3], [4, 5], [6, 7], [1, 2], [3, 4]], np.int32)
+    wts = np.full((tokens, top_k), 0.5, np.float32)
+    y_good, _ = run_experts(ctx, pool, offs, hidden, inter, experts, x, good, wts)
+    for bad_row in ([5, 5], [1, 9], [-1, 2]):
+        ids = good.copy()
+        ids[2] = bad_row
+        pool_d = dev(pool)
+        pools = ops.Context.moe_pools(pool_d, hidden, inter, experts, offs["gate_off"], offs["up_off"], offs["down_off"])
+        y = ctx.moe_experts_q4_0(pools, dev(x), dev(ids), dev(wts), top_k, tokens)
+        with pytest.raises(LevError) as e:
+            ctx.sync()
+        assert e.value.status == capi.BAD_DIMENSIONS
+        y = y.cpu().numpy()
+        for t in (0, 1, 3, 4, 5):
+            assert np.array_equal(y[t].view(np.uint32), y_good[t].view(np.uint32))
+        assert np.all(np.isfinite(y[2]))
+
+
 def test_moe_rejects_bad_expert_ids(ctx):
     """MoEModelBinding.offsets (MoEModelBinding.swift:174-214): ids must be in
     range and distinct; nothing is written through a bad id."""
