@@ -35,7 +35,13 @@
 // not the bytes, kept the L1 busy for more than half of the kernel), parks them in
 // a small wave-private LDS area, and every lane reads from there the four code
 // bytes (both nibbles: eight weights) and the scale it multiplies.
+//
+// Batches of at most four pairs per expert on average, with rows of up to 2048 activations, take
+// the integer matrix cores instead (moe_grouped_i8_kernel below: the digit planes of the few-token
+// kernels, four tokens of an expert per product, operands in registers): they cost less per
+// product and more per token, and win while most experts hold no more than a handful of pairs.
 #include "moe_grouped.hpp"
+#include "q4_0_mfma.hpp"
 
 #include <cstdlib>
 
@@ -103,9 +109,11 @@ moe_group_kernel(const int32_t *__restrict__ ids, uint32_t pairs, uint32_t exper
                  int32_t *__restrict__ goff, int32_t *__restrict__ glist,
                  uint8_t *__restrict__ valid, int *__restrict__ flag, const float *__restrict__ x,
                  uint32_t hidden, _Float16 *__restrict__ xh, _Float16 *__restrict__ xl,
-                 uint32_t *__restrict__ xmax, uint32_t *__restrict__ amax) {
-    extern __shared__ int32_t s_cnt[];          // [experts] counts, then [experts] cursors
-    int32_t *s_cur = s_cnt + experts;
+                 uint32_t *__restrict__ xmax, uint32_t *__restrict__ amax, lev_grp_item *items,
+                 int32_t *__restrict__ n_items, uint32_t item_pairs) {
+    // [experts] counts | cursors | with items: first pair | first item of more than four pairs | first other item
+    extern __shared__ int32_t s_cnt[];
+    int32_t *s_cur = s_cnt + experts, *s_first = s_cur + experts, *s_big = s_first + experts, *s_small = s_big + experts;
     const uint32_t tid = threadIdx.x;
     if (blockIdx.x != 0u) {
         __shared__ float s_max[16];
@@ -132,10 +140,12 @@ moe_group_kernel(const int32_t *__restrict__ ids, uint32_t pairs, uint32_t exper
         }
         return;
     }
-    for (uint32_t p = tid; p < pairs; p += 1024u) amax[p] = 0u;
+    if (amax)
+        for (uint32_t p = tid; p < pairs; p += 1024u) amax[p] = 0u;
     for (uint32_t e = tid; e < experts; e += 1024u) s_cnt[e] = 0;
     __syncthreads();
     bool bad_seen = false;
+    int32_t e_own = -1;                          // the thread's first pair, kept for the placement: its expert, or -1
     for (uint32_t p = tid; p < pairs; p += 1024u) {
         const int32_t e = ids[p];
         bool ok = e >= 0 && (uint32_t)e < experts;
@@ -144,31 +154,46 @@ moe_group_kernel(const int32_t *__restrict__ ids, uint32_t pairs, uint32_t exper
             if (k != slot && ids[first + k] == e) ok = false;   // both copies of a duplicate are dropped
         valid[p] = ok ? 1 : 0;
         if (ok) atomicAdd(&s_cnt[e], 1);
+        if (p == tid && ok) e_own = e;
         bad_seen = bad_seen || !ok;
     }
     if (bad_seen) atomicOr(flag, kFlagBadExpertId);
     __syncthreads();
     // exclusive scan of the counts (experts <= 4096): thread i takes experts 4i..4i+3, the waves scan
-    // their threads' sums by shuffles and meet in LDS
+    // their threads' sums by shuffles and meet in LDS.  One scan carries three counts of at most
+    // 2^20 each in 21-bit fields: pairs, items of more than four pairs, other items.
+    __shared__ uint64_t s_wave[16];
     {
-        __shared__ int32_t s_wave[16];
-        int32_t c4[4], local = 0;
+        int32_t c4[4], big4[4], small4[4];
+        const int32_t ip = items ? (int32_t)item_pairs : 1, ish = ip == 8 ? 3 : ip == 4 ? 2 : 0;   // (4 or 8 pairs an item)
+        uint64_t local = 0;
 #pragma unroll
         for (uint32_t k = 0; k < 4u; ++k) {
             const uint32_t e = 4u * tid + k;
             c4[k] = e < experts ? s_cnt[e] : 0;
-            local += c4[k];
+            // work items of the integer matrix-core kernels: runs of at most item_pairs pairs of one expert
+            const int32_t full = c4[k] >> ish, rem = c4[k] - (full << ish);
+            big4[k] = items ? (ip > 4 ? full : 0) + (rem > 4 ? 1 : 0) : 0;
+            small4[k] = items ? (ip > 4 ? 0 : full) + (rem > 0 && rem <= 4 ? 1 : 0) : 0;
+            local += (uint64_t)c4[k] | (uint64_t)big4[k] << 21 | (uint64_t)small4[k] << 42;
         }
-        int32_t incl = local;
+        uint64_t incl = local;
 #pragma unroll
         for (int off = 1; off < 64; off <<= 1) {
-            const int32_t o = __shfl_up(incl, off);
+            const uint64_t o = __shfl_up(incl, off);
             if ((int)(tid & 63u) >= off) incl += o;
         }
         if ((tid & 63u) == 63u) s_wave[tid >> 6] = incl;
         __syncthreads();
-        int32_t run = incl - local;
-        for (uint32_t w = 0; w < (tid >> 6); ++w) run += s_wave[w];
+        uint64_t before = incl - local, all = 0;
+#pragma unroll
+        for (uint32_t w = 0; w < 16u; ++w) {
+            const uint64_t v = s_wave[w];
+            before += w < (tid >> 6) ? v : 0u;
+            all += v;
+        }
+        int32_t run = (int32_t)(before & 0x1FFFFFu);
+        const int32_t first_pair = run;
 #pragma unroll
         for (uint32_t k = 0; k < 4u; ++k) {
             const uint32_t e = 4u * tid + k;
@@ -178,12 +203,62 @@ moe_group_kernel(const int32_t *__restrict__ ids, uint32_t pairs, uint32_t exper
         }
         // 4096 experts: the total has no thread of its own (thread i owns 4i..4i+3 <= 4095)
         if (4u * tid + 4u == experts && experts == 4096u) goff[experts] = run;
+        if (items) {
+            // Items of more than four pairs (two products a block) come first, in expert order, the
+            // others behind them: what a round costs then depends on its position in the line of
+            // rounds alone.
+            const int32_t nbig = (int32_t)(all >> 21 & 0x1FFFFFu), nsmall = (int32_t)(all >> 42);
+            int32_t brun = (int32_t)(before >> 21 & 0x1FFFFFu), srun = nbig + (int32_t)(before >> 42);
+            if (tid == 0u) {
+                n_items[0] = nbig + nsmall;
+                n_items[1] = nbig;
+            }
+            int32_t prun = first_pair;
+#pragma unroll
+            for (uint32_t k = 0; k < 4u; ++k) {
+                const uint32_t e = 4u * tid + k;
+                if (e < experts) {
+                    s_first[e] = prun;
+                    s_big[e] = brun;
+                    s_small[e] = srun;
+                }
+                const int32_t n = big4[k] + small4[k];
+                for (int32_t j = 0; j < n; ++j) {
+                    const int32_t left = c4[k] - j * ip, count = left < ip ? left : ip;
+                    lev_grp_item *it = items + (count > 4 ? brun++ : srun++);
+                    it->expert = (int32_t)e;
+                    it->count = count;
+                    it->first = prun + j * ip;
+                }
+                prun += c4[k];
+            }
+        }
     }
     __syncthreads();
     // The order of an expert's pairs in the list depends on the atomics; no
     // result does: every pair is computed independently and owns its outputs.
     for (uint32_t p = tid; p < pairs; p += 1024u)
-        if (valid[p]) glist[atomicAdd(&s_cur[ids[p]], 1)] = (int32_t)p;
+        if (p == tid ? e_own >= 0 : valid[p] != 0) {
+            const int32_t e = p == tid ? e_own : ids[p];
+            const int32_t at = atomicAdd(&s_cur[e], 1);
+            glist[at] = (int32_t)p;
+            if (items) {
+                // the pair's column in its item: the expert's items of more than four pairs come
+                // first in the expert's list (whole items, then a remainder of more than four)
+                const int32_t ip = (int32_t)item_pairs, ish = ip == 8 ? 3 : 2, c = s_cnt[e], pos = at - s_first[e];
+                const int32_t full = c >> ish, rem = c - (full << ish), nbig = (ip > 4 ? full : 0) + (rem > 4 ? 1 : 0);
+                const int32_t j = pos >> ish;
+                lev_grp_item *it = items + (j < nbig ? s_big[e] + j : s_small[e] + (j - nbig));
+                const int32_t left = c - j * ip, count = left < ip ? left : ip, col = pos - j * ip;
+                it->pair[col] = (int32_t)p;
+                it->src[col] = (int32_t)(p / top_k);
+                if (col == count - 1)   // the columns past the count repeat the last pair
+                    for (int32_t k = count; k < 8; ++k) {
+                        it->pair[k] = (int32_t)p;
+                        it->src[k] = (int32_t)(p / top_k);
+                    }
+            }
+        }
 }
 
 // ---------------------------------------------------------------------------
@@ -437,6 +512,349 @@ moe_grouped_kernel(lev_moe_grouped_args a, uint32_t tiles_per_wg, const float *_
     }
 }
 
+// ---------------------------------------------------------------------------
+// 2./3. on the integer matrix cores, four tokens of an expert per product.
+//
+// v_mfma_i32_16x16x32_i8 multiplies 16 A rows x 32 k x 16 weight rows: ONE Q4_0 block of 16 weight
+// rows.  A row 4t + p is digit plane p of token t (x as integers X = rint(x * 2^(156 - ex)), ex
+// the exponent of the largest magnitude among the task's 256 activations, cut into four balanced
+// base-256 digits: the arithmetic of the few-token kernels), so the output lane (row, t) holds
+// the four plane sums of token t against its row's block: they are recombined in 32-bit integers
+// and f32 and scaled by the block's d there, with nothing exchanged between lanes.  B: lane
+// (row, g) supplies code bytes 4g..4g+3 of the block, low nibbles then high nibbles, as int8
+// 16 * (n - 8) (flip the top bit of every nibble, mask; the low nibbles shifted up first).
+//
+// A task is fetched as in the decode GEMV (a quad of lanes reads the 144 contiguous bytes of a
+// row's four block pairs; one lane permutation per dword brings pair g of row r to lane (r, g));
+// the dwords of a block are then spread over the four lanes of its row by a 4 x 4 transpose
+// between the lane groups (four row swaps), and the scales of the row's eight blocks are
+// gathered the same way.
+//
+// A work ITEM is up to kG8NT pairs of one expert (the grouping kernel cuts each expert's list into
+// such runs).  Every item takes the same number of ROUNDS over its expert's rows, so the rounds of
+// all items form one line that the grid's workgroups cut into equal stretches, whatever the
+// routing: a workgroup works through `total * L / G .. total * (L + 1) / G` and stages the
+// activations of each item its stretch touches.  Stretches that follow each other go to
+// workgroups of one XCD (an expert with more than kG8NT pairs is streamed by neighbours, through
+// one L2).
+//
+// Workgroup = wpr * slots waves (eight for gate/up, twelve for down), as in the decode GEMV: wave (slot, pos) owns
+// column task `pos` (256 activations) of the row groups of its slot, stages the task's
+// activations for all of the item's tokens by itself and keeps the operands in registers (16 per
+// four tokens).  A round of a wave is NTILE tiles of 16 rows x 256 codes: gate and up rows of one
+// row group (PAIRED), or NTILE consecutive row groups (down); the next round's bytes are
+// requested as soon as this round's have been handed to the lanes that multiply them.  The wpr
+// partial sums of a (row, token) meet in LDS behind one barrier a batch of rounds; wave u adds
+// unit u of the batch (a slot's 16 rows x four tokens), applies the activation function (PAIRED)
+// and stores.
+// ---------------------------------------------------------------------------
+constexpr int kG8MaxWpr = 8;                              // waves that share a row group: one task each
+constexpr int kG8WavesGateUp = 8;                         // 2048 activations: eight column tasks, one slot
+constexpr int kG8WavesDown = 12;                          // 768 activations: three column tasks, four slots (three
+                                                          // waves a SIMD; eight waves leave two SIMDs with one)
+constexpr int kG8NT = 8;                                  // tokens per item
+static_assert(kG8NT == 4 || kG8NT == 8, "an item is one or two groups of four tokens");
+constexpr uint32_t kG8Batch = 4;                          // rounds between two barriers of a workgroup (2: 55.4
+                                                          // against 53.6 us for gate/up, 1: 64.9)
+constexpr uint32_t kG8MaxInLen = 256u * kG8MaxWpr;
+constexpr uint32_t kG8Plane = 272u;                       // a digit plane of a staged task: 256 bytes + 16, so that
+constexpr uint32_t kG8TokArea = 4u * kG8Plane;            // the 64 lanes of an operand read hit 64 different banks
+constexpr uint32_t kG8WaveLds = 4u * kG8TokArea;           // four tokens are staged at a time
+
+// LDS: part [parity 2][round of the batch][tile NTILE][token / 4][wave][row 16][token % 4] f32 | per wave four
+// staged tasks
+template <int NTILE, int NW>
+constexpr size_t g8_lds() {
+    return (size_t)2 * kG8Batch * NTILE * (kG8NT / 4) * (NW * 256u) + (size_t)NW * kG8WaveLds;
+}
+
+// Digit planes of one token's task into `tok` (kG8TokArea bytes, this wave's own): lane i holds
+// elements 4i..4i+3 of the task's 256 activations; plane p, byte e = digit p of element e.
+// Returns the power of two that undoes the scaling (and the 16 of the codes); NaN when the task
+// holds a NaN or an infinity.
+__device__ __forceinline__ float g8_stage_token(const lev_f32x4 v, uint8_t *tok) {
+    const uint32_t lane = threadIdx.x & 63u;
+    uint32_t mb = 0u;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const uint32_t bits = __float_as_uint(v[k]) & 0x7FFFFFFFu;
+        mb = bits > mb ? bits : mb;
+    }
+#define LEV_G8_MAXSTEP(CTRL)                                                                             \
+    {                                                                                                    \
+        const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp((int)mb, (int)mb, CTRL, 0xF, 0xF, false); \
+        mb = o > mb ? o : mb;                                                                            \
+    }
+    LEV_G8_MAXSTEP(0xB1)    // quad_perm [1,0,3,2]
+    LEV_G8_MAXSTEP(0x4E)    // quad_perm [2,3,0,1]
+    LEV_G8_MAXSTEP(0x141)   // row_half_mirror
+    LEV_G8_MAXSTEP(0x140)   // row_mirror: the 16 lanes of a row hold the row's maximum
+#undef LEV_G8_MAXSTEP
+    {
+        const auto s0 = __builtin_amdgcn_permlane32_swap(mb, mb, false, false);
+        mb = s0[0] > s0[1] ? s0[0] : s0[1];
+        const auto s1 = __builtin_amdgcn_permlane16_swap(mb, mb, false, false);
+        mb = s1[0] > s1[1] ? s1[0] : s1[1];                    // every lane: the task's maximum
+    }
+    uint32_t ex = mb >> 23;                                    // |x| < 2^(ex - 126)
+    const bool bad = ex == 255u;
+    ex = ex < 34u ? 34u : (ex > 254u ? 254u : ex);             // keeps both powers of two normal numbers
+    const float scale = __uint_as_float((283u - ex) << 23);    // 2^(156 - ex): |x * scale| < 2^30
+    uint32_t Y[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) Y[k] = ((uint32_t)(int)rintf(v[k] * scale) + 0x00808080u) ^ 0x00808080u;
+    // 4x4 byte transpose: digit p of the lane's four values in one dword
+    const uint32_t t0 = __builtin_amdgcn_perm(Y[1], Y[0], 0x05010400u);
+    const uint32_t t1 = __builtin_amdgcn_perm(Y[1], Y[0], 0x07030602u);
+    const uint32_t t2 = __builtin_amdgcn_perm(Y[3], Y[2], 0x05010400u);
+    const uint32_t t3 = __builtin_amdgcn_perm(Y[3], Y[2], 0x07030602u);
+    uint32_t *at = reinterpret_cast<uint32_t *>(tok + 4u * lane);
+    at[0u * (kG8Plane / 4u)] = __builtin_amdgcn_perm(t2, t0, 0x05040100u);
+    at[1u * (kG8Plane / 4u)] = __builtin_amdgcn_perm(t2, t0, 0x07060302u);
+    at[2u * (kG8Plane / 4u)] = __builtin_amdgcn_perm(t3, t1, 0x05040100u);
+    at[3u * (kG8Plane / 4u)] = __builtin_amdgcn_perm(t3, t1, 0x07060302u);
+    return bad ? __builtin_nanf("") : __uint_as_float((ex - 33u) << 23);   // 2^(ex - 160)
+}
+
+// A operands of four staged tokens (`toks`: their kG8TokArea areas, one behind the other): lane
+// (a, g) = (lane % 16, lane / 16) supplies, for block b of the task, plane a % 4 of token a / 4
+// at the block's elements 4g..4g+3 and 16+4g..16+4g+3 (the elements whose codes lie in bytes
+// 4g..4g+3 of the block).
+__device__ __forceinline__ void g8_read_operands(const uint8_t *toks, long (&A)[8]) {
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t a = lane & 15u, g = lane >> 4;
+    const uint32_t *p = reinterpret_cast<const uint32_t *>(toks + (a >> 2) * kG8TokArea + (a & 3u) * kG8Plane + 4u * g);
+#pragma unroll
+    for (int b = 0; b < 8; ++b) A[b] = (long)(((uint64_t)p[8 * b + 4] << 32) | (uint64_t)p[8 * b]);
+}
+
+// In: lane (r, g) holds q[j] = dword j of a record of lane group g.  Out: q[P] = dword g of the
+// record of lane group P (a 4 x 4 transpose between the four lanes of a row, by row swaps).
+__device__ __forceinline__ void g8_transpose4(uint32_t (&q)[4]) {
+    const auto a = __builtin_amdgcn_permlane16_swap(q[0], q[1], false, false);
+    const auto b = __builtin_amdgcn_permlane16_swap(q[2], q[3], false, false);
+    const auto c = __builtin_amdgcn_permlane32_swap(a[0], b[0], false, false);
+    const auto d = __builtin_amdgcn_permlane32_swap(a[1], b[1], false, false);
+    q[0] = c[0]; q[1] = d[0]; q[2] = c[1]; q[3] = d[1];
+}
+
+// One tile (16 rows x 256 codes; W: the lane's pair, already turned) against NJ groups of four
+// tokens, of which the first ng take part: val[j] = the task's sum for (row lane % 16, token
+// 4j + lane / 16), blocks added in their order.
+template <uint32_t NJ>
+__device__ __forceinline__ void g8_tile_dot(const uint32_t W[9], const long (&A)[NJ][8], uint32_t ng,
+                                            const float (&unscale)[NJ], float (&val)[NJ]) {
+    uint32_t qa[4], qb[4];
+    qa[0] = __builtin_amdgcn_alignbit(W[1], W[0], 16);
+    qa[1] = __builtin_amdgcn_alignbit(W[2], W[1], 16);
+    qa[2] = __builtin_amdgcn_alignbit(W[3], W[2], 16);
+    qa[3] = __builtin_amdgcn_alignbit(W[4], W[3], 16);
+    qb[0] = W[5]; qb[1] = W[6]; qb[2] = W[7]; qb[3] = W[8];
+    g8_transpose4(qa);
+    g8_transpose4(qb);
+    // the pair's two scales in one dword, then every lane of a row gets the row's four dwords
+    const uint32_t dd = __builtin_amdgcn_perm(W[4], W[0], 0x07060100u);
+    const auto s = __builtin_amdgcn_permlane16_swap(dd, dd, false, false);      // pairs g & ~1, g | 1
+    const auto e = __builtin_amdgcn_permlane32_swap(s[0], s[0], false, false);  // pairs 0, 2
+    const auto o = __builtin_amdgcn_permlane32_swap(s[1], s[1], false, false);  // pairs 1, 3
+    const uint32_t dp[4] = {e[0], o[0], e[1], o[1]};
+    long B[8];
+    float d[8];
+#pragma unroll
+    for (int b = 0; b < 8; ++b) {
+        const uint32_t q = ((b & 1) ? qb[b >> 1] : qa[b >> 1]) ^ 0x88888888u;
+        B[b] = (long)(((uint64_t)(q & 0xF0F0F0F0u) << 32) | (uint64_t)((q << 4) & 0xF0F0F0F0u));
+        d[b] = lev_f16_bits_to_f32((b & 1) ? dp[b >> 1] >> 16 : dp[b >> 1] & 0xFFFFu);
+    }
+    // a group's eight products are independent: they issue back to back, the sums follow
+    auto group = [&](const long (&Aj)[8]) {
+        lev_i32x4 acc[8];
+#pragma unroll
+        for (int b = 0; b < 8; ++b)
+            acc[b] = __builtin_amdgcn_mfma_i32_16x16x32_i8(Aj[b], B[b], lev_i32x4{0, 0, 0, 0}, 0, 0, 0);
+        float v = 0.f;
+#pragma unroll
+        for (int b = 0; b < 8; ++b) {
+            // |plane sum| <= 32 * 128 * 128 = 2^19: two planes recombine in 32 bits, the halves in f32
+            const float f = fmaf((float)(acc[b][2] + (acc[b][3] << 8)), 65536.0f, (float)(acc[b][0] + (acc[b][1] << 8)));
+            v = fmaf(d[b], f, v);
+        }
+        return v;
+    };
+    val[0] = group(A[0]);
+#pragma unroll
+    for (uint32_t j = 1; j < NJ; ++j) {
+        val[j] = 0.f;
+        if (j < ng) val[j] = group(A[j]);
+    }
+#pragma unroll
+    for (uint32_t j = 0; j < NJ; ++j) val[j] *= unscale[j];
+}
+
+template <int NTILE, bool PAIRED, int NW>
+__global__ void __launch_bounds__(NW * LEV_WAVE)
+moe_grouped_i8_kernel(lev_moe_grouped_args a, const float *__restrict__ src, const lev_grp_item *__restrict__ items,
+                      const int32_t *__restrict__ n_items, float *__restrict__ out, uint32_t wpr, uint32_t slots,
+                      uint32_t rpi, uint64_t slot_of_wave, uint64_t pos_of_wave, uint32_t w1, uint32_t w2) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    constexpr uint32_t NT = kG8NT, NJ = NT / 4u;
+    constexpr uint32_t TO = PAIRED ? 1u : (uint32_t)NTILE;       // row groups a slot finishes per round
+    constexpr uint32_t kG8Unit = NW * 256u;                       // bytes of part[wave][row][token % 4]: one tile's sums of four tokens
+    constexpr uint32_t kRound = NTILE * NJ * kG8Unit;             // one round's sums in `part`
+    constexpr uint32_t kHalf = kG8Batch * kRound;                 // one parity of `part`: a batch of rounds
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    const uint32_t nwaves = blockDim.x >> 6;                      // wpr * slots: every wave has a task
+    const uint32_t slot = (uint32_t)(slot_of_wave >> (4u * wave)) & 15u;
+    const uint32_t tw = (uint32_t)(pos_of_wave >> (4u * wave)) & 15u;
+    const uint32_t in_len = PAIRED ? a.hidden : a.inter, out_rows = PAIRED ? a.inter : a.hidden;
+    const uint32_t ngroups = (out_rows + 15u) >> 4;
+    const uint64_t row_bytes = (uint64_t)(in_len >> 6) * 36u;
+    const uint32_t r = lane & 15u, g = lane >> 4, lrow = lane >> 2;
+
+    // this workgroup's stretch of the line of rounds
+    const uint32_t G = gridDim.x;
+    const uint32_t L = (G & 7u) == 0u ? (blockIdx.x & 7u) * (G >> 3) + (blockIdx.x >> 3) : blockIdx.x;
+    // A round of an item of more than four pairs costs w2, any other w1; the line is cut into
+    // stretches of equal COST.  The items of more than four pairs come first, so a position in
+    // cost is a position in rounds by two divisions (32-bit arithmetic: rounds * w < 2^29,
+    // G <= 2^10; a 64-bit division is a hundred instructions).
+    const uint32_t R2 = (uint32_t)n_items[1] * rpi, C2 = R2 * w2;
+    const uint32_t total = C2 + ((uint32_t)n_items[0] * rpi - R2) * w1, per = total / G, rest = total - per * G;
+    auto rounds_before = [&](uint32_t c) { return c <= C2 ? (c + w2 - 1u) / w2 : R2 + (c - C2 + w1 - 1u) / w1; };
+    uint32_t R = rounds_before(per * L + rest * L / G);
+    const uint32_t Rend = rounds_before(per * (L + 1u) + rest * (L + 1u) / G);
+
+    uint8_t *area = smem + 2u * kHalf + (size_t)wave * kG8WaveLds;
+    // byte offsets into the workgroup's LDS, not pointers; lane (r, g) writes row r, token 4j + g
+    uint32_t pw = ((wave * 16u + r) * 4u + g) * 4u;
+    uint32_t half = 0u;                                           // byte offset of the round's parity
+
+    while (R < Rend) {
+        const uint32_t it = R / rpi, r0 = R - it * rpi;
+        const uint32_t nr = rpi - r0 < Rend - R ? rpi - r0 : Rend - R;   // rounds r0 .. r0 + nr of item `it`
+        // request order = return order: the item (one scalar load), the activations of the wave's
+        // task for every token, and the first round's weights behind them, so that the staging
+        // does not wait for the weights
+        const lev_grp_item *item = items + it;
+        const uint32_t e = (uint32_t)item->expert, cnt = (uint32_t)item->count;
+        const uint32_t ng = (cnt + 3u) >> 2;                      // groups of four tokens that take part
+        int32_t pk[NT];
+        lev_f32x4 v[NT];
+#pragma unroll
+        for (uint32_t k = 0; k < NT; ++k) {
+            pk[k] = item->pair[k];
+            const uint32_t srow = (uint32_t)(PAIRED ? item->src[k] : item->pair[k]);
+            v[k] = reinterpret_cast<const lev_f32x4 *>(src + (uint64_t)srow * in_len)[64u * tw + lane];
+        }
+        const uint8_t *m0 = a.base + (PAIRED ? a.gate_off + e * a.gate_stride : a.down_off + e * a.down_stride);
+        const uint8_t *m1 = PAIRED ? a.base + a.up_off + e * a.up_stride : m0;
+        auto issue = [&](uint32_t rho, uint32_t (&D)[NTILE][9]) {
+#pragma unroll
+            for (int t = 0; t < NTILE; ++t) {
+                uint32_t rg = PAIRED ? rho * slots + slot : (rho * slots + slot) * (uint32_t)NTILE + (uint32_t)t;
+                rg = rg < ngroups ? rg : ngroups - 1u;
+                uint32_t row = rg * 16u + lrow;
+                row = row < out_rows ? row : out_rows - 1u;
+                q4m_load_task((PAIRED && t == 1 ? m1 : m0) + (uint64_t)row * row_bytes, 4u * tw, D[t]);
+            }
+        };
+        __builtin_amdgcn_sched_barrier(0);
+        const uint32_t r_last = r0 + nr - 1u;
+        uint32_t Da[NTILE][9];
+        issue(r0, Da);
+        __builtin_amdgcn_sched_barrier(0);
+        // the activations are requested for every column, whatever the item's count (columns past
+        // the count repeat the last pair), in front of the weights: a request inside the branch
+        // below would queue behind them
+#pragma unroll
+        for (uint32_t k = 0; k < NT; ++k) lev_pin(v[k]);
+        long A[NJ][8];
+        float unscale[NJ];
+#pragma unroll
+        for (uint32_t j = 0; j < NJ; ++j) {
+#pragma unroll
+            for (int b = 0; b < 8; ++b) A[j][b] = 0;
+            unscale[j] = 0.f;
+            if (j < ng) {
+                // the area belongs to this wave alone: LDS runs a wave's accesses in order, the fences
+                // only keep the compiler from moving reads above writes (and the next group's writes
+                // above these reads)
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                float us[4];
+#pragma unroll
+                for (uint32_t k = 0; k < 4u; ++k) us[k] = g8_stage_token(v[4u * j + k], area + k * kG8TokArea);
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                g8_read_operands(area, A[j]);
+                unscale[j] = g == 0u ? us[0] : g == 1u ? us[1] : g == 2u ? us[2] : us[3];
+            }
+        }
+        // the operands are read back before the wait for the weights, not behind it
+        __builtin_amdgcn_sched_barrier(0);
+
+        uint32_t batch0 = r0, nb = 0u;                            // the batch's first round, rounds in it so far
+        auto round = [&](uint32_t rho, uint32_t (&D)[NTILE][9]) {
+            // lane (r, g) <- lane 4r + g; the registers the bytes came in take a later round's
+            // request at once (unconditional, clamped: a branch around the loads would make the
+            // compiler wait for them before this round is multiplied)
+            uint32_t W[NTILE][9];
+#pragma unroll
+            for (int t = 0; t < NTILE; ++t) q4m_turn_task(D[t], W[t]);
+            __builtin_amdgcn_sched_barrier(0);
+            issue(rho + 1u < r_last ? rho + 1u : r_last, D);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int t = 0; t < NTILE; ++t) {
+                float val[NJ];
+                g8_tile_dot<NJ>(W[t], A, ng, unscale, val);
+#pragma unroll
+                for (uint32_t j = 0; j < NJ; ++j)
+                    if (j < ng)
+                        *reinterpret_cast<float *>(smem + half + nb * kRound + pw + ((uint32_t)t * NJ + j) * kG8Unit) = val[j];
+            }
+            // the waves meet once per batch of rounds (and at the item's end): between two barriers
+            // they run at their own pace, and the batch's sums are finished by several waves at once
+            if (++nb < kG8Batch && rho != r_last) return;
+            lev_barrier_lds();
+            // unit u = (round b of the batch, slot s, row group t of the slot's round, tokens 4j .. 4j + 3):
+            // lane (r, g) adds the slot's waves' sums of row r and token 4j + g in a fixed order
+            static_assert(NJ <= 2u, "the unit index is split by a shift");
+            const uint32_t per_round = slots * TO * ng;
+            for (uint32_t u = wave; u < nb * per_round; u += nwaves) {
+                const uint32_t b = u / per_round, ur = u - b * per_round;
+                const uint32_t j = ur & (ng - 1u), us_ = ur >> (ng - 1u), s = us_ / TO, t = us_ % TO;
+                const uint32_t k = 4u * j + g;
+                const uint32_t rg = PAIRED ? (batch0 + b) * slots + s : ((batch0 + b) * slots + s) * (uint32_t)NTILE + t;
+                const uint32_t row = rg * 16u + r;
+                const float *pp = reinterpret_cast<const float *>(
+                    smem + half + b * kRound + (t * NJ + j) * kG8Unit + ((s * wpr * 16u + r) * 4u + g) * 4u);
+                auto slot_sum = [&](const float *q) {
+                    float p[kG8MaxWpr];
+#pragma unroll
+                    for (uint32_t w = 0; w < (uint32_t)kG8MaxWpr; ++w) p[w] = q[(w < wpr ? w : 0u) * 64u];   // eight reads in flight
+#pragma unroll
+                    for (uint32_t w = 0; w < (uint32_t)kG8MaxWpr; ++w) p[w] = w < wpr ? p[w] : 0.f;
+                    return ((p[0] + p[4]) + (p[2] + p[6])) + ((p[1] + p[5]) + (p[3] + p[7]));
+                };
+                float res = slot_sum(pp);
+                if (PAIRED) res = lev_gelu_up_value(res, slot_sum(pp + NJ * (kG8Unit / 4u)));
+                int32_t pair = pk[0];
+#pragma unroll
+                for (uint32_t q = 1; q < NT; ++q) pair = k == q ? pk[q] : pair;
+                if (k < cnt && row < out_rows) out[(uint64_t)(uint32_t)pair * out_rows + row] = res;
+            }
+            half ^= kHalf;
+            batch0 = rho + 1u;
+            nb = 0u;
+        };
+        for (uint32_t rho = r0; rho <= r_last; ++rho) round(rho, Da);
+        R += nr;
+    }
+}
+
 // 4. merge in slot order (g4_axpy chain, Gemma4.swift:2171-2175); dropped pairs add nothing.
 // grid (ceil(hidden / 1024), tokens), 256 threads, four outputs a thread.  Eight slots' rows are
 // requested together (a row of a dropped pair was never written: it is read all the same, so that
@@ -484,7 +902,7 @@ moe_merge_kernel(const float *__restrict__ dn, const float *__restrict__ weights
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct grouped_layout {
-    size_t goff, glist, valid, xh, xl, xmax, amax, dn, total;
+    size_t goff, glist, valid, xh, xl, xmax, amax, dn, items, n_items, total;
 };
 
 grouped_layout layout_of(const lev_moe_grouped_args &a) {
@@ -499,6 +917,8 @@ grouped_layout layout_of(const lev_moe_grouped_args &a) {
     L.xmax = o; o += align256((size_t)a.tokens * 4);
     L.amax = o; o += align256(pairs * 4);
     L.dn = o; o += align256(pairs * a.hidden * 4);
+    L.items = o; o += align256((pairs / 8 + a.experts + 1) * sizeof(lev_grp_item));   // an expert with c pairs: ceil(c / 8) items
+    L.n_items = o; o += 256;
     L.total = o;
     return L;
 }
@@ -522,6 +942,49 @@ uint32_t tiles_per_wg(const lev_ctx *ctx, const lev_moe_grouped_args &a, uint32_
     if (t < 1) t = 1;
     if (t > tiles) t = tiles;
     return (uint32_t)t;
+}
+
+// Where the integer matrix-core kernels serve: rows of whole 256-value tasks, one task per wave, and
+// at most four pairs per expert on average -- they multiply four tokens at a time and are the
+// faster ones while most experts hold no more than four or eight pairs; the fp16 kernel above takes
+// twelve tokens a pass at one price.  LEV_MOE_GROUPED_I8=0 keeps the fp16 kernel, =1 takes the
+// integer kernels for any token count (for comparison and for the tests).
+bool g8_usable(const lev_moe_grouped_args &a) {
+    static const int mode = [] {
+        const char *v = getenv("LEV_MOE_GROUPED_I8");
+        return v && v[0] == '0' ? 0 : v && v[0] == '1' ? 1 : 2;
+    }();
+    if (mode == 0) return false;
+    const bool shape = a.hidden % 256u == 0u && a.hidden <= kG8MaxInLen && a.inter % 256u == 0u && a.inter <= kG8MaxInLen;
+    return shape && (mode == 1 || (uint64_t)a.tokens * a.top_k <= 4u * (uint64_t)a.experts);
+}
+
+template <int NTILE, bool PAIRED, int NW>
+hipError_t g8_launch(lev_ctx *ctx, const lev_moe_grouped_args &a, const float *src, const lev_grp_item *items,
+                     const int32_t *n_items, float *out) {
+    const uint32_t in_len = PAIRED ? a.hidden : a.inter, out_rows = PAIRED ? a.inter : a.hidden;
+    const uint32_t wpr = in_len >> 8, slots = (uint32_t)NW / wpr;
+    const uint32_t ngroups = (out_rows + 15u) / 16u;
+    const uint32_t per_round = slots * (PAIRED ? 1u : (uint32_t)NTILE);   // row groups a round finishes
+    const uint32_t rpi = (ngroups + per_round - 1u) / per_round;
+    uint64_t slot_of_wave, pos_of_wave;
+    lev_wave_tables(wpr, &slot_of_wave, &pos_of_wave);
+    constexpr size_t lds = g8_lds<NTILE, NW>();
+    static bool configured = false;   // per instantiation: raise the dynamic LDS limit once
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&moe_grouped_i8_kernel<NTILE, PAIRED, NW>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        configured = true;
+    }
+    const uint32_t grid = (uint32_t)ctx->num_cus;
+    // what a round of an item of up to four pairs and of a larger one cost, relative to each other
+    // (gate/up 52 against 62 us, down 33 against 38 with every item of the one or the other kind;
+    // equal weights: 62 + 39 us at 64 tokens, these: 58 + 36.5)
+    const uint32_t w1 = 5u, w2 = 6u;
+    hipLaunchKernelGGL((moe_grouped_i8_kernel<NTILE, PAIRED, NW>), dim3(grid), dim3(64u * wpr * slots), lds, ctx->stream, a,
+                       src, items, n_items, out, wpr, slots, rpi, slot_of_wave, pos_of_wave, w1, w2);
+    return hipGetLastError();
 }
 
 }  // namespace
@@ -553,9 +1016,31 @@ hipError_t lev_moe_grouped_launch(lev_ctx *ctx, const lev_moe_grouped_args &a, c
     const uint32_t pairs = a.tokens * a.top_k;
     hipError_t e;
 
+    if (g8_usable(a)) {
+        int32_t *n_items = reinterpret_cast<int32_t *>(s + L.n_items);
+        lev_grp_item *items = reinterpret_cast<lev_grp_item *>(s + L.items);
+        const size_t lds_group = (size_t)5 * a.experts * 4;
+        static size_t lds_group_set = 0;
+        if (lds_group > 48 * 1024 && lds_group > lds_group_set) {
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(&moe_group_kernel),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_group);
+            if (e != hipSuccess) return e;
+            lds_group_set = lds_group;
+        }
+        hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), lds_group, ctx->stream, ids, pairs,
+                           a.experts, a.top_k, goff, glist, valid, ctx->d_flag, x, a.hidden, nullptr, nullptr, nullptr,
+                           nullptr, items, n_items, (uint32_t)kG8NT);
+        if ((e = hipGetLastError()) != hipSuccess) return e;
+        if ((e = g8_launch<2, true, kG8WavesGateUp>(ctx, a, x, items, n_items, act)) != hipSuccess) return e;
+        // rows of act that belong to dropped pairs are never written and never read
+        if ((e = g8_launch<2, false, kG8WavesDown>(ctx, a, act, items, n_items, dn)) != hipSuccess) return e;
+        hipLaunchKernelGGL(moe_merge_kernel, dim3((a.hidden + 1023) / 1024, a.tokens), dim3(256), 0, ctx->stream, dn,
+                           weights, valid, y, a.hidden, a.top_k);
+        return hipGetLastError();
+    }
     hipLaunchKernelGGL(moe_group_kernel, dim3(1 + a.tokens), dim3(1024), (size_t)2 * a.experts * 4,
                        ctx->stream, ids, pairs, a.experts, a.top_k, goff, glist, valid, ctx->d_flag, x,
-                       a.hidden, xh, xl, xmax, amax);
+                       a.hidden, xh, xl, xmax, amax, nullptr, nullptr, 0u);
     if ((e = hipGetLastError()) != hipSuccess) return e;
 
     static size_t lds_set[2] = {0, 0};

@@ -11,6 +11,14 @@ struct lev_moe_grouped_args {
     uint32_t hidden, inter, experts, top_k, tokens;
 };
 
+// A work item of the integer matrix-core kernels: `count` (1..8) pairs of one expert, the pairs
+// `first ..` of the expert-ordered list.  pair[k] is the (token * top_k + slot) index of column k,
+// src[k] its token; columns past `count` repeat the last.
+struct alignas(16) lev_grp_item {
+    int32_t expert, count, first, pad;
+    int32_t pair[8], src[8];
+};
+
 size_t lev_moe_grouped_scratch_bytes(const lev_moe_grouped_args &a);
 // Geometry the grouped path serves (the caller also checks 4-byte aligned pools).
 bool lev_moe_grouped_usable(const lev_ctx *ctx, const lev_moe_grouped_args &a);

@@ -322,27 +322,40 @@ def test_moe_grouped_path_many_experts(ctx, experts):
         assert O.max_rel_err(y[t], ref["y"]) < TOL
 
 
-@pytest.mark.parametrize("experts", [16, 1500])
-def test_moe_grouped_path_many_tokens(ctx, experts):
-    """2100 tokens through the grouped path: with 16 experts every expert takes many passes of
-    twelve columns over its weights, with 1500 the scan over the expert counts crosses waves and
-    most experts hold a handful of pairs.  Sampled tokens against the FP64 chain, and the first 64
-    tokens as a batch of their own bit for bit (a pair's result does not depend on the batch)."""
-    hidden, inter, top_k, tokens = 256, 256, 4, 2100
+@pytest.mark.parametrize("experts,tokens,again", [(16, 2100, 64), (1500, 2100, 1600), (1500, 1400, 64), (40, 36, 20)])
+def test_moe_grouped_path_many_tokens(ctx, experts, tokens, again):
+    """Many tokens through the grouped path.  More than four pairs per expert on average take the
+    fp16 kernels: with 16 experts every expert takes many passes of twelve columns over its weights,
+    with 1500 the scan over the expert counts crosses waves.  Up to four pairs per expert take the
+    integer kernels (1400 tokens over 1500 experts: work items of one to eight pairs, those of more
+    than four in front of the others; 36 tokens of which most go to two experts: several whole
+    items per expert).  Sampled tokens against the FP64 chain, and the first `again` tokens as a
+    batch of their own, on the same kernels, bit for bit: a pair's result does not depend on the
+    batch."""
+    hidden, inter, top_k = 256, 256, 4
     wr, pool, offs, x = H.config5(hidden, inter, experts, tokens, seed=experts + 7)
     rng = np.random.default_rng(experts + 7)
     ids = np.stack([rng.permutation(experts)[:top_k] for _ in range(tokens)]).astype(np.int32)
     ids[0, 0], ids[1, 1] = experts - 1, 0
+    if experts == 40:
+        # experts 3 and 4 in nearly every token: 30 and 27 pairs -> three whole items and a remainder
+        for t in range(tokens):
+            if t % 6 != 5:
+                ids[t] = [3, 5 + t % 30, 4 if t % 10 else 36, 37 + t % 3]
+        for t in range(tokens):
+            assert len(set(ids[t].tolist())) == top_k
+    # which kernels a batch takes (integer matrix cores up to four pairs per expert on average)
+    assert (tokens * top_k <= 4 * experts) == (again * top_k <= 4 * experts)
     wts = rng.random((tokens, top_k)).astype(np.float32)
     y, act = run_experts(ctx, pool, offs, hidden, inter, experts, x, ids, wts)
     g, u, d = (pool[offs["gate_off"]:], pool[offs["up_off"]:], pool[offs["down_off"]:])
-    for t in list(range(0, tokens, 97)) + [1, tokens - 1]:
+    for t in list(range(0, tokens, 97 if tokens > 100 else 5)) + [1, tokens - 1]:
         ref = O.moe_experts_f64(g, u, d, hidden, inter, ids[t], wts[t], x[t])
         assert O.max_rel_err(act[t], ref["act"]) < TOL
         assert O.max_rel_err(y[t], ref["y"]) < TOL
-    y64, act64 = run_experts(ctx, pool, offs, hidden, inter, experts, x[:64], ids[:64], wts[:64])
-    assert np.array_equal(y64.view(np.uint32), y[:64].view(np.uint32))
-    assert np.array_equal(act64.view(np.uint32), act[:64].view(np.uint32))
+    y2, act2 = run_experts(ctx, pool, offs, hidden, inter, experts, x[:again], ids[:again], wts[:again])
+    assert np.array_equal(y2.view(np.uint32), y[:again].view(np.uint32))
+    assert np.array_equal(act2.view(np.uint32), act[:again].view(np.uint32))
 
 
 def test_moe_grouped_path_rejects_bad_expert_ids(ctx):
