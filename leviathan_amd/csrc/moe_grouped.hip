@@ -110,7 +110,8 @@ moe_group_kernel(const int32_t *__restrict__ ids, uint32_t pairs, uint32_t exper
                  uint8_t *__restrict__ valid, int *__restrict__ flag, const float *__restrict__ x,
                  uint32_t hidden, _Float16 *__restrict__ xh, _Float16 *__restrict__ xl,
                  uint32_t *__restrict__ xmax, uint32_t *__restrict__ amax, lev_grp_item *items,
-                 int32_t *__restrict__ n_items, uint32_t item_pairs) {
+                 uint32_t item_pairs, lev_grp_start *__restrict__ starts, uint32_t grid, uint32_t rpi_gu,
+                 uint32_t rpi_dn, uint32_t w1, uint32_t w2) {
     // [experts] counts | cursors | with items: first pair | first item of more than four pairs | first other item
     extern __shared__ int32_t s_cnt[];
     int32_t *s_cur = s_cnt + experts, *s_first = s_cur + experts, *s_big = s_first + experts, *s_small = s_big + experts;
@@ -163,6 +164,7 @@ moe_group_kernel(const int32_t *__restrict__ ids, uint32_t pairs, uint32_t exper
     // their threads' sums by shuffles and meet in LDS.  One scan carries three counts of at most
     // 2^20 each in 21-bit fields: pairs, items of more than four pairs, other items.
     __shared__ uint64_t s_wave[16];
+    uint32_t n_big = 0u, n_all = 0u;            // items of more than four pairs, all items
     {
         int32_t c4[4], big4[4], small4[4];
         const int32_t ip = items ? (int32_t)item_pairs : 1, ish = ip == 8 ? 3 : ip == 4 ? 2 : 0;   // (4 or 8 pairs an item)
@@ -209,10 +211,8 @@ moe_group_kernel(const int32_t *__restrict__ ids, uint32_t pairs, uint32_t exper
             // rounds alone.
             const int32_t nbig = (int32_t)(all >> 21 & 0x1FFFFFu), nsmall = (int32_t)(all >> 42);
             int32_t brun = (int32_t)(before >> 21 & 0x1FFFFFu), srun = nbig + (int32_t)(before >> 42);
-            if (tid == 0u) {
-                n_items[0] = nbig + nsmall;
-                n_items[1] = nbig;
-            }
+            n_big = (uint32_t)nbig;
+            n_all = (uint32_t)(nbig + nsmall);
             int32_t prun = first_pair;
 #pragma unroll
             for (uint32_t k = 0; k < 4u; ++k) {
@@ -235,6 +235,26 @@ moe_group_kernel(const int32_t *__restrict__ ids, uint32_t pairs, uint32_t exper
         }
     }
     __syncthreads();
+    const uint32_t sid = 1023u - tid;   // (the high threads: the low ones place the first 1024 pairs below)
+    if (items && sid < 2u * grid) {
+        // Where the workgroups of the two expert kernels start.  A round of an item of more than
+        // four pairs costs w2, any other w1; the line of rounds is cut into stretches of equal
+        // COST.  The items of more than four pairs come first, so a position in cost is a position
+        // in rounds by two divisions (32-bit arithmetic: rounds * w < 2^29, grid <= 2^9).
+        const uint32_t down = sid >= grid ? 1u : 0u, L = sid - down * grid, rpi = down ? rpi_dn : rpi_gu;
+        const uint32_t R2 = n_big * rpi, C2 = R2 * w2;
+        const uint32_t total = C2 + (n_all * rpi - R2) * w1, per = total / grid, rest = total - per * grid;
+        auto rounds_before = [&](uint32_t c) { return c <= C2 ? (c + w2 - 1u) / w2 : R2 + (c - C2 + w1 - 1u) / w1; };
+        lev_grp_start st;
+        st.first_round = rounds_before(per * L + rest * L / grid);
+        st.end_round = rounds_before(per * (L + 1u) + rest * (L + 1u) / grid);
+        st.item = st.first_round / rpi;
+        const lev_grp_item *it = items + (st.item < n_all ? st.item : 0u);   // (written before the barrier)
+        st.expert = it->expert;
+        st.count = it->count;
+        st.pad[0] = st.pad[1] = st.pad[2] = 0u;
+        starts[sid] = st;
+    }
     // The order of an expert's pairs in the list depends on the atomics; no
     // result does: every pair is computed independently and owns its outputs.
     for (uint32_t p = tid; p < pairs; p += 1024u)
@@ -548,6 +568,7 @@ moe_grouped_kernel(lev_moe_grouped_args a, uint32_t tiles_per_wg, const float *_
 // unit u of the batch (a slot's 16 rows x four tokens), applies the activation function (PAIRED)
 // and stores.
 // ---------------------------------------------------------------------------
+constexpr uint32_t kG8MaxGrid = 512;                      // workgroups of an expert kernel (one per CU)
 constexpr int kG8MaxWpr = 8;                              // waves that share a row group: one task each
 constexpr int kG8WavesGateUp = 8;                         // 2048 activations: eight column tasks, one slot
 constexpr int kG8WavesDown = 12;                          // 768 activations: three column tasks, four slots (three
@@ -561,8 +582,8 @@ constexpr uint32_t kG8Plane = 272u;                       // a digit plane of a 
 constexpr uint32_t kG8TokArea = 4u * kG8Plane;            // the 64 lanes of an operand read hit 64 different banks
 constexpr uint32_t kG8WaveLds = 4u * kG8TokArea;           // four tokens are staged at a time
 
-// LDS: part [parity 2][round of the batch][tile NTILE][token / 4][wave][row 16][token % 4] f32 | per wave four
-// staged tasks
+// LDS: part [parity 2][round of the batch][tile NTILE][token group of the item][wave][row 16][token % 4] f32 | per
+// wave four staged tasks
 template <int NTILE, int NW>
 constexpr size_t g8_lds() {
     return (size_t)2 * kG8Batch * NTILE * (kG8NT / 4) * (NW * 256u) + (size_t)NW * kG8WaveLds;
@@ -694,14 +715,14 @@ __device__ __forceinline__ void g8_tile_dot(const uint32_t W[9], const long (&A)
 template <int NTILE, bool PAIRED, int NW>
 __global__ void __launch_bounds__(NW * LEV_WAVE)
 moe_grouped_i8_kernel(lev_moe_grouped_args a, const float *__restrict__ src, const lev_grp_item *__restrict__ items,
-                      const int32_t *__restrict__ n_items, float *__restrict__ out, uint32_t wpr, uint32_t slots,
-                      uint32_t rpi, uint64_t slot_of_wave, uint64_t pos_of_wave, uint32_t w1, uint32_t w2) {
+                      const lev_grp_start *__restrict__ starts, float *__restrict__ out, uint32_t wpr, uint32_t slots,
+                      uint32_t rpi, uint64_t slot_of_wave, uint64_t pos_of_wave) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     constexpr uint32_t NT = kG8NT, NJ = NT / 4u;
     constexpr uint32_t TO = PAIRED ? 1u : (uint32_t)NTILE;       // row groups a slot finishes per round
     constexpr uint32_t kG8Unit = NW * 256u;                       // bytes of part[wave][row][token % 4]: one tile's sums of four tokens
-    constexpr uint32_t kRound = NTILE * NJ * kG8Unit;             // one round's sums in `part`
-    constexpr uint32_t kHalf = kG8Batch * kRound;                 // one parity of `part`: a batch of rounds
+    constexpr uint32_t kHalf = kG8Batch * NTILE * NJ * kG8Unit;   // one parity of `part`: a batch of rounds (with one
+                                                                  // token group an item: twice as many rounds)
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
     const uint32_t nwaves = blockDim.x >> 6;                      // wpr * slots: every wave has a task
@@ -715,15 +736,11 @@ moe_grouped_i8_kernel(lev_moe_grouped_args a, const float *__restrict__ src, con
     // this workgroup's stretch of the line of rounds
     const uint32_t G = gridDim.x;
     const uint32_t L = (G & 7u) == 0u ? (blockIdx.x & 7u) * (G >> 3) + (blockIdx.x >> 3) : blockIdx.x;
-    // A round of an item of more than four pairs costs w2, any other w1; the line is cut into
-    // stretches of equal COST.  The items of more than four pairs come first, so a position in
-    // cost is a position in rounds by two divisions (32-bit arithmetic: rounds * w < 2^29,
-    // G <= 2^10; a 64-bit division is a hundred instructions).
-    const uint32_t R2 = (uint32_t)n_items[1] * rpi, C2 = R2 * w2;
-    const uint32_t total = C2 + ((uint32_t)n_items[0] * rpi - R2) * w1, per = total / G, rest = total - per * G;
-    auto rounds_before = [&](uint32_t c) { return c <= C2 ? (c + w2 - 1u) / w2 : R2 + (c - C2 + w1 - 1u) / w1; };
-    uint32_t R = rounds_before(per * L + rest * L / G);
-    const uint32_t Rend = rounds_before(per * (L + 1u) + rest * (L + 1u) / G);
+    // (stretches of equal cost, laid out by the grouping kernel together with the first item's header)
+    const lev_grp_start st = starts[L];
+    uint32_t R = st.first_round, it = st.item;
+    const uint32_t Rend = st.end_round;
+    uint32_t e = (uint32_t)st.expert, cnt = (uint32_t)st.count;
 
     uint8_t *area = smem + 2u * kHalf + (size_t)wave * kG8WaveLds;
     // byte offsets into the workgroup's LDS, not pointers; lane (r, g) writes row r, token 4j + g
@@ -731,13 +748,14 @@ moe_grouped_i8_kernel(lev_moe_grouped_args a, const float *__restrict__ src, con
     uint32_t half = 0u;                                           // byte offset of the round's parity
 
     while (R < Rend) {
-        const uint32_t it = R / rpi, r0 = R - it * rpi;
+        const uint32_t r0 = R - it * rpi;
         const uint32_t nr = rpi - r0 < Rend - R ? rpi - r0 : Rend - R;   // rounds r0 .. r0 + nr of item `it`
-        // request order = return order: the item (one scalar load), the activations of the wave's
-        // task for every token, and the first round's weights behind them, so that the staging
-        // does not wait for the weights
+        // request order = return order: the item's columns (scalar loads), the activations of the
+        // wave's task for every token, and the first round's weights behind them, so that the
+        // staging does not wait for the weights.  The header of the NEXT item is requested here as
+        // well (the list has one record past its end): its expert is known when its turn comes.
         const lev_grp_item *item = items + it;
-        const uint32_t e = (uint32_t)item->expert, cnt = (uint32_t)item->count;
+        const uint32_t e_next = (uint32_t)item[1].expert, cnt_next = (uint32_t)item[1].count;
         const uint32_t ng = (cnt + 3u) >> 2;                      // groups of four tokens that take part
         int32_t pk[NT];
         lev_f32x4 v[NT];
@@ -796,6 +814,8 @@ moe_grouped_i8_kernel(lev_moe_grouped_args a, const float *__restrict__ src, con
         __builtin_amdgcn_sched_barrier(0);
 
         uint32_t batch0 = r0, nb = 0u;                            // the batch's first round, rounds in it so far
+        const uint32_t round_bytes = NTILE * ng * kG8Unit;        // one round's sums in `part`: [tile][token group][wave][row][token % 4]
+        const uint32_t batch_rounds = kG8Batch * NJ / ng;
         auto round = [&](uint32_t rho, uint32_t (&D)[NTILE][9]) {
             // lane (r, g) <- lane 4r + g; the registers the bytes came in take a later round's
             // request at once (unconditional, clamped: a branch around the loads would make the
@@ -813,11 +833,11 @@ moe_grouped_i8_kernel(lev_moe_grouped_args a, const float *__restrict__ src, con
 #pragma unroll
                 for (uint32_t j = 0; j < NJ; ++j)
                     if (j < ng)
-                        *reinterpret_cast<float *>(smem + half + nb * kRound + pw + ((uint32_t)t * NJ + j) * kG8Unit) = val[j];
+                        *reinterpret_cast<float *>(smem + half + nb * round_bytes + pw + ((uint32_t)t * ng + j) * kG8Unit) = val[j];
             }
             // the waves meet once per batch of rounds (and at the item's end): between two barriers
             // they run at their own pace, and the batch's sums are finished by several waves at once
-            if (++nb < kG8Batch && rho != r_last) return;
+            if (++nb < batch_rounds && rho != r_last) return;
             lev_barrier_lds();
             // unit u = (round b of the batch, slot s, row group t of the slot's round, tokens 4j .. 4j + 3):
             // lane (r, g) adds the slot's waves' sums of row r and token 4j + g in a fixed order
@@ -830,7 +850,7 @@ moe_grouped_i8_kernel(lev_moe_grouped_args a, const float *__restrict__ src, con
                 const uint32_t rg = PAIRED ? (batch0 + b) * slots + s : ((batch0 + b) * slots + s) * (uint32_t)NTILE + t;
                 const uint32_t row = rg * 16u + r;
                 const float *pp = reinterpret_cast<const float *>(
-                    smem + half + b * kRound + (t * NJ + j) * kG8Unit + ((s * wpr * 16u + r) * 4u + g) * 4u);
+                    smem + half + b * round_bytes + (t * ng + j) * kG8Unit + ((s * wpr * 16u + r) * 4u + g) * 4u);
                 auto slot_sum = [&](const float *q) {
                     float p[kG8MaxWpr];
 #pragma unroll
@@ -840,7 +860,7 @@ moe_grouped_i8_kernel(lev_moe_grouped_args a, const float *__restrict__ src, con
                     return ((p[0] + p[4]) + (p[2] + p[6])) + ((p[1] + p[5]) + (p[3] + p[7]));
                 };
                 float res = slot_sum(pp);
-                if (PAIRED) res = lev_gelu_up_value(res, slot_sum(pp + NJ * (kG8Unit / 4u)));
+                if (PAIRED) res = lev_gelu_up_value(res, slot_sum(pp + ng * (kG8Unit / 4u)));
                 int32_t pair = pk[0];
 #pragma unroll
                 for (uint32_t q = 1; q < NT; ++q) pair = k == q ? pk[q] : pair;
@@ -852,6 +872,9 @@ moe_grouped_i8_kernel(lev_moe_grouped_args a, const float *__restrict__ src, con
         };
         for (uint32_t rho = r0; rho <= r_last; ++rho) round(rho, Da);
         R += nr;
+        ++it;
+        e = e_next;
+        cnt = cnt_next;
     }
 }
 
@@ -902,7 +925,7 @@ moe_merge_kernel(const float *__restrict__ dn, const float *__restrict__ weights
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct grouped_layout {
-    size_t goff, glist, valid, xh, xl, xmax, amax, dn, items, n_items, total;
+    size_t goff, glist, valid, xh, xl, xmax, amax, dn, items, starts, total;
 };
 
 grouped_layout layout_of(const lev_moe_grouped_args &a) {
@@ -917,8 +940,8 @@ grouped_layout layout_of(const lev_moe_grouped_args &a) {
     L.xmax = o; o += align256((size_t)a.tokens * 4);
     L.amax = o; o += align256(pairs * 4);
     L.dn = o; o += align256(pairs * a.hidden * 4);
-    L.items = o; o += align256((pairs / 8 + a.experts + 1) * sizeof(lev_grp_item));   // an expert with c pairs: ceil(c / 8) items
-    L.n_items = o; o += 256;
+    L.items = o; o += align256((pairs / 8 + a.experts + 1) * sizeof(lev_grp_item));   // an expert with c pairs: ceil(c / 8) items; one past the end
+    L.starts = o; o += 2 * kG8MaxGrid * sizeof(lev_grp_start);
     L.total = o;
     return L;
 }
@@ -959,16 +982,27 @@ bool g8_usable(const lev_moe_grouped_args &a) {
     return shape && (mode == 1 || (uint64_t)a.tokens * a.top_k <= 4u * (uint64_t)a.experts);
 }
 
+struct g8_geometry {
+    uint32_t wpr, slots, rpi;   // waves a row, row-group slots a workgroup, rounds an item
+};
+template <int NTILE, bool PAIRED, int NW>
+g8_geometry g8_geometry_of(const lev_moe_grouped_args &a) {
+    const uint32_t in_len = PAIRED ? a.hidden : a.inter, out_rows = PAIRED ? a.inter : a.hidden;
+    g8_geometry q;
+    q.wpr = in_len >> 8;
+    q.slots = (uint32_t)NW / q.wpr;
+    const uint32_t ngroups = (out_rows + 15u) / 16u;
+    const uint32_t per_round = q.slots * (PAIRED ? 1u : (uint32_t)NTILE);   // row groups a round finishes
+    q.rpi = (ngroups + per_round - 1u) / per_round;
+    return q;
+}
+
 template <int NTILE, bool PAIRED, int NW>
 hipError_t g8_launch(lev_ctx *ctx, const lev_moe_grouped_args &a, const float *src, const lev_grp_item *items,
-                     const int32_t *n_items, float *out) {
-    const uint32_t in_len = PAIRED ? a.hidden : a.inter, out_rows = PAIRED ? a.inter : a.hidden;
-    const uint32_t wpr = in_len >> 8, slots = (uint32_t)NW / wpr;
-    const uint32_t ngroups = (out_rows + 15u) / 16u;
-    const uint32_t per_round = slots * (PAIRED ? 1u : (uint32_t)NTILE);   // row groups a round finishes
-    const uint32_t rpi = (ngroups + per_round - 1u) / per_round;
+                     const lev_grp_start *starts, uint32_t grid, float *out) {
+    const g8_geometry q = g8_geometry_of<NTILE, PAIRED, NW>(a);
     uint64_t slot_of_wave, pos_of_wave;
-    lev_wave_tables(wpr, &slot_of_wave, &pos_of_wave);
+    lev_wave_tables(q.wpr, &slot_of_wave, &pos_of_wave);
     constexpr size_t lds = g8_lds<NTILE, NW>();
     static bool configured = false;   // per instantiation: raise the dynamic LDS limit once
     if (!configured) {
@@ -977,13 +1011,8 @@ hipError_t g8_launch(lev_ctx *ctx, const lev_moe_grouped_args &a, const float *s
         if (e != hipSuccess) return e;
         configured = true;
     }
-    const uint32_t grid = (uint32_t)ctx->num_cus;
-    // what a round of an item of up to four pairs and of a larger one cost, relative to each other
-    // (gate/up 52 against 62 us, down 33 against 38 with every item of the one or the other kind;
-    // equal weights: 62 + 39 us at 64 tokens, these: 58 + 36.5)
-    const uint32_t w1 = 5u, w2 = 6u;
-    hipLaunchKernelGGL((moe_grouped_i8_kernel<NTILE, PAIRED, NW>), dim3(grid), dim3(64u * wpr * slots), lds, ctx->stream, a,
-                       src, items, n_items, out, wpr, slots, rpi, slot_of_wave, pos_of_wave, w1, w2);
+    hipLaunchKernelGGL((moe_grouped_i8_kernel<NTILE, PAIRED, NW>), dim3(grid), dim3(64u * q.wpr * q.slots), lds,
+                       ctx->stream, a, src, items, starts, out, q.wpr, q.slots, q.rpi, slot_of_wave, pos_of_wave);
     return hipGetLastError();
 }
 
@@ -1017,8 +1046,14 @@ hipError_t lev_moe_grouped_launch(lev_ctx *ctx, const lev_moe_grouped_args &a, c
     hipError_t e;
 
     if (g8_usable(a)) {
-        int32_t *n_items = reinterpret_cast<int32_t *>(s + L.n_items);
         lev_grp_item *items = reinterpret_cast<lev_grp_item *>(s + L.items);
+        lev_grp_start *starts = reinterpret_cast<lev_grp_start *>(s + L.starts);
+        const uint32_t grid = (uint32_t)ctx->num_cus < kG8MaxGrid ? (uint32_t)ctx->num_cus : kG8MaxGrid;
+        const g8_geometry q_gu = g8_geometry_of<2, true, kG8WavesGateUp>(a), q_dn = g8_geometry_of<2, false, kG8WavesDown>(a);
+        // what a round of an item of up to four pairs and of a larger one cost, relative to each other
+        // (gate/up 52 against 62 us, down 33 against 38 with every item of the one or the other kind;
+        // equal weights: 62 + 39 us at 64 tokens, these: 58 + 36.5)
+        const uint32_t w1 = 5u, w2 = 6u;
         const size_t lds_group = (size_t)5 * a.experts * 4;
         static size_t lds_group_set = 0;
         if (lds_group > 48 * 1024 && lds_group > lds_group_set) {
@@ -1029,18 +1064,18 @@ hipError_t lev_moe_grouped_launch(lev_ctx *ctx, const lev_moe_grouped_args &a, c
         }
         hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), lds_group, ctx->stream, ids, pairs,
                            a.experts, a.top_k, goff, glist, valid, ctx->d_flag, x, a.hidden, nullptr, nullptr, nullptr,
-                           nullptr, items, n_items, (uint32_t)kG8NT);
+                           nullptr, items, (uint32_t)kG8NT, starts, grid, q_gu.rpi, q_dn.rpi, w1, w2);
         if ((e = hipGetLastError()) != hipSuccess) return e;
-        if ((e = g8_launch<2, true, kG8WavesGateUp>(ctx, a, x, items, n_items, act)) != hipSuccess) return e;
+        if ((e = g8_launch<2, true, kG8WavesGateUp>(ctx, a, x, items, starts, grid, act)) != hipSuccess) return e;
         // rows of act that belong to dropped pairs are never written and never read
-        if ((e = g8_launch<2, false, kG8WavesDown>(ctx, a, act, items, n_items, dn)) != hipSuccess) return e;
+        if ((e = g8_launch<2, false, kG8WavesDown>(ctx, a, act, items, starts + grid, grid, dn)) != hipSuccess) return e;
         hipLaunchKernelGGL(moe_merge_kernel, dim3((a.hidden + 1023) / 1024, a.tokens), dim3(256), 0, ctx->stream, dn,
                            weights, valid, y, a.hidden, a.top_k);
         return hipGetLastError();
     }
     hipLaunchKernelGGL(moe_group_kernel, dim3(1 + a.tokens), dim3(1024), (size_t)2 * a.experts * 4,
                        ctx->stream, ids, pairs, a.experts, a.top_k, goff, glist, valid, ctx->d_flag, x,
-                       a.hidden, xh, xl, xmax, amax, nullptr, nullptr, 0u);
+                       a.hidden, xh, xl, xmax, amax, nullptr, 0u, nullptr, 0u, 0u, 0u, 0u, 0u);
     if ((e = hipGetLastError()) != hipSuccess) return e;
 
     static size_t lds_set[2] = {0, 0};

@@ -19,6 +19,15 @@ struct alignas(16) lev_grp_item {
     int32_t pair[8], src[8];
 };
 
+// Where a workgroup of the integer matrix-core kernels starts: its stretch of the line of rounds
+// and the header of the first item it touches (one load in front of the first weight request
+// instead of three that depend on each other).
+struct alignas(32) lev_grp_start {
+    uint32_t first_round, end_round, item;
+    int32_t expert, count;
+    uint32_t pad[3];
+};
+
 size_t lev_moe_grouped_scratch_bytes(const lev_moe_grouped_args &a);
 // Geometry the grouped path serves (the caller also checks 4-byte aligned pools).
 bool lev_moe_grouped_usable(const lev_ctx *ctx, const lev_moe_grouped_args &a);
