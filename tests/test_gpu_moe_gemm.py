@@ -418,11 +418,13 @@ def test_moe_layer_config5(ctx, tokens):
         assert float(np.min(np.diff(-order[:top_k + 1]))) > 1e-5, "degenerate seed"
         H.check_moe_layer_token(y[t], ids[t], wts[t], ref_ids, ref_w, g, u, d, hidden, inter, x[t], TOL)
     # batch invariance (main.swift:9053-9056: a schedule gives the same bits whatever
-    # else is in the batch).  Two schedules exist here: up to four tokens every
-    # (token, slot) streams its expert alone on the vector ALU; from five tokens
-    # pairs are grouped by expert on the matrix cores.  Within the grouped
-    # schedule a token's bits do not depend on the rest of the batch; across the
-    # two schedules the same token agrees to the summation-order noise.
+    # else is in the batch).  Three schedules exist here: up to four tokens every
+    # (token, slot) streams its expert alone; from five tokens pairs are grouped
+    # by expert on the matrix cores, by the integer kernels up to four pairs per
+    # expert on average (64 and 8 tokens over 128 experts both) and by the fp16
+    # kernels beyond.  Within a schedule a token's bits do not depend on the rest
+    # of the batch; across schedules the same token agrees to the
+    # summation-order noise.
     if tokens > 1:
         y8, _, _ = ctx.moe_layer_q4_0(pools, dev(wr), dev(x[:8]), top_k, 8)
         y1, _, _ = ctx.moe_layer_q4_0(pools, dev(wr), dev(x[:1]), top_k, 1)
