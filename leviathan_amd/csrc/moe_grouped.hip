@@ -972,14 +972,19 @@ uint32_t tiles_per_wg(const lev_ctx *ctx, const lev_moe_grouped_args &a, uint32_
 // faster ones while most experts hold no more than four or eight pairs; the fp16 kernel above takes
 // twelve tokens a pass at one price.  LEV_MOE_GROUPED_I8=0 keeps the fp16 kernel, =1 takes the
 // integer kernels for any token count (for comparison and for the tests).
-bool g8_usable(const lev_moe_grouped_args &a) {
+bool g8_usable(const lev_ctx *ctx, const lev_moe_grouped_args &a) {
     static const int mode = [] {
         const char *v = getenv("LEV_MOE_GROUPED_I8");
         return v && v[0] == '0' ? 0 : v && v[0] == '1' ? 1 : 2;
     }();
     if (mode == 0) return false;
     const bool shape = a.hidden % 256u == 0u && a.hidden <= kG8MaxInLen && a.inter % 256u == 0u && a.inter <= kG8MaxInLen;
-    return shape && (mode == 1 || (uint64_t)a.tokens * a.top_k <= 4u * (uint64_t)a.experts);
+    const size_t limit = ctx->props.sharedMemPerBlockOptin > ctx->props.sharedMemPerBlock
+                             ? ctx->props.sharedMemPerBlockOptin
+                             : ctx->props.sharedMemPerBlock;
+    const size_t lds_group = (size_t)5 * a.experts * 4;
+    const bool fits = g8_lds<2, kG8WavesGateUp>() <= limit && g8_lds<2, kG8WavesDown>() <= limit && lds_group <= limit;
+    return shape && fits && (mode == 1 || (uint64_t)a.tokens * a.top_k <= 4u * (uint64_t)a.experts);
 }
 
 struct g8_geometry {
@@ -1045,7 +1050,7 @@ hipError_t lev_moe_grouped_launch(lev_ctx *ctx, const lev_moe_grouped_args &a, c
     const uint32_t pairs = a.tokens * a.top_k;
     hipError_t e;
 
-    if (g8_usable(a)) {
+    if (g8_usable(ctx, a)) {
         lev_grp_item *items = reinterpret_cast<lev_grp_item *>(s + L.items);
         lev_grp_start *starts = reinterpret_cast<lev_grp_start *>(s + L.starts);
         const uint32_t grid = (uint32_t)ctx->num_cus < kG8MaxGrid ? (uint32_t)ctx->num_cus : kG8MaxGrid;
