@@ -151,8 +151,16 @@ moe_group_kernel(const int32_t *__restrict__ ids, uint32_t pairs, uint32_t exper
         const int32_t e = ids[p];
         bool ok = e >= 0 && (uint32_t)e < experts;
         const uint32_t slot = p % top_k, first = p - slot;
-        for (uint32_t k = 0; k < top_k && ok; ++k)
-            if (k != slot && ids[first + k] == e) ok = false;   // both copies of a duplicate are dropped
+        // both copies of a duplicate are dropped; the token's ids are requested eight at a time (one
+        // wait for eight, not one after the other)
+        for (uint32_t k0 = 0; k0 < top_k; k0 += 8u) {
+            int32_t other[8];
+#pragma unroll
+            for (uint32_t u = 0; u < 8u; ++u) other[u] = ids[first + (k0 + u < top_k ? k0 + u : slot)];
+#pragma unroll
+            for (uint32_t u = 0; u < 8u; ++u)
+                if (k0 + u < top_k && k0 + u != slot && other[u] == e) ok = false;
+        }
         valid[p] = ok ? 1 : 0;
         if (ok) atomicAdd(&s_cnt[e], 1);
         if (p == tid && ok) e_own = e;
