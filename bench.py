@@ -563,8 +563,9 @@ def main():
                     alg = experts * hidden * 4 + distinct * expert_bytes + 2 * T * hidden * 4
                     # a pool is used again after the two other pools have been streamed
                     extra_fields = {"distinct_bytes_between_reuse": (npool - 1) * distinct * expert_bytes,
-                                    # an expert with more pairs than a pass of the grouped kernel holds
-                                    # (twelve) takes a second pass over its weights
+                                    # up to four pairs per expert on average the integer grouped kernels
+                                    # run: four tokens a product, a second product for an expert's pairs
+                                    # five to eight, another work item (and pass) beyond
                                     "max_pairs_per_expert": int(torch.bincount(ids.flatten().long()).max())}
 
                 def moe_extra(ms, T=T, distinct=distinct, alg=alg, extra_fields=extra_fields):
