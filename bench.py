@@ -563,7 +563,7 @@ def main():
                     alg = experts * hidden * 4 + distinct * expert_bytes + 2 * T * hidden * 4
                     # a pool is used again after the two other pools have been streamed
                     extra_fields = {"distinct_bytes_between_reuse": (npool - 1) * distinct * expert_bytes,
-                                    # up to four pairs per expert on average the integer grouped kernels
+                                    # up to 5.5 pairs per expert on average the integer grouped kernels
                                     # run: four tokens a product, a second product for an expert's pairs
                                     # five to eight, another work item (and pass) beyond
                                     "max_pairs_per_expert": int(torch.bincount(ids.flatten().long()).max())}
