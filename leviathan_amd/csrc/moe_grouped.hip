@@ -24,7 +24,7 @@
 //   B = 16 weight rows x the block's 32 codes as exact fp16 integers n-8
 //       (mask, OR in 1024's exponent, subtract 1032: two instructions per two
 //       weights, no conversion);
-//   A = up to 8 tokens' activations of that block, fp16 high and low halves
+//   A = up to twelve tokens' activations of that block, fp16 high and low halves
 //       (two MFMAs), x = hi + lo to 2^-22;
 //   the output lane of weight row n is the lane that holds row n's block scale
 //   d, so y += d * (A.B) needs no exchange.
@@ -36,10 +36,12 @@
 // a small wave-private LDS area, and every lane reads from there the four code
 // bytes (both nibbles: eight weights) and the scale it multiplies.
 //
-// Batches of at most five and a half pairs per expert on average, with rows of up to 2048 activations, take
-// the integer matrix cores instead (moe_grouped_i8_kernel below: the digit planes of the few-token
-// kernels, four tokens of an expert per product, operands in registers): they cost less per
-// product and more per token, and win while most experts hold no more than a handful of pairs.
+// Batches of at most five and a half pairs per expert on average, with rows of up to 2048
+// activations, take the integer matrix cores instead (moe_grouped_i8_kernel below: the digit
+// planes of the few-token kernels, four tokens of an expert per product, operands in registers;
+// its grouping step also cuts the pair lists into work items and lays out where each workgroup
+// starts): they cost less per product and more per token, and win while most experts hold no
+// more than a handful of pairs.
 #include "moe_grouped.hpp"
 #include "q4_0_mfma.hpp"
 
