@@ -200,6 +200,32 @@ __device__ __forceinline__ double lev_row_sum_f64(double v) {
     return __hiloint2double((int)a1[0], (int)a0[0]) + __hiloint2double((int)a1[1], (int)a0[1]);
 }
 
+// Largest of an unsigned value over the 16 lanes of a row of the wave, in every lane of the row:
+// quad swaps, then the two row mirrors (DPP: no LDS, no other unit).  Magnitudes of floats
+// compare as their bit patterns do; NaN and infinity sort above every number.
+__device__ __forceinline__ uint32_t lev_row16_max_u32(uint32_t v) {
+#define LEV_ROW16_MAX_STEP(CTRL)                                                                        \
+    {                                                                                                   \
+        const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, CTRL, 0xF, 0xF, false); \
+        v = o > v ? o : v;                                                                              \
+    }
+    LEV_ROW16_MAX_STEP(0xB1)    // quad_perm [1,0,3,2]
+    LEV_ROW16_MAX_STEP(0x4E)    // quad_perm [2,3,0,1]
+    LEV_ROW16_MAX_STEP(0x141)   // row_half_mirror
+    LEV_ROW16_MAX_STEP(0x140)   // row_mirror
+#undef LEV_ROW16_MAX_STEP
+    return v;
+}
+
+// The same over all 64 lanes: the four rows' maxima meet by two row swaps.
+__device__ __forceinline__ uint32_t lev_wave_max_u32(uint32_t v) {
+    v = lev_row16_max_u32(v);
+    const auto s0 = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+    v = s0[0] > s0[1] ? s0[0] : s0[1];
+    const auto s1 = __builtin_amdgcn_permlane16_swap(v, v, false, false);
+    return s1[0] > s1[1] ? s1[0] : s1[1];
+}
+
 // Four values per lane whose sums over lanes l, l ^ 16, l ^ 32, l ^ 48 are wanted: lane group
 // g = lane / 16 gets the sum of v[g], by two exchanges between the halves of the wave and one
 // between the rows of a half (three swaps for four sums; the additions pair the lane groups as

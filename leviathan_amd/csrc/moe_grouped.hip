@@ -525,16 +525,7 @@ moe_grouped_kernel(lev_moe_grouped_args a, uint32_t tiles_per_wg, const float *_
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 uint32_t m = cmax[i];
-#define LEV_GRP_MAXSTEP(CTRL)                                                                          \
-                {                                                                                      \
-                    const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp((int)m, (int)m, CTRL, 0xF, 0xF, false); \
-                    m = o > m ? o : m;                                                                 \
-                }
-                LEV_GRP_MAXSTEP(0xB1);    // quad_perm [1,0,3,2]
-                LEV_GRP_MAXSTEP(0x4E);    // quad_perm [2,3,0,1]
-                LEV_GRP_MAXSTEP(0x141);   // row_half_mirror
-                LEV_GRP_MAXSTEP(0x140);   // row_mirror
-#undef LEV_GRP_MAXSTEP
+                m = lev_row16_max_u32(m);
                 const uint32_t col = 4u * g + (uint32_t)i;
                 if (r == 0u && col < ncols && m != 0u) atomicMax(out_max + s_pair[col], m);
             }
@@ -611,22 +602,7 @@ __device__ __forceinline__ float g8_stage_token(const lev_f32x4 v, uint8_t *tok)
         const uint32_t bits = __float_as_uint(v[k]) & 0x7FFFFFFFu;
         mb = bits > mb ? bits : mb;
     }
-#define LEV_G8_MAXSTEP(CTRL)                                                                             \
-    {                                                                                                    \
-        const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp((int)mb, (int)mb, CTRL, 0xF, 0xF, false); \
-        mb = o > mb ? o : mb;                                                                            \
-    }
-    LEV_G8_MAXSTEP(0xB1)    // quad_perm [1,0,3,2]
-    LEV_G8_MAXSTEP(0x4E)    // quad_perm [2,3,0,1]
-    LEV_G8_MAXSTEP(0x141)   // row_half_mirror
-    LEV_G8_MAXSTEP(0x140)   // row_mirror: the 16 lanes of a row hold the row's maximum
-#undef LEV_G8_MAXSTEP
-    {
-        const auto s0 = __builtin_amdgcn_permlane32_swap(mb, mb, false, false);
-        mb = s0[0] > s0[1] ? s0[0] : s0[1];
-        const auto s1 = __builtin_amdgcn_permlane16_swap(mb, mb, false, false);
-        mb = s1[0] > s1[1] ? s1[0] : s1[1];                    // every lane: the task's maximum
-    }
+    mb = lev_wave_max_u32(mb);   // every lane: the task's maximum
     uint32_t ex = mb >> 23;                                    // |x| < 2^(ex - 126)
     const bool bad = ex == 255u;
     ex = ex < 34u ? 34u : (ex > 254u ? 254u : ex);             // keeps both powers of two normal numbers

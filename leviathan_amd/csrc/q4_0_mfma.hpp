@@ -57,16 +57,7 @@ __device__ __forceinline__ void q4m_stage_task(const lev_f32x4 v, uint8_t *area,
         const uint32_t bits = __float_as_uint(v[k]) & 0x7FFFFFFFu;
         mb = bits > mb ? bits : mb;
     }
-#define LEV_Q4M_MAXSTEP(CTRL)                                                                            \
-    {                                                                                                    \
-        const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp((int)mb, (int)mb, CTRL, 0xF, 0xF, false); \
-        mb = o > mb ? o : mb;                                                                            \
-    }
-    LEV_Q4M_MAXSTEP(0xB1)    // quad_perm [1,0,3,2]
-    LEV_Q4M_MAXSTEP(0x4E)    // quad_perm [2,3,0,1]
-    LEV_Q4M_MAXSTEP(0x141)   // row_half_mirror
-    LEV_Q4M_MAXSTEP(0x140)   // row_mirror: the 16 lanes of a pair hold the pair's maximum
-#undef LEV_Q4M_MAXSTEP
+    mb = lev_row16_max_u32(mb);   // the 16 lanes of a pair hold the pair's maximum
     uint32_t ex = mb >> 23;                                    // |x| < 2^(ex - 126)
     const bool bad = ex == 255u;
     ex = ex < 34u ? 34u : (ex > 254u ? 254u : ex);             // keeps both powers of two normal numbers

@@ -264,16 +264,7 @@ q4_k_mfma_gemv(const uint8_t *__restrict__ w, const float *__restrict__ x,
             const uint32_t bits = __float_as_uint(v[k]) & 0x7FFFFFFFu;
             mb = bits > mb ? bits : mb;
         }
-#define LEV_Q4K_MAXSTEP(CTRL)                                                                       \
-        {                                                                                          \
-            const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp((int)mb, (int)mb, CTRL, 0xF, 0xF, false); \
-            mb = o > mb ? o : mb;                                                                  \
-        }
-        LEV_Q4K_MAXSTEP(0xB1);    // quad_perm [1,0,3,2]
-        LEV_Q4K_MAXSTEP(0x4E);    // quad_perm [2,3,0,1]
-        LEV_Q4K_MAXSTEP(0x141);   // row_half_mirror
-        LEV_Q4K_MAXSTEP(0x140);   // row_mirror: all 16 lanes of a row hold the row's maximum
-#undef LEV_Q4K_MAXSTEP
+        mb = lev_row16_max_u32(mb);   // all 16 lanes of a row hold the row's maximum
         {
             const uint32_t o = (uint32_t)__builtin_amdgcn_ds_swizzle((int)mb, 0x401F);   // lane ^ 16
             mb = o > mb ? o : mb;
@@ -627,16 +618,7 @@ q4_k_mfma_gemv_narrow(const uint8_t *__restrict__ w, const float *__restrict__ x
             const uint32_t bits = __float_as_uint(v[k]) & 0x7FFFFFFFu;
             mb = bits > mb ? bits : mb;
         }
-#define LEV_Q4K_MAXSTEP(CTRL)                                                                       \
-        {                                                                                          \
-            const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp((int)mb, (int)mb, CTRL, 0xF, 0xF, false); \
-            mb = o > mb ? o : mb;                                                                  \
-        }
-        LEV_Q4K_MAXSTEP(0xB1);    // quad_perm [1,0,3,2]
-        LEV_Q4K_MAXSTEP(0x4E);    // quad_perm [2,3,0,1]
-        LEV_Q4K_MAXSTEP(0x141);   // row_half_mirror
-        LEV_Q4K_MAXSTEP(0x140);   // row_mirror: all 16 lanes of a row hold the row's maximum
-#undef LEV_Q4K_MAXSTEP
+        mb = lev_row16_max_u32(mb);   // all 16 lanes of a row hold the row's maximum
         {
             const uint32_t o = (uint32_t)__builtin_amdgcn_ds_swizzle((int)mb, 0x401F);   // lane ^ 16
             mb = o > mb ? o : mb;

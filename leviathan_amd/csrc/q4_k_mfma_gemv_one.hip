@@ -63,24 +63,9 @@ __device__ __forceinline__ void q4k_one_stage(const lev_f32x4 v, uint8_t *area, 
         const uint32_t bits = __float_as_uint(v[k]) & 0x7FFFFFFFu;
         mb = bits > mb ? bits : mb;
     }
-#define LEV_Q4K1_MAXSTEP(CTRL)                                                                           \
-    {                                                                                                    \
-        const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp((int)mb, (int)mb, CTRL, 0xF, 0xF, false); \
-        mb = o > mb ? o : mb;                                                                            \
-    }
-    LEV_Q4K1_MAXSTEP(0xB1)    // quad_perm [1,0,3,2]
-    LEV_Q4K1_MAXSTEP(0x4E)    // quad_perm [2,3,0,1]
-    LEV_Q4K1_MAXSTEP(0x141)   // row_half_mirror
-    LEV_Q4K1_MAXSTEP(0x140)   // row_mirror: the 16 lanes of a chunk hold the chunk's maximum
-#undef LEV_Q4K1_MAXSTEP
     // one power of two per superblock, as in the kernels for several columns: the same integers,
     // so a column gives the same bits whichever kernel multiplies it
-    {
-        const auto s0 = __builtin_amdgcn_permlane32_swap(mb, mb, false, false);
-        mb = s0[0] > s0[1] ? s0[0] : s0[1];
-        const auto s1 = __builtin_amdgcn_permlane16_swap(mb, mb, false, false);
-        mb = s1[0] > s1[1] ? s1[0] : s1[1];
-    }
+    mb = lev_wave_max_u32(mb);
     uint32_t ex = mb >> 23;                                    // |x| < 2^(ex - 126)
     const bool bad = ex == 255u;                               // NaN or infinity among the 256
     ex = ex < 25u ? 25u : (ex > 254u ? 254u : ex);             // keeps both powers of two normal numbers

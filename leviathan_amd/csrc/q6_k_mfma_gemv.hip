@@ -434,16 +434,7 @@ q6_k_mfma_gemv(const uint8_t *__restrict__ w, const float *__restrict__ x, const
             const uint32_t bits = __float_as_uint(e4[k]) & 0x7FFFFFFFu;
             mb = bits > mb ? bits : mb;
         }
-#define LEV_Q6M_MAXSTEP(CTRL)                                                                       \
-        {                                                                                          \
-            const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp((int)mb, (int)mb, CTRL, 0xF, 0xF, false); \
-            mb = o > mb ? o : mb;                                                                  \
-        }
-        LEV_Q6M_MAXSTEP(0xB1);    // quad_perm [1,0,3,2]
-        LEV_Q6M_MAXSTEP(0x4E);    // quad_perm [2,3,0,1]
-        LEV_Q6M_MAXSTEP(0x141);   // row_half_mirror
-        LEV_Q6M_MAXSTEP(0x140);   // row_mirror: all 16 lanes of a row hold the row's maximum
-#undef LEV_Q6M_MAXSTEP
+        mb = lev_row16_max_u32(mb);   // all 16 lanes of a row hold the row's maximum
         {
             const uint32_t m0 = (uint32_t)__builtin_amdgcn_readlane((int)mb, 0);
             const uint32_t m1 = (uint32_t)__builtin_amdgcn_readlane((int)mb, 16);
@@ -728,22 +719,7 @@ q6_k_mfma_gemv_one(const uint8_t *__restrict__ w, const float *__restrict__ x, c
             const uint32_t bits = __float_as_uint(v[c][k]) & 0x7FFFFFFFu;
             mb = bits > mb ? bits : mb;
         }
-#define LEV_Q6M_MAXSTEP(CTRL)                                                                           \
-        {                                                                                              \
-            const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp((int)mb, (int)mb, CTRL, 0xF, 0xF, false); \
-            mb = o > mb ? o : mb;                                                                      \
-        }
-        LEV_Q6M_MAXSTEP(0xB1);
-        LEV_Q6M_MAXSTEP(0x4E);
-        LEV_Q6M_MAXSTEP(0x141);
-        LEV_Q6M_MAXSTEP(0x140);
-#undef LEV_Q6M_MAXSTEP
-        {
-            const auto s0 = __builtin_amdgcn_permlane32_swap(mb, mb, false, false);
-            mb = s0[0] > s0[1] ? s0[0] : s0[1];
-            const auto s1 = __builtin_amdgcn_permlane16_swap(mb, mb, false, false);
-            mb = s1[0] > s1[1] ? s1[0] : s1[1];
-        }
+        mb = lev_wave_max_u32(mb);
         uint32_t ex = mb >> 23;                             // biased exponent: |x| < 2^(ex-126)
         const bool bad = ex == 255u;                        // NaN or infinity in the superblock
         ex = ex < 30u ? 30u : (ex > 254u ? 254u : ex);      // keeps both powers of two normal numbers
