@@ -358,6 +358,29 @@ def test_moe_grouped_path_many_tokens(ctx, experts, tokens, again):
     assert np.array_equal(act2.view(np.uint32), act[:again].view(np.uint32))
 
 
+@pytest.mark.parametrize("experts,tokens,top_k", [(16, 2, 2), (16, 6, 2), (4, 12, 2)])
+def test_moe_non_finite_activation_stays_in_its_token(ctx, experts, tokens, top_k):
+    """A NaN or an infinity in one token's activations makes every output of THAT token non-finite
+    (as the reference's f32 dot products do: each of them contains the element) and leaves the
+    other tokens' bits alone, on the per-pair kernels (2 tokens), the integer grouped kernels
+    (6 tokens over 16 experts) and the fp16 grouped kernels (12 tokens over 4 experts)."""
+    hidden, inter = 256, 256
+    wr, pool, offs, x = H.config5(hidden, inter, experts, tokens, seed=91 + tokens)
+    rng = np.random.default_rng(91 + tokens)
+    ids = np.stack([rng.permutation(experts)[:top_k] for _ in range(tokens)]).astype(np.int32)
+    wts = rng.random((tokens, top_k)).astype(np.float32)
+    y_good, _ = run_experts(ctx, pool, offs, hidden, inter, experts, x, ids, wts)
+    assert np.isfinite(y_good).all()
+    for bad_value, where in ((np.float32(np.nan), 77), (np.float32(np.inf), 3), (np.float32(-np.inf), 255)):
+        xb = x.copy()
+        xb[1, where] = bad_value
+        y, _ = run_experts(ctx, pool, offs, hidden, inter, experts, xb, ids, wts)
+        assert not np.isfinite(y[1]).any(), (bad_value, where)
+        for t in range(tokens):
+            if t != 1:
+                assert np.array_equal(y[t].view(np.uint32), y_good[t].view(np.uint32)), (bad_value, t)
+
+
 def test_moe_grouped_path_rejects_bad_expert_ids(ctx):
     """The same rule on the many-token path: a pair whose id is out of range or repeats another
     slot of its token is dropped (it adds nothing to its token) and reported; the other tokens
