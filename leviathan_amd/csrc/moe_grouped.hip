@@ -68,17 +68,21 @@ typedef uint32_t g_u4 __attribute__((ext_vector_type(4)));
 typedef uint32_t g_u2 __attribute__((ext_vector_type(2)));
 
 // ---------------------------------------------------------------------------
-// Activation planes.  A row is scaled by the power of two that brings its maximum into [1, 2)
-// (zero, denormal and non-finite maxima: no scaling) and split into fp16 high and low halves;
+// Activation planes.  A row is scaled by the power of two that brings its maximum into
+// [2^14, 2^15) (zero, denormal and non-finite maxima: no scaling) and split into fp16 high and low
+// halves.  At the top of fp16's range the low half of every element down to 2^-17 of the row's
+// maximum is still a normal number: x = hi + lo to 2^-22 of the element (with the maximum in
+// [1, 2) an element 2^-6 below it kept 18 bits, 2^-10 below it 14);
 // run 4b + g of a row holds elements 4g, 4g+2, 4g+1, 4g+3, then 16+4g, 16+4g+2, 16+4g+1, 16+4g+3 of
 // block b: the weights in code bytes 4g..4g+3 of the block (low nibbles, then high nibbles), in the
 // order in which the masks of the matrix-core kernel deliver them.
 // ---------------------------------------------------------------------------
 struct grp_scale { float scale, unscale; };
 __device__ __forceinline__ grp_scale grp_row_scale(uint32_t max_bits) {
-    uint32_t ex = (max_bits >> 23) & 0xFFu;
-    if (ex == 0u || ex >= 254u) ex = 127u;
-    return grp_scale{__uint_as_float((254u - ex) << 23), __uint_as_float(ex << 23)};
+    uint32_t ex = (max_bits >> 23) & 0xFFu;                    // maximum in [2^(ex - 127), 2^(ex - 126))
+    if (ex == 0u || ex >= 254u) ex = 141u;                     // (no scaling)
+    ex = ex < 15u ? 15u : ex;                                  // keeps both powers of two normal numbers
+    return grp_scale{__uint_as_float((268u - ex) << 23), __uint_as_float((ex - 14u) << 23)};   // 2^(141 - ex), 2^(ex - 141)
 }
 __device__ __forceinline__ void grp_split_run(lev_f32x4 a, lev_f32x4 b, float scale, g_h8 &h, g_h8 &l) {
     typedef float f32x2 __attribute__((ext_vector_type(2)));

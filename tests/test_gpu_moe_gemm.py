@@ -381,6 +381,39 @@ def test_moe_non_finite_activation_stays_in_its_token(ctx, experts, tokens, top_
                 assert np.array_equal(y[t].view(np.uint32), y_good[t].view(np.uint32)), (bad_value, t)
 
 
+@pytest.mark.parametrize("experts,tokens,top_k", [(16, 2, 2), (16, 6, 2), (4, 12, 2)])
+def test_moe_block_scale_edge_cases(ctx, experts, tokens, top_k):
+    """Block scales the synthetic pools do not draw: zero, negative, the smallest fp16 subnormal
+    and a large one, sprinkled over every matrix, and activations spanning forty-six binades within a
+    row; the three schedules (per-pair, integer grouped, fp16 grouped) against the FP64 chain."""
+    hidden, inter = 256, 256
+    wr, pool, offs, x = H.config5(hidden, inter, experts, tokens, seed=311 + tokens)
+    pool = pool.copy()
+    d = np.ascontiguousarray(pool.reshape(-1, 18)[:, 0:2]).view(np.float16).reshape(-1)   # one scale per block
+    n = d.size
+    d[0:n:7] = np.float16(0.0)
+    d[3:n:11] = -d[3:n:11]
+    d[5:n:13] = np.float16(5.96e-8)                                     # 2^-24: the smallest subnormal
+    d[6:n:17] = np.float16(0.0625)
+    pool.reshape(-1, 18)[:, 0:2] = d.view(np.uint8).reshape(-1, 2)
+    x = x.copy()
+    x[:, 0::5] *= np.float32(2.0 ** -40)
+    x[:, 1::9] *= np.float32(2.0 ** 6)
+    rng = np.random.default_rng(311 + tokens)
+    ids = np.stack([rng.permutation(experts)[:top_k] for _ in range(tokens)]).astype(np.int32)
+    wts = rng.random((tokens, top_k)).astype(np.float32)
+    y, act = run_experts(ctx, pool, offs, hidden, inter, experts, x, ids, wts)
+    g, u, dwn = (pool[offs["gate_off"]:], pool[offs["up_off"]:], pool[offs["down_off"]:])
+    for t in range(tokens):
+        ref = O.moe_experts_f64(g, u, dwn, hidden, inter, ids[t], wts[t], x[t])
+        assert np.isfinite(ref["y"]).all()
+        assert O.max_rel_err(act[t], ref["act"]) < TOL
+        # y sums f32 activations of mixed sign and size 1e3: the reference's own f32 chain is off by up
+        # to 5e-4 of small outputs here; the HIP path must stay within the gate or within that chain's error
+        y32, _ = O.moe_experts_f32(g, u, dwn, hidden, inter, ids[t], wts[t], x[t])
+        assert O.max_rel_err(y[t], ref["y"]) <= max(TOL, 1.5 * O.max_rel_err(y32, ref["y"]))
+
+
 def test_moe_grouped_path_rejects_bad_expert_ids(ctx):
     """The same rule on the many-token path: a pair whose id is out of range or repeats another
     slot of its token is dropped (it adds nothing to its token) and reported; the other tokens
