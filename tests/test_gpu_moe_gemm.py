@@ -414,6 +414,26 @@ def test_moe_block_scale_edge_cases(ctx, experts, tokens, top_k):
         assert O.max_rel_err(y[t], ref["y"]) <= max(TOL, 1.5 * O.max_rel_err(y32, ref["y"]))
 
 
+@pytest.mark.parametrize("hidden,inter", [(1280, 512), (1536, 1280), (1792, 256), (768, 1792), (2048, 2048)])
+def test_moe_grouped_integer_kernels_wave_geometries(ctx, hidden, inter):
+    """The integer grouped kernels give a wave one 256-value column task of its row groups: rows of
+    three, five, six, seven and eight tasks, whose workgroups hold five to twelve waves in one to
+    four row-group slots (gate/up over hidden, down over the intermediate size).  Seven tokens over
+    six experts; one expert takes six pairs (a second product), one a single pair."""
+    experts, top_k, tokens = 6, 2, 7
+    wr, pool, offs, x = H.config5(hidden, inter, experts, tokens, seed=hidden + inter)
+    ids = np.array([[0, 1], [0, 2], [0, 3], [0, 4], [0, 1], [0, 2], [5, 3]], dtype=np.int32)
+    rng = np.random.default_rng(hidden + inter)
+    wts = rng.random((tokens, top_k)).astype(np.float32)
+    assert 2 * tokens * top_k <= 11 * experts            # the integer kernels' share of the grouped path
+    y, act = run_experts(ctx, pool, offs, hidden, inter, experts, x, ids, wts)
+    g, u, d = (pool[offs["gate_off"]:], pool[offs["up_off"]:], pool[offs["down_off"]:])
+    for t in range(tokens):
+        ref = O.moe_experts_f64(g, u, d, hidden, inter, ids[t], wts[t], x[t])
+        assert O.max_rel_err(act[t], ref["act"]) < TOL
+        assert O.max_rel_err(y[t], ref["y"]) < TOL
+
+
 def test_moe_grouped_path_rejects_bad_expert_ids(ctx):
     """The same rule on the many-token path: a pair whose id is out of range or repeats another
     slot of its token is dropped (it adds nothing to its token) and reported; the other tokens
