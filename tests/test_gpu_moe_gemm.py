@@ -434,6 +434,34 @@ def test_moe_grouped_integer_kernels_wave_geometries(ctx, hidden, inter):
         assert O.max_rel_err(y[t], ref["y"]) < TOL
 
 
+@pytest.mark.parametrize("experts,top_k,tokens", [(40, 12, 6), (9, 1, 40), (24, 8, 5)])
+def test_moe_grouped_integer_kernels_fused_layout_and_top_k(ctx, experts, top_k, tokens):
+    """The integer grouped kernels on the reference's fused gate|up tensor ([2I, H] per expert: the up
+    rows of an expert lie behind its gate rows, both strides are the fused record's size) and with
+    more and fewer slots per token than eight: twelve (the merge and the duplicate check take the
+    slots in runs of eight), one, and five tokens, the fewest the grouped path takes."""
+    hidden, inter = 512, 256
+    wr, pool, offs, x = H.config5(hidden, inter, experts, tokens, seed=experts + top_k)
+    gu = offs["gate_stride"]
+    g, u, d = (pool[offs["gate_off"]:offs["up_off"]], pool[offs["up_off"]:offs["down_off"]], pool[offs["down_off"]:])
+    fused = np.concatenate([np.concatenate([g[e * gu:(e + 1) * gu], u[e * gu:(e + 1) * gu]]) for e in range(experts)])
+    pool2 = np.concatenate([fused, d])
+    offs2 = dict(gate_off=0, up_off=gu, down_off=fused.size, gate_stride=2 * gu, up_stride=2 * gu,
+                 down_stride=offs["down_stride"])
+    rng = np.random.default_rng(experts + top_k)
+    ids = np.stack([rng.permutation(experts)[:top_k] for _ in range(tokens)]).astype(np.int32)
+    wts = rng.random((tokens, top_k)).astype(np.float32)
+    assert tokens >= 5 and 2 * tokens * top_k <= 11 * experts
+    y, act = run_experts(ctx, pool2, offs2, hidden, inter, experts, x, ids, wts)
+    y_packed, act_packed = run_experts(ctx, pool, offs, hidden, inter, experts, x, ids, wts)
+    assert np.array_equal(y.view(np.uint32), y_packed.view(np.uint32))          # the layout does not show
+    assert np.array_equal(act.view(np.uint32), act_packed.view(np.uint32))
+    for t in range(tokens):
+        ref = O.moe_experts_f64(g, u, d, hidden, inter, ids[t], wts[t], x[t])
+        assert O.max_rel_err(act[t], ref["act"]) < TOL
+        assert O.max_rel_err(y[t], ref["y"]) < TOL
+
+
 def test_moe_grouped_path_rejects_bad_expert_ids(ctx):
     """The same rule on the many-token path: a pair whose id is out of range or repeats another
     slot of its token is dropped (it adds nothing to its token) and reported; the other tokens
