@@ -112,10 +112,12 @@ def test_recorded_step_replays_bit_exact():
     ctx.close()
 
 
-def test_recorded_prefill_like_sequence_replays_bit_exact():
+@pytest.mark.parametrize("experts", [12, 16])
+def test_recorded_prefill_like_sequence_replays_bit_exact(experts):
     """f32 -> f16, the two prefill GEMMs (first use of the kernels happens while recording),
-    grouped MoE over 24 tokens, and a Q4_0 GEMV under a forge selection made before
-    recording: three replays with changed inputs equal the eager results bit for bit."""
+    grouped MoE over 24 tokens (72 pairs: over 12 experts the fp16 grouped kernels, over 16 the
+    integer ones with their work items and start records), and a Q4_0 GEMV under a forge selection
+    made before recording: three replays with changed inputs equal the eager results bit for bit."""
     from leviathan_amd import capi, ops
     stream = torch.cuda.Stream()
     ctx = ops.Context(0, stream=stream)
@@ -126,7 +128,7 @@ def test_recorded_prefill_like_sequence_replays_bit_exact():
             raise RuntimeError(lib.lev_hip_last_error(c).decode())
 
     T, K, R = 24, 512, 200
-    hidden, inter, experts, top_k = 512, 256, 12, 3
+    hidden, inter, top_k = 512, 256, 3
     wk = dev(O.synth_q4_k(11, R * K // 256))
     w6 = dev(O.synth_q6_k(17, R * K // 256))
     w0 = dev(O.synth_q4_0(12, 300 * 2048 // 32))
