@@ -37,6 +37,9 @@
 // activations take 64 KB of LDS).  The waves of a workgroup share 16 weight rows,
 // one superblock column each; their partial sums meet in LDS.
 //
+// Five to eight columns of at most sixteen superblocks: the planes are made once per launch
+// by a small kernel in front (q4k_planes_kernel, below) instead of by every workgroup.
+//
 // A NaN or infinity in a column of x makes every output of that column NaN.
 #include "lev_common.hpp"
 
@@ -111,11 +114,134 @@ struct q4k_lds {
     }
 };
 
+// ---------------------------------------------------------------------------
+// The digit planes made ONCE per launch instead of once per workgroup.
+//
+// Turning a column of activations into digit planes costs a compute unit about a
+// microsecond whoever does it, and in q4_k_mfma_gemv every workgroup does it for every
+// column: at eight columns that is more than half of the kernel's instructions.  For five
+// to eight columns of at most sixteen superblocks q4k_planes_kernel (one workgroup per
+// column) writes the planes to device scratch in the order the matrix cores read them, and
+// the workgroups of q4_k_mfma_gemv<NC, SHORT, true> load the planes of their wave's
+// superblock column straight into registers: no staging, no digit area in LDS, no LDS read
+// per product.  The numbers are the same integers, so the outputs are the same bits.
+//
+// Scratch, for NX groups of four layout columns and SB superblocks:
+//   planes [SB][4 sub-block pairs][NX][64 lanes][16 B]   lane (r, g): A row r (4 * (column % 4) + plane,
+//          plane 0 the highest digit), k-group g, of sub-blocks 2jp (low 8 bytes) and 2jp + 1 (high)
+//   psb    [SB][4 * NX] f64                               2^(e-151) per superblock and column
+//   bad    [4 * NX] u32                                   a NaN or infinity in the column
+// The sum of X per sub-block (for the mins) is not stored: the matrix cores form
+// sum_j m_j * sum_k digit directly, with the min of a sub-block in all of its B bytes.
+// ---------------------------------------------------------------------------
+constexpr int kPThreads = 512;   // one run of 8 activations per thread: in_dim <= 4096
+__host__ __device__ constexpr size_t q4k_planes_bytes(uint32_t sb, uint32_t nx) { return (size_t)sb * nx * 4096u; }
+__host__ __device__ constexpr size_t q4k_planes_total(uint32_t sb, uint32_t nx) {
+    return q4k_planes_bytes(sb, nx) + (size_t)sb * 4u * nx * 8u + 4u * nx * 4u;
+}
+
+// grid (ncol), kPThreads threads; cols % 256 == 0, cols <= 8 * kPThreads; x and gain 16-byte aligned.
+__global__ void __launch_bounds__(kPThreads)
+q4k_planes_kernel(const float *__restrict__ x, const float *__restrict__ gain, float eps, uint8_t *__restrict__ scratch,
+                  uint32_t cols, uint32_t nx, double rcols) {
+    __shared__ double run[kPThreads / 4];
+    __shared__ double s_inv;
+    __shared__ uint32_t s_bad;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t c = blockIdx.x, SB = cols >> 8, subs = cols >> 5, NL = 4u * nx;
+    uint8_t *planes = scratch;
+    double *psb = reinterpret_cast<double *>(scratch + q4k_planes_bytes(SB, nx));
+    uint32_t *bad = reinterpret_cast<uint32_t *>(psb + (size_t)SB * NL);
+    const bool real = tid < (cols >> 3);
+    const uint32_t k8 = real ? tid : 0u;
+    const lev_f32x4 *xp = reinterpret_cast<const lev_f32x4 *>(x + (uint64_t)c * cols) + 2u * k8;
+    lev_f32x4 va = xp[0], vb = xp[1];
+    if (tid == 0u) s_bad = 0u;
+    if (gain) {
+        const lev_f32x4 *gp = reinterpret_cast<const lev_f32x4 *>(gain) + 2u * k8;
+        const lev_f32x4 ga = gp[0], gb = gp[1];
+        // RMSNorm as the reference computes it (rmsnorm, rust/crates/lev-model/src/lib.rs:110-114):
+        // mean square and 1/sqrt in f64, then (f32)(x * inv) * gain; the additions in the order of
+        // q4_k_mfma_gemv (a sub-block's four runs, the sub-blocks lane by lane, the lanes)
+        double ss = (double)va.x * (double)va.x;
+        ss = fma((double)va.y, (double)va.y, ss); ss = fma((double)va.z, (double)va.z, ss);
+        ss = fma((double)va.w, (double)va.w, ss); ss = fma((double)vb.x, (double)vb.x, ss);
+        ss = fma((double)vb.y, (double)vb.y, ss); ss = fma((double)vb.z, (double)vb.z, ss);
+        ss = fma((double)vb.w, (double)vb.w, ss);
+        ss = lev_group_sum_f64<4>(ss);
+        if (real && (k8 & 3u) == 3u) run[k8 >> 2] = ss;
+        lev_barrier_lds();
+        if (wave == 0u) {
+            double tot = 0.0;
+            for (uint32_t k = lane; k < subs; k += 64u) tot += run[k];
+            tot = lev_group_sum_f64<64>(tot);
+            const double a = fma(tot, rcols, (double)eps);
+            double rs = __builtin_amdgcn_rsq(a);
+            rs = rs * fma(-0.5 * a * rs, rs, 1.5);
+            rs = rs * fma(-0.5 * a * rs, rs, 1.5);
+            if (lane == 63u) s_inv = rs;
+        }
+        lev_barrier_lds();
+        const double inv = s_inv;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            va[k] = (float)((double)va[k] * inv) * ga[k];
+            vb[k] = (float)((double)vb[k] * inv) * gb[k];
+        }
+    } else {
+        lev_barrier_lds();   // s_bad is zero before anybody raises it
+    }
+    const float v[8] = {va.x, va.y, va.z, va.w, vb.x, vb.y, vb.z, vb.w};
+    uint32_t mb = 0u;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        const uint32_t bits = __float_as_uint(v[k]) & 0x7FFFFFFFu;
+        mb = bits > mb ? bits : mb;
+    }
+    mb = lev_row16_max_u32(mb);
+    {
+        const uint32_t o = (uint32_t)__builtin_amdgcn_ds_swizzle((int)mb, 0x401F);   // lane ^ 16: the superblock's 32 runs
+        mb = o > mb ? o : mb;
+    }
+    uint32_t ex = mb >> 23;
+    if (real && ex == 255u) atomicOr(&s_bad, 1u);
+    ex = ex < 25u ? 25u : (ex > 254u ? 254u : ex);
+    const float scale = __uint_as_float((278u - ex) << 23);   // 2^(151-ex): |x*scale| < 2^25
+    uint32_t dw[4][2];                                        // dw[3] = highest digit
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        uint32_t Y[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) Y[k] = ((uint32_t)(int)rintf(v[4 * h + k] * scale) + 0x00808080u) ^ 0x00808080u;
+        const uint32_t t0 = __builtin_amdgcn_perm(Y[1], Y[0], 0x05010400u);
+        const uint32_t t1 = __builtin_amdgcn_perm(Y[1], Y[0], 0x07030602u);
+        const uint32_t t2 = __builtin_amdgcn_perm(Y[3], Y[2], 0x05010400u);
+        const uint32_t t3 = __builtin_amdgcn_perm(Y[3], Y[2], 0x07030602u);
+        dw[0][h] = __builtin_amdgcn_perm(t2, t0, 0x05040100u);
+        dw[1][h] = __builtin_amdgcn_perm(t2, t0, 0x07060302u);
+        dw[2][h] = __builtin_amdgcn_perm(t3, t1, 0x05040100u);
+        dw[3][h] = __builtin_amdgcn_perm(t3, t1, 0x07060302u);
+    }
+    if (real) {
+        const uint32_t j = k8 >> 2, kg = k8 & 3u;             // sub-block of the row, k-group
+        const uint32_t sb = j >> 3, jp = (j & 7u) >> 1, half = j & 1u, q = c >> 2;
+        uint8_t *at = planes + ((((size_t)sb * 4u + jp) * nx + q) * 64u + 16u * kg + 4u * (c & 3u)) * 16u + 8u * half;
+#pragma unroll
+        for (int p = 0; p < 4; ++p) *reinterpret_cast<lev_u2 *>(at + 16 * p) = lev_u2{dw[3 - p][0], dw[3 - p][1]};
+        if ((k8 & 31u) == 31u) psb[sb * NL + c] = __hiloint2double((int)((ex + 872u) << 20), 0);   // 2^(ex-151)
+    }
+    lev_barrier_lds();
+    if (tid == 0u) bad[c] = s_bad;
+}
+
 // NC: columns staged (1, 2, 4 or 8; >= ncol).  SHORT: no wave has more than
 // three tasks (every decode-sized matrix); the kernel is then straight-line
 // code, so the wait before each task covers exactly that task's loads and each
 // task is multiplied while the next streams in.
-template <int NC, bool SHORT>
+// PLANES: the digit planes come from q4k_planes_kernel (`x` then points at its scratch; gain
+// and eps are not used): SB <= 16, so a wave has one superblock column and keeps its A
+// operands in registers; LDS holds the partial sums only.
+template <int NC, bool SHORT, bool PLANES = false>
 __global__ void __launch_bounds__(kMThreads)
 q4_k_mfma_gemv(const uint8_t *__restrict__ w, const float *__restrict__ x,
                const float *__restrict__ gain, float eps, float *__restrict__ y, uint32_t cols,
@@ -124,7 +250,7 @@ q4_k_mfma_gemv(const uint8_t *__restrict__ w, const float *__restrict__ x,
     using L = q4k_lds<NX>;
     constexpr uint32_t NL = L::NL;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    const uint32_t SB = cols >> 8, subs = cols >> 5;
+    const uint32_t SB = cols >> 8, subs = PLANES ? 0u : cols >> 5;
     uint8_t *dig = smem;
     double *sxd = reinterpret_cast<double *>(smem + L::dig_bytes(subs));
     double *part = sxd + (size_t)subs * NL;
@@ -165,156 +291,181 @@ q4_k_mfma_gemv(const uint8_t *__restrict__ w, const float *__restrict__ x,
     cursor ci{0u, blockIdx.x, 0u}, cc{0u, blockIdx.x, 0u};
     q4k_regs W0, W1, W2;
 
-    // ---- stage the activations ----
-    // A thread takes runs of 8 consecutive elements (the 8 k-slots one lane
-    // feeds to one MFMA).  Slot q = tid + i*1024: the 32 runs of one superblock
-    // of one column sit in 32 adjacent lanes (q % 32), superblocks of the NC
-    // columns alternate (q / 32 % NC).  The loads are unconditional (clamped) so
-    // that they are in flight together; whole passes beyond the data are skipped.
-    constexpr int CH = 4;                                   // slots per thread: NC*cols/8 <= 4096
-    constexpr uint32_t kLogNC = NC == 8 ? 3u : NC == 4 ? 2u : NC == 2 ? 1u : 0u;
-    const uint32_t total_slots = (cols >> 3) * NC;
-    auto slot_of = [&](uint32_t q, uint32_t &c, uint32_t &k8) {
-        c = (q >> 5) & (NC - 1u);
-        k8 = ((q >> (5u + kLogNC)) << 5) | (q & 31u);
-        return q < total_slots && c < ncol;
-    };
-    lev_f32x4 va[CH], vb[CH];
-    {
-        lev_f32x4 ga[CH], gb[CH];
+    // ---- the planes of this wave's superblock column, from q4k_planes_kernel's scratch ----
+    lev_i4 Areg[4][NX];      // [sub-block pair][group of four columns]: A of sub-blocks 2jp (x, y) and 2jp + 1 (z, w)
+    double pwreg[NX];        // 2^(e-151) of column 4q + g
+    if constexpr (PLANES) {
+        const uint8_t *scratch = reinterpret_cast<const uint8_t *>(x);
+        const uint32_t sbw = wave < SB ? wave : SB - 1u;
+        const double *psb_g = reinterpret_cast<const double *>(scratch + q4k_planes_bytes(SB, NX));
 #pragma unroll
-        for (int i = 0; i < CH; ++i) {
-            if ((uint32_t)i * kMThreads >= total_slots) break;   // workgroup-uniform
-            uint32_t c, k8;
-            if (!slot_of(tid + (uint32_t)i * kMThreads, c, k8)) c = 0u, k8 = 0u;
-            const lev_f32x4 *xp = reinterpret_cast<const lev_f32x4 *>(x + (uint64_t)c * cols) + 2u * k8;
-            va[i] = xp[0];
-            vb[i] = xp[1];
-            const lev_f32x4 *gp = reinterpret_cast<const lev_f32x4 *>(gain ? gain : x) + 2u * k8;
-            ga[i] = gp[0];
-            gb[i] = gp[1];
-        }
-        if (tid < NL) s_bad[tid] = 0u;
-        // RMSNorm as the reference computes it (rmsnorm, rust/crates/lev-model/src/lib.rs:110-114):
-        // mean square and 1/sqrt in f64, then (f32)(x * inv) * gain
-        if (gain) {
+        for (int jp = 0; jp < 4; ++jp)
 #pragma unroll
-            for (int i = 0; i < CH; ++i) {
-                if ((uint32_t)i * kMThreads >= total_slots) break;
-                uint32_t c, k8;
-                const bool real = slot_of(tid + (uint32_t)i * kMThreads, c, k8);
-                const lev_f32x4 a = va[i], b = vb[i];
-                double ss = (double)a.x * (double)a.x;
-                ss = fma((double)a.y, (double)a.y, ss); ss = fma((double)a.z, (double)a.z, ss);
-                ss = fma((double)a.w, (double)a.w, ss); ss = fma((double)b.x, (double)b.x, ss);
-                ss = fma((double)b.y, (double)b.y, ss); ss = fma((double)b.z, (double)b.z, ss);
-                ss = fma((double)b.w, (double)b.w, ss);
-                ss = lev_group_sum_f64<4>(ss);   // the four runs of a sub-block sit in four adjacent lanes
-                if (real && (k8 & 3u) == 3u) run[c * subs + (k8 >> 2)] = ss;
-            }
-        }
-        // every wave of the workgroup has its activations: a CU's memory pipeline is
-        // one queue, and weight loads of early waves would hold up the activation
-        // loads of late ones.  The first weights stream in while the digits are made.
-        lev_barrier_lds();
+            for (int q = 0; q < NX; ++q)
+                Areg[jp][q] = *reinterpret_cast<const lev_i4 *>(
+                    scratch + ((((size_t)sbw * 4u + (uint32_t)jp) * NX + (uint32_t)q) * 64u + lane) * 16u);
+#pragma unroll
+        for (int q = 0; q < NX; ++q) pwreg[q] = psb_g[sbw * NL + 4u * (uint32_t)q + g];
+        if (tid < NL) s_bad[tid] = reinterpret_cast<const uint32_t *>(psb_g + (size_t)SB * NL)[tid];
         issue(ci, W0);
         if constexpr (!SHORT) {
             issue(ci, W1);
             issue(ci, W2);
         }
-        if (gain) {
-            // one wave per column adds the column's sums of squares
-            if (wave < ncol) {
-                double ss = 0.0;
-                for (uint32_t k = lane; k < subs; k += 64u) ss += run[wave * subs + k];
-                ss = lev_group_sum_f64<64>(ss);
-                // 1/sqrt(mean + eps): the hardware estimate and two Newton steps (full f64 accuracy)
-                const double a = fma(ss, rcols, (double)eps);
-                double rs = __builtin_amdgcn_rsq(a);
-                rs = rs * fma(-0.5 * a * rs, rs, 1.5);
-                rs = rs * fma(-0.5 * a * rs, rs, 1.5);
-                if (lane == 63u) s_inv[wave] = rs;
-            }
-            lev_barrier_lds();   // the sums (in the digit area) are dead from here
-#pragma unroll
+        lev_barrier_lds();
+    }
+    if constexpr (!PLANES) {
+        // ---- stage the activations ----
+        // A thread takes runs of 8 consecutive elements (the 8 k-slots one lane
+        // feeds to one MFMA).  Slot q = tid + i*1024: the 32 runs of one superblock
+        // of one column sit in 32 adjacent lanes (q % 32), superblocks of the NC
+        // columns alternate (q / 32 % NC).  The loads are unconditional (clamped) so
+        // that they are in flight together; whole passes beyond the data are skipped.
+        constexpr int CH = 4;                                   // slots per thread: NC*cols/8 <= 4096
+        constexpr uint32_t kLogNC = NC == 8 ? 3u : NC == 4 ? 2u : NC == 2 ? 1u : 0u;
+        const uint32_t total_slots = (cols >> 3) * NC;
+        auto slot_of = [&](uint32_t q, uint32_t &c, uint32_t &k8) {
+            c = (q >> 5) & (NC - 1u);
+            k8 = ((q >> (5u + kLogNC)) << 5) | (q & 31u);
+            return q < total_slots && c < ncol;
+        };
+        lev_f32x4 va[CH], vb[CH];
+        {
+            lev_f32x4 ga[CH], gb[CH];
+    #pragma unroll
             for (int i = 0; i < CH; ++i) {
-                if ((uint32_t)i * kMThreads >= total_slots) break;
+                if ((uint32_t)i * kMThreads >= total_slots) break;   // workgroup-uniform
                 uint32_t c, k8;
-                const bool real = slot_of(tid + (uint32_t)i * kMThreads, c, k8);
-                const double inv = s_inv[real ? c : 0u];
-#pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    va[i][k] = (float)((double)va[i][k] * inv) * ga[i][k];
-                    vb[i][k] = (float)((double)vb[i][k] * inv) * gb[i][k];
+                if (!slot_of(tid + (uint32_t)i * kMThreads, c, k8)) c = 0u, k8 = 0u;
+                const lev_f32x4 *xp = reinterpret_cast<const lev_f32x4 *>(x + (uint64_t)c * cols) + 2u * k8;
+                va[i] = xp[0];
+                vb[i] = xp[1];
+                const lev_f32x4 *gp = reinterpret_cast<const lev_f32x4 *>(gain ? gain : x) + 2u * k8;
+                ga[i] = gp[0];
+                gb[i] = gp[1];
+            }
+            if (tid < NL) s_bad[tid] = 0u;
+            // RMSNorm as the reference computes it (rmsnorm, rust/crates/lev-model/src/lib.rs:110-114):
+            // mean square and 1/sqrt in f64, then (f32)(x * inv) * gain
+            if (gain) {
+    #pragma unroll
+                for (int i = 0; i < CH; ++i) {
+                    if ((uint32_t)i * kMThreads >= total_slots) break;
+                    uint32_t c, k8;
+                    const bool real = slot_of(tid + (uint32_t)i * kMThreads, c, k8);
+                    const lev_f32x4 a = va[i], b = vb[i];
+                    double ss = (double)a.x * (double)a.x;
+                    ss = fma((double)a.y, (double)a.y, ss); ss = fma((double)a.z, (double)a.z, ss);
+                    ss = fma((double)a.w, (double)a.w, ss); ss = fma((double)b.x, (double)b.x, ss);
+                    ss = fma((double)b.y, (double)b.y, ss); ss = fma((double)b.z, (double)b.z, ss);
+                    ss = fma((double)b.w, (double)b.w, ss);
+                    ss = lev_group_sum_f64<4>(ss);   // the four runs of a sub-block sit in four adjacent lanes
+                    if (real && (k8 & 3u) == 3u) run[c * subs + (k8 >> 2)] = ss;
+                }
+            }
+            // every wave of the workgroup has its activations: a CU's memory pipeline is
+            // one queue, and weight loads of early waves would hold up the activation
+            // loads of late ones.  The first weights stream in while the digits are made.
+            lev_barrier_lds();
+            issue(ci, W0);
+            if constexpr (!SHORT) {
+                issue(ci, W1);
+                issue(ci, W2);
+            }
+            if (gain) {
+                // one wave per column adds the column's sums of squares
+                if (wave < ncol) {
+                    double ss = 0.0;
+                    for (uint32_t k = lane; k < subs; k += 64u) ss += run[wave * subs + k];
+                    ss = lev_group_sum_f64<64>(ss);
+                    // 1/sqrt(mean + eps): the hardware estimate and two Newton steps (full f64 accuracy)
+                    const double a = fma(ss, rcols, (double)eps);
+                    double rs = __builtin_amdgcn_rsq(a);
+                    rs = rs * fma(-0.5 * a * rs, rs, 1.5);
+                    rs = rs * fma(-0.5 * a * rs, rs, 1.5);
+                    if (lane == 63u) s_inv[wave] = rs;
+                }
+                lev_barrier_lds();   // the sums (in the digit area) are dead from here
+    #pragma unroll
+                for (int i = 0; i < CH; ++i) {
+                    if ((uint32_t)i * kMThreads >= total_slots) break;
+                    uint32_t c, k8;
+                    const bool real = slot_of(tid + (uint32_t)i * kMThreads, c, k8);
+                    const double inv = s_inv[real ? c : 0u];
+    #pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        va[i][k] = (float)((double)va[i][k] * inv) * ga[i][k];
+                        vb[i][k] = (float)((double)vb[i][k] * inv) * gb[i][k];
+                    }
                 }
             }
         }
-    }
-#pragma unroll
-    for (int i = 0; i < CH; ++i) {
-        if ((uint32_t)i * kMThreads >= total_slots) break;
-        uint32_t c, k8;
-        const bool real = slot_of(tid + (uint32_t)i * kMThreads, c, k8);
-        const lev_f32x4 a = va[i], b = vb[i];
-        const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
-        // largest magnitude of the superblock as an integer: NaN and infinity sort above every number
-        uint32_t mb = 0u;
-#pragma unroll
-        for (int k = 0; k < 8; ++k) {
-            const uint32_t bits = __float_as_uint(v[k]) & 0x7FFFFFFFu;
-            mb = bits > mb ? bits : mb;
+    #pragma unroll
+        for (int i = 0; i < CH; ++i) {
+            if ((uint32_t)i * kMThreads >= total_slots) break;
+            uint32_t c, k8;
+            const bool real = slot_of(tid + (uint32_t)i * kMThreads, c, k8);
+            const lev_f32x4 a = va[i], b = vb[i];
+            const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+            // largest magnitude of the superblock as an integer: NaN and infinity sort above every number
+            uint32_t mb = 0u;
+    #pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const uint32_t bits = __float_as_uint(v[k]) & 0x7FFFFFFFu;
+                mb = bits > mb ? bits : mb;
+            }
+            mb = lev_row16_max_u32(mb);   // all 16 lanes of a row hold the row's maximum
+            {
+                const uint32_t o = (uint32_t)__builtin_amdgcn_ds_swizzle((int)mb, 0x401F);   // lane ^ 16
+                mb = o > mb ? o : mb;
+            }
+            uint32_t ex = mb >> 23;                             // biased exponent: |x| < 2^(ex-126)
+            if (real && ex == 255u) atomicOr(&s_bad[c], 1u);
+            ex = ex < 25u ? 25u : (ex > 254u ? 254u : ex);      // keeps both powers of two normal numbers
+            const float scale = __uint_as_float((278u - ex) << 23);   // 2^(151-ex): |x*scale| < 2^25
+            int sum = 0, X[8];
+    #pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                X[k] = (int)rintf(v[k] * scale);
+                sum += X[k];
+            }
+            // balanced base-256 digits: adding 0x80 to each of the low three bytes carries
+            // into the next digit where a byte exceeds 127, and flipping bit 7 subtracts the
+            // 0x80 again, so the bytes of (X + 0x808080) ^ 0x808080 read as int8 are the
+            // digits.  A 4x4 byte transpose puts digit k of four neighbours into one dword.
+            uint32_t dw[4][2];                                  // dw[3] = highest digit
+    #pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                uint32_t Y[4];
+    #pragma unroll
+                for (int k = 0; k < 4; ++k) Y[k] = ((uint32_t)X[4 * h + k] + 0x00808080u) ^ 0x00808080u;
+                const uint32_t t0 = __builtin_amdgcn_perm(Y[1], Y[0], 0x05010400u);   // a0 b0 a1 b1
+                const uint32_t t1 = __builtin_amdgcn_perm(Y[1], Y[0], 0x07030602u);   // a2 b2 a3 b3
+                const uint32_t t2 = __builtin_amdgcn_perm(Y[3], Y[2], 0x05010400u);   // c0 d0 c1 d1
+                const uint32_t t3 = __builtin_amdgcn_perm(Y[3], Y[2], 0x07030602u);   // c2 d2 c3 d3
+                dw[0][h] = __builtin_amdgcn_perm(t2, t0, 0x05040100u);                // a0 b0 c0 d0
+                dw[1][h] = __builtin_amdgcn_perm(t2, t0, 0x07060302u);
+                dw[2][h] = __builtin_amdgcn_perm(t3, t1, 0x05040100u);
+                dw[3][h] = __builtin_amdgcn_perm(t3, t1, 0x07060302u);
+            }
+            sum += __builtin_amdgcn_update_dpp(0, sum, 0xB1, 0xF, 0xF, true);   // 32 values of at most 2^25
+            sum += __builtin_amdgcn_update_dpp(0, sum, 0x4E, 0xF, 0xF, true);
+            if (real) {
+                const uint32_t j = k8 >> 2, kg = k8 & 3u;       // sub-block, k-group
+                // 16-byte unit u = 8*kg + (A row)/2 of the sub-block's 512 bytes, stored at q4k_unit(u, kg, j)
+                uint8_t *blk = dig + ((size_t)j * NX + (c >> 2)) * 512u;
+                const uint32_t u = 8u * kg + 2u * (c & 3u);
+                *reinterpret_cast<lev_u4 *>(blk + q4k_unit(u, kg, j)) = lev_u4{dw[3][0], dw[3][1], dw[2][0], dw[2][1]};
+                *reinterpret_cast<lev_u4 *>(blk + q4k_unit(u + 1u, kg, j)) = lev_u4{dw[1][0], dw[1][1], dw[0][0], dw[0][1]};
+                if (kg == 3u) sxd[((j >> 3) * NL + c) * 8u + (j & 7u)] = (double)sum;
+                if ((k8 & 31u) == 31u) psb[(j >> 3) * NL + c] = __hiloint2double((int)((ex + 872u) << 20), 0);   // 2^(ex-151)
+            }
         }
-        mb = lev_row16_max_u32(mb);   // all 16 lanes of a row hold the row's maximum
-        {
-            const uint32_t o = (uint32_t)__builtin_amdgcn_ds_swizzle((int)mb, 0x401F);   // lane ^ 16
-            mb = o > mb ? o : mb;
-        }
-        uint32_t ex = mb >> 23;                             // biased exponent: |x| < 2^(ex-126)
-        if (real && ex == 255u) atomicOr(&s_bad[c], 1u);
-        ex = ex < 25u ? 25u : (ex > 254u ? 254u : ex);      // keeps both powers of two normal numbers
-        const float scale = __uint_as_float((278u - ex) << 23);   // 2^(151-ex): |x*scale| < 2^25
-        int sum = 0, X[8];
-#pragma unroll
-        for (int k = 0; k < 8; ++k) {
-            X[k] = (int)rintf(v[k] * scale);
-            sum += X[k];
-        }
-        // balanced base-256 digits: adding 0x80 to each of the low three bytes carries
-        // into the next digit where a byte exceeds 127, and flipping bit 7 subtracts the
-        // 0x80 again, so the bytes of (X + 0x808080) ^ 0x808080 read as int8 are the
-        // digits.  A 4x4 byte transpose puts digit k of four neighbours into one dword.
-        uint32_t dw[4][2];                                  // dw[3] = highest digit
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            uint32_t Y[4];
-#pragma unroll
-            for (int k = 0; k < 4; ++k) Y[k] = ((uint32_t)X[4 * h + k] + 0x00808080u) ^ 0x00808080u;
-            const uint32_t t0 = __builtin_amdgcn_perm(Y[1], Y[0], 0x05010400u);   // a0 b0 a1 b1
-            const uint32_t t1 = __builtin_amdgcn_perm(Y[1], Y[0], 0x07030602u);   // a2 b2 a3 b3
-            const uint32_t t2 = __builtin_amdgcn_perm(Y[3], Y[2], 0x05010400u);   // c0 d0 c1 d1
-            const uint32_t t3 = __builtin_amdgcn_perm(Y[3], Y[2], 0x07030602u);   // c2 d2 c3 d3
-            dw[0][h] = __builtin_amdgcn_perm(t2, t0, 0x05040100u);                // a0 b0 c0 d0
-            dw[1][h] = __builtin_amdgcn_perm(t2, t0, 0x07060302u);
-            dw[2][h] = __builtin_amdgcn_perm(t3, t1, 0x05040100u);
-            dw[3][h] = __builtin_amdgcn_perm(t3, t1, 0x07060302u);
-        }
-        sum += __builtin_amdgcn_update_dpp(0, sum, 0xB1, 0xF, 0xF, true);   // 32 values of at most 2^25
-        sum += __builtin_amdgcn_update_dpp(0, sum, 0x4E, 0xF, 0xF, true);
-        if (real) {
-            const uint32_t j = k8 >> 2, kg = k8 & 3u;       // sub-block, k-group
-            // 16-byte unit u = 8*kg + (A row)/2 of the sub-block's 512 bytes, stored at q4k_unit(u, kg, j)
-            uint8_t *blk = dig + ((size_t)j * NX + (c >> 2)) * 512u;
-            const uint32_t u = 8u * kg + 2u * (c & 3u);
-            *reinterpret_cast<lev_u4 *>(blk + q4k_unit(u, kg, j)) = lev_u4{dw[3][0], dw[3][1], dw[2][0], dw[2][1]};
-            *reinterpret_cast<lev_u4 *>(blk + q4k_unit(u + 1u, kg, j)) = lev_u4{dw[1][0], dw[1][1], dw[0][0], dw[0][1]};
-            if (kg == 3u) sxd[((j >> 3) * NL + c) * 8u + (j & 7u)] = (double)sum;
-            if ((k8 & 31u) == 31u) psb[(j >> 3) * NL + c] = __hiloint2double((int)((ex + 872u) << 20), 0);   // 2^(ex-151)
-        }
-    }
-    // columns of the layout beyond ncol hold no data: the lanes that read them
-    // only feed outputs that are never stored
-    lev_barrier_lds();
+        // columns of the layout beyond ncol hold no data: the lanes that read them
+        // only feed outputs that are never stored
+        lev_barrier_lds();
 
+    }
     // ---- stream the weights ----
     double yacc[NX];
 #pragma unroll
@@ -336,14 +487,20 @@ q4_k_mfma_gemv(const uint8_t *__restrict__ w, const float *__restrict__ x,
         double acc2[NX];
         lev_d2 SX[NX][4];
         double pw[NX];
+        lev_i4 M[NX];            // PLANES: sum_j m_j * (sum of the sub-block's digits), per plane
 #pragma unroll
         for (int q = 0; q < NX; ++q) {
             E[q][0] = E[q][1] = E[q][2] = E[q][3] = 0;
             acc2[q] = 0.0;
-            const uint32_t m = sb * NL + 4u * q + g;
-            pw[q] = psb[m];
+            M[q] = lev_i4{0, 0, 0, 0};
+            if constexpr (PLANES) {
+                pw[q] = pwreg[q];
+            } else {
+                const uint32_t m = sb * NL + 4u * q + g;
+                pw[q] = psb[m];
 #pragma unroll
-            for (int h = 0; h < 4; ++h) SX[q][h] = *reinterpret_cast<const lev_d2 *>(sxd + m * 8u + 2u * h);
+                for (int h = 0; h < 4; ++h) SX[q][h] = *reinterpret_cast<const lev_d2 *>(sxd + m * 8u + 2u * h);
+            }
         }
         // lane (r, g) reads A row r, k-group g: unit 8g + r/2, its low or high 8 bytes
         const uint8_t *ablk = dig + (size_t)sb * 8u * NX * 512u;
@@ -362,7 +519,13 @@ q4_k_mfma_gemv(const uint8_t *__restrict__ w, const float *__restrict__ x,
             const long B = __builtin_bit_cast(long, wv);
 #pragma unroll
             for (int q = 0; q < NX; ++q) {
-                const long A = *reinterpret_cast<const long *>(ablk + ((size_t)j * NX + q) * 512u + (aoff ^ (32u * (j & 1))));
+                long A;
+                if constexpr (PLANES) {
+                    const lev_i4 a4 = Areg[j >> 1][q];
+                    A = __builtin_bit_cast(long, (j & 1) ? lev_u2{(uint32_t)a4.z, (uint32_t)a4.w} : lev_u2{(uint32_t)a4.x, (uint32_t)a4.y});
+                } else {
+                    A = *reinterpret_cast<const long *>(ablk + ((size_t)j * NX + q) * 512u + (aoff ^ (32u * (j & 1))));
+                }
                 const lev_i4 D = __builtin_amdgcn_mfma_i32_16x16x32_i8(A, B, lev_i4{0, 0, 0, 0}, 0, 0, 0);
                 // |D| <= 32*15*128 < 2^16, sc < 2^6: eight of the products fit 32 bits with room
 #pragma unroll
@@ -370,7 +533,21 @@ q4_k_mfma_gemv(const uint8_t *__restrict__ w, const float *__restrict__ x,
                     E[q][p] += __mul24(D[p], sc);
                     asm("" : "+v"(E[q][p]));   // one multiply-add per plane: keeps the sums from being regrouped
                 }
-                acc2[q] = fma(mnd, SX[q][j >> 1][j & 1], acc2[q]);
+                if constexpr (!PLANES) acc2[q] = fma(mnd, SX[q][j >> 1][j & 1], acc2[q]);
+            }
+            if constexpr (PLANES) {
+                if (j & 1) {
+                    // the mins of sub-blocks j - 1 and j in every B byte of their halves of a 64-deep product:
+                    // the sum over the pair of m * (sum of the sub-block's digits), per plane (below 2^21 over
+                    // the superblock)
+                    const uint32_t mw = mn_w[j >> 2];
+                    const uint32_t m0 = __builtin_amdgcn_perm(0u, mw, 0x01010101u * (uint32_t)((j - 1) & 3));
+                    const uint32_t m1 = __builtin_amdgcn_perm(0u, mw, 0x01010101u * (uint32_t)(j & 3));
+                    const lev_i4 Bm = __builtin_bit_cast(lev_i4, lev_u4{m0, m0, m1, m1});
+#pragma unroll
+                    for (int q = 0; q < NX; ++q)
+                        M[q] = __builtin_amdgcn_mfma_i32_16x16x64_i8(Areg[j >> 1][q], Bm, M[q], 0, 0, 0);
+                }
             }
         }
         // a task past the wave's last superblock contributes nothing
@@ -382,6 +559,11 @@ q4_k_mfma_gemv(const uint8_t *__restrict__ w, const float *__restrict__ x,
             const double hi = fma((double)E[q][0], 256.0, (double)E[q][1]);
             const double lo = fma((double)E[q][2], 256.0, (double)E[q][3]);
             const double dot = fma(hi, 65536.0, lo);
+            if constexpr (PLANES) {
+                const double mhi = fma((double)M[q][0], 256.0, (double)M[q][1]);
+                const double mlo = fma((double)M[q][2], 256.0, (double)M[q][3]);
+                acc2[q] = fma(mhi, 65536.0, mlo);
+            }
             yacc[q] = fma(pw[q], fma(d, dot, -dmin * acc2[q]), yacc[q]);
         }
 
@@ -842,6 +1024,46 @@ hipError_t launch_mfma(lev_ctx *ctx, const uint8_t *w, const float *x, const flo
     return launch_mfma_variant<NC, false>(ctx, w, x, gain, eps, y, cols, rows, ncol);
 }
 
+// Five to eight columns of at most sixteen superblocks: the planes once per launch (q4k_planes_kernel), then the
+// products.  Returns hipErrorOutOfMemory when the scratch cannot be had (a program is being recorded and the
+// context's scratch is still too small): the caller then takes the kernel that stages for itself (same bits).
+template <bool SHORT>
+hipError_t launch_planes_variant(lev_ctx *ctx, const uint8_t *w, const uint8_t *scratch, float *y, uint32_t cols,
+                                 uint32_t rows, uint32_t ncol) {
+    constexpr uint32_t NL = 8u, pb = 2u;
+    const size_t lds = (size_t)pb * kMWaves * 16u * NL * 8u + (size_t)(cols >> 8) * NL * 8u + (size_t)NL * 12u;   // 34 KB
+    const uint32_t groups = (rows + 15u) / 16u;
+    const uint32_t blocks = groups < (uint32_t)ctx->num_cus ? groups : (uint32_t)ctx->num_cus;
+    hipLaunchKernelGGL((q4_k_mfma_gemv<8, SHORT, true>), dim3(blocks), dim3(kMThreads), lds, ctx->stream, w,
+                       reinterpret_cast<const float *>(scratch), static_cast<const float *>(nullptr), 0.f, y, cols,
+                       rows, ncol, pb, 0.0);
+    return hipGetLastError();
+}
+
+bool q4k_planes_serves(uint32_t cols, uint32_t ncol) {
+    static const bool off = [] {
+        const char *e = getenv("LEV_Q4K_PLANES");   // LEV_Q4K_PLANES=0: every workgroup stages the planes, for comparison
+        return e && e[0] == '0';
+    }();
+    return !off && ncol > 4u && ncol <= 8u && cols % 256u == 0u && cols != 0u && cols <= 8u * kPThreads &&
+           (cols >> 8) <= (uint32_t)kMWaves;
+}
+
+hipError_t launch_planes(lev_ctx *ctx, const uint8_t *w, const float *x, const float *gain, float eps, float *y,
+                         uint32_t cols, uint32_t rows, uint32_t ncol) {
+    const uint32_t SB = cols >> 8;
+    uint8_t *scratch = static_cast<uint8_t *>(lev_scratch(ctx, q4k_planes_total(SB, 2u)));
+    if (!scratch) return hipErrorOutOfMemory;
+    hipLaunchKernelGGL(q4k_planes_kernel, dim3(ncol), dim3(kPThreads), 0, ctx->stream, x, gain, eps, scratch, cols, 2u,
+                       1.0 / (double)cols);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    const uint32_t groups = (rows + 15u) / 16u;
+    const uint32_t blocks = groups < (uint32_t)ctx->num_cus ? groups : (uint32_t)ctx->num_cus;
+    if ((groups + blocks - 1u) / blocks <= 3u) return launch_planes_variant<true>(ctx, w, scratch, y, cols, rows, ncol);
+    return launch_planes_variant<false>(ctx, w, scratch, y, cols, rows, ncol);
+}
+
 size_t q4k_narrow_lds_bytes(uint32_t cols, uint32_t nc, uint32_t pb) {
     return nc > 1u ? q4k_narrow_lds<2>::total(cols, pb) : q4k_narrow_lds<1>::total(cols, pb);
 }
@@ -922,6 +1144,10 @@ hipError_t lev_q4_k_mfma_gemv_launch(lev_ctx *ctx, const uint8_t *w, const float
     if (ncol <= lev_q4_k_mfma_narrow_cols(ctx, in_dim) && (ncol == 1u || lev_q4_k_mfma_cols(ctx, in_dim) < ncol)) {
         if (ncol > 1) return launch_narrow<2>(ctx, w, x, gain, eps, y, in_dim, rows, ncol);
         return launch_narrow<1>(ctx, w, x, gain, eps, y, in_dim, rows, ncol);
+    }
+    if (q4k_planes_serves(in_dim, ncol)) {
+        const hipError_t e = launch_planes(ctx, w, x, gain, eps, y, in_dim, rows, ncol);
+        if (e != hipErrorOutOfMemory) return e;
     }
     if (ncol > 4) return launch_mfma<8>(ctx, w, x, gain, eps, y, in_dim, rows, ncol);
     if (ncol > 2) return launch_mfma<4>(ctx, w, x, gain, eps, y, in_dim, rows, ncol);

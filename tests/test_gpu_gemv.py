@@ -696,6 +696,40 @@ def test_q4_k_one_column_kernel_shapes(ctx, rows, cols):
     assert np.isnan(q4k_gemv(ctx, w, xb, rows, cols, 1, gain)).all()
 
 
+@pytest.mark.parametrize("rows,cols,ncol", [(50, 4096, 8), (33, 3840, 5), (100, 2048, 7), (11205, 512, 6), (16, 768, 8),
+                                            (4099, 4096, 8), (1, 256, 5)])
+def test_q4_k_five_to_eight_columns_planes_made_once(ctx, rows, cols, ncol):
+    """Five to eight columns of at most sixteen superblocks: one small kernel writes the digit planes of every
+    column, the product kernel's waves keep the planes of their superblock column in registers and the matrix cores
+    form the sum of min * digit sums as well.  Same integers as in the kernels that stage per workgroup: every column
+    is the same bits as through the four-column kernel, scaling x by a power of two scales y by exactly that power,
+    superblocks of very different magnitude keep their own power of two, and a NaN or an infinity stays in its column."""
+    w, x, gain = H.config3(rows, cols, ncol, seed=rows % 83 + cols // 256 + ncol)
+    x = x.copy()
+    x[:, :256] *= 1e-6
+    x[ncol - 1, cols - 256:] *= 2.0 ** -9   # (made smaller only: the error measure is absolute below 1)
+    got = q4k_gemv(ctx, w, x, rows, cols, ncol, gain)
+    xn = H.rmsnorm_rows(x, gain)
+    for c in range(ncol):
+        assert O.max_rel_err(got[c], O.q4_k_matvec_f64(w, rows, cols, xn[c])) < TOL, c
+    first = q4k_gemv(ctx, w, x[:4], rows, cols, 4, gain)
+    rest = q4k_gemv(ctx, w, x[4:], rows, cols, ncol - 4, gain)
+    assert np.array_equal(bits(got[:4]), bits(first)) and np.array_equal(bits(got[4:]), bits(rest))
+    plain = q4k_gemv(ctx, w, x, rows, cols, ncol)
+    for c in range(ncol):
+        assert O.max_rel_err(plain[c], O.q4_k_matvec_f64(w, rows, cols, x[c])) < TOL, c
+    for e in (-47, 38):
+        scaled = q4k_gemv(ctx, w, np.ldexp(x, e).astype(np.float32), rows, cols, ncol)
+        assert np.array_equal(bits(scaled), bits(np.ldexp(plain, e).astype(np.float32))), e
+    for bad in (np.nan, -np.inf):
+        xb = x.copy()
+        xb[ncol - 2, cols - 5] = bad
+        hit = q4k_gemv(ctx, w, xb, rows, cols, ncol)
+        assert np.isnan(hit[ncol - 2]).all(), bad
+        keep = [c for c in range(ncol) if c != ncol - 2]
+        assert np.array_equal(bits(hit[keep]), bits(plain[keep])), bad
+
+
 def test_q4_k_mixed_magnitudes_within_a_row(ctx):
     """Superblocks of very different magnitude in one row: each carries its own power of two."""
     rows, cols = 48, 4096
