@@ -1027,41 +1027,51 @@ hipError_t launch_mfma(lev_ctx *ctx, const uint8_t *w, const float *x, const flo
 // Five to eight columns of at most sixteen superblocks: the planes once per launch (q4k_planes_kernel), then the
 // products.  Returns hipErrorOutOfMemory when the scratch cannot be had (a program is being recorded and the
 // context's scratch is still too small): the caller then takes the kernel that stages for itself (same bits).
-template <bool SHORT>
+template <int NC, bool SHORT>
 hipError_t launch_planes_variant(lev_ctx *ctx, const uint8_t *w, const uint8_t *scratch, float *y, uint32_t cols,
                                  uint32_t rows, uint32_t ncol) {
-    constexpr uint32_t NL = 8u, pb = 2u;
+    constexpr uint32_t NL = NC > 4 ? 8u : 4u, pb = 2u;
     const size_t lds = (size_t)pb * kMWaves * 16u * NL * 8u + (size_t)(cols >> 8) * NL * 8u + (size_t)NL * 12u;   // 34 KB
     const uint32_t groups = (rows + 15u) / 16u;
     const uint32_t blocks = groups < (uint32_t)ctx->num_cus ? groups : (uint32_t)ctx->num_cus;
-    hipLaunchKernelGGL((q4_k_mfma_gemv<8, SHORT, true>), dim3(blocks), dim3(kMThreads), lds, ctx->stream, w,
+    hipLaunchKernelGGL((q4_k_mfma_gemv<NC, SHORT, true>), dim3(blocks), dim3(kMThreads), lds, ctx->stream, w,
                        reinterpret_cast<const float *>(scratch), static_cast<const float *>(nullptr), 0.f, y, cols,
                        rows, ncol, pb, 0.0);
     return hipGetLastError();
 }
 
-bool q4k_planes_serves(uint32_t cols, uint32_t ncol) {
-    static const bool off = [] {
-        const char *e = getenv("LEV_Q4K_PLANES");   // LEV_Q4K_PLANES=0: every workgroup stages the planes, for comparison
-        return e && e[0] == '0';
+// From how many columns the planes are made in front (LEV_Q4K_PLANES: 0 never, 3..8 from that many; built-in 5).
+uint32_t q4k_planes_min_cols() {
+    static const uint32_t v = [] {
+        const char *e = getenv("LEV_Q4K_PLANES");
+        const int n = e ? atoi(e) : 5;
+        return e && e[0] == '0' ? 0xFFFFFFFFu : (uint32_t)(n < 3 ? 3 : n > 8 ? 8 : n);
     }();
-    return !off && ncol > 4u && ncol <= 8u && cols % 256u == 0u && cols != 0u && cols <= 8u * kPThreads &&
+    return v;
+}
+
+bool q4k_planes_serves(uint32_t cols, uint32_t ncol) {
+    return ncol >= q4k_planes_min_cols() && ncol <= 8u && cols % 256u == 0u && cols != 0u && cols <= 8u * kPThreads &&
            (cols >> 8) <= (uint32_t)kMWaves;
 }
 
 hipError_t launch_planes(lev_ctx *ctx, const uint8_t *w, const float *x, const float *gain, float eps, float *y,
                          uint32_t cols, uint32_t rows, uint32_t ncol) {
-    const uint32_t SB = cols >> 8;
-    uint8_t *scratch = static_cast<uint8_t *>(lev_scratch(ctx, q4k_planes_total(SB, 2u)));
+    const uint32_t SB = cols >> 8, nx = ncol > 4u ? 2u : 1u;
+    uint8_t *scratch = static_cast<uint8_t *>(lev_scratch(ctx, q4k_planes_total(SB, nx)));
     if (!scratch) return hipErrorOutOfMemory;
-    hipLaunchKernelGGL(q4k_planes_kernel, dim3(ncol), dim3(kPThreads), 0, ctx->stream, x, gain, eps, scratch, cols, 2u,
+    hipLaunchKernelGGL(q4k_planes_kernel, dim3(ncol), dim3(kPThreads), 0, ctx->stream, x, gain, eps, scratch, cols, nx,
                        1.0 / (double)cols);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     const uint32_t groups = (rows + 15u) / 16u;
     const uint32_t blocks = groups < (uint32_t)ctx->num_cus ? groups : (uint32_t)ctx->num_cus;
-    if ((groups + blocks - 1u) / blocks <= 3u) return launch_planes_variant<true>(ctx, w, scratch, y, cols, rows, ncol);
-    return launch_planes_variant<false>(ctx, w, scratch, y, cols, rows, ncol);
+    const bool few = (groups + blocks - 1u) / blocks <= 3u;
+    if (nx == 2u)
+        return few ? launch_planes_variant<8, true>(ctx, w, scratch, y, cols, rows, ncol)
+                   : launch_planes_variant<8, false>(ctx, w, scratch, y, cols, rows, ncol);
+    return few ? launch_planes_variant<4, true>(ctx, w, scratch, y, cols, rows, ncol)
+               : launch_planes_variant<4, false>(ctx, w, scratch, y, cols, rows, ncol);
 }
 
 size_t q4k_narrow_lds_bytes(uint32_t cols, uint32_t nc, uint32_t pb) {
