@@ -240,6 +240,59 @@ def test_scratch_growth_after_recording_keeps_the_program_valid():
     ctx.close()
 
 
+def test_q4_k_eight_columns_record_with_and_without_scratch():
+    """Five to eight f32 columns of Q4_K make their digit planes in the context's scratch.  Recorded on a context
+    that never ran anything (no scratch yet, and nothing may be allocated while recording) the launch takes the kernel
+    that stages per workgroup; recorded once the scratch exists it takes the planes kernel and the program holds the
+    scratch address, which a later eager call that grows the scratch must not free.  Same bits every way."""
+    from leviathan_amd import ops
+    from tests import helpers as H
+    rows, cols, ncol = 333, 2048, 8
+    w, x, gain = H.config3(rows, cols, ncol, seed=77)
+    results = []
+    for warm in (False, True):
+        stream = torch.cuda.Stream()
+        ctx = ops.Context(0, stream=stream)
+        with torch.cuda.stream(stream):
+            w_d, x_d, g_d = dev(w), dev(x), dev(gain)
+            y = torch.empty(ncol, rows, device="cuda")
+        if warm:
+            ctx.q4_k_gemv_ncol(w_d, x_d, cols, rows, ncol, gain=g_d, y=y)      # sizes the scratch
+            ctx.sync()
+        ctx.program_begin()
+        ctx.q4_k_gemv_ncol(w_d, x_d, cols, rows, ncol, gain=g_d, y=y)
+        prog = ctx.program_end()
+        # an eager call that needs more scratch than the planes while the program is alive
+        hidden, inter, experts, top_k = 512, 256, 16, 4
+        wr, pool, offs, xm = H.config5(hidden, inter, experts, 300, seed=5)
+        pools = ops.Context.moe_pools(dev(pool), hidden, inter, experts, offs["gate_off"], offs["up_off"], offs["down_off"])
+        with torch.cuda.stream(stream):
+            wr_d, xm_d = dev(wr), dev(xm)
+        ym, _, _ = ctx.moe_layer_q4_0(pools, wr_d, xm_d, top_k, 300)
+        ctx.sync()
+        for _ in range(3):
+            with torch.cuda.stream(stream):
+                y.fill_(float("nan"))
+            prog.run()
+            ctx.sync()
+            results.append(y.cpu().numpy().copy())
+            ym2, _, _ = ctx.moe_layer_q4_0(pools, wr_d, xm_d, top_k, 300)      # eager work on the scratch in between
+            ctx.sync()
+            assert torch.equal(ym2, ym)
+        with torch.cuda.stream(stream):
+            y.fill_(float("nan"))
+        ctx.q4_k_gemv_ncol(w_d, x_d, cols, rows, ncol, gain=g_d, y=y)          # eager: the planes kernel
+        ctx.sync()
+        results.append(y.cpu().numpy().copy())
+        prog.destroy()
+        ctx.close()
+    xn = H.rmsnorm_rows(x, gain)
+    for c in range(ncol):
+        assert O.max_rel_err(results[0][c], O.q4_k_matvec_f64(w, rows, cols, xn[c])) < 1e-4, c
+    for r in results[1:]:
+        assert np.array_equal(r.view(np.uint32), results[0].view(np.uint32))
+
+
 def test_q6_k_argmax_records_on_a_fresh_context():
     """The greedy-token epilogue needs no grow-on-demand scratch: a GEMV with argmax can be
     recorded on a context that never ran anything eagerly."""
