@@ -159,7 +159,11 @@ int lev_hip_q6_k_gemv(lev_ctx *ctx, const void *d_w, size_t w_bytes, uint64_t w_
  * q4k.matvec nb columns, lev-forge/src/glsl.rs:157-281) with the RMSNorm of
  * the input fused in front (Builder::norm_quant, gpu.rs:295; rmsnorm,
  * lev-model/src/lib.rs:110-114).  x is [ncol][in_dim], y is [ncol][rows]
- * (y[col*rows + row], glsl.rs:247).  d_gain == NULL skips the norm. */
+ * (y[col*rows + row], glsl.rs:247).  d_gain == NULL skips the norm.
+ * Five to eight columns of in_dim <= 4096 keep ncol*in_dim*4 bytes (+ 1 KB) of
+ * digit planes in the context's scratch between two kernels; while a program is
+ * being recorded and the scratch is still smaller than that, a kernel that needs
+ * none runs instead (same results), so the call never fails for want of scratch. */
 int lev_hip_q4_k_gemv_ncol(lev_ctx *ctx, const void *d_w, size_t w_bytes, uint64_t w_off,
                            const float *d_x, size_t x_count, const float *d_gain, float eps,
                            float *d_y, size_t y_capacity, uint32_t in_dim, uint32_t rows,
