@@ -117,7 +117,8 @@ moe_group_kernel(const int32_t *__restrict__ ids, uint32_t pairs, uint32_t exper
                  uint32_t hidden, _Float16 *__restrict__ xh, _Float16 *__restrict__ xl,
                  uint32_t *__restrict__ xmax, uint32_t *__restrict__ amax, lev_grp_item *items,
                  uint32_t item_pairs, lev_grp_start *__restrict__ starts, uint32_t grid, uint32_t rpi_gu,
-                 uint32_t rpi_dn, uint32_t w1, uint32_t w2) {
+                 uint32_t rpi_dn, uint32_t w1_gu, uint32_t w2_gu, uint32_t w1_dn, uint32_t w2_dn, uint32_t s0_gu,
+                 uint32_t s0_dn) {
     // [experts] counts | cursors | with items: first pair | first item of more than four pairs | first other item
     extern __shared__ int32_t s_cnt[];
     int32_t *s_cur = s_cnt + experts, *s_first = s_cur + experts, *s_big = s_first + experts, *s_small = s_big + experts;
@@ -252,13 +253,24 @@ moe_group_kernel(const int32_t *__restrict__ ids, uint32_t pairs, uint32_t exper
     const uint32_t sid = 1023u - tid;   // (the high threads: the low ones place the first 1024 pairs below)
     if (items && sid < 2u * grid) {
         // Where the workgroups of the two expert kernels start.  A round of an item of more than
-        // four pairs costs w2, any other w1; the line of rounds is cut into stretches of equal
-        // COST.  The items of more than four pairs come first, so a position in cost is a position
-        // in rounds by two divisions (32-bit arithmetic: rounds * w < 2^29, grid <= 2^9).
+        // four pairs costs w2, any other w1, and beginning an item (its header, its activations,
+        // their staging) costs s0 wherever the item begins; the line of items is cut into
+        // stretches of equal COST.  The items of more than four pairs come first, so a position in
+        // cost is a position in rounds by a few divisions (32-bit arithmetic: cost < 2^29,
+        // grid <= 2^9).
         const uint32_t down = sid >= grid ? 1u : 0u, L = sid - down * grid, rpi = down ? rpi_dn : rpi_gu;
-        const uint32_t R2 = n_big * rpi, C2 = R2 * w2;
-        const uint32_t total = C2 + (n_all * rpi - R2) * w1, per = total / grid, rest = total - per * grid;
-        auto rounds_before = [&](uint32_t c) { return c <= C2 ? (c + w2 - 1u) / w2 : R2 + (c - C2 + w1 - 1u) / w1; };
+        const uint32_t w1 = down ? w1_dn : w1_gu, w2 = down ? w2_dn : w2_gu, s0 = down ? s0_dn : s0_gu;
+        const uint32_t I2 = s0 + rpi * w2, I1 = s0 + rpi * w1;       // cost of a whole item
+        const uint32_t R2 = n_big * rpi, C2 = n_big * I2;
+        const uint32_t total = C2 + (n_all - n_big) * I1, per = total / grid, rest = total - per * grid;
+        // rounds that lie wholly or partly before cost position c
+        auto rounds_before = [&](uint32_t c) {
+            const bool big = c <= C2;
+            const uint32_t cc = big ? c : c - C2, I = big ? I2 : I1, w = big ? w2 : w1;
+            const uint32_t item = cc / I, in_item = cc - item * I;
+            const uint32_t r = in_item <= s0 ? 0u : (in_item - s0 + w - 1u) / w;
+            return (big ? 0u : R2) + item * rpi + r;
+        };
         lev_grp_start st;
         st.first_round = rounds_before(per * L + rest * L / grid);
         st.end_round = rounds_before(per * (L + 1u) + rest * (L + 1u) / grid);
@@ -1050,7 +1062,10 @@ hipError_t lev_moe_grouped_launch(lev_ctx *ctx, const lev_moe_grouped_args &a, c
         // what a round of an item of up to four pairs and of a larger one cost, relative to each other
         // (gate/up 52 against 62 us, down 33 against 38 with every item of the one or the other kind;
         // equal weights: 62 + 39 us at 64 tokens, these: 58 + 36.5)
-        const uint32_t w1 = 5u, w2 = 6u;
+        // cost of a round of an item of at most four pairs / of more, and of beginning an item, per kernel
+        // (64 tokens over 128 experts, us a layer: rounds 5:6 and no cost of beginning 106.4; beginning 12 / 6: 104.5;
+        // 30 / 10: 107.2; rounds 1:1 107; 6:5 109)
+        const uint32_t w1 = 5u, w2 = 6u, w1_dn = 5u, w2_dn = 6u, s0_gu = 12u, s0_dn = 6u;
         const size_t lds_group = (size_t)5 * a.experts * 4;
         static size_t lds_group_set = 0;
         if (lds_group > 48 * 1024 && lds_group > lds_group_set) {
@@ -1061,7 +1076,8 @@ hipError_t lev_moe_grouped_launch(lev_ctx *ctx, const lev_moe_grouped_args &a, c
         }
         hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), lds_group, ctx->stream, ids, pairs,
                            a.experts, a.top_k, goff, glist, valid, ctx->d_flag, x, a.hidden, nullptr, nullptr, nullptr,
-                           nullptr, items, (uint32_t)kG8NT, starts, grid, q_gu.rpi, q_dn.rpi, w1, w2);
+                           nullptr, items, (uint32_t)kG8NT, starts, grid, q_gu.rpi, q_dn.rpi, w1, w2, w1_dn, w2_dn,
+                           s0_gu, s0_dn);
         if ((e = hipGetLastError()) != hipSuccess) return e;
         if ((e = g8_launch<2, true, kG8WavesGateUp>(ctx, a, x, items, starts, grid, act)) != hipSuccess) return e;
         // rows of act that belong to dropped pairs are never written and never read
@@ -1072,7 +1088,7 @@ hipError_t lev_moe_grouped_launch(lev_ctx *ctx, const lev_moe_grouped_args &a, c
     }
     hipLaunchKernelGGL(moe_group_kernel, dim3(1 + a.tokens), dim3(1024), (size_t)2 * a.experts * 4,
                        ctx->stream, ids, pairs, a.experts, a.top_k, goff, glist, valid, ctx->d_flag, x,
-                       a.hidden, xh, xl, xmax, amax, nullptr, 0u, nullptr, 0u, 0u, 0u, 0u, 0u);
+                       a.hidden, xh, xl, xmax, amax, nullptr, 0u, nullptr, 0u, 0u, 0u, 0u, 0u, 0u, 0u, 0u, 0u);
     if ((e = hipGetLastError()) != hipSuccess) return e;
 
     static size_t lds_set[2] = {0, 0};
