@@ -590,6 +590,9 @@ constexpr int kG8MaxWpr = 8;                              // waves that share a 
 constexpr int kG8WavesGateUp = 8;                         // 2048 activations: eight column tasks, one slot
 constexpr int kG8WavesDown = 12;                          // 768 activations: three column tasks, four slots (three
                                                           // waves a SIMD; eight waves leave two SIMDs with one)
+constexpr int kG8TilesDown = 1;                          // row groups a wave of the down kernel takes per round (2: rounds twice
+                                                          // as long, the stretches a workgroup gets then differ by more: 106.8
+                                                          // against 104.4 us a layer at 64 tokens)
 constexpr int kG8NT = 8;                                  // tokens per item
 static_assert(kG8NT == 4 || kG8NT == 8, "an item is one or two groups of four tokens");
 constexpr uint32_t kG8Batch = 4;                          // rounds between two barriers of a workgroup (2: 55.4
@@ -985,7 +988,7 @@ bool g8_usable(const lev_ctx *ctx, const lev_moe_grouped_args &a) {
                              ? ctx->props.sharedMemPerBlockOptin
                              : ctx->props.sharedMemPerBlock;
     const size_t lds_group = (size_t)5 * a.experts * 4;
-    const bool fits = g8_lds<2, kG8WavesGateUp>() <= limit && g8_lds<2, kG8WavesDown>() <= limit && lds_group <= limit;
+    const bool fits = g8_lds<2, kG8WavesGateUp>() <= limit && g8_lds<kG8TilesDown, kG8WavesDown>() <= limit && lds_group <= limit;
     // (64 tokens x top-8 over 128 experts, experts only, us: 72 tokens 106 against 119, 88 tokens 117 against 119,
     // 96 tokens 132 against 124)
     return shape && fits && (mode == 1 || 2u * (uint64_t)a.tokens * a.top_k <= 11u * (uint64_t)a.experts);
@@ -1058,14 +1061,14 @@ hipError_t lev_moe_grouped_launch(lev_ctx *ctx, const lev_moe_grouped_args &a, c
         lev_grp_item *items = reinterpret_cast<lev_grp_item *>(s + L.items);
         lev_grp_start *starts = reinterpret_cast<lev_grp_start *>(s + L.starts);
         const uint32_t grid = (uint32_t)ctx->num_cus < kG8MaxGrid ? (uint32_t)ctx->num_cus : kG8MaxGrid;
-        const g8_geometry q_gu = g8_geometry_of<2, true, kG8WavesGateUp>(a), q_dn = g8_geometry_of<2, false, kG8WavesDown>(a);
+        const g8_geometry q_gu = g8_geometry_of<2, true, kG8WavesGateUp>(a), q_dn = g8_geometry_of<kG8TilesDown, false, kG8WavesDown>(a);
         // what a round of an item of up to four pairs and of a larger one cost, relative to each other
         // (gate/up 52 against 62 us, down 33 against 38 with every item of the one or the other kind;
         // equal weights: 62 + 39 us at 64 tokens, these: 58 + 36.5)
         // cost of a round of an item of at most four pairs / of more, and of beginning an item, per kernel
-        // (64 tokens over 128 experts, us a layer: rounds 5:6 and no cost of beginning 106.4; beginning 12 / 6: 104.5;
-        // 30 / 10: 107.2; rounds 1:1 107; 6:5 109)
-        const uint32_t w1 = 5u, w2 = 6u, w1_dn = 5u, w2_dn = 6u, s0_gu = 12u, s0_dn = 6u;
+        // (64 tokens over 128 experts, us a layer on one box: rounds 5:6 and no cost of beginning 106.4, with it
+        // 104.5; beginning 30 / 10: 107.2; rounds 1:1 107; 6:5 109)
+        const uint32_t w1 = 5u, w2 = 6u, w1_dn = 5u, w2_dn = 6u, s0_gu = 12u, s0_dn = 12u;
         const size_t lds_group = (size_t)5 * a.experts * 4;
         static size_t lds_group_set = 0;
         if (lds_group > 48 * 1024 && lds_group > lds_group_set) {
@@ -1081,7 +1084,7 @@ hipError_t lev_moe_grouped_launch(lev_ctx *ctx, const lev_moe_grouped_args &a, c
         if ((e = hipGetLastError()) != hipSuccess) return e;
         if ((e = g8_launch<2, true, kG8WavesGateUp>(ctx, a, x, items, starts, grid, act)) != hipSuccess) return e;
         // rows of act that belong to dropped pairs are never written and never read
-        if ((e = g8_launch<2, false, kG8WavesDown>(ctx, a, act, items, starts + grid, grid, dn)) != hipSuccess) return e;
+        if ((e = g8_launch<kG8TilesDown, false, kG8WavesDown>(ctx, a, act, items, starts + grid, grid, dn)) != hipSuccess) return e;
         hipLaunchKernelGGL(moe_merge_kernel, dim3((a.hidden + 1023) / 1024, a.tokens), dim3(256), 0, ctx->stream, dn,
                            weights, valid, y, a.hidden, a.top_k);
         return hipGetLastError();
