@@ -1065,10 +1065,12 @@ hipError_t lev_moe_grouped_launch(lev_ctx *ctx, const lev_moe_grouped_args &a, c
         // what a round of an item of up to four pairs and of a larger one cost, relative to each other
         // (gate/up 52 against 62 us, down 33 against 38 with every item of the one or the other kind;
         // equal weights: 62 + 39 us at 64 tokens, these: 58 + 36.5)
-        // cost of a round of an item of at most four pairs / of more, and of beginning an item, per kernel
-        // (64 tokens over 128 experts, us a layer on one box: rounds 5:6 and no cost of beginning 106.4, with it
-        // 104.5; beginning 30 / 10: 107.2; rounds 1:1 107; 6:5 109)
-        const uint32_t w1 = 5u, w2 = 6u, w1_dn = 5u, w2_dn = 6u, s0_gu = 12u, s0_dn = 12u;
+        // cost of a round of an item of at most four pairs / of more, and of beginning an item, per kernel.
+        // Measured at 64 tokens over 128 experts, us a layer in alternating runs on one box: no cost of
+        // beginning 106.4, with it 104.5; down rounds 10:12 103.5, 10:14 101.6, 10:16 103.4 (the items of more
+        // than four pairs come first in the line and go to the first XCDs, which finished 8 % after the others
+        // at 5:6); gate/up rounds 10:13 and 10:14 no better than 5:6
+        const uint32_t w1 = 5u, w2 = 6u, w1_dn = 10u, w2_dn = 14u, s0_gu = 12u, s0_dn = 24u;
         const size_t lds_group = (size_t)5 * a.experts * 4;
         static size_t lds_group_set = 0;
         if (lds_group > 48 * 1024 && lds_group > lds_group_set) {
