@@ -43,6 +43,9 @@
 // starts): they cost less per product and more per token, and win while most experts hold no
 // more than a handful of pairs.
 #include "moe_grouped.hpp"
+
+#include <array>
+#include <cstdio>
 #include "q4_0_mfma.hpp"
 
 #include <cstdlib>
@@ -1069,8 +1072,20 @@ hipError_t lev_moe_grouped_launch(lev_ctx *ctx, const lev_moe_grouped_args &a, c
         // Measured at 64 tokens over 128 experts, us a layer in alternating runs on one box: no cost of
         // beginning 106.4, with it 104.5; down rounds 10:12 103.5, 10:14 101.6, 10:16 103.4 (the items of more
         // than four pairs come first in the line and go to the first XCDs, which finished 8 % after the others
-        // at 5:6); gate/up rounds 10:13 and 10:14 no better than 5:6
-        const uint32_t w1 = 5u, w2 = 6u, w1_dn = 10u, w2_dn = 14u, s0_gu = 12u, s0_dn = 24u;
+        // at 5:6); gate/up rounds 10:13 and 10:14 no better than 5:6.  Thirteen settings around these, five
+        // alternating runs each: medians 101.4 to 103.7, these 102.0
+        // (LEV_MOE_CUT="w1,w2,s0,w1,w2,s0", gate/up then down, each 1..64 resp. 0..256: other weights, for measurement)
+        static const std::array<uint32_t, 6> cut = [] {
+            std::array<uint32_t, 6> c = {5u, 6u, 12u, 10u, 14u, 24u};
+            unsigned v[6];
+            const char *e = getenv("LEV_MOE_CUT");
+            if (e && sscanf(e, "%u,%u,%u,%u,%u,%u", &v[0], &v[1], &v[2], &v[3], &v[4], &v[5]) == 6 && v[0] >= 1u &&
+                v[0] <= 64u && v[1] >= 1u && v[1] <= 64u && v[2] <= 256u && v[3] >= 1u && v[3] <= 64u && v[4] >= 1u &&
+                v[4] <= 64u && v[5] <= 256u)
+                for (int i = 0; i < 6; ++i) c[i] = v[i];
+            return c;
+        }();
+        const uint32_t w1 = cut[0], w2 = cut[1], s0_gu = cut[2], w1_dn = cut[3], w2_dn = cut[4], s0_dn = cut[5];
         const size_t lds_group = (size_t)5 * a.experts * 4;
         static size_t lds_group_set = 0;
         if (lds_group > 48 * 1024 && lds_group > lds_group_set) {
